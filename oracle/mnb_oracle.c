@@ -1,0 +1,349 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- CPU oracle for com.microsoft::MatMulNBits.
+ *
+ * A plain-C restatement of the reference's arithmetic contract for the op at
+ * accuracy_level 0.  It is the checker used by tests/, __graft_entry__.smoke()
+ * and the cpu_baseline leg of bench.py.  Nothing in the shipped library or the
+ * Python host package may link, import or call it.
+ *
+ * What each function follows in the reference (onnxruntime 1.30.0):
+ *   layout + dequantisation   onnxruntime/core/mlas/lib/q4_dq.cpp:587-641
+ *                             (BlockwiseQuantizer::dequantize, column-wise blocks)
+ *   default zero point        onnxruntime/core/mlas/lib/q4_dq.cpp:323,634 (kMid = 2^(bits-1))
+ *   zero-point row length     onnxruntime/contrib_ops/cpu/quantization/matmul_nbits_helper.h:33-35
+ *   fp32 op semantics         onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc:940-1065
+ *   fp16 op semantics         onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc:1069-1180
+ *                             (A, scales, bias widened to fp32; fp32 accumulate; one RNE narrowing of Y)
+ *   bias                      onnxruntime/core/mlas/lib/qnbitgemm.cpp:500-524 (added once per output)
+ *   fp16 <-> fp32             onnxruntime/core/mlas/inc/mlas_float16.h:46-86 (round to nearest even,
+ *                             NaN -> 0x7e00, overflow -> Inf); restated here from IEEE-754, not copied
+ *
+ * Parity status of each function (what pins it is in tests/test_oracle_*.py):
+ *   mnbo_f16_to_f32 / mnbo_f32_to_f16   pinned: exhaustive over all 65536 halves and against numpy's
+ *                                       independent float16 conversion on edge + random floats
+ *   mnbo_dequantize_{f32,f16}           pinned: the reference's own 23 op-test vectors (through the matmul),
+ *                                       exhaustive (q, zp) tables against integer arithmetic, unit-vector
+ *                                       recovery, and an independent numpy implementation
+ *   mnbo_matmul_{f32,f16,f64}           pinned: the 23 vectors (exact), integer special cases against
+ *                                       numpy int64 matmul, linearity, fp64 agreement
+ *   mnbo_quantize_*                     see the header comment of that section
+ */
+#include <math.h>
+#include <pthread.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ fp16 */
+
+float mnbo_f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else { /* subnormal: normalise */
+      int e = -1;
+      do {
+        man <<= 1;
+        ++e;
+      } while ((man & 0x400u) == 0);
+      bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ffu) << 13);
+    }
+  } else if (exp == 31) {
+    bits = sign | 0x7f800000u | (man << 13);
+  } else {
+    bits = sign | ((exp + (127 - 15)) << 23) | (man << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+uint16_t mnbo_f32_to_f16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  uint32_t ax = x & 0x7fffffffu;
+  if (ax > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);   /* NaN -> quiet NaN */
+  if (ax >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);  /* >= 65536 (or Inf) -> Inf */
+  int32_t e = (int32_t)(ax >> 23) - 127;
+  uint32_t m = (ax & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+  if (ax < 0x33000000u) return sign;         /* < 2^-25 rounds to zero (2^-25 itself ties to even = 0) */
+  int shift;                                 /* bits to drop from the 24-bit significand */
+  uint32_t base;
+  if (e < -14) { /* result is subnormal: value = m * 2^(e-23); unit = 2^-24 */
+    shift = -e - 1; /* 13 + (-14 - e) */
+    base = 0;
+  } else {
+    shift = 13;
+    base = (uint32_t)(e + 15) << 10;
+    m &= 0x7fffffu;
+  }
+  uint32_t q = m >> shift;
+  uint32_t rem = m & ((1u << shift) - 1u);
+  uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (q & 1u))) ++q;
+  uint32_t r = base + q; /* a carry out of the mantissa correctly bumps the exponent */
+  if (r >= 0x7c00u) r = 0x7c00u;
+  return (uint16_t)(sign | r);
+}
+
+void mnbo_f16_to_f32_buffer(const uint16_t* src, float* dst, size_t n) {
+  for (size_t i = 0; i < n; ++i) dst[i] = mnbo_f16_to_f32(src[i]);
+}
+
+void mnbo_f32_to_f16_buffer(const float* src, uint16_t* dst, size_t n) {
+  for (size_t i = 0; i < n; ++i) dst[i] = mnbo_f32_to_f16(src[i]);
+}
+
+/* ------------------------------------------------------------------ layout */
+
+static inline int64_t k_blocks_of(int64_t K, int64_t bs) { return (K + bs - 1) / bs; }
+static inline int64_t blob_of(int64_t bs, int64_t bits) { return bs * bits / 8; }
+static inline int64_t zp_row_of(int64_t kb, int64_t bits) { return (kb * bits + 7) / 8; }
+
+/* quantised element (n, k): 4-bit packs two per byte, low nibble = even k; 8-bit one per byte */
+static inline int q_at(const uint8_t* B, int64_t n, int64_t k, int64_t kb_count, int64_t bs, int bits) {
+  int64_t kb = k / bs, r = k % bs;
+  const uint8_t* blob = B + (n * kb_count + kb) * blob_of(bs, bits);
+  if (bits == 8) return blob[r];
+  if (bits == 4) return (blob[r >> 1] >> ((r & 1) * 4)) & 0xf;
+  return (blob[r >> 2] >> ((r & 3) * 2)) & 0x3; /* bits == 2 */
+}
+
+/* zero point of block (n, kb): packed like the weights, row length ceil(kb_count*bits/8); absent -> 2^(bits-1) */
+static inline int zp_at(const uint8_t* zp, int64_t n, int64_t kb, int64_t kb_count, int bits) {
+  if (!zp) return 1 << (bits - 1);
+  const uint8_t* row = zp + n * zp_row_of(kb_count, bits);
+  if (bits == 8) return row[kb];
+  if (bits == 4) return (row[kb >> 1] >> ((kb & 1) * 4)) & 0xf;
+  return (row[kb >> 2] >> ((kb & 3) * 2)) & 0x3;
+}
+
+/* ------------------------------------------------------------------ dequantise */
+
+/* dst is column-major [N][K] (stride K): dst[n*K + k] = (q - zp) * scale, one fp32 rounding. */
+void mnbo_dequantize_f32(float* dst, const uint8_t* B, const float* scales, const uint8_t* zp, int64_t N, int64_t K,
+                         int bits, int64_t bs) {
+  int64_t kbc = k_blocks_of(K, bs);
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t k = 0; k < K; ++k) {
+      int64_t kb = k / bs;
+      int d = q_at(B, n, k, kbc, bs, bits) - zp_at(zp, n, kb, kbc, bits);
+      volatile float v = (float)d * scales[n * kbc + kb];
+      dst[n * K + k] = v;
+    }
+}
+
+/* fp16 model: the fp32 product of an integer |d| <= 255 and a widened half is exact; one RNE narrowing. */
+void mnbo_dequantize_f16(uint16_t* dst, const uint8_t* B, const uint16_t* scales, const uint8_t* zp, int64_t N,
+                         int64_t K, int bits, int64_t bs) {
+  int64_t kbc = k_blocks_of(K, bs);
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t k = 0; k < K; ++k) {
+      int64_t kb = k / bs;
+      int d = q_at(B, n, k, kbc, bs, bits) - zp_at(zp, n, kb, kbc, bits);
+      volatile float v = (float)d * mnbo_f16_to_f32(scales[n * kbc + kb]);
+      dst[n * K + k] = mnbo_f32_to_f16(v);
+    }
+}
+
+/* ------------------------------------------------------------------ matmul */
+
+typedef struct {
+  const float* A;
+  const uint8_t* B;
+  const float* scales;
+  const uint8_t* zp;
+  const float* bias;
+  float* Y;
+  double* Y64;
+  double* bound;
+  int64_t M, N, K, bs, lda, ldc;
+  int bits;
+  int64_t n0, n1;
+} mm_job;
+
+/* One output column slice [n0, n1): dequantise the column once, reuse it for every row of A. */
+static void* mm_worker(void* p) {
+  mm_job* j = (mm_job*)p;
+  int64_t kbc = k_blocks_of(j->K, j->bs);
+  float* w = (float*)malloc((size_t)(kbc * j->bs) * sizeof(float));
+  for (int64_t n = j->n0; n < j->n1; ++n) {
+    for (int64_t kb = 0; kb < kbc; ++kb) {
+      int z = zp_at(j->zp, n, kb, kbc, j->bits);
+      float s = j->scales[n * kbc + kb];
+      const uint8_t* blob = j->B + (n * kbc + kb) * blob_of(j->bs, j->bits);
+      float* wb = w + kb * j->bs;
+      if (j->bits == 4) {
+        for (int64_t r = 0; r < j->bs / 2; ++r) {
+          wb[2 * r] = (float)((blob[r] & 0xf) - z) * s;
+          wb[2 * r + 1] = (float)((blob[r] >> 4) - z) * s;
+        }
+      } else if (j->bits == 8) {
+        for (int64_t r = 0; r < j->bs; ++r) wb[r] = (float)(blob[r] - z) * s;
+      } else {
+        for (int64_t r = 0; r < j->bs; ++r) wb[r] = (float)(((blob[r >> 2] >> ((r & 3) * 2)) & 3) - z) * s;
+      }
+    }
+    for (int64_t m = 0; m < j->M; ++m) {
+      const float* a = j->A + m * j->lda;
+      if (j->Y) {
+        float acc = 0.f;
+        for (int64_t k = 0; k < j->K; ++k) acc += a[k] * w[k];
+        if (j->bias) acc += j->bias[n];
+        j->Y[m * j->ldc + n] = acc;
+      }
+      if (j->Y64) {
+        double acc = 0.0, bnd = 0.0;
+        for (int64_t k = 0; k < j->K; ++k) {
+          double t = (double)a[k] * (double)w[k];
+          acc += t;
+          bnd += fabs(t);
+        }
+        if (j->bias) {
+          acc += (double)j->bias[n];
+          bnd += fabs((double)j->bias[n]);
+        }
+        j->Y64[m * j->ldc + n] = acc;
+        if (j->bound) j->bound[m * j->ldc + n] = bnd;
+      }
+    }
+  }
+  free(w);
+  return NULL;
+}
+
+static void mm_run(mm_job base, int nthreads) {
+  if (nthreads < 1) nthreads = 1;
+  if (nthreads > 256) nthreads = 256;
+  if ((int64_t)nthreads > base.N) nthreads = (int)(base.N > 0 ? base.N : 1);
+  pthread_t th[256];
+  mm_job jobs[256];
+  int64_t per = (base.N + nthreads - 1) / nthreads;
+  int started = 0;
+  for (int t = 0; t < nthreads; ++t) {
+    jobs[t] = base;
+    jobs[t].n0 = t * per;
+    jobs[t].n1 = (t + 1) * per < base.N ? (t + 1) * per : base.N;
+    if (jobs[t].n0 >= jobs[t].n1) break;
+    if (nthreads == 1) {
+      mm_worker(&jobs[t]);
+    } else {
+      pthread_create(&th[t], NULL, mm_worker, &jobs[t]);
+      ++started;
+    }
+  }
+  for (int t = 0; t < started; ++t) pthread_join(th[t], NULL);
+}
+
+/* Y[m][n] = sum_k A[m][k] * W[k][n] (+ bias[n]); fp32 accumulation in k order; elements k >= K ignored. */
+void mnbo_matmul_f32(const float* A, const uint8_t* B, const float* scales, const uint8_t* zp, const float* bias,
+                     float* Y, int64_t M, int64_t N, int64_t K, int bits, int64_t bs, int nthreads) {
+  mm_job j = {A, B, scales, zp, bias, Y, NULL, NULL, M, N, K, bs, K, N, bits, 0, N};
+  mm_run(j, nthreads);
+}
+
+/* fp64 accumulation of the same fp32 products, plus the row bound sum_k |a*w| (+|bias|) used by the error gate. */
+void mnbo_matmul_f64(const float* A, const uint8_t* B, const float* scales, const uint8_t* zp, const float* bias,
+                     double* Y64, double* bound, int64_t M, int64_t N, int64_t K, int bits, int64_t bs,
+                     int nthreads) {
+  mm_job j = {A, B, scales, zp, bias, NULL, Y64, bound, M, N, K, bs, K, N, bits, 0, N};
+  mm_run(j, nthreads);
+}
+
+/* fp16 model on the reference's x64 path: widen A/scales/bias, compute in fp32, narrow Y once (RNE). */
+void mnbo_matmul_f16(const uint16_t* A, const uint8_t* B, const uint16_t* scales, const uint8_t* zp,
+                     const uint16_t* bias, uint16_t* Y, int64_t M, int64_t N, int64_t K, int bits, int64_t bs,
+                     int nthreads) {
+  int64_t kbc = k_blocks_of(K, bs);
+  float* a32 = (float*)malloc((size_t)(M * K) * sizeof(float));
+  float* s32 = (float*)malloc((size_t)(N * kbc) * sizeof(float));
+  float* b32 = bias ? (float*)malloc((size_t)N * sizeof(float)) : NULL;
+  float* y32 = (float*)malloc((size_t)(M * N) * sizeof(float));
+  mnbo_f16_to_f32_buffer(A, a32, (size_t)(M * K));
+  mnbo_f16_to_f32_buffer(scales, s32, (size_t)(N * kbc));
+  if (bias) mnbo_f16_to_f32_buffer(bias, b32, (size_t)N);
+  mnbo_matmul_f32(a32, B, s32, zp, b32, y32, M, N, K, bits, bs, nthreads);
+  mnbo_f32_to_f16_buffer(y32, Y, (size_t)(M * N));
+  free(a32);
+  free(s32);
+  free(b32);
+  free(y32);
+}
+
+/* ------------------------------------------------------------------ quantise (producer of the format)
+ *
+ * Follows BlockwiseQuantizer::quantizeAndTranspose with column-wise blocks
+ * (onnxruntime/core/mlas/lib/q4_dq.cpp:468-574) and range2scalezp / range2scale (:347-386):
+ *   asymmetric: min = min(min, 0), max = max(max, 0); scale = (max - min) / (2^bits - 1);
+ *               zp = clamp(round(-min / scale)) (0 when scale is 0); q = clamp(round(v / scale + zp))
+ *   symmetric : s = max if |max| > |min| else min; scale = -s / 2^(bits-1);
+ *               zp = 2^(bits-1); q = clamp(round(v / scale + zp))  (computed with the reciprocal of scale)
+ * src is row-major [K][N].  Rounding is roundf (half away from zero), as in the reference.
+ * Parity: pinned only by round-trip and closed-form properties (tests/test_oracle_quantize.py); tie-breaking
+ * on exact .5 values is "parity unpinned" because the compiled reference is not available in this build.
+ */
+void mnbo_quantize_f32(uint8_t* B, float* scales, uint8_t* zp, const float* src, int64_t K, int64_t N, int bits,
+                       int64_t bs, int symmetric) {
+  int64_t kbc = k_blocks_of(K, bs);
+  int64_t blob = blob_of(bs, bits);
+  int64_t zrow = zp_row_of(kbc, bits);
+  const int maxq = (1 << bits) - 1;
+  const int mid = 1 << (bits - 1);
+  memset(B, 0, (size_t)(N * kbc * blob));
+  if (zp) memset(zp, 0, (size_t)(N * zrow));
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t kb = 0; kb < kbc; ++kb) {
+      int64_t k0 = kb * bs, k1 = k0 + bs < K ? k0 + bs : K;
+      float scale, rscale;
+      int z;
+      if (!symmetric) {
+        float mn = 0.f, mx = 0.f;
+        for (int64_t k = k0; k < k1; ++k) {
+          float v = src[k * N + n];
+          if (v < mn) mn = v;
+          if (v > mx) mx = v;
+        }
+        scale = (mx - mn) / (float)maxq;
+        float zf = scale == 0.f ? mn : -mn / scale;
+        if (zf < 0.f) zf = 0.f;
+        if (zf > (float)maxq) zf = (float)maxq;
+        z = (int)roundf(zf);
+        rscale = scale == 0.f ? 0.f : 1.f / scale;
+      } else {
+        float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+        for (int64_t k = k0; k < k1; ++k) {
+          float v = src[k * N + n];
+          if (v < mn) mn = v;
+          if (v > mx) mx = v;
+        }
+        float smax = fabsf(mx) > fabsf(mn) ? mx : mn; /* the larger half maps to [-2^(bits-1), 0] */
+        scale = -smax / (float)mid;
+        rscale = scale == 0.f ? 0.f : 1.f / scale;
+        z = mid;
+      }
+      scales[n * kbc + kb] = scale;
+      if (zp) {
+        uint8_t* row = zp + n * zrow;
+        if (bits == 8) row[kb] = (uint8_t)z;
+        else if (bits == 4) row[kb >> 1] |= (uint8_t)(z << ((kb & 1) * 4));
+        else row[kb >> 2] |= (uint8_t)(z << ((kb & 3) * 2));
+      }
+      uint8_t* out = B + (n * kbc + kb) * blob;
+      for (int64_t k = k0; k < k0 + bs; ++k) {
+        float v = k < k1 ? src[k * N + n] : 0.f;
+        float qf = roundf(v * rscale + (float)z);
+        if (qf < 0.f) qf = 0.f;
+        if (qf > (float)maxq) qf = (float)maxq;
+        int q = k < k1 ? (int)qf : z; /* padding dequantises to 0 */
+        int64_t r = k - k0;
+        if (bits == 8) out[r] = (uint8_t)q;
+        else if (bits == 4) out[r >> 1] |= (uint8_t)(q << ((r & 1) * 4));
+        else out[r >> 2] |= (uint8_t)(q << ((r & 3) * 2));
+      }
+    }
+}

@@ -1,0 +1,224 @@
+"""TEST INFRASTRUCTURE ONLY -- Python face of the CPU oracle for MatMulNBits.
+
+Two independent restatements of the reference's arithmetic contract live here:
+
+* ``C``: ctypes bindings of ``libmnb_oracle.so`` (``mnb_oracle.c``), used for full-size checks and as the
+  ``cpu_baseline`` of ``bench.py``;
+* ``np_*``: a vectorised numpy restatement written separately from the C code, so that the two can be
+  checked against each other and against the reference's own test vectors.
+
+Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this module.
+The product (``onnxruntime_amd``) never does.
+
+Reference definitions followed (onnxruntime 1.30.0):
+  canonical layout + ``(q - zp) * scale``      onnxruntime/core/mlas/lib/q4_dq.cpp:587-641
+  operator contract (shapes, optional inputs)   onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3782-3849
+  zero-point packing                            onnxruntime/contrib_ops/cpu/quantization/matmul_nbits_helper.h:33-35
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_HERE = Path(__file__).resolve().parent
+_LIB_PATH = _HERE / "libmnb_oracle.so"
+
+
+def build(force: bool = False) -> Path:
+    """Compile the C oracle (gcc, a second or two)."""
+    if force or not _LIB_PATH.exists() or _LIB_PATH.stat().st_mtime < (_HERE / "mnb_oracle.c").stat().st_mtime:
+        subprocess.check_call(["make", "-C", str(_HERE), "-B" if force else "-s", "libmnb_oracle.so"])
+    return _LIB_PATH
+
+
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+
+def _ptr(a, typ):
+    if a is None:
+        return ctypes.cast(None, typ)
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(typ)
+
+
+class _C:
+    """Lazy ctypes handle of the C oracle."""
+
+    def __init__(self):
+        self._lib = None
+
+    @property
+    def lib(self):
+        if self._lib is None:
+            if not _LIB_PATH.exists():
+                build()
+            lib = ctypes.CDLL(str(_LIB_PATH))
+            lib.mnbo_f16_to_f32.restype = ctypes.c_float
+            lib.mnbo_f16_to_f32.argtypes = [ctypes.c_uint16]
+            lib.mnbo_f32_to_f16.restype = ctypes.c_uint16
+            lib.mnbo_f32_to_f16.argtypes = [ctypes.c_float]
+            lib.mnbo_f16_to_f32_buffer.argtypes = [_u16p, _f32p, ctypes.c_size_t]
+            lib.mnbo_f32_to_f16_buffer.argtypes = [_f32p, _u16p, ctypes.c_size_t]
+            lib.mnbo_dequantize_f32.argtypes = [_f32p, _u8p, _f32p, _u8p, _i64, _i64, _int, _i64]
+            lib.mnbo_dequantize_f16.argtypes = [_u16p, _u8p, _u16p, _u8p, _i64, _i64, _int, _i64]
+            lib.mnbo_matmul_f32.argtypes = [_f32p, _u8p, _f32p, _u8p, _f32p, _f32p, _i64, _i64, _i64, _int, _i64, _int]
+            lib.mnbo_matmul_f64.argtypes = [_f32p, _u8p, _f32p, _u8p, _f32p, _f64p, _f64p, _i64, _i64, _i64, _int,
+                                            _i64, _int]
+            lib.mnbo_matmul_f16.argtypes = [_u16p, _u8p, _u16p, _u8p, _u16p, _u16p, _i64, _i64, _i64, _int, _i64, _int]
+            lib.mnbo_quantize_f32.argtypes = [_u8p, _f32p, _u8p, _f32p, _i64, _i64, _int, _i64, _int]
+            for f in (lib.mnbo_f16_to_f32_buffer, lib.mnbo_f32_to_f16_buffer, lib.mnbo_dequantize_f32,
+                      lib.mnbo_dequantize_f16, lib.mnbo_matmul_f32, lib.mnbo_matmul_f64, lib.mnbo_matmul_f16,
+                      lib.mnbo_quantize_f32):
+                f.restype = None
+            self._lib = lib
+        return self._lib
+
+    # -- fp16 -----------------------------------------------------------------
+    def f16_to_f32(self, h: np.ndarray) -> np.ndarray:
+        h = np.ascontiguousarray(h).view(np.uint16)
+        out = np.empty(h.shape, np.float32)
+        self.lib.mnbo_f16_to_f32_buffer(_ptr(h, _u16p), _ptr(out, _f32p), h.size)
+        return out
+
+    def f32_to_f16(self, f: np.ndarray) -> np.ndarray:
+        f = np.ascontiguousarray(f, np.float32)
+        out = np.empty(f.shape, np.uint16)
+        self.lib.mnbo_f32_to_f16_buffer(_ptr(f, _f32p), _ptr(out, _u16p), f.size)
+        return out.view(np.float16)
+
+    # -- dequantise -----------------------------------------------------------
+    def dequantize(self, B, scales, zp, N, K, bits, bs) -> np.ndarray:
+        """Returns W as [N, K] in the dtype of ``scales`` (the reference's column-major output)."""
+        B = np.ascontiguousarray(B, np.uint8)
+        zp = None if zp is None else np.ascontiguousarray(zp, np.uint8)
+        if scales.dtype == np.float16:
+            s = np.ascontiguousarray(scales).view(np.uint16)
+            out = np.empty((N, K), np.uint16)
+            self.lib.mnbo_dequantize_f16(_ptr(out, _u16p), _ptr(B, _u8p), _ptr(s, _u16p), _ptr(zp, _u8p), N, K, bits,
+                                         bs)
+            return out.view(np.float16)
+        s = np.ascontiguousarray(scales, np.float32)
+        out = np.empty((N, K), np.float32)
+        self.lib.mnbo_dequantize_f32(_ptr(out, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), N, K, bits, bs)
+        return out
+
+    # -- matmul ---------------------------------------------------------------
+    def matmul(self, A, B, scales, zp, bias, N, K, bits, bs, nthreads=1) -> np.ndarray:
+        """Y = A x dequant(B)^T (+ bias) with the reference's CPU semantics for the dtype of A."""
+        lead = A.shape[:-1]
+        M = int(np.prod(lead)) if lead else 1
+        B = np.ascontiguousarray(B, np.uint8)
+        zp = None if zp is None else np.ascontiguousarray(zp, np.uint8)
+        if A.dtype == np.float16:
+            a = np.ascontiguousarray(A).view(np.uint16)
+            s = np.ascontiguousarray(scales, np.float16).view(np.uint16)
+            b = None if bias is None else np.ascontiguousarray(bias, np.float16).view(np.uint16)
+            y = np.empty((M, N), np.uint16)
+            self.lib.mnbo_matmul_f16(_ptr(a, _u16p), _ptr(B, _u8p), _ptr(s, _u16p), _ptr(zp, _u8p), _ptr(b, _u16p),
+                                     _ptr(y, _u16p), M, N, K, bits, bs, nthreads)
+            return y.view(np.float16).reshape(*lead, N)
+        a = np.ascontiguousarray(A, np.float32)
+        s = np.ascontiguousarray(scales, np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+        y = np.empty((M, N), np.float32)
+        self.lib.mnbo_matmul_f32(_ptr(a, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), _ptr(b, _f32p),
+                                 _ptr(y, _f32p), M, N, K, bits, bs, nthreads)
+        return y.reshape(*lead, N)
+
+    def matmul_f64(self, A, B, scales, zp, bias, N, K, bits, bs, nthreads=1):
+        """fp64 accumulation of the fp32 products and the row bound sum_k |a*w| (+|bias|).
+
+        fp16 inputs are widened exactly first, as the reference does."""
+        lead = A.shape[:-1]
+        M = int(np.prod(lead)) if lead else 1
+        a = np.ascontiguousarray(A.astype(np.float32))
+        s = np.ascontiguousarray(scales.astype(np.float32))
+        b = None if bias is None else np.ascontiguousarray(bias.astype(np.float32))
+        B = np.ascontiguousarray(B, np.uint8)
+        zp = None if zp is None else np.ascontiguousarray(zp, np.uint8)
+        y = np.empty((M, N), np.float64)
+        bound = np.empty((M, N), np.float64)
+        self.lib.mnbo_matmul_f64(_ptr(a, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), _ptr(b, _f32p),
+                                 _ptr(y, _f64p), _ptr(bound, _f64p), M, N, K, bits, bs, nthreads)
+        return y.reshape(*lead, N), bound.reshape(*lead, N)
+
+    # -- quantise -------------------------------------------------------------
+    def quantize(self, W, bits, bs, symmetric):
+        """W is [K, N] fp32 row-major. Returns (B[N,kb,blob], scales[N,kb], zp[N,zrow] or None)."""
+        W = np.ascontiguousarray(W, np.float32)
+        K, N = W.shape
+        kb = (K + bs - 1) // bs
+        Bq = np.empty((N, kb, bs * bits // 8), np.uint8)
+        sc = np.empty((N, kb), np.float32)
+        zp = None if symmetric else np.empty((N, (kb * bits + 7) // 8), np.uint8)
+        self.lib.mnbo_quantize_f32(_ptr(Bq, _u8p), _ptr(sc, _f32p), _ptr(zp, _u8p), _ptr(W, _f32p), K, N, bits, bs,
+                                   1 if symmetric else 0)
+        return Bq, sc, zp
+
+
+C = _C()
+
+
+# ----------------------------------------------------------------------------- numpy restatement
+
+def np_unpack_q(B: np.ndarray, N: int, K: int, bits: int, bs: int) -> np.ndarray:
+    """Quantised integers as int32 [N, k_blocks*bs] from canonical B [N, k_blocks, bs*bits/8]."""
+    kb = (K + bs - 1) // bs
+    b = np.asarray(B, np.uint8).reshape(N, kb, bs * bits // 8).astype(np.int32)
+    if bits == 8:
+        q = b
+    elif bits == 4:
+        q = np.stack([b & 0xF, b >> 4], axis=-1).reshape(N, kb, bs)
+    elif bits == 2:
+        q = np.stack([b & 3, (b >> 2) & 3, (b >> 4) & 3, b >> 6], axis=-1).reshape(N, kb, bs)
+    else:
+        raise ValueError(bits)
+    return q.reshape(N, kb * bs)
+
+
+def np_unpack_zp(zp, N: int, K: int, bits: int, bs: int) -> np.ndarray:
+    """Zero points as int32 [N, k_blocks]; ``None`` means the default 2^(bits-1)."""
+    kb = (K + bs - 1) // bs
+    if zp is None:
+        return np.full((N, kb), 1 << (bits - 1), np.int32)
+    row = (kb * bits + 7) // 8
+    z = np.asarray(zp, np.uint8).reshape(N, row).astype(np.int32)
+    if bits == 8:
+        return z[:, :kb]
+    if bits == 4:
+        return np.stack([z & 0xF, z >> 4], axis=-1).reshape(N, row * 2)[:, :kb]
+    return np.stack([z & 3, (z >> 2) & 3, (z >> 4) & 3, z >> 6], axis=-1).reshape(N, row * 4)[:, :kb]
+
+
+def np_dequantize(B, scales, zp, N, K, bits, bs) -> np.ndarray:
+    """W [N, K] in the dtype of ``scales``: fp32 -> one fp32 multiply; fp16 -> RNE of the exact fp32 product."""
+    kb = (K + bs - 1) // bs
+    q = np_unpack_q(B, N, K, bits, bs).reshape(N, kb, bs)
+    z = np_unpack_zp(zp, N, K, bits, bs)[:, :, None]
+    s = np.asarray(scales).reshape(N, kb)
+    d = (q - z).astype(np.float32)
+    w = d * s.astype(np.float32)[:, :, None]
+    return w.reshape(N, kb * bs)[:, :K].astype(s.dtype if s.dtype == np.float16 else np.float32)
+
+
+def np_matmul_f64(A, B, scales, zp, bias, N, K, bits, bs) -> np.ndarray:
+    """fp64 matmul over the exactly-widened dequantised weights (kept in fp32 precision, not rounded to fp16)."""
+    kb = (K + bs - 1) // bs
+    q = np_unpack_q(B, N, K, bits, bs).reshape(N, kb, bs)
+    z = np_unpack_zp(zp, N, K, bits, bs)[:, :, None]
+    s = np.asarray(scales).reshape(N, kb).astype(np.float32)
+    w = ((q - z).astype(np.float32) * s[:, :, None]).reshape(N, kb * bs)[:, :K].astype(np.float64)
+    lead = A.shape[:-1]
+    y = A.reshape(-1, K).astype(np.float64) @ w.T
+    if bias is not None:
+        y = y + np.asarray(bias).astype(np.float64)[None, :]
+    return y.reshape(*lead, N)
