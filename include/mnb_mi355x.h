@@ -1,0 +1,139 @@
+/*
+ * mnb_mi355x.h -- C ABI of libmnb_mi355x.so: com.microsoft::MatMulNBits for AMD Instinct MI355X (gfx950).
+ *
+ * The library is the device-side replacement of the routines the reference CPU kernel
+ * (onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc) calls in MLAS.  Every entry point takes plain
+ * pointers and sizes; pointers named *_dev are HIP device pointers on the current device, `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream).  All functions are asynchronous with respect to the
+ * host unless stated otherwise, return 0 on success or an MnbStatus code, and leave a message retrievable with
+ * MnbGetLastErrorMessage() (thread local) on failure.  No function throws.
+ *
+ * Canonical (on-disk) operand layout, as defined by the operator schema
+ * (onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3782-3849):
+ *   k_blocks = ceil(K / block_size)
+ *   B           u8 [N][k_blocks][block_size*bits/8]   4-bit: low nibble = even k;  8-bit: one byte per element
+ *   scales      T  [N][k_blocks]                       T = fp32 or fp16, same as A
+ *   zero_points u8 [N][ceil(k_blocks*bits/8)]          packed like B; absent -> 2^(bits-1)
+ *   bias        T  [N]
+ *   W[k][n] = (q - zp) * scale;  Y[m][n] = sum_k A[m][k] * W[k][n] (+ bias[n]);  k >= K is ignored.
+ */
+#ifndef MNB_MI355X_H_
+#define MNB_MI355X_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MNB_API __attribute__((visibility("default")))
+
+/* Status codes; numeric values are those of OrtErrorCode
+ * (include/onnxruntime/core/session/onnxruntime_error_code.h) so a caller inside an execution provider can
+ * forward them to OrtApi::CreateStatus unchanged. */
+typedef enum MnbStatus {
+  MNB_OK = 0,
+  MNB_FAIL = 1,
+  MNB_INVALID_ARGUMENT = 2,
+  MNB_NOT_IMPLEMENTED = 9,
+  MNB_EP_FAIL = 11
+} MnbStatus;
+
+/* Element types; numeric values are those of ONNXTensorElementDataType
+ * (include/onnxruntime/core/session/onnxruntime_c_api.h:195-222). */
+typedef enum MnbDataType {
+  MNB_DTYPE_FLOAT = 1,
+  MNB_DTYPE_UINT8 = 2,
+  MNB_DTYPE_INT32 = 6,
+  MNB_DTYPE_FLOAT16 = 10
+} MnbDataType;
+
+/* Shape of one operator input for MnbCheckInputs; dims == NULL means the optional input is absent. */
+typedef struct MnbTensorInfo {
+  const int64_t* dims;
+  size_t rank;
+  int dtype; /* MnbDataType */
+} MnbTensorInfo;
+
+/* Message of the last failure on the calling thread ("" if none). The pointer stays valid until the next
+ * failing call on the same thread. */
+MNB_API const char* MnbGetLastErrorMessage(void);
+
+/* Library ABI version (bumped when a signature or the packed layout changes). */
+MNB_API int MnbGetVersion(void);
+
+/* Number of usable gfx950 devices seen by HIP, or 0. Never fails. */
+MNB_API int MnbGetDeviceCount(void);
+
+/* Replaces MlasIsQNBitGemmAvailable (onnxruntime/core/mlas/inc/mlas_qnbit.h:134-139).
+ * 1 if (bits, block_size, a_dtype) has a device kernel: bits in {4, 8}, block_size in {16,32,64,128,256},
+ * a_dtype in {MNB_DTYPE_FLOAT, MNB_DTYPE_FLOAT16}; else 0. */
+MNB_API int MnbIsAvailable(int bits, int block_size, int a_dtype);
+
+/* Replaces matmul_nbits_helper::CheckInputs
+ * (onnxruntime/contrib_ops/cpu/quantization/matmul_nbits_helper.h:38-109): validates the shapes of the
+ * operator inputs against the attributes, with the same messages. quantized_weight may be absent (already
+ * packed). group_index values are not inspected (they live on the device). */
+MNB_API int MnbCheckInputs(const MnbTensorInfo* quantized_weight, const MnbTensorInfo* scales,
+                           const MnbTensorInfo* zero_points, const MnbTensorInfo* group_index,
+                           const MnbTensorInfo* bias, int64_t n, int64_t k, int64_t block_size, int64_t bits);
+
+/* Replaces MlasQNBitGemmPackQuantBDataSize (mlas_qnbit.h:206-215): bytes of the packed buffer that holds
+ * weights, scales and zero points of one [N, K] matrix in the gfx950 tiled layout; 0 if unsupported.
+ * has_zero_points: 1 if the operator has a zero_points input (the packed meta then carries them). */
+MNB_API size_t MnbPackQuantBDataSize(size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype);
+
+/* Replaces MlasQNBitGemmPackQuantBData (mlas_qnbit.h:244-258): repacks canonical B, scales and zero points
+ * (all on the device) into packed_dev (MnbPackQuantBDataSize bytes, 256-byte aligned). zero_points_dev may be
+ * NULL (default zero point; has_zero_points = 0 everywhere else). The inputs may be freed once the stream has run
+ * the call. */
+MNB_API int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype, const void* b_dev,
+                              const void* scales_dev, const void* zero_points_dev, void* packed_dev, void* stream);
+
+/* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call scratch MnbGemm can use for
+ * this problem (split-K partial sums of the GEMV); may be 0. */
+MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                                    int a_dtype);
+
+/* Replaces MlasQNBitGemmBatch at SQNBIT_CompFp32 (mlas_qnbit.h:111-125) for one B matrix:
+ *   C[M][N] (ldc) = A[M][K] (lda) x dequant(packed)^T (+ bias[N]).
+ * a_dev, bias_dev (optional) and c_dev have element type a_dtype; lda and ldc count elements. M <= 16 runs the
+ * dequantising GEMV, larger M the LDS-staged MFMA GEMM (fp16) or the fp32 tile kernel. M == 0 or N == 0 is a
+ * no-op. workspace_dev (optional, MnbGemmWorkspaceSize bytes, 256-byte aligned) must not be shared by calls that
+ * may overlap; without it the GEMV does not split K over workgroups (same result up to summation order). */
+MNB_API int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                    const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev,
+                    size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* Workspace bytes MnbGemmUnpacked needs (packed copy + MnbGemmWorkspaceSize). */
+MNB_API size_t MnbGemmUnpackedWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size,
+                                            int has_zero_points, int a_dtype);
+
+/* The Compute path when the weights were not packed at session initialisation (session.disable_prepacking, or B
+ * not a constant initializer): counterpart of MatMulNBits<T1>::ComputeBUnpacked
+ * (onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc:1184-1333). Packs into workspace_dev on the stream,
+ * then runs MnbGemm. */
+MNB_API int MnbGemmUnpacked(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, const void* a_dev,
+                            size_t lda, const void* b_dev, const void* scales_dev, const void* zero_points_dev,
+                            const void* bias_dev, void* c_dev, size_t ldc, void* workspace_dev,
+                            size_t workspace_bytes, void* stream);
+
+/* Replaces MlasDequantizeBlockwise<T, bits> with column-wise blocks (onnxruntime/core/mlas/inc/mlas_q4.h:352-362,
+ * definition onnxruntime/core/mlas/lib/q4_dq.cpp:587-641): dst_dev[n*K + k] = (q - zp) * scale in a_dtype.
+ * fp32: one multiply; fp16: round-to-nearest-even of the exact product. */
+MNB_API int MnbDequantizeBlockwise(void* dst_dev, const void* b_dev, const void* scales_dev,
+                                   const void* zero_points_dev, int block_size, int bits, size_t K, size_t N,
+                                   int a_dtype, void* stream);
+
+/* Same output as MnbDequantizeBlockwise, read back from a packed buffer: proves that packing loses nothing. */
+MNB_API int MnbDequantizePacked(void* dst_dev, const void* packed_dev, size_t N, size_t K, int bits, int block_size,
+                                int has_zero_points, int a_dtype, void* stream);
+
+/* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
+MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MNB_MI355X_H_ */

@@ -1,0 +1,78 @@
+"""ctypes binding of libmnb_mi355x.so -- the only way this package reaches the device kernels.
+
+There is no fallback: if the shared library is missing or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_int, c_int64, c_size_t, c_void_p, c_char_p
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libmnb_mi355x.so"
+
+DTYPE_FLOAT = 1
+DTYPE_UINT8 = 2
+DTYPE_INT32 = 6
+DTYPE_FLOAT16 = 10
+
+OK, FAIL, INVALID_ARGUMENT, NOT_IMPLEMENTED, EP_FAIL = 0, 1, 2, 9, 11
+
+
+class MnbError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(message)
+        self.code = code
+
+
+class MnbTensorInfo(ctypes.Structure):
+    _fields_ = [("dims", ctypes.POINTER(c_int64)), ("rank", c_size_t), ("dtype", c_int)]
+
+
+# name -> (restype, argtypes); every symbol include/mnb_mi355x.h declares
+SIGNATURES = {
+    "MnbGetLastErrorMessage": (c_char_p, []),
+    "MnbGetVersion": (c_int, []),
+    "MnbGetDeviceCount": (c_int, []),
+    "MnbIsAvailable": (c_int, [c_int, c_int, c_int]),
+    "MnbCheckInputs": (c_int, [ctypes.POINTER(MnbTensorInfo)] * 5 + [c_int64] * 4),
+    "MnbPackQuantBDataSize": (c_size_t, [c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
+    "MnbPackQuantBData": (c_int, [c_size_t, c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p]),
+    "MnbGemmWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
+    "MnbGemm": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
+                        c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "MnbGemmUnpackedWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
+    "MnbGemmUnpacked": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "MnbDequantizeBlockwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_size_t,
+                                       c_int, c_void_p]),
+    "MnbDequantizePacked": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
+    "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the shared library (once). Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(f"{LIB_PATH} is missing: build it with `python -m onnxruntime_amd.build` "
+                               "(there is no CPU fallback)")
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().MnbGetLastErrorMessage().decode()
+
+
+def check(code: int) -> None:
+    if code != OK:
+        raise MnbError(code, last_error())

@@ -1,0 +1,284 @@
+// C ABI of libmnb_mi355x.so (declared in include/mnb_mi355x.h): argument validation, error reporting and kernel
+// selection.  No exception leaves this file.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/mnb_mi355x.h"
+#include "mnb_internal.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(MNB_EP_FAIL, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool supported(int bits, int bs, int dtype) {
+  const bool b = bits == 4 || bits == 8;
+  const bool s = bs == 16 || bs == 32 || bs == 64 || bs == 128 || bs == 256;
+  const bool d = dtype == MNB_DTYPE_FLOAT || dtype == MNB_DTYPE_FLOAT16;
+  return b && s && d;
+}
+
+int check_config(const char* fn, int bits, int bs, int dtype) {
+  // Same wording as the reference kernel's constructor (matmul_nbits.cc:130-135).
+  if (bits != 2 && bits != 4 && bits != 8)
+    return fail(MNB_INVALID_ARGUMENT,
+                "%s: Only 2b, 4b and 8b quantization is supported for MatMulNBits op, additional bits support is "
+                "planned.", fn);
+  if (!(bs == 16 || bs == 32 || bs == 64 || bs == 128 || bs == 256))
+    return fail(MNB_INVALID_ARGUMENT,
+                "%s: Only block sizes 16, 32, 64, 128, and 256 are supported for MatMulNBits op, got: %d", fn, bs);
+  if (bits == 2) return fail(MNB_NOT_IMPLEMENTED, "%s: 2-bit weights have no MI355X kernel", fn);
+  if (dtype != MNB_DTYPE_FLOAT && dtype != MNB_DTYPE_FLOAT16)
+    return fail(MNB_NOT_IMPLEMENTED, "%s: element type %d has no MI355X kernel (float and float16 only)", fn, dtype);
+  return MNB_OK;
+}
+
+std::string shape_str(const int64_t* d, size_t r) {
+  std::string s = "{";
+  for (size_t i = 0; i < r; ++i) {
+    if (i) s += ",";
+    s += std::to_string(d[i]);
+  }
+  return s + "}";
+}
+
+bool shape_is(const MnbTensorInfo* t, std::initializer_list<int64_t> want) {
+  if (t->rank != want.size()) return false;
+  size_t i = 0;
+  for (int64_t w : want)
+    if (t->dims[i++] != w) return false;
+  return true;
+}
+
+std::string want_str(std::initializer_list<int64_t> want) {
+  std::string s = "{";
+  bool first = true;
+  for (int64_t w : want) {
+    if (!first) s += ",";
+    s += std::to_string(w);
+    first = false;
+  }
+  return s + "}";
+}
+
+bool present(const MnbTensorInfo* t) { return t != nullptr && t->dims != nullptr; }
+
+}  // namespace
+
+extern "C" {
+
+const char* MnbGetLastErrorMessage(void) { return g_last_error.c_str(); }
+
+int MnbGetVersion(void) { return 1; }
+
+int MnbGetDeviceCount(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  int usable = 0;
+  for (int i = 0; i < n; ++i) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, i) == hipSuccess && strncmp(prop.gcnArchName, "gfx950", 6) == 0) ++usable;
+  }
+  return usable;
+}
+
+int MnbIsAvailable(int bits, int block_size, int a_dtype) { return supported(bits, block_size, a_dtype) ? 1 : 0; }
+
+int MnbCheckInputs(const MnbTensorInfo* quantized_weight, const MnbTensorInfo* scales,
+                   const MnbTensorInfo* zero_points, const MnbTensorInfo* group_index, const MnbTensorInfo* bias,
+                   int64_t n, int64_t k, int64_t block_size, int64_t bits) {
+  if (bits != 2 && bits != 4 && bits != 8)
+    return fail(MNB_INVALID_ARGUMENT, "bits should be 2, 4 or 8, got %lld", (long long)bits);
+  if (block_size < 16 || (block_size & (block_size - 1)) != 0)
+    return fail(MNB_INVALID_ARGUMENT, "block_size must be a power of 2, and >= 16. Got %lld", (long long)block_size);
+  const int64_t k_blocks = (k + block_size - 1) / block_size;
+  const int64_t blob_size = block_size * bits / 8;
+
+  auto mismatch1 = [&](const char* name, const MnbTensorInfo* t, std::initializer_list<int64_t> want) {
+    return fail(MNB_INVALID_ARGUMENT, "Input '%s' is expected to have shape %s, got %s", name, want_str(want).c_str(),
+                shape_str(t->dims, t->rank).c_str());
+  };
+  auto mismatch2 = [&](const char* name, const MnbTensorInfo* t, std::initializer_list<int64_t> w1,
+                       std::initializer_list<int64_t> w2) {
+    return fail(MNB_INVALID_ARGUMENT, "Input '%s' is expected to have shape %s or %s, got %s", name,
+                want_str(w1).c_str(), want_str(w2).c_str(), shape_str(t->dims, t->rank).c_str());
+  };
+
+  if (present(quantized_weight) && !shape_is(quantized_weight, {n, k_blocks, blob_size}))
+    return mismatch1("quantized_weight", quantized_weight, {n, k_blocks, blob_size});
+  if (present(scales) && !shape_is(scales, {n * k_blocks}) && !shape_is(scales, {n, k_blocks}))
+    return mismatch2("scales", scales, {n * k_blocks}, {n, k_blocks});
+  if (present(zero_points)) {
+    if (zero_points->dtype == MNB_DTYPE_UINT8) {
+      const int64_t zb = (k_blocks * bits + 7) / 8;
+      if (!shape_is(zero_points, {n * zb}) && !shape_is(zero_points, {n, zb}))
+        return mismatch2("zero_points", zero_points, {n * zb}, {n, zb});
+    } else {
+      if (present(scales) && zero_points->dtype != scales->dtype)
+        return fail(MNB_INVALID_ARGUMENT,
+                    "Input 'zero_points' and 'scales' should have the same data type when zero_points is not uint8");
+      if (!shape_is(zero_points, {n * k_blocks}) && !shape_is(zero_points, {n, k_blocks}))
+        return mismatch2("zero_points", zero_points, {n * k_blocks}, {n, k_blocks});
+    }
+  }
+  if (present(group_index) && !shape_is(group_index, {k}) && !shape_is(group_index, {k_blocks * block_size}))
+    return mismatch2("group_index", group_index, {k}, {k_blocks * block_size});
+  if (present(bias) && !shape_is(bias, {n})) return mismatch1("bias", bias, {n});
+  return MNB_OK;
+}
+
+size_t MnbPackQuantBDataSize(size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype) {
+  if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0) return 0;
+  return (size_t)mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points).total_bytes;
+}
+
+int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype, const void* b_dev,
+                      const void* scales_dev, const void* zero_points_dev, void* packed_dev, void* stream) {
+  if (int rc = check_config("MnbPackQuantBData", bits, block_size, a_dtype)) return rc;
+  if (N == 0 || K == 0) return MNB_OK;
+  if (!b_dev || !scales_dev || !packed_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbPackQuantBData: B, scales and the packed buffer must not be NULL");
+  if (reinterpret_cast<uintptr_t>(packed_dev) % 256 != 0)
+    return fail(MNB_INVALID_ARGUMENT, "MnbPackQuantBData: the packed buffer must be 256-byte aligned");
+  MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, zero_points_dev != nullptr);
+  hipError_t e = mnb_launch_pack(L, b_dev, scales_dev, zero_points_dev, packed_dev, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbPackQuantBData");
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------------------------------------ kernel choice
+MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
+  if (a.M <= 16) return kMnbKernelGemv;
+  if (a.L.dtype == kMnbDtypeFloat16) {
+    // 16-byte activation loads: base and row pitch aligned, no partial 8-element chunk at the end of a row
+    const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (a.L.K % 8 == 0);
+    if (aligned) return kMnbKernelGemmMfma;
+  }
+  return kMnbKernelGemmGeneric;
+}
+
+const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout&) {
+  switch (k) {
+    case kMnbKernelGemv: return "mnb_gemv_kernel";
+    case kMnbKernelGemmMfma: return "mnb_gemm_mfma_kernel";
+    case kMnbKernelGemmGeneric: return "mnb_gemm_generic_kernel";
+    default: return "none";
+  }
+}
+
+extern "C" {
+
+size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                            int a_dtype) {
+  if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0 || M == 0) return 0;
+  MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  return mnb_gemv_workspace_bytes(L, (int64_t)M);
+}
+
+int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+            const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev, size_t ldc,
+            void* workspace_dev, size_t workspace_bytes, void* stream) {
+  if (int rc = check_config("MnbGemm", bits, block_size, a_dtype)) return rc;
+  if (M == 0 || N == 0) return MNB_OK;  // empty output: nothing to compute (matmul_nbits.cc:1533-1536)
+  if (K == 0) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: K must be positive");
+  if (!a_dev || !packed_dev || !c_dev) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: A, packed B and C must not be NULL");
+  if (lda < K || ldc < N) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: lda (%zu) < K (%zu) or ldc (%zu) < N (%zu)", lda, K, ldc, N);
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff)
+    return fail(MNB_INVALID_ARGUMENT, "MnbGemm: M, N and K must fit in 31 bits");
+  MnbGemmArgs a;
+  a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  a.M = (int64_t)M;
+  a.A = a_dev;
+  a.lda = (int64_t)lda;
+  a.packed = packed_dev;
+  a.bias = bias_dev;
+  a.C = c_dev;
+  a.ldc = (int64_t)ldc;
+  a.workspace = workspace_dev;
+  a.workspace_bytes = workspace_dev ? workspace_bytes : 0;
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e;
+  switch (mnb_select_kernel(a)) {
+    case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
+    case kMnbKernelGemmMfma: e = mnb_launch_gemm_mfma(a, s); break;
+    default: e = mnb_launch_gemm_generic(a, s); break;
+  }
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbGemm");
+}
+
+size_t MnbGemmUnpackedWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                                    int a_dtype) {
+  const size_t pack = MnbPackQuantBDataSize(N, K, bits, block_size, has_zero_points, a_dtype);
+  if (pack == 0) return 0;
+  return pack + MnbGemmWorkspaceSize(M, N, K, bits, block_size, has_zero_points, a_dtype);
+}
+
+int MnbGemmUnpacked(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, const void* a_dev, size_t lda,
+                    const void* b_dev, const void* scales_dev, const void* zero_points_dev, const void* bias_dev,
+                    void* c_dev, size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  if (int rc = check_config("MnbGemmUnpacked", bits, block_size, a_dtype)) return rc;
+  if (M == 0 || N == 0) return MNB_OK;
+  const int has_zp = zero_points_dev != nullptr;
+  const size_t pack = MnbPackQuantBDataSize(N, K, bits, block_size, has_zp, a_dtype);
+  if (!workspace_dev || workspace_bytes < pack)
+    return fail(MNB_INVALID_ARGUMENT, "MnbGemmUnpacked: workspace of %zu bytes needed, %zu given", pack,
+                workspace_dev ? workspace_bytes : (size_t)0);
+  if (int rc = MnbPackQuantBData(N, K, bits, block_size, a_dtype, b_dev, scales_dev, zero_points_dev, workspace_dev,
+                                 stream))
+    return rc;
+  return MnbGemm(M, N, K, bits, block_size, has_zp, a_dtype, a_dev, lda, workspace_dev, bias_dev, c_dev, ldc,
+                 static_cast<char*>(workspace_dev) + pack, workspace_bytes - pack, stream);
+}
+
+int MnbDequantizeBlockwise(void* dst_dev, const void* b_dev, const void* scales_dev, const void* zero_points_dev,
+                           int block_size, int bits, size_t K, size_t N, int a_dtype, void* stream) {
+  if (int rc = check_config("MnbDequantizeBlockwise", bits, block_size, a_dtype)) return rc;
+  if (N == 0 || K == 0) return MNB_OK;
+  if (!dst_dev || !b_dev || !scales_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbDequantizeBlockwise: dst, B and scales must not be NULL");
+  hipError_t e = mnb_launch_dequant_canonical(dst_dev, b_dev, scales_dev, zero_points_dev, (int64_t)N, (int64_t)K,
+                                              bits, block_size, a_dtype, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbDequantizeBlockwise");
+}
+
+int MnbDequantizePacked(void* dst_dev, const void* packed_dev, size_t N, size_t K, int bits, int block_size,
+                        int has_zero_points, int a_dtype, void* stream) {
+  if (int rc = check_config("MnbDequantizePacked", bits, block_size, a_dtype)) return rc;
+  if (N == 0 || K == 0) return MNB_OK;
+  if (!dst_dev || !packed_dev) return fail(MNB_INVALID_ARGUMENT, "MnbDequantizePacked: dst and packed must not be NULL");
+  MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  hipError_t e = mnb_launch_dequant_packed(dst_dev, packed_dev, L, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbDequantizePacked");
+}
+
+const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype) {
+  if (!supported(bits, block_size, a_dtype)) return "none";
+  MnbGemmArgs a{};
+  a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, 0);
+  a.M = (int64_t)M;
+  a.lda = (int64_t)K;
+  return mnb_kernel_name(mnb_select_kernel(a), a.L);
+}
+
+}  // extern "C"

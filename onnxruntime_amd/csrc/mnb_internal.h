@@ -1,0 +1,39 @@
+// Launchers implemented in the .hip translation units; called by the C ABI in mnb_api.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "mnb_layout.h"
+
+struct MnbGemmArgs {
+  MnbLayout L;
+  int64_t M;
+  const void* A;
+  int64_t lda;
+  const void* packed;
+  const void* bias;
+  void* C;
+  int64_t ldc;
+  void* workspace;
+  size_t workspace_bytes;
+};
+
+enum MnbKernelKind {
+  kMnbKernelNone = 0,
+  kMnbKernelGemv,       // M <= 16, dequantising GEMV (VALU dot products)
+  kMnbKernelGemmMfma,   // fp16, LDS-staged MFMA GEMM
+  kMnbKernelGemmGeneric // any shape / fp32 large M: simple tile kernel
+};
+
+MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a);
+const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout& L);
+
+hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
+                           hipStream_t s);
+hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,
+                                        int64_t K, int bits, int bs, int dtype, hipStream_t s);
+hipError_t mnb_launch_dequant_packed(void* dst, const void* packed, const MnbLayout& L, hipStream_t s);
+
+size_t mnb_gemv_workspace_bytes(const MnbLayout& L, int64_t M);
+hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
+hipError_t mnb_launch_gemm_mfma(const MnbGemmArgs& a, hipStream_t s);
+hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);

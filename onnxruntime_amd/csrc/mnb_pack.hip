@@ -1,0 +1,223 @@
+// PrePack and dequantise kernels.
+//
+// PrePack replaces the CPU-specific nibble interleave of the reference
+// (onnxruntime/core/mlas/lib/sqnbitgemm_kernel_avx_common.h:39-115) with the gfx950 k-group-major layout described
+// in mnb_layout.h.  The dequantise kernels restate BlockwiseQuantizer::dequantize
+// (onnxruntime/core/mlas/lib/q4_dq.cpp:587-641) on the device.
+#include "mnb_device.cuh"
+#include "mnb_internal.h"
+
+// ------------------------------------------------------------------------------------------------ pack weights
+// One thread per (column n, group g).  Consecutive threads take consecutive groups of one column, so the reads of
+// the canonical matrix are contiguous; the 16-byte writes are strided by Npad.
+template <int BITS>
+__global__ void __launch_bounds__(256) mnb_pack_weights_kernel(const uint8_t* __restrict__ B, uint4* __restrict__ W,
+                                                               MnbLayout L) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t n = idx / L.KG;
+  const int64_t g = idx % L.KG;
+  if (n >= L.Npad) return;
+  uint32_t w[4] = {0, 0, 0, 0};
+  const int64_t col_bytes = L.k_blocks * L.bs * BITS / 8;  // bytes of one canonical column
+  if (n < L.N) {
+    const uint8_t* src = B + n * col_bytes + g * 16;
+    for (int i = 0; i < 4; ++i) {
+      uint32_t v = 0;
+      for (int b = 0; b < 4; ++b) {
+        int64_t off = g * 16 + i * 4 + b;
+        uint32_t byte = off < col_bytes ? src[i * 4 + b] : 0u;
+        v |= byte << (8 * b);
+      }
+      if constexpr (BITS == 4) {
+        // canonical nibble i of the word holds element e_i; store e0 e2 e4 e6 e1 e3 e5 e7
+        uint32_t r = 0;
+        for (int e = 0; e < 8; ++e) {
+          uint32_t q = (v >> (4 * e)) & 0xFu;
+          int pos = (e & 1) ? 4 + (e >> 1) : (e >> 1);
+          r |= q << (4 * pos);
+        }
+        v = r;
+      }
+      w[i] = v;
+    }
+  }
+  W[g * L.Npad + n] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ------------------------------------------------------------------------------------------------ pack meta
+// One thread per (block kb, column n).
+template <typename T, int BITS, bool HAS_ZP>
+__global__ void __launch_bounds__(256) mnb_pack_meta_kernel(const T* __restrict__ scales,
+                                                            const uint8_t* __restrict__ zp, uint8_t* __restrict__ meta,
+                                                            MnbLayout L) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= L.KBp * L.Npad) return;
+  const int64_t kb = idx / L.Npad;
+  const int64_t n = idx % L.Npad;
+  const bool valid = n < L.N && kb < L.k_blocks;
+  T s = valid ? scales[n * L.k_blocks + kb] : (T)0;
+  int z = 0;
+  if constexpr (HAS_ZP) {
+    if (valid) {
+      const int64_t row = (L.k_blocks * BITS + 7) / 8;
+      if constexpr (BITS == 8) {
+        z = zp[n * row + kb];
+      } else {
+        z = (zp[n * row + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
+      }
+    }
+  }
+  if constexpr (sizeof(T) == 2) {
+    if constexpr (HAS_ZP) {
+      h2_t m;
+      m.x = s;
+      m.y = (_Float16)(-(1024.0f + (float)z));
+      reinterpret_cast<uint32_t*>(meta)[idx] = mnb_as_u32(m);
+    } else {
+      reinterpret_cast<_Float16*>(meta)[idx] = s;
+    }
+  } else {
+    if constexpr (HAS_ZP) {
+      reinterpret_cast<float2*>(meta)[idx] = make_float2(s, (float)z);
+    } else {
+      reinterpret_cast<float*>(meta)[idx] = s;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ dequantise
+// Canonical operands -> dst[n*K + k].  One thread per element.
+template <typename T, int BITS>
+__global__ void __launch_bounds__(256) mnb_dequant_canonical_kernel(T* __restrict__ dst, const uint8_t* __restrict__ B,
+                                                                    const T* __restrict__ scales,
+                                                                    const uint8_t* __restrict__ zp, int64_t N,
+                                                                    int64_t K, int bs) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= N * K) return;
+  const int64_t n = idx / K, k = idx % K;
+  const int64_t kbc = (K + bs - 1) / bs;
+  const int64_t kb = k / bs, r = k % bs;
+  const uint8_t* blob = B + (n * kbc + kb) * (bs * BITS / 8);
+  int q, z = 1 << (BITS - 1);
+  if constexpr (BITS == 8) {
+    q = blob[r];
+    if (zp) z = zp[n * kbc + kb];
+  } else {
+    q = (blob[r >> 1] >> ((r & 1) * 4)) & 0xF;
+    if (zp) z = (zp[n * ((kbc + 1) / 2) + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
+  }
+  const T s = scales[n * kbc + kb];
+  if constexpr (sizeof(T) == 2) {
+    dst[idx] = (_Float16)(q - z) * s;  // exact integer half times half: one RNE rounding
+  } else {
+    dst[idx] = (float)(q - z) * s;
+  }
+}
+
+// Packed buffer -> dst[n*K + k], through the same unpack code the GEMV/GEMM kernels use.
+template <typename T, int BITS, bool HAS_ZP>
+__global__ void __launch_bounds__(256) mnb_dequant_packed_kernel(T* __restrict__ dst, const uint8_t* __restrict__ packed,
+                                                                 MnbLayout L) {
+  constexpr int GK = 128 / BITS;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t g = idx / L.Npad;
+  const int64_t n = idx % L.Npad;
+  if (g >= L.KG || n >= L.N) return;
+  const uint4 v = reinterpret_cast<const uint4*>(packed)[g * L.Npad + n];
+  const uint8_t* meta = packed + L.meta_off;
+  T out[GK];
+  if constexpr (sizeof(T) == 2) {
+    mnb_dequant_group_h<BITS, HAS_ZP>(v, meta, g, n, L.Npad, L.bs, out);
+  } else {
+    mnb_dequant_group_f<BITS, HAS_ZP>(v, meta, g, n, L.Npad, L.bs, out);
+  }
+  for (int i = 0; i < GK; ++i) {
+    const int64_t k = g * GK + i;
+    if (k < L.K) dst[n * L.K + k] = out[i];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ launchers
+template <typename T>
+static hipError_t pack_t(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
+                         hipStream_t s) {
+  uint4* W = reinterpret_cast<uint4*>(packed);
+  uint8_t* meta = reinterpret_cast<uint8_t*>(packed) + L.meta_off;
+  const int64_t wn = L.Npad * L.KG;
+  const int64_t mn = L.KBp * L.Npad;
+  dim3 blk(256);
+  if (L.bits == 4) {
+    mnb_pack_weights_kernel<4><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>((const uint8_t*)B, W, L);
+    if (zp)
+      mnb_pack_meta_kernel<T, 4, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales,
+                                                                                         (const uint8_t*)zp, meta, L);
+    else
+      mnb_pack_meta_kernel<T, 4, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales, nullptr,
+                                                                                          meta, L);
+  } else {
+    mnb_pack_weights_kernel<8><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>((const uint8_t*)B, W, L);
+    if (zp)
+      mnb_pack_meta_kernel<T, 8, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales,
+                                                                                         (const uint8_t*)zp, meta, L);
+    else
+      mnb_pack_meta_kernel<T, 8, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales, nullptr,
+                                                                                          meta, L);
+  }
+  return hipGetLastError();
+}
+
+hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
+                           hipStream_t s) {
+  return L.dtype == kMnbDtypeFloat16 ? pack_t<_Float16>(L, B, scales, zp, packed, s)
+                                     : pack_t<float>(L, B, scales, zp, packed, s);
+}
+
+hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,
+                                        int64_t K, int bits, int bs, int dtype, hipStream_t s) {
+  const int64_t total = N * K;
+  if (total == 0) return hipSuccess;
+  dim3 grid((unsigned)((total + 255) / 256)), blk(256);
+  if (dtype == kMnbDtypeFloat16) {
+    if (bits == 4)
+      mnb_dequant_canonical_kernel<_Float16, 4><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,
+                                                                     (const _Float16*)scales, (const uint8_t*)zp, N, K,
+                                                                     bs);
+    else
+      mnb_dequant_canonical_kernel<_Float16, 8><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,
+                                                                     (const _Float16*)scales, (const uint8_t*)zp, N, K,
+                                                                     bs);
+  } else {
+    if (bits == 4)
+      mnb_dequant_canonical_kernel<float, 4><<<grid, blk, 0, s>>>((float*)dst, (const uint8_t*)B, (const float*)scales,
+                                                                  (const uint8_t*)zp, N, K, bs);
+    else
+      mnb_dequant_canonical_kernel<float, 8><<<grid, blk, 0, s>>>((float*)dst, (const uint8_t*)B, (const float*)scales,
+                                                                  (const uint8_t*)zp, N, K, bs);
+  }
+  return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t dequant_packed_t(void* dst, const void* packed, const MnbLayout& L, hipStream_t s) {
+  const int64_t total = L.KG * L.Npad;
+  dim3 grid((unsigned)((total + 255) / 256)), blk(256);
+  const uint8_t* p = (const uint8_t*)packed;
+  if (L.bits == 4) {
+    if (L.has_zp)
+      mnb_dequant_packed_kernel<T, 4, true><<<grid, blk, 0, s>>>((T*)dst, p, L);
+    else
+      mnb_dequant_packed_kernel<T, 4, false><<<grid, blk, 0, s>>>((T*)dst, p, L);
+  } else {
+    if (L.has_zp)
+      mnb_dequant_packed_kernel<T, 8, true><<<grid, blk, 0, s>>>((T*)dst, p, L);
+    else
+      mnb_dequant_packed_kernel<T, 8, false><<<grid, blk, 0, s>>>((T*)dst, p, L);
+  }
+  return hipGetLastError();
+}
+
+hipError_t mnb_launch_dequant_packed(void* dst, const void* packed, const MnbLayout& L, hipStream_t s) {
+  if (L.N == 0 || L.K == 0) return hipSuccess;
+  return L.dtype == kMnbDtypeFloat16 ? dequant_packed_t<_Float16>(dst, packed, L, s)
+                                     : dequant_packed_t<float>(dst, packed, L, s);
+}

@@ -1,0 +1,86 @@
+"""The benchmark configurations at their full sizes: oracle on what the CPU finishes in seconds, size-independent
+properties (unit vectors, linearity, absent-zp identity) on the rest."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import check_against_oracle, dev, make_op, run_case
+from onnxruntime_amd import synthetic
+from onnxruntime_amd.synthetic import make_case
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits_view(a):
+    return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+def test_config1_fp32_decode(oracle):
+    c = synthetic.config_c1()
+    y = run_case(c)
+    worst = check_against_oracle(oracle, c, y)
+    print(f"C1 max|err|/bound = {worst:.2e}")
+
+
+def test_config2_fp16_decode(oracle):
+    c = synthetic.config_c2()
+    y = run_case(c)
+    rel = check_against_oracle(oracle, c, y)
+    print(f"C2 rel L2 = {rel:.2e}")
+    # unit vector at full size: row k of W comes back bit for bit
+    op = make_op(c)
+    w = oracle.C.dequantize(c.B, c.scales, None, c.N, c.K, 4, 128)
+    for k in (0, 1, 127, 128, 2049, 4095):
+        e = np.zeros((1, c.K), np.float16)
+        e[0, k] = 1
+        yk = op.Compute(dev(e)).cpu().numpy()[0]
+        assert np.array_equal(_bits_view(yk), _bits_view(np.ascontiguousarray(w[:, k])))
+
+
+@pytest.mark.parametrize("shape", list(synthetic.C3_SHAPES))
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 16])
+def test_config3_small_batch(oracle, shape, M):
+    K, N = synthetic.C3_SHAPES[shape]
+    c = make_case(M, N, K, 4, 64, np.float16, has_zp=True, seed=0)
+    y = run_case(c)
+    check_against_oracle(oracle, c, y)
+
+
+def test_config4_prefill(oracle):
+    c = synthetic.config_c4()
+    op = make_op(c)
+    a = dev(c.A)
+    y = op.Compute(a, bias=dev(c.bias))
+    torch.cuda.synchronize()
+    yh = y.cpu().numpy()
+    # oracle on a sample of rows (the CPU needs ~1 s per 8 rows at this size)
+    rows = np.array([0, 1, 31, 32, 63, 64, 127, 128, 1000, 1023, 1024, 2046, 2047])
+    sub = make_case(len(rows), c.N, c.K, 4, 32, np.float16, has_zp=True, has_bias=True, seed=0)
+    sub.B, sub.scales, sub.zero_points, sub.bias = c.B, c.scales, c.zero_points, c.bias
+    sub.A = c.A[rows]
+    check_against_oracle(oracle, sub, yh[rows], A=sub.A)
+    # linearity over the whole output: f(A) - bias is linear in A; compare f(2A) - bias with 2 (f(A) - bias)
+    y2 = op.Compute(a * 2, bias=dev(c.bias)).float()
+    b = dev(c.bias).float()
+    lhs = y2 - b
+    rhs = 2 * (y.float() - b)
+    rel = (torch.linalg.norm(lhs - rhs) / torch.linalg.norm(rhs)).item()
+    assert rel < 2e-3, rel
+    # every 128 x 128 tile of the output is finite and non-trivial
+    assert torch.isfinite(y).all()
+    t = y.float().view(16, 128, 112, 128).abs().amax(dim=(1, 3))
+    assert (t > 0).all()
+
+
+@pytest.mark.parametrize("bits,bs", [(4, 128), (8, 64)])
+@pytest.mark.parametrize("shape", list(synthetic.C5_SHAPES))
+def test_config5_layer_sweep(oracle, bits, bs, shape):
+    K, N = synthetic.C5_SHAPES[shape]
+    for M in (1, 64, 256):
+        c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, seed=0)
+        y = run_case(c)
+        rows = np.unique(np.linspace(0, M - 1, 6).astype(int))
+        sub = make_case(len(rows), N, K, bits, bs, np.float16, has_zp=True, seed=0)
+        sub.B, sub.scales, sub.zero_points = c.B, c.scales, c.zero_points
+        sub.A = c.A[rows]
+        check_against_oracle(oracle, sub, y[rows], A=sub.A)

@@ -1,0 +1,167 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle and the golden vectors."""
+import numpy as np
+import pytest
+import torch
+
+from golden_cases import load_js_cases
+from gpu_util import check_against_oracle, dev, make_op, run_case, tdtype
+from onnxruntime_amd.matmul_nbits import MatMulNBits, dequantize_blockwise
+from onnxruntime_amd.synthetic import make_case
+
+pytestmark = pytest.mark.gpu
+
+JS = load_js_cases()
+
+
+def _bits_view(a):
+    return a.view(np.uint16 if a.dtype == np.float16 else np.uint32)
+
+
+# ----------------------------------------------------------------------------------------------- golden vectors
+@pytest.mark.parametrize("prepack", [True, False])
+@pytest.mark.parametrize("case", JS, ids=[f"{i}" for i in range(len(JS))])
+def test_reference_vectors(case, prepack):
+    c = case
+    op = MatMulNBits(c["K"], c["N"], c["bits"], c["block_size"], dtype=torch.float32,
+                     has_zero_points=c["zero_points"] is not None)
+    a, b, s, z = dev(c["A"]), dev(c["B"]), dev(c["scales"]), dev(c["zero_points"])
+    if prepack:
+        assert op.PrePack(b, s, z)
+        y = op.Compute(a)
+    else:
+        y = op.Compute(a, b, s, z)
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == c["Y"].shape
+    assert np.array_equal(y.cpu().numpy(), c["Y"]), c["name"]
+
+
+# ----------------------------------------------------------------------------------------------- dequant, bit exact
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128, 256])
+@pytest.mark.parametrize("zp", [False, True])
+def test_dequant_bit_exact(oracle, dtype, bits, bs, zp):
+    for (N, K) in [(8, 64), (33, 93), (300, 260), (5, 1234)]:
+        c = make_case(1, N, K, bits, bs, dtype, has_zp=zp, seed=N + K)
+        want = oracle.C.dequantize(c.B, c.scales, c.zero_points, N, K, bits, bs)
+        got = dequantize_blockwise(dev(c.B), dev(c.scales), dev(c.zero_points), N, K, bits, bs).cpu().numpy()
+        assert np.array_equal(_bits_view(got), _bits_view(want)), "canonical dequantise"
+        op = make_op(c)
+        got_p = op.dequantize_packed().cpu().numpy()
+        assert np.array_equal(_bits_view(got_p), _bits_view(want)), "packed dequantise"
+
+
+@pytest.mark.parametrize("bits,bs", [(4, 16), (8, 16), (4, 32)])
+def test_dequant_exhaustive_q_zp(bits, bs):
+    """All 2^bits x 2^bits (q, zp) pairs against integer arithmetic, for both model types."""
+    levels = 1 << bits
+    N, K = levels, max(levels, bs) * 2
+    kb = K // bs
+    q = np.broadcast_to(np.arange(K)[None, :] % levels, (N, K)).copy()
+    zpv = (np.arange(N)[:, None] + np.arange(kb)[None, :]) % levels
+    per = 8 // bits
+    B = np.zeros((N, kb, bs * bits // 8), np.uint8)
+    Z = np.zeros((N, (kb * bits + 7) // 8), np.uint8)
+    qq = q.reshape(N, kb, bs // per, per)
+    for j in range(per):
+        B |= (qq[..., j] << (bits * j)).astype(np.uint8)
+    zz = np.zeros((N, Z.shape[1] * per), np.int64)
+    zz[:, :kb] = zpv
+    zz = zz.reshape(N, Z.shape[1], per)
+    for j in range(per):
+        Z |= (zz[..., j] << (bits * j)).astype(np.uint8)
+    scales = (0.5 ** (np.arange(N * kb) % 5)).astype(np.float32).reshape(N, kb) * 3
+    want = (q - np.repeat(zpv, bs, axis=1)).astype(np.float64) * np.repeat(scales, bs, axis=1)
+    for dt in (np.float32, np.float16):
+        s = scales.astype(dt)
+        got = dequantize_blockwise(dev(B), dev(s), dev(Z), N, K, bits, bs).cpu().numpy()
+        assert np.array_equal(got.astype(np.float64), want)
+        op = MatMulNBits(K, N, bits, bs, dtype=tdtype(dt), has_zero_points=True)
+        op.PrePack(dev(B), dev(s), dev(Z))
+        assert np.array_equal(op.dequantize_packed().cpu().numpy().astype(np.float64), want)
+
+
+# ----------------------------------------------------------------------------------------------- unit vectors
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits,bs,K,N", [(4, 32, 96, 70), (4, 16, 48, 9), (8, 64, 256, 130), (4, 128, 256, 64),
+                                         (8, 16, 40, 11), (4, 64, 93, 17)])
+def test_unit_vectors_recover_dequant(oracle, dtype, bits, bs, K, N):
+    """A = I pushes every weight through the compute kernels unchanged: Y must equal the dequantised bits.
+
+    M = K rows exercises the large-M kernel; the first rows alone (M <= 16) exercise the GEMV."""
+    c = make_case(K, N, K, bits, bs, dtype, has_zp=True, seed=9)
+    want = oracle.C.dequantize(c.B, c.scales, c.zero_points, N, K, bits, bs).T.copy()  # [K, N]
+    eye = np.eye(K, dtype=dtype)
+    y = run_case(c, A=eye)
+    assert np.array_equal(_bits_view(y), _bits_view(want)), "large-M kernel"
+    for m in (1, 3, 16):
+        y = run_case(c, A=eye[:m])
+        assert np.array_equal(_bits_view(y), _bits_view(want[:m])), f"GEMV M={m}"
+
+
+# ----------------------------------------------------------------------------------------------- random parity
+SHAPES_SMALL_M = [(1, 33, 93), (1, 1031, 1027), (2, 64, 64), (3, 401, 500), (4, 128, 4096), (5, 17, 260),
+                  (8, 2131, 527), (11, 1031, 1027), (16, 64, 1234), (16, 256, 2048), (1, 32, 80), (7, 300, 16)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits,bs,zp,bias", [(4, 32, True, False), (4, 128, False, True), (4, 16, True, True),
+                                             (8, 64, True, True), (8, 256, False, False), (4, 64, False, False),
+                                             (4, 256, True, True), (8, 16, True, False), (8, 32, False, True),
+                                             (8, 128, True, False)])
+def test_gemv_parity(oracle, dtype, bits, bs, zp, bias):
+    for (M, N, K) in SHAPES_SMALL_M:
+        c = make_case(M, N, K, bits, bs, dtype, has_zp=zp, has_bias=bias, seed=M * 7 + N)
+        y = run_case(c)
+        check_against_oracle(oracle, c, y)
+
+
+SHAPES_LARGE_M = [(17, 64, 64), (43, 401, 500), (64, 256, 512), (100, 130, 264), (128, 128, 128), (129, 257, 1032),
+                  (300, 512, 1024), (33, 1031, 1027), (257, 384, 96)]
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("bits,bs,zp,bias", [(4, 32, True, True), (4, 128, False, False), (4, 16, True, False),
+                                             (8, 64, True, True), (8, 16, False, True), (4, 64, True, False),
+                                             (8, 256, True, False), (4, 256, False, True)])
+def test_gemm_parity(oracle, dtype, bits, bs, zp, bias):
+    for (M, N, K) in SHAPES_LARGE_M:
+        c = make_case(M, N, K, bits, bs, dtype, has_zp=zp, has_bias=bias, seed=M + N + K)
+        y = run_case(c)
+        check_against_oracle(oracle, c, y)
+
+
+def test_unpacked_route_matches_packed():
+    for dtype in (np.float16, np.float32):
+        for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128)]:
+            c = make_case(M, N, K, bits, bs, dtype, has_zp=True, has_bias=True, seed=4)
+            assert np.array_equal(run_case(c, prepack=True), run_case(c, prepack=False))
+
+
+def test_batched_leading_dims_and_strided_a(oracle):
+    c = make_case(6, 96, 128, 4, 32, np.float16, has_zp=True, seed=2, a_shape=(2, 3, 128))
+    op = make_op(c)
+    y = op.Compute(dev(c.A))
+    assert tuple(y.shape) == (2, 3, 96)
+    check_against_oracle(oracle, c, y.cpu().numpy().reshape(6, 96), A=c.A.reshape(6, 128))
+    # rows of A with a pitch larger than K
+    big = torch.zeros(6, 160, dtype=torch.float16, device="cuda")
+    big[:, :128] = dev(c.A.reshape(6, 128))
+    y2 = op.Compute(big[:, :128])
+    assert torch.equal(y2, y.view(6, 96))
+
+
+def test_empty_output():
+    c = make_case(1, 64, 64, 4, 32, np.float16, seed=1)
+    op = make_op(c)
+    y = op.Compute(torch.empty(0, 64, dtype=torch.float16, device="cuda"))
+    assert tuple(y.shape) == (0, 64)
+
+
+def test_deterministic_run_to_run():
+    c = make_case(4, 4096, 4096, 4, 64, np.float16, has_zp=True, seed=3)
+    op = make_op(c)
+    a = dev(c.A)
+    y0 = op.Compute(a).clone()
+    for _ in range(3):
+        assert torch.equal(op.Compute(a), y0)

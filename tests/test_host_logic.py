@@ -1,0 +1,109 @@
+"""CPU-side tests: the C ABI library loads and exports every declared symbol; shape validation and error text."""
+import re
+from pathlib import Path
+
+import pytest
+
+from onnxruntime_amd import _lib
+from onnxruntime_amd._lib import MnbError
+from onnxruntime_amd.matmul_nbits import MatMulNBits, check_inputs
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "mnb_mi355x.h").read_text()
+    declared = set(re.findall(r"MNB_API\s+[\w\s\*]+?\b(Mnb\w+)\s*\(", header))
+    assert len(declared) >= 14
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.MnbGetVersion() >= 1
+
+
+def test_availability_and_sizes():
+    lib = _lib.load()
+    for bits in (4, 8):
+        for bs in (16, 32, 64, 128, 256):
+            for dt in (_lib.DTYPE_FLOAT, _lib.DTYPE_FLOAT16):
+                assert lib.MnbIsAvailable(bits, bs, dt) == 1
+    assert lib.MnbIsAvailable(2, 32, _lib.DTYPE_FLOAT16) == 0
+    assert lib.MnbIsAvailable(4, 512, _lib.DTYPE_FLOAT16) == 0
+    assert lib.MnbIsAvailable(4, 32, 16) == 0  # bf16
+    # packed size: weights (N*K/2) + fp16 scales for the headline decode shape, no padding needed
+    assert lib.MnbPackQuantBDataSize(14336, 4096, 4, 128, 0, _lib.DTYPE_FLOAT16) == 14336 * 2048 + 14336 * 32 * 2
+    assert lib.MnbPackQuantBDataSize(14336, 4096, 4, 32, 1, _lib.DTYPE_FLOAT16) == 14336 * 2048 + 14336 * 128 * 4
+    assert lib.MnbPackQuantBDataSize(0, 4096, 4, 32, 1, _lib.DTYPE_FLOAT16) == 0
+
+
+def _fails(substr, *args, **kw):
+    with pytest.raises(MnbError) as e:
+        check_inputs(*args, **kw)
+    assert substr in str(e.value), str(e.value)
+    assert e.value.code == _lib.INVALID_ARGUMENT
+
+
+def test_check_inputs_messages():
+    # N=8, K=32, bs=16, bits=4: B [8,2,8], scales [8,2] or [16], zp [8,1] or [8]
+    check_inputs((8, 2, 8), (8, 2), (8, 1), None, (8,), 8, 32, 16, 4)
+    check_inputs((8, 2, 8), (16,), (8,), None, None, 8, 32, 16, 4)          # legacy 1-D shapes
+    check_inputs(None, (8, 2), None, (32,), None, 8, 32, 16, 4)            # B already packed, g_idx [K]
+    _fails("bits should be 2, 4 or 8, got 3", (8, 2, 6), (8, 2), None, None, None, 8, 32, 16, 3)
+    _fails("block_size must be a power of 2, and >= 16. Got 8", (8, 4, 4), (8, 4), None, None, None, 8, 32, 8, 4)
+    _fails("block_size must be a power of 2, and >= 16. Got 48", (8, 1, 24), (8, 1), None, None, None, 8, 32, 48, 4)
+    _fails("Input 'quantized_weight' is expected to have shape {8,2,8}, got {8,2,16}", (8, 2, 16), (8, 2), None,
+           None, None, 8, 32, 16, 4)
+    _fails("Input 'scales' is expected to have shape {16} or {8,2}, got {8,3}", (8, 2, 8), (8, 3), None, None, None,
+           8, 32, 16, 4)
+    _fails("Input 'zero_points' is expected to have shape {8} or {8,1}, got {8,2}", (8, 2, 8), (8, 2), (8, 2), None,
+           None, 8, 32, 16, 4)
+    _fails("Input 'bias' is expected to have shape {8}, got {9}", (8, 2, 8), (8, 2), None, None, (9,), 8, 32, 16, 4)
+    _fails("Input 'group_index' is expected to have shape {30} or {32}, got {31}", (8, 2, 8), (8, 2), None, (31,),
+           None, 8, 30, 16, 4)
+    # typed (non-uint8) zero points: same dtype as scales, shape [N, k_blocks]
+    import torch
+    check_inputs((8, 2, 8), (8, 2), (8, 2), None, None, 8, 32, 16, 4, scales_dtype=torch.float16,
+                 zp_dtype=torch.float16)
+    _fails("should have the same data type when zero_points is not uint8", (8, 2, 8), (8, 2), (8, 2), None, None, 8,
+           32, 16, 4, scales_dtype=torch.float16, zp_dtype=torch.float32)
+
+
+def test_constructor_and_prepack_guards():
+    import torch
+    with pytest.raises(MnbError, match="Only 2b, 4b and 8b quantization is supported"):
+        MatMulNBits(32, 8, bits=3)
+    with pytest.raises(MnbError, match="Only block sizes 16, 32, 64, 128, and 256 are supported for MatMulNBits op, "
+                                       "got: 512"):
+        MatMulNBits(1024, 8, block_size=512)
+    op = MatMulNBits(32, 8, bits=4, block_size=16, has_zero_points=True)
+    b = torch.zeros(8, 2, 8, dtype=torch.uint8)
+    s = torch.zeros(8, 2, dtype=torch.float16)
+    z = torch.zeros(8, 1, dtype=torch.uint8)
+    with pytest.raises(MnbError, match=r"MatMulNBits PrePack: B initializer shape \{8,2,16\} does not match "
+                                       r"attribute-derived shape \[8,2,8\]"):
+        op.PrePack(torch.zeros(8, 2, 16, dtype=torch.uint8), s, z)
+    with pytest.raises(MnbError, match=r"MatMulNBits PrePack: scales initializer shape \{8,3\}"):
+        op.PrePack(b, torch.zeros(8, 3, dtype=torch.float16), z)
+    with pytest.raises(MnbError, match=r"MatMulNBits PrePack: zero_points initializer shape \{8,2\}"):
+        op.PrePack(b, s, torch.zeros(8, 2, dtype=torch.uint8))
+    # configurations the device path declines (they stay on the CPU provider)
+    assert not MatMulNBits(32, 8, bits=2, block_size=16).supported
+    assert not MatMulNBits(32, 8, has_g_idx=True).supported
+    assert not MatMulNBits(32, 8, has_zero_points=True, zero_points_dtype=torch.float16).supported
+    assert not MatMulNBits(32, 8, dtype=torch.bfloat16).supported
+
+
+def test_c_abi_rejects_bad_arguments_without_a_gpu():
+    lib = _lib.load()
+    rc = lib.MnbGemm(1, 8, 32, 3, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
+    assert rc == _lib.INVALID_ARGUMENT and "Only 2b, 4b and 8b" in _lib.last_error()
+    rc = lib.MnbGemm(1, 8, 32, 4, 48, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
+    assert rc == _lib.INVALID_ARGUMENT and "got: 48" in _lib.last_error()
+    rc = lib.MnbGemm(1, 8, 32, 2, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
+    assert rc == _lib.NOT_IMPLEMENTED
+    rc = lib.MnbGemm(1, 8, 32, 4, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
+    assert rc == _lib.INVALID_ARGUMENT and "must not be NULL" in _lib.last_error()
+    assert lib.MnbGemm(0, 8, 32, 4, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None) == 0
+    rc = lib.MnbPackQuantBData(8, 32, 4, 16, _lib.DTYPE_FLOAT16, None, None, None, None, None)
+    assert rc == _lib.INVALID_ARGUMENT
