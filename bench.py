@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X MatMulNBits hot path.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--sweep]
+
+Prints ONE JSON line on stdout.  Headline workload (BASELINE.json configs[1]): the decode GEMV
+M=1, K=4096, N=14336, int4, block_size 128, symmetric, fp16.  One *step* is one decode pass of that projection
+through the 32 decoder layers of Llama-3-8B: 32 launches, each on its own packed weight matrix (32 x 30 MB is
+four times the 256 MB Infinity Cache, so every launch streams its weights from HBM).  `value` is algorithmic GB/s
+of the whole step, inputs resident in HBM.  The same line carries the prefill GEMM (configs[3], M=2048) as
+`prefill`, the roofline of the dominant kernel and the CPU baseline (the oracle, timed on this host).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
+LAYERS = 32
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+class Problem:
+    """One MatMulNBits shape with `copies` independently packed weight matrices, run through the C ABI."""
+
+    def __init__(self, case, copies: int, torch, lib_mod):
+        from onnxruntime_amd.matmul_nbits import MatMulNBits
+        self.torch, self.case = torch, case
+        self.lib = lib_mod.load()
+        self.lib_mod = lib_mod
+        tdt = torch.float16 if case.dtype == np.float16 else torch.float32
+        self.dt = lib_mod.DTYPE_FLOAT16 if case.dtype == np.float16 else lib_mod.DTYPE_FLOAT
+        dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()
+        self.has_zp = int(case.zero_points is not None)
+        b, s, z = dev(case.B), dev(case.scales), dev(case.zero_points)
+        self.packed = []
+        t0 = time.perf_counter()
+        for i in range(copies):
+            op = MatMulNBits(case.K, case.N, case.bits, case.block_size, dtype=tdt,
+                             has_zero_points=bool(self.has_zp), has_bias=case.bias is not None)
+            # distinct contents per copy (rolled columns) so no two copies alias in any cache
+            bi = torch.roll(b, shifts=i, dims=0) if i else b
+            assert op.PrePack(bi, s, z)
+            self.packed.append(op.packed)
+        torch.cuda.synchronize()
+        self.prepack_ms = (time.perf_counter() - t0) * 1e3 / copies
+        self.a = dev(case.A.reshape(-1, case.K))
+        self.bias = dev(case.bias)
+        self.M = self.a.shape[0]
+        self.y = [torch.empty(self.M, case.N, dtype=tdt, device="cuda") for _ in range(copies)]
+        wsz = self.lib.MnbGemmWorkspaceSize(self.M, case.N, case.K, case.bits, case.block_size, self.has_zp, self.dt)
+        self.wsz = wsz
+        self.ws = torch.zeros(max(wsz, 256), dtype=torch.uint8, device="cuda")
+        self.kernel = self.lib.MnbGemmKernelName(self.M, case.N, case.K, case.bits, case.block_size, self.dt).decode()
+
+    def launch(self, i: int):
+        c = self.case
+        stream = ctypes.c_void_p(self.torch.cuda.current_stream().cuda_stream)
+        rc = self.lib.MnbGemm(self.M, c.N, c.K, c.bits, c.block_size, self.has_zp, self.dt, _ptr(self.a), c.K,
+                              _ptr(self.packed[i]), _ptr(self.bias), _ptr(self.y[i]), c.N, _ptr(self.ws), self.wsz,
+                              stream)
+        self.lib_mod.check(rc)
+
+    def step(self):
+        for i in range(len(self.packed)):
+            self.launch(i)
+
+
+def time_steps(torch, run_step, steps: int, warmup: int) -> float:
+    """Milliseconds per step, HIP events on the launch stream, barrier + synchronize on both sides."""
+    for _ in range(warmup):
+        run_step()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        run_step()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def graph_of(torch, run_step):
+    """Captures one step into a HIP graph (the launches are ~5 us each: Python cannot issue them that fast)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run_step()  # warm every code path on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        run_step()
+    return g
+
+
+def cpu_baseline(case, budget_s: float, threads: int):
+    """The oracle (a port of the reference arithmetic) timed on this host for a bounded number of calls."""
+    from oracle import oracle
+    oracle.build()
+    run = lambda: oracle.C.matmul(case.A, case.B, case.scales, case.zero_points, case.bias, case.N, case.K,
+                                  case.bits, case.block_size, nthreads=threads)
+    run()
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        run()
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= 200:
+            break
+    return el / n, n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 GEMM")
+    ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the op shards along N without communication; nothing "
+              "here uses a second device). Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+    from onnxruntime_amd import _lib, synthetic
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    _lib.load()
+
+    # ---- decode GEMV (headline) ------------------------------------------------------------------------------
+    c2 = synthetic.config_c2(seed=0)
+    p2 = Problem(c2, LAYERS, torch, _lib)
+    g2 = graph_of(torch, p2.step)
+    ms_step = time_steps(torch, g2.replay, args.steps, args.warmup)
+    bytes_per_launch = c2.algorithmic_bytes()
+    us_per_launch = ms_step * 1e3 / LAYERS
+    gbs = bytes_per_launch / (us_per_launch * 1e-6) / 1e9
+    # same launches with the weights resident in the Infinity Cache (one matrix re-used), for reference only
+    g2hot = graph_of(torch, lambda: [p2.launch(0) for _ in range(LAYERS)])
+    ms_hot = time_steps(torch, g2hot.replay, args.steps, args.warmup)
+
+    out = {
+        "metric": "int4 MatMulNBits decode GEMV (M=1, K=4096, N=14336) algorithmic HBM GB/s",
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[1]: MatMulNBits M=1 K=4096 N=14336 bits=4 block_size=128 symmetric fp16; "
+                        f"one step = {LAYERS} launches on {LAYERS} distinct packed weight matrices (HIP graph)",
+            "launches_per_step": LAYERS,
+            "algorithmic_bytes_per_launch": bytes_per_launch,
+            "kernel": p2.kernel,
+            "prepack_ms_per_matrix": round(p2.prepack_ms, 3),
+            "us_per_launch_weights_in_infinity_cache": round(ms_hot * 1e3 / LAYERS, 3),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "kernel": p2.kernel,
+            "us_per_launch": round(us_per_launch, 3),
+        },
+    }
+    del g2, g2hot, p2
+    torch.cuda.empty_cache()
+
+    # ---- prefill GEMM ----------------------------------------------------------------------------------------
+    if not args.no_prefill:
+        c4 = synthetic.config_c4(seed=0)
+        p4 = Problem(c4, 2, torch, _lib)
+        k4 = max(4, args.steps // 5)
+        ms4 = time_steps(torch, p4.step, k4, max(1, args.warmup // 2)) / 2
+        tflops = c4.flops() / (ms4 * 1e-3) / 1e12
+        out["prefill"] = {
+            "workload": "BASELINE configs[3]: M=2048 K=4096 N=14336 bits=4 block_size=32 zero_points bias fp16",
+            "value": round(tflops, 1),
+            "unit": "TFLOP/s",
+            "ms_per_launch": round(ms4, 4),
+            "kernel": p4.kernel,
+            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None},
+        }
+        del p4
+        torch.cuda.empty_cache()
+
+    # ---- the other configurations (not part of the JSON contract) ---------------------------------------------
+    if args.sweep:
+        sweep(torch, _lib, synthetic)
+
+    # ---- CPU baseline ----------------------------------------------------------------------------------------
+    if not args.no_cpu:
+        threads = max(1, min(16, os.cpu_count() or 1))
+        sec, n = cpu_baseline(c2, args.cpu_seconds, threads)
+        out["cpu_baseline"] = {
+            "value": round(bytes_per_launch / sec / 1e9, 2),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{n} calls of the same M=1 K=4096 N=14336 problem on the C oracle, N sliced over {threads} "
+                      f"threads, {sec * 1e3:.2f} ms per call",
+        }
+    print(json.dumps(out))
+    return 0
+
+
+def sweep(torch, _lib, synthetic):
+    """Times BASELINE configs 1, 3 and 5 (one launch each, rotating weight copies); table on stderr."""
+    from onnxruntime_amd.synthetic import make_case
+    rows = []
+
+    def one(name, case, copies):
+        p = Problem(case, copies, torch, _lib)
+        if p.M <= 64:
+            g = graph_of(torch, p.step)
+            ms = time_steps(torch, g.replay, 20, 3) / copies
+        else:
+            ms = time_steps(torch, p.step, 5, 1) / copies
+        gb = case.algorithmic_bytes() / (ms * 1e-3) / 1e9
+        tf = case.flops() / (ms * 1e-3) / 1e12
+        rows.append((name, p.kernel, ms * 1e3, gb, tf))
+        print(f"{name:44s} {p.kernel:26s} {ms * 1e3:10.2f} us {gb:9.1f} GB/s {tf:9.2f} TFLOP/s", file=sys.stderr)
+        del p
+        torch.cuda.empty_cache()
+
+    one("C1 fp32 M=1 4096x4096 bs32 zp", synthetic.config_c1(), 16)
+    for nm, (K, N) in synthetic.C3_SHAPES.items():
+        for M in (1, 2, 4, 8, 16):
+            one(f"C3 {nm} M={M} K={K} N={N} bs64 zp", make_case(M, N, K, 4, 64, np.float16, has_zp=True), 16)
+    for bits, bs in ((4, 128), (8, 64)):
+        for nm, (K, N) in synthetic.C5_SHAPES.items():
+            for M in (1, 64, 256, 1024, 4096):
+                copies = 8 if M <= 64 else 1
+                one(f"C5 {nm} M={M} K={K} N={N} b{bits} bs{bs} zp",
+                    make_case(M, N, K, bits, bs, np.float16, has_zp=True), copies)
+    return rows
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -91,8 +91,8 @@ MNB_API size_t MnbPackQuantBDataSize(size_t N, size_t K, int bits, int block_siz
 MNB_API int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype, const void* b_dev,
                               const void* scales_dev, const void* zero_points_dev, void* packed_dev, void* stream);
 
-/* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call scratch MnbGemm can use for
- * this problem (split-K partial sums of the GEMV); may be 0. */
+/* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call scratch MnbGemm wants for
+ * this problem. Currently always 0: no kernel needs scratch. */
 MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                     int a_dtype);
 
@@ -100,8 +100,8 @@ MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int 
  *   C[M][N] (ldc) = A[M][K] (lda) x dequant(packed)^T (+ bias[N]).
  * a_dev, bias_dev (optional) and c_dev have element type a_dtype; lda and ldc count elements. M <= 16 runs the
  * dequantising GEMV, larger M the LDS-staged MFMA GEMM (fp16) or the fp32 tile kernel. M == 0 or N == 0 is a
- * no-op. workspace_dev (optional, MnbGemmWorkspaceSize bytes, 256-byte aligned) must not be shared by calls that
- * may overlap; without it the GEMV does not split K over workgroups (same result up to summation order). */
+ * no-op. workspace_dev / workspace_bytes: per-call scratch of MnbGemmWorkspaceSize bytes (may be NULL / 0 when
+ * that size is 0); it must not be shared by calls that may overlap. */
 MNB_API int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
                     const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev,
                     size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream);

@@ -169,7 +169,8 @@ int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype,
 
 // ------------------------------------------------------------------------------------------------ kernel choice
 MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
-  if (a.M <= 16) return kMnbKernelGemv;
+  if (mnb_skinny_applicable(a)) return kMnbKernelSkinny;
+  if (mnb_gemv_applicable(a)) return kMnbKernelGemv;
   if (a.L.dtype == kMnbDtypeFloat16) {
     // 16-byte activation loads: base and row pitch aligned, no partial 8-element chunk at the end of a row
     const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (a.L.K % 8 == 0);
@@ -180,6 +181,7 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
 
 const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout&) {
   switch (k) {
+    case kMnbKernelSkinny: return "mnb_skinny_kernel";
     case kMnbKernelGemv: return "mnb_gemv_kernel";
     case kMnbKernelGemmMfma: return "mnb_gemm_mfma_kernel";
     case kMnbKernelGemmGeneric: return "mnb_gemm_generic_kernel";
@@ -192,8 +194,7 @@ extern "C" {
 size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                             int a_dtype) {
   if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0 || M == 0) return 0;
-  MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
-  return mnb_gemv_workspace_bytes(L, (int64_t)M);
+  return 0;  // no kernel needs per-call scratch at present
 }
 
 int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
@@ -220,6 +221,7 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
   hipStream_t s = (hipStream_t)stream;
   hipError_t e;
   switch (mnb_select_kernel(a)) {
+    case kMnbKernelSkinny: e = mnb_launch_skinny(a, s); break;
     case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
     case kMnbKernelGemmMfma: e = mnb_launch_gemm_mfma(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
@@ -277,7 +279,8 @@ const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_
   MnbGemmArgs a{};
   a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, 0);
   a.M = (int64_t)M;
-  a.lda = (int64_t)K;
+  a.lda = (int64_t)((K + 7) / 8 * 8);  // assume the usual aligned activations
+  a.A = nullptr;
   return mnb_kernel_name(mnb_select_kernel(a), a.L);
 }
 

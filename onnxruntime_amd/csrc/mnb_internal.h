@@ -19,7 +19,8 @@ struct MnbGemmArgs {
 
 enum MnbKernelKind {
   kMnbKernelNone = 0,
-  kMnbKernelGemv,       // M <= 16, dequantising GEMV (VALU dot products)
+  kMnbKernelSkinny,     // fp16, M <= 16: dequantising skinny GEMM on the matrix cores
+  kMnbKernelGemv,       // fp32, M <= 16: dequantising GEMV (VALU dot products, activations in SGPRs)
   kMnbKernelGemmMfma,   // fp16, LDS-staged MFMA GEMM
   kMnbKernelGemmGeneric // any shape / fp32 large M: simple tile kernel
 };
@@ -33,7 +34,9 @@ hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* sc
                                         int64_t K, int bits, int bs, int dtype, hipStream_t s);
 hipError_t mnb_launch_dequant_packed(void* dst, const void* packed, const MnbLayout& L, hipStream_t s);
 
-size_t mnb_gemv_workspace_bytes(const MnbLayout& L, int64_t M);
+bool mnb_skinny_applicable(const MnbGemmArgs& a);
+hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s);
+bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_mfma(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);

@@ -1,0 +1,489 @@
+// fp16 decode kernel for 1 <= M <= 16: dequantising "skinny" GEMM on the matrix cores.
+//
+// Same contract as the reference's decode loop (MlasQ4GemmKernelBlkLen32PlusAvx512f,
+// onnxruntime/core/mlas/lib/sqnbitgemm_kernel_avx_common_fp32.h:288-639): Y = A x dequant(B)^T (+ bias), fp32
+// accumulation, one narrowing of Y.  The job is HBM-bound; the point of this design is to spend as few VALU
+// instructions per weight byte as possible so the load pipe never waits for arithmetic:
+//
+//  * v_mfma_f32_16x16x32_f16 does the dot products: rows = the (up to 16) rows of A, columns = 16 output columns.
+//    Lane (j = lane%16, kq = lane/16) reads ONE 16-byte vector of column j, k-group kq of a chunk of 4 k-groups, and
+//    each of its 32-bit words is the B operand of one MFMA (the contraction index may be permuted freely as long
+//    as A uses the same permutation).
+//  * MODE 0 (block_size >= chunk): the B operand is the raw "magic" half 1024+q (low nibbles, bytes) or 64+q (high
+//    nibbles: (w & 0x00F000F0) | 0x5400 is the half 64+q) -- 5 bit operations per 8 weights, no subtraction, no
+//    multiplication.  The offsets and the zero point are removed afterwards, exactly, per (row, column, block):
+//        sum_k a_k (q_k - zp) = D - C1 - zp * C2,   C1 = sum_k off_k a_k,  C2 = sum_k a_k
+//    where -C1 and -C2 come out of MFMAs of the same A operands against constant operands (-off_k and -1 in every
+//    lane, so each lane receives the values of its own rows), -C1 seeds the accumulator of the weight MFMAs, and
+//    the scale is applied to the block sum in fp32.
+//  * MODE 1 (smaller blocks): exact (q - zp) halves times the fp16 scale (bit-identical to the reference's fp16
+//    dequantisation), accumulated across blocks by the MFMA.
+//  * The A operands come straight from global memory (L2 hits after the first workgroup) when the rows of A are
+//    16-byte aligned -- every load of a wavefront's first two chunks is issued before anything is waited for;
+//    otherwise the rows are staged in LDS phase by phase (zero-filled beyond K, any alignment).
+//  * K is split over the wavefronts of a workgroup and reduced through LDS in a fixed order; nothing is split over
+//    workgroups, so there is no cross-workgroup synchronisation and no workspace.
+#include <cstdio>
+#include <cstdlib>
+
+#include "mnb_device.cuh"
+#include "mnb_internal.h"
+
+namespace {
+
+struct SkinnyParams {
+  const _Float16* A;
+  const uint4* W;
+  const uint8_t* meta;
+  const _Float16* bias;
+  _Float16* C;
+  int64_t lda, ldc, Npad;
+  int M, N, K;
+  int bs_shift;
+  int chunks;       // chunks that hold elements below K
+  int phase_chunks; // chunks staged in LDS at a time
+  int mtr;          // rows of A staged (power of two >= M, <= 16)
+  int a_vec_ok;     // A allows 16-byte loads
+  uint32_t uc[4];   // UnpackConsts
+};
+
+constexpr int kLdsPad = 8;  // halves of padding per staged row
+
+// The four constants of the nibble unpack.  They are passed as kernel arguments rather than written as literals:
+// VOP3 encodings of this ISA family take no literal, so with literals the compiler emits v_and_b32 + v_or_b32
+// (two instructions); with register operands it selects the single v_and_or_b32.
+struct UnpackConsts {
+  uint32_t mask_lo, mask_hi, magic_lo, magic_hi;  // 0x000F000F, 0x00F000F0, 0x64006400 (1024), 0x54005400 (64)
+};
+
+// One SGPR operand per VALU instruction: the masks stay scalar, the magics are moved to VGPRs once per kernel.
+// The move is opaque to the optimiser so that it cannot fold the value back into a literal.
+__device__ __forceinline__ UnpackConsts make_unpack_consts(const uint32_t* k) {
+  UnpackConsts u;
+  u.mask_lo = k[0];
+  u.mask_hi = k[1];
+  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic_lo) : "s"(k[2]));
+  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic_hi) : "s"(k[3]));
+  return u;
+}
+
+// raw magic halves of one 32-bit word: 4-bit -> 8 halves {1024+e0,1024+e1,64+e2,64+e3,1024+e4,1024+e5,64+e6,64+e7}
+__device__ __forceinline__ h8_t raw4(uint32_t w, const UnpackConsts& u) {
+  const uint32_t w8 = w >> 8;
+  uint4 r;
+  r.x = (w & u.mask_lo) | u.magic_lo;
+  r.y = (w & u.mask_hi) | u.magic_hi;
+  r.z = (w8 & u.mask_lo) | u.magic_lo;
+  r.w = (w8 & u.mask_hi) | u.magic_hi;
+  return __builtin_bit_cast(h8_t, r);
+}
+// 8-bit: two words -> 8 halves 1024+b
+__device__ __forceinline__ h8_t raw8(uint32_t w0, uint32_t w1) {
+  uint4 r;
+  r.x = __builtin_amdgcn_perm(kMagic, w0, 0x07010700u);
+  r.y = __builtin_amdgcn_perm(kMagic, w0, 0x07030702u);
+  r.z = __builtin_amdgcn_perm(kMagic, w1, 0x07010700u);
+  r.w = __builtin_amdgcn_perm(kMagic, w1, 0x07030702u);
+  return __builtin_bit_cast(h8_t, r);
+}
+
+// ---- registers of one chunk: weights, meta and (direct variant) the A operands ---------------------------------
+template <int BITS, int T>
+struct ChunkRegs {
+  uint4 w[T];
+  uint32_t m0[T];  // meta entry of the lane's (first) block: raw bits (32 with zero points, else 16)
+  uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
+};
+
+template <int BITS, bool HAS_ZP, int MODE, int T>
+__device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq, int64_t col0, ChunkRegs<BITS, T>& R) {
+  constexpr int GK = 128 / BITS;
+  constexpr int CK = 4 * GK;
+  // small loads first: memory returns in issue order, and the weights are waited for tile by tile
+  auto meta_at = [&](int64_t idx) -> uint32_t {
+    if constexpr (HAS_ZP)
+      return reinterpret_cast<const uint32_t*>(p.meta)[idx];
+    else
+      return reinterpret_cast<const uint16_t*>(p.meta)[idx];
+  };
+  if constexpr (MODE == 0) {
+    const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
+#pragma unroll
+    for (int t = 0; t < T; ++t) R.m0[t] = meta_at(kb * p.Npad + col0 + t * 16);
+  } else {
+    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      R.m0[t] = meta_at((k0 >> p.bs_shift) * p.Npad + col0 + t * 16);
+      if constexpr (BITS == 4) R.m1[t] = meta_at(((k0 + 16) >> p.bs_shift) * p.Npad + col0 + t * 16);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < T; ++t) R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + col0 + t * 16];
+}
+
+template <int BITS, bool HAS_ZP>
+__device__ __forceinline__ void decode_meta(uint32_t raw, _Float16& s, _Float16& neg_1024_plus_zp) {
+  if constexpr (HAS_ZP) {
+    const h2_t m = mnb_as_h2(raw);
+    s = m.x;
+    neg_1024_plus_zp = m.y;
+  } else {
+    s = __builtin_bit_cast(_Float16, (uint16_t)raw);
+    neg_1024_plus_zp = (_Float16)(-(1024.0f + (float)(1 << (BITS - 1))));
+  }
+}
+
+// constant MFMA B operands (identical in every lane) that turn the A operands into the correction terms
+struct BConst {
+  h8_t off;  // -(offset of the raw half at each of the 8 positions of a word [+ default zero point])
+  h8_t one;  // -1
+};
+
+// One chunk: T column tiles x (4 k-groups) against the 16-row A operands af[].
+template <int BITS, bool HAS_ZP, int MODE, int T>
+__device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t* af, const BConst& bc,
+                                              const UnpackConsts& uc, f4_t* y) {
+  constexpr int NI = (128 / BITS) / 8;
+  if constexpr (MODE == 0) {
+    // init[m] = -sum_k (off_k + zp) a[m][k] (no zero points) or -sum_k off_k a[m][k]; nc2[m] = -sum_k a[m][k].
+    // The constant operands are the same in every lane, so every lane receives the value of its own rows.
+    const f4_t zero = f4_t{0.f, 0.f, 0.f, 0.f};
+    f4_t init = zero, nc2 = zero;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) init = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bc.off, init, 0, 0, 0);
+    if constexpr (HAS_ZP) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) nc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bc.one, nc2, 0, 0, 0);
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      _Float16 s, nz;
+      decode_meta<BITS, HAS_ZP>(R.m0[t], s, nz);
+      const float sf = (float)s;
+      const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
+      f4_t d = init;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        h8_t b;
+        if constexpr (BITS == 4)
+          b = raw4(wd[i], uc);
+        else
+          b = raw8(wd[2 * i], wd[2 * i + 1]);
+        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], b, d, 0, 0, 0);
+      }
+      if constexpr (HAS_ZP) {
+        const float zp = -(float)nz - 1024.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, __builtin_fmaf(zp, nc2[r], d[r]), y[t][r]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, d[r], y[t][r]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
+      _Float16 s0, s1, nz0, nz1;
+      decode_meta<BITS, HAS_ZP>(R.m0[t], s0, nz0);
+      if constexpr (BITS == 4) {
+        decode_meta<BITS, HAS_ZP>(R.m1[t], s1, nz1);
+      } else {
+        s1 = s0;
+        nz1 = nz0;
+      }
+      const ZpH z0 = mnb_zp_h(nz0), z1 = mnb_zp_h(nz1);
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        h2_t d[4];
+        const bool second = (BITS == 4) && i >= 2;
+        const ZpH& z = second ? z1 : z0;
+        const h2_t s2 = mnb_h2(second ? s1 : s0);
+        if constexpr (BITS == 4) {
+          mnb_unpack4_h(wd[i], z, d);
+        } else {
+          mnb_unpack8_h(wd[2 * i], z, d);
+          mnb_unpack8_h(wd[2 * i + 1], z, d + 2);
+        }
+        uint4 bw;
+        bw.x = mnb_as_u32(d[0] * s2);
+        bw.y = mnb_as_u32(d[1] * s2);
+        bw.z = mnb_as_u32(d[2] * s2);
+        bw.w = mnb_as_u32(d[3] * s2);
+        y[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], __builtin_bit_cast(h8_t, bw), y[t], 0, 0, 0);
+      }
+    }
+  }
+}
+
+template <int BITS, bool HAS_ZP>
+__device__ __forceinline__ BConst make_bconst() {
+  // offsets the raw halves carry: 1024 (low nibbles, bytes) and 64 (high nibbles); without zero points the
+  // default zero point 2^(bits-1) is folded in.  All values are integers below 2048: exact in fp16.
+  const float zp = HAS_ZP ? 0.f : (float)(1 << (BITS - 1));
+  const _Float16 lo = (_Float16)(-(1024.0f + zp));
+  const _Float16 hi = (_Float16)(-((BITS == 4 ? 64.0f : 1024.0f) + zp));
+  const _Float16 m1 = (_Float16)(-1.0f);
+  BConst bc;
+  bc.off = h8_t{lo, lo, hi, hi, lo, lo, hi, hi};
+  bc.one = h8_t{m1, m1, m1, m1, m1, m1, m1, m1};
+  return bc;
+}
+
+// Reduce the per-wavefront tiles through LDS in wavefront order and write Y.
+// Lane (j, kq), register r of tile t holds row 4*kq + r, column n0 + 16 t + j; only rows < M travel.
+template <int T, int NW>
+__device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* red, const f4_t* y, int wave, int lane,
+                                                int64_t n0) {
+  const int kq = lane >> 4;
+  if constexpr (NW > 1) {
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (4 * kq + r < p.M) red[(wave * T * 4 + t * 4 + r) * 64 + lane] = y[t][r];
+    __syncthreads();
+  }
+  for (int i = threadIdx.x; i < T * 4 * 64; i += NW * 64) {
+    const int l = i & 63, tr = i >> 6;
+    const int t = tr >> 2, r = tr & 3;
+    const int m = 4 * (l >> 4) + r;
+    const int64_t n = n0 + t * 16 + (l & 15);
+    if (m >= p.M || n >= p.N) continue;
+    float sum = 0.f;
+    if constexpr (NW > 1) {
+#pragma unroll
+      for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * T * 4 + tr) * 64 + l];
+    } else {
+      sum = y[t][r];
+    }
+    if (p.bias) sum += (float)p.bias[n];
+    p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
+  }
+}
+
+// ---- direct variant: A operands straight from global memory (16-byte aligned rows), no barrier before the end ----
+// Two chunks are always in flight per wavefront (all of them when a wavefront owns at most two).
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW>
+__global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams p) {
+  constexpr int GK = 128 / BITS;
+  constexpr int NI = GK / 8;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, kq = lane >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
+  const int64_t col0 = n0 + j;
+  int arow = j & (p.mtr - 1);
+  if (arow >= p.M) arow = p.M - 1;
+  const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
+
+  f4_t y[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const BConst bconst = make_bconst<BITS, HAS_ZP>();
+  const UnpackConsts uc = make_unpack_consts(p.uc);
+
+  auto load_a = [&](int c, h8_t* af) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      af[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
+    }
+  };
+
+  ChunkRegs<BITS, T> R0, R1;
+  h8_t a0[NI], a1[NI];
+  int c = wave;
+  if (c < p.chunks) {
+    load_a(c, a0);
+    load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R0);
+  }
+  if (c + NW < p.chunks) {
+    load_a(c + NW, a1);
+    load_chunk<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, col0, R1);
+  }
+  for (; c < p.chunks; c += 2 * NW) {
+    compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
+    if (c + 2 * NW < p.chunks) {
+      load_a(c + 2 * NW, a0);
+      load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 2 * NW, kq, col0, R0);
+    }
+    if (c + NW < p.chunks) {
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
+      if (c + 3 * NW < p.chunks) {
+        load_a(c + 3 * NW, a1);
+        load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 3 * NW, kq, col0, R1);
+      }
+    }
+  }
+  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
+}
+
+// ---- staged variant: any alignment of A; rows staged in LDS phase by phase -------------------------------------
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW>
+__global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams p) {
+  constexpr int GK = 128 / BITS;  // k per 16-byte vector: 32 or 16
+  constexpr int NI = GK / 8;      // MFMAs per vector: 4 or 2
+  constexpr int CK = 4 * GK;      // k per chunk: 128 or 64
+  extern __shared__ __align__(16) unsigned char smem[];
+  _Float16* As = reinterpret_cast<_Float16*>(smem);
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, kq = lane >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
+  const int64_t col0 = n0 + j;
+  const int row_stride = p.phase_chunks * CK + kLdsPad;  // halves
+  const int arow = j & (p.mtr - 1);                      // staged row this lane feeds to the MFMA A operand
+
+  f4_t y[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const BConst bconst = make_bconst<BITS, HAS_ZP>();
+  const UnpackConsts uc = make_unpack_consts(p.uc);
+
+  for (int ph0 = 0; ph0 < p.chunks; ph0 += p.phase_chunks) {
+    const int ph1 = min(ph0 + p.phase_chunks, p.chunks);
+    // this wavefront's first weight loads go out before the staging barrier
+    const int c_first = ph0 + wave;
+    ChunkRegs<BITS, T> Rn;
+    if (c_first < ph1) load_chunk<BITS, HAS_ZP, MODE, T>(p, c_first, kq, col0, Rn);
+    // stage rows [0, mtr) of A for k in [ph0*CK, ph1*CK): zero beyond K, rows >= M repeat row M-1
+    __syncthreads();
+    {
+      const int kbase = ph0 * CK;
+      const int kext = (ph1 - ph0) * CK;
+      for (int i = threadIdx.x; i < p.mtr * kext; i += NW * 64) {
+        const int r = i / kext, kk = i % kext;
+        const int k = kbase + kk;
+        const int rr = r < p.M ? r : p.M - 1;
+        As[r * row_stride + kk] = (k < p.K) ? p.A[(int64_t)rr * p.lda + k] : (_Float16)0.0f;
+      }
+    }
+    __syncthreads();
+    for (int c = c_first; c < ph1; c += NW) {
+      const ChunkRegs<BITS, T> Rc = Rn;
+      if (c + NW < ph1) load_chunk<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, col0, Rn);
+      h8_t af[NI];
+      const _Float16* abase = As + arow * row_stride + ((c - ph0) * 4 + kq) * GK;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) af[i] = *reinterpret_cast<const h8_t*>(abase + 8 * i);
+      compute_chunk<BITS, HAS_ZP, MODE, T>(Rc, af, bconst, uc, y);
+    }
+  }
+  __syncthreads();
+  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
+}
+
+struct SkinnyPlan {
+  int mode, t, nw, phase_chunks, mtr;
+  size_t smem;
+};
+
+int pow2_ceil(int v) {
+  int r = 1;
+  while (r < v) r <<= 1;
+  return r;
+}
+
+SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct) {
+  SkinnyPlan pl;
+  const int GK = L.group_k, CK = 4 * GK;
+  const int chunks = (int)((L.K + CK - 1) / CK);
+  pl.mode = (L.bs >= CK) ? 0 : 1;
+  pl.mtr = pow2_ceil((int)M);
+  // workgroups: as many column slabs as fill the chip; wide slabs (T = 4) amortise the A operands best
+  const int64_t tiles = (L.N + 15) / 16;
+  pl.t = tiles >= 4 * 200 ? 4 : tiles >= 2 * 200 ? 2 : 1;
+  // wavefronts per workgroup: aim for >= 2 chunks per wavefront
+  pl.nw = chunks >= 32 ? 16 : chunks >= 16 ? 8 : 4;
+  if (const char* e = getenv("MNB_SKINNY_PLAN")) {  // tuning override "<T>,<NW>"
+    int t = 0, nw = 0;
+    if (sscanf(e, "%d,%d", &t, &nw) == 2 && (t == 1 || t == 2 || t == 4) && (nw == 4 || nw == 8 || nw == 16)) {
+      pl.t = t;
+      pl.nw = nw;
+    }
+  }
+  // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
+  const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
+  pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
+  if (!direct) pl.nw = 4;
+  const size_t a_bytes = direct ? 0 : (size_t)pl.mtr * (pl.phase_chunks * CK + kLdsPad) * 2;
+  const size_t red_bytes = (size_t)pl.nw * pl.t * 4 * 64 * 4;
+  pl.smem = a_bytes > red_bytes ? a_bytes : red_bytes;
+  return pl;
+}
+
+template <int BITS, bool HAS_ZP, int MODE, int T>
+hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
+  dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)));
+  if (p.a_vec_ok) {
+    switch (pl.nw) {
+      case 16: mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, 16><<<grid, dim3(1024), pl.smem, s>>>(p); break;
+      case 8: mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, 8><<<grid, dim3(512), pl.smem, s>>>(p); break;
+      default: mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, 4><<<grid, dim3(256), pl.smem, s>>>(p); break;
+    }
+  } else {
+    // rare: A not 16-byte aligned or K not a multiple of 8 -- one configuration is enough
+    mnb_skinny_staged_kernel<BITS, HAS_ZP, MODE, T, 4><<<grid, dim3(256), pl.smem, s>>>(p);
+  }
+  return hipGetLastError();
+}
+
+template <int BITS, bool HAS_ZP, int MODE>
+hipError_t launch_mode(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
+  switch (pl.t) {
+    case 4: return launch_t<BITS, HAS_ZP, MODE, 4>(p, pl, s);
+    case 2: return launch_t<BITS, HAS_ZP, MODE, 2>(p, pl, s);
+    default: return launch_t<BITS, HAS_ZP, MODE, 1>(p, pl, s);
+  }
+}
+
+template <int BITS, bool HAS_ZP>
+hipError_t launch_zp(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
+  return pl.mode == 0 ? launch_mode<BITS, HAS_ZP, 0>(p, pl, s) : launch_mode<BITS, HAS_ZP, 1>(p, pl, s);
+}
+
+int log2i(int v) {
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+
+}  // namespace
+
+bool mnb_skinny_applicable(const MnbGemmArgs& a) {
+  return a.L.dtype == kMnbDtypeFloat16 && a.M >= 1 && a.M <= 16;
+}
+
+hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
+  const MnbLayout& L = a.L;
+  // direct variant: 16-byte loads of whole chunks of A
+  const bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
+  SkinnyPlan pl = skinny_plan(L, a.M, a_vec_ok);
+  SkinnyParams p{};
+  p.A = reinterpret_cast<const _Float16*>(a.A);
+  p.W = reinterpret_cast<const uint4*>(a.packed);
+  p.meta = reinterpret_cast<const uint8_t*>(a.packed) + L.meta_off;
+  p.bias = reinterpret_cast<const _Float16*>(a.bias);
+  p.C = reinterpret_cast<_Float16*>(a.C);
+  p.lda = a.lda;
+  p.ldc = a.ldc;
+  p.Npad = L.Npad;
+  p.M = (int)a.M;
+  p.N = (int)L.N;
+  p.K = (int)L.K;
+  p.bs_shift = log2i(L.bs);
+  const int CK = 4 * L.group_k;
+  p.chunks = (int)((L.K + CK - 1) / CK);
+  p.phase_chunks = pl.phase_chunks;
+  p.mtr = pl.mtr;
+  p.a_vec_ok = a_vec_ok;
+  p.uc[0] = 0x000F000Fu;
+  p.uc[1] = 0x00F000F0u;
+  p.uc[2] = 0x64006400u;
+  p.uc[3] = 0x54005400u;
+  if (L.bits == 4) return L.has_zp ? launch_zp<4, true>(p, pl, s) : launch_zp<4, false>(p, pl, s);
+  return L.has_zp ? launch_zp<8, true>(p, pl, s) : launch_zp<8, false>(p, pl, s);
+}

@@ -134,7 +134,7 @@ class MatMulNBits:
         key = (device, torch.cuda.current_stream(device).cuda_stream)
         ws = self._workspace.get(key)
         if ws is None or ws.numel() < nbytes:
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)  # tickets start at zero
             self._workspace[key] = ws
         return ws
 
