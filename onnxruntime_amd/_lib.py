@@ -8,7 +8,10 @@ import ctypes
 from ctypes import c_int, c_int64, c_size_t, c_void_p, c_char_p
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libmnb_mi355x.so"
+import os
+
+# MNB_LIB_PATH points at an alternative build of the same library (kernel experiments); default: the in-tree one.
+LIB_PATH = Path(os.environ.get("MNB_LIB_PATH") or Path(__file__).resolve().parent / "libmnb_mi355x.so")
 
 DTYPE_FLOAT = 1
 DTYPE_UINT8 = 2

@@ -174,7 +174,7 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
   if (a.L.dtype == kMnbDtypeFloat16) {
     // 16-byte activation loads: base and row pitch aligned, no partial 8-element chunk at the end of a row
     const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (a.L.K % 8 == 0);
-    if (aligned) return kMnbKernelGemmMfma;
+    if (aligned) return a.M > 128 ? kMnbKernelGemm256 : kMnbKernelGemmMfma;
   }
   return kMnbKernelGemmGeneric;
 }
@@ -184,6 +184,7 @@ const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout&) {
     case kMnbKernelSkinny: return "mnb_skinny_kernel";
     case kMnbKernelGemv: return "mnb_gemv_kernel";
     case kMnbKernelGemmMfma: return "mnb_gemm_mfma_kernel";
+    case kMnbKernelGemm256: return "mnb_gemm256_kernel";
     case kMnbKernelGemmGeneric: return "mnb_gemm_generic_kernel";
     default: return "none";
   }
@@ -224,6 +225,7 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
     case kMnbKernelSkinny: e = mnb_launch_skinny(a, s); break;
     case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
     case kMnbKernelGemmMfma: e = mnb_launch_gemm_mfma(a, s); break;
+    case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }
   return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbGemm");

@@ -119,7 +119,7 @@ __device__ __forceinline__ void mnb_dequant_group_h(const uint4& v, const uint8_
   for (int b = 0; b < nblk; ++b) {
     _Float16 s;
     ZpH z;
-    mnb_load_meta_h<HAS_ZP, BITS>(meta, ((k0 + b * bs) / bs) * Npad + n, s, z);
+    mnb_load_meta_h<HAS_ZP, BITS>(meta, ((k0 + b * bs) / bs) * Npad + mnb_meta_col(n), s, z);
     const h2_t s2 = mnb_h2(s);
     const int words = 4 / nblk;
     for (int i = 0; i < words; ++i) {
@@ -154,7 +154,7 @@ __device__ __forceinline__ void mnb_dequant_group_f(const uint4& v, const uint8_
   const int nblk = (bs < GK) ? GK / bs : 1;
   for (int b = 0; b < nblk; ++b) {
     float s, zp;
-    mnb_load_meta_f<HAS_ZP, BITS>(meta, ((k0 + b * bs) / bs) * Npad + n, s, zp);
+    mnb_load_meta_f<HAS_ZP, BITS>(meta, ((k0 + b * bs) / bs) * Npad + mnb_meta_col(n), s, zp);
     const int words = 4 / nblk;
     for (int i = 0; i < words; ++i) {
       const int wi = b * words + i;

@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_gemv_kernel(GemvParams p) {
       const int g = c + u;
       if (g < kg1) {
         const int64_t kb = SMALL_BS ? (int64_t)g * 2 : (((int64_t)g * GK) >> p.bs_shift);
-        mnb_gemv_group<T, BITS, HAS_ZP, SMALL_BS, MT>(w[u], meta, kb * p.Npad + n, p.Npad, A + (int64_t)g * GK, p.lda,
+        mnb_gemv_group<T, BITS, HAS_ZP, SMALL_BS, MT>(w[u], meta, kb * p.Npad + mnb_meta_col(n), p.Npad, A + (int64_t)g * GK, p.lda,
                                                       p.M, acc);
       }
     }
@@ -189,7 +189,7 @@ __global__ void __launch_bounds__(64) mnb_gemm_generic_kernel(GemvParams p) {
     float wv[GK];
 #pragma unroll
     for (int b = 0; b < NBLK; ++b) {
-      const int64_t midx = (kb + b) * p.Npad + n;
+      const int64_t midx = (kb + b) * p.Npad + mnb_meta_col(n);
       if constexpr (sizeof(T) == 2) {
         // exact integers times the widened scale: the fp32 product is exact, as on the reference's x64 path
         _Float16 s;

@@ -21,7 +21,8 @@ enum MnbKernelKind {
   kMnbKernelNone = 0,
   kMnbKernelSkinny,     // fp16, M <= 16: dequantising skinny GEMM on the matrix cores
   kMnbKernelGemv,       // fp32, M <= 16: dequantising GEMV (VALU dot products, activations in SGPRs)
-  kMnbKernelGemmMfma,   // fp16, LDS-staged MFMA GEMM
+  kMnbKernelGemmMfma,   // fp16, LDS-staged MFMA GEMM, 128 x 128 tiles (17 <= M <= 128)
+  kMnbKernelGemm256,    // fp16, LDS-staged MFMA GEMM, 256 x 256 tiles (M > 128)
   kMnbKernelGemmGeneric // any shape / fp32 large M: simple tile kernel
 };
 
@@ -39,4 +40,5 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s);
 bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_mfma(const MnbGemmArgs& a, hipStream_t s);
+hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);

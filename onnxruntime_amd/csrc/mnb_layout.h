@@ -11,7 +11,9 @@
 //                             8-bit: bytes stay in k order.
 //   meta[KBp][Npad]           per (block, column): fp16 model {half scale, half -(1024+zp)} (4 B) or {half scale}
 //                             (2 B) when there are no zero points; fp32 model {float scale, float zp} (8 B) or
-//                             {float scale} (4 B).
+//                             {float scale} (4 B).  Inside every slab of 64 columns the entries are stored in the
+//                             order (n%16)*4 + (n%64)/16, so that the four 16-column tiles a matrix-core lane
+//                             works on are adjacent and arrive with one vector load (mnb_meta_col).
 //
 //   Npad = N rounded up to 256, Kpad = k_blocks*block_size rounded up to 128, KG = Kpad*bits/128, KBp = Kpad/bs.
 //   Padding columns and padding k hold zero weights and zero scales, so loads never need a bounds check.
@@ -43,6 +45,9 @@ struct MnbLayout {
 };
 
 MNB_HD int64_t mnb_round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+// position of column n inside a meta row
+MNB_HD int64_t mnb_meta_col(int64_t n) { return (n & ~(int64_t)63) | ((n & 15) << 2) | ((n >> 4) & 3); }
 
 MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dtype, int has_zp) {
   MnbLayout L;

@@ -54,6 +54,7 @@ __global__ void __launch_bounds__(256) mnb_pack_meta_kernel(const T* __restrict_
   if (idx >= L.KBp * L.Npad) return;
   const int64_t kb = idx / L.Npad;
   const int64_t n = idx % L.Npad;
+  const int64_t dst = kb * L.Npad + mnb_meta_col(n);
   const bool valid = n < L.N && kb < L.k_blocks;
   T s = valid ? scales[n * L.k_blocks + kb] : (T)0;
   int z = 0;
@@ -72,15 +73,15 @@ __global__ void __launch_bounds__(256) mnb_pack_meta_kernel(const T* __restrict_
       h2_t m;
       m.x = s;
       m.y = (_Float16)(-(1024.0f + (float)z));
-      reinterpret_cast<uint32_t*>(meta)[idx] = mnb_as_u32(m);
+      reinterpret_cast<uint32_t*>(meta)[dst] = mnb_as_u32(m);
     } else {
-      reinterpret_cast<_Float16*>(meta)[idx] = s;
+      reinterpret_cast<_Float16*>(meta)[dst] = s;
     }
   } else {
     if constexpr (HAS_ZP) {
-      reinterpret_cast<float2*>(meta)[idx] = make_float2(s, (float)z);
+      reinterpret_cast<float2*>(meta)[dst] = make_float2(s, (float)z);
     } else {
-      reinterpret_cast<float*>(meta)[idx] = s;
+      reinterpret_cast<float*>(meta)[dst] = s;
     }
   }
 }

@@ -95,28 +95,48 @@ struct ChunkRegs {
   uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
 };
 
+// T adjacent meta entries (2 or 4 bytes each) with one load; dst holds the raw bits of each entry
+template <bool HAS_ZP, int T>
+__device__ __forceinline__ void load_meta_vec(const uint8_t* __restrict__ meta, int64_t first, uint32_t* dst) {
+  if constexpr (HAS_ZP) {
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(meta) + first;
+    if constexpr (T == 4) {
+      const uint4 v = *reinterpret_cast<const uint4*>(q);
+      dst[0] = v.x, dst[1] = v.y, dst[2] = v.z, dst[3] = v.w;
+    } else if constexpr (T == 2) {
+      const uint2 v = *reinterpret_cast<const uint2*>(q);
+      dst[0] = v.x, dst[1] = v.y;
+    } else {
+      dst[0] = *q;
+    }
+  } else {
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(meta) + first;
+    if constexpr (T == 4) {
+      const uint2 v = *reinterpret_cast<const uint2*>(q);
+      dst[0] = v.x & 0xFFFFu, dst[1] = v.x >> 16, dst[2] = v.y & 0xFFFFu, dst[3] = v.y >> 16;
+    } else if constexpr (T == 2) {
+      const uint32_t v = *reinterpret_cast<const uint32_t*>(q);
+      dst[0] = v & 0xFFFFu, dst[1] = v >> 16;
+    } else {
+      dst[0] = *q;
+    }
+  }
+}
+
+// col0 = first column of the workgroup + j; the T tiles of a lane are columns col0 + 16 t.
 template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq, int64_t col0, ChunkRegs<BITS, T>& R) {
   constexpr int GK = 128 / BITS;
   constexpr int CK = 4 * GK;
   // small loads first: memory returns in issue order, and the weights are waited for tile by tile
-  auto meta_at = [&](int64_t idx) -> uint32_t {
-    if constexpr (HAS_ZP)
-      return reinterpret_cast<const uint32_t*>(p.meta)[idx];
-    else
-      return reinterpret_cast<const uint16_t*>(p.meta)[idx];
-  };
+  const int64_t mcol = mnb_meta_col(col0);  // entries of columns col0 + 16 t follow at mcol + t
   if constexpr (MODE == 0) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
-#pragma unroll
-    for (int t = 0; t < T; ++t) R.m0[t] = meta_at(kb * p.Npad + col0 + t * 16);
+    load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
   } else {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-      R.m0[t] = meta_at((k0 >> p.bs_shift) * p.Npad + col0 + t * 16);
-      if constexpr (BITS == 4) R.m1[t] = meta_at(((k0 + 16) >> p.bs_shift) * p.Npad + col0 + t * 16);
-    }
+    load_meta_vec<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0);
+    if constexpr (BITS == 4) load_meta_vec<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1);
   }
 #pragma unroll
   for (int t = 0; t < T; ++t) R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + col0 + t * 16];
@@ -145,6 +165,14 @@ template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t* af, const BConst& bc,
                                               const UnpackConsts& uc, f4_t* y) {
   constexpr int NI = (128 / BITS) / 8;
+#if defined(MNB_EXPERIMENT) && MNB_EXPERIMENT == 1
+  // loads only: fold every loaded register into y so nothing is optimised away
+  for (int t = 0; t < T; ++t) {
+    y[t][0] += __builtin_bit_cast(float, R.w[t].x ^ R.w[t].y ^ R.w[t].z ^ R.w[t].w ^ R.m0[t]);
+    y[t][1] += (float)af[t % NI][0];
+  }
+  return;
+#endif
   if constexpr (MODE == 0) {
     // init[m] = -sum_k (off_k + zp) a[m][k] (no zero points) or -sum_k off_k a[m][k]; nc2[m] = -sum_k a[m][k].
     // The constant operands are the same in every lane, so every lane receives the value of its own rows.
@@ -264,8 +292,10 @@ __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* re
 }
 
 // ---- direct variant: A operands straight from global memory (16-byte aligned rows), no barrier before the end ----
-// Two chunks are always in flight per wavefront (all of them when a wavefront owns at most two).
-template <int BITS, bool HAS_ZP, int MODE, int T, int NW>
+// CPW = chunks per wavefront when that is 1 or 2 for every wavefront (chunks == CPW * NW): everything is loaded up
+// front in straight-line code, so the compiler's s_waitcnt counts are exact and each tile is processed as soon as
+// its own vector has landed.  CPW = 0: general loop with two chunks in flight.
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW>
 __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams p) {
   constexpr int GK = 128 / BITS;
   constexpr int NI = GK / 8;
@@ -275,8 +305,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams
   const int j = lane & 15, kq = lane >> 4;
   const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
   const int64_t col0 = n0 + j;
-  int arow = j & (p.mtr - 1);
-  if (arow >= p.M) arow = p.M - 1;
+  const int arow = j < p.M ? j : p.M - 1;
   const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
 
   f4_t y[T];
@@ -285,35 +314,45 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams
   const BConst bconst = make_bconst<BITS, HAS_ZP>();
   const UnpackConsts uc = make_unpack_consts(p.uc);
 
+  // rows >= M of the MFMA A operand re-read row M-1: they are never stored
   auto load_a = [&](int c, h8_t* af) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      af[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
-    }
+    for (int i = 0; i < NI; ++i) af[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
   };
 
-  ChunkRegs<BITS, T> R0, R1;
-  h8_t a0[NI], a1[NI];
-  int c = wave;
-  if (c < p.chunks) {
-    load_a(c, a0);
-    load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R0);
-  }
-  if (c + NW < p.chunks) {
-    load_a(c + NW, a1);
-    load_chunk<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, col0, R1);
-  }
-  for (; c < p.chunks; c += 2 * NW) {
-    compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-    if (c + 2 * NW < p.chunks) {
-      load_a(c + 2 * NW, a0);
-      load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 2 * NW, kq, col0, R0);
+  if constexpr (CPW > 0) {
+    ChunkRegs<BITS, T> R[CPW];
+    h8_t a[CPW][NI];
+#pragma unroll
+    for (int q = 0; q < CPW; ++q) load_a(wave + q * NW, a[q]);
+#pragma unroll
+    for (int q = 0; q < CPW; ++q) load_chunk<BITS, HAS_ZP, MODE, T>(p, wave + q * NW, kq, col0, R[q]);
+#pragma unroll
+    for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, y);
+  } else {
+    ChunkRegs<BITS, T> R0, R1;
+    h8_t a0[NI], a1[NI];
+    int c = wave;
+    if (c < p.chunks) {
+      load_a(c, a0);
+      load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R0);
     }
     if (c + NW < p.chunks) {
-      compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
-      if (c + 3 * NW < p.chunks) {
-        load_a(c + 3 * NW, a1);
-        load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 3 * NW, kq, col0, R1);
+      load_a(c + NW, a1);
+      load_chunk<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, col0, R1);
+    }
+    for (; c < p.chunks; c += 2 * NW) {
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
+      if (c + 2 * NW < p.chunks) {
+        load_a(c + 2 * NW, a0);
+        load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 2 * NW, kq, col0, R0);
+      }
+      if (c + NW < p.chunks) {
+        compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
+        if (c + 3 * NW < p.chunks) {
+          load_a(c + 3 * NW, a1);
+          load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 3 * NW, kq, col0, R1);
+        }
       }
     }
   }
@@ -419,11 +458,25 @@ template <int BITS, bool HAS_ZP, int MODE, int T>
 hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
   dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)));
   if (p.a_vec_ok) {
+    const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
+#define MNB_SKINNY_LAUNCH(NW_, CPW_) \
+  mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
+#define MNB_SKINNY_CPW(NW_)               \
+  do {                                    \
+    if (cpw == 1)                         \
+      MNB_SKINNY_LAUNCH(NW_, 1);          \
+    else if (cpw == 2)                    \
+      MNB_SKINNY_LAUNCH(NW_, 2);          \
+    else                                  \
+      MNB_SKINNY_LAUNCH(NW_, 0);          \
+  } while (0)
     switch (pl.nw) {
-      case 16: mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, 16><<<grid, dim3(1024), pl.smem, s>>>(p); break;
-      case 8: mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, 8><<<grid, dim3(512), pl.smem, s>>>(p); break;
-      default: mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, 4><<<grid, dim3(256), pl.smem, s>>>(p); break;
+      case 16: MNB_SKINNY_CPW(16); break;
+      case 8: MNB_SKINNY_CPW(8); break;
+      default: MNB_SKINNY_CPW(4); break;
     }
+#undef MNB_SKINNY_CPW
+#undef MNB_SKINNY_LAUNCH
   } else {
     // rare: A not 16-byte aligned or K not a multiple of 8 -- one configuration is enough
     mnb_skinny_staged_kernel<BITS, HAS_ZP, MODE, T, 4><<<grid, dim3(256), pl.smem, s>>>(p);
