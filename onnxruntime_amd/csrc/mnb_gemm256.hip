@@ -15,6 +15,8 @@
 
 namespace {
 
+typedef uint32_t u4_t __attribute__((ext_vector_type(4)));  // plain register quad (HIP's uint4 struct resists SROA)
+
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // halves per staged row
 constexpr int THREADS = 256;
@@ -55,11 +57,18 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  uint4 a_reg[A_LOADS];
-  uint4 b_reg[GPK];
+  u4_t a_reg[A_LOADS];
+  u4_t b_reg[GPK];
   uint32_t m_reg[GPK * (SMALL_BS ? 2 : 1)];
 
   const int a_row = tid >> 3, a_kc = tid & 7;  // thread's first A chunk: row a_row (+32 per load), k chunk a_kc
+  const _Float16* a_ptr[A_LOADS];
+#pragma unroll
+  for (int i = 0; i < A_LOADS; ++i) {
+    int m = m0 + a_row + i * 32;
+    m = m < p.M ? m : p.M - 1;
+    a_ptr[i] = p.A + (int64_t)m * p.lda + a_kc * 8;
+  }
   const int64_t bcol = n0 + tid;
   const int64_t mcol = mnb_meta_col(bcol);
 
@@ -74,14 +83,14 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
     const int k0 = ks * BK;
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
-      const int m = m0 + a_row + i * 32, k = k0 + a_kc * 8;
-      a_reg[i] = (m < p.M && k < p.K) ? *reinterpret_cast<const uint4*>(p.A + (int64_t)m * p.lda + k)
-                                      : make_uint4(0, 0, 0, 0);
+      // unconditional loads (a predicated load serialises on its own zero fill): rows beyond M re-read row M-1
+      // and are never stored; K is a multiple of BK for this kernel
+      a_reg[i] = *reinterpret_cast<const u4_t*>(a_ptr[i] + k0);
     }
 #pragma unroll
     for (int g = 0; g < GPK; ++g) {
       const int64_t kg = (int64_t)ks * GPK + g;
-      b_reg[g] = p.W[kg * p.Npad + bcol];
+      b_reg[g] = *reinterpret_cast<const u4_t*>(p.W + kg * p.Npad + bcol);
       if constexpr (SMALL_BS) {
         m_reg[2 * g] = meta_at((kg * 2) * p.Npad + mcol);
         m_reg[2 * g + 1] = meta_at((kg * 2 + 1) * p.Npad + mcol);
@@ -105,7 +114,7 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
   // dequantise group g of this thread's column and write its GK halves to buffer `buf`
   auto store_b_group = [&](int buf, int g) {
     _Float16* brow = lds + buf * STAGE_HALVES + (BM + tid) * LDS_STRIDE + g * GK;
-    const uint32_t wd[4] = {b_reg[g].x, b_reg[g].y, b_reg[g].z, b_reg[g].w};
+    const uint32_t wd[4] = {b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]};
     h2_t s2a, s2b;
     ZpH za, zb;
     if constexpr (SMALL_BS) {
@@ -122,12 +131,8 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
         h2_t d[4];
         mnb_unpack4_h(wd[i], i < 2 ? za : zb, d);
         const h2_t s2 = i < 2 ? s2a : s2b;
-        uint4 o;
-        o.x = mnb_as_u32(d[0] * s2);
-        o.y = mnb_as_u32(d[1] * s2);
-        o.z = mnb_as_u32(d[2] * s2);
-        o.w = mnb_as_u32(d[3] * s2);
-        *reinterpret_cast<uint4*>(brow + i * 8) = o;
+        const u4_t o = {mnb_as_u32(d[0] * s2), mnb_as_u32(d[1] * s2), mnb_as_u32(d[2] * s2), mnb_as_u32(d[3] * s2)};
+        *reinterpret_cast<u4_t*>(brow + i * 8) = o;
       }
     } else {
 #pragma unroll
@@ -135,18 +140,15 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
         h2_t d[4];
         mnb_unpack8_h(wd[2 * i], za, d);
         mnb_unpack8_h(wd[2 * i + 1], za, d + 2);
-        uint4 o;
-        o.x = mnb_as_u32(d[0] * s2a);
-        o.y = mnb_as_u32(d[1] * s2a);
-        o.z = mnb_as_u32(d[2] * s2a);
-        o.w = mnb_as_u32(d[3] * s2a);
-        *reinterpret_cast<uint4*>(brow + i * 8) = o;
+        const u4_t o = {mnb_as_u32(d[0] * s2a), mnb_as_u32(d[1] * s2a), mnb_as_u32(d[2] * s2a),
+                        mnb_as_u32(d[3] * s2a)};
+        *reinterpret_cast<u4_t*>(brow + i * 8) = o;
       }
     }
   };
 
   auto store_a = [&](int buf, int i) {
-    *reinterpret_cast<uint4*>(lds + buf * STAGE_HALVES + (a_row + i * 32) * LDS_STRIDE + a_kc * 8) = a_reg[i];
+    *reinterpret_cast<u4_t*>(lds + buf * STAGE_HALVES + (a_row + i * 32) * LDS_STRIDE + a_kc * 8) = a_reg[i];
   };
 
   auto mfma_slab = [&](int buf, int kk) {

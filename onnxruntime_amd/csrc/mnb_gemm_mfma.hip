@@ -59,9 +59,14 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm_mfma_kernel(GemmParams p) {
     for (int i = 0; i < A_LOADS; ++i) {
       const int c = tid + i * THREADS;
       const int row = c >> 3, kc = c & 7;
-      const int m = m0 + row, k = k0 + kc * 8;
-      a_reg[i] = (m < p.M && k < p.K) ? *reinterpret_cast<const uint4*>(p.A + (int64_t)m * p.lda + k)
-                                      : make_uint4(0, 0, 0, 0);
+      // unconditional load from a clamped address, then a select: a predicated load would serialise the loop
+      int m = m0 + row;
+      m = m < p.M ? m : p.M - 1;
+      const int k = k0 + kc * 8;
+      const int kc_safe = k < p.K ? k : p.K - 8;
+      uint4 v = *reinterpret_cast<const uint4*>(p.A + (int64_t)m * p.lda + kc_safe);
+      if (k >= p.K) v = make_uint4(0, 0, 0, 0);
+      a_reg[i] = v;
     }
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
