@@ -174,7 +174,7 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
   if (a.L.dtype == kMnbDtypeFloat16) {
     // 16-byte activation loads: base and row pitch aligned, no partial 8-element chunk at the end of a row
     const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (a.L.K % 8 == 0);
-    if (aligned) return (a.M > 128 && a.L.K % 64 == 0) ? kMnbKernelGemm256 : kMnbKernelGemmMfma;
+    if (aligned) return (a.M > 128 && a.L.K % 128 == 0) ? kMnbKernelGemm256 : kMnbKernelGemmMfma;
   }
   return kMnbKernelGemmGeneric;
 }

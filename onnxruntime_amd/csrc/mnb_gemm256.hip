@@ -33,6 +33,24 @@ struct Gemm256Params {
   int ksteps;
 };
 
+// Scheduling pipeline of one slab section (16 MFMAs): after every MFMA a few of the other instructions of the
+// section, so they run in the MFMA's shadow; the 8 fragment reads go behind the first 8 MFMAs.  The closing
+// sched_barrier keeps the scheduler from mixing the MFMAs of different slabs (they reuse the same accumulators).
+template <bool VMEM, int VALU, int LDS_WRITE_EVERY>
+__device__ __forceinline__ void slab_pipeline() {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // 1 MFMA
+    if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // 1 LDS read
+    if (VMEM && i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // 1 VMEM read
+    if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
+    if constexpr (LDS_WRITE_EVERY > 0) {
+      if (i % LDS_WRITE_EVERY == LDS_WRITE_EVERY - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // 1 LDS write
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int BITS, bool HAS_ZP, bool SMALL_BS>
 __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int GK = 128 / BITS;                    // k per 16-byte group
@@ -57,20 +75,30 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  u4_t a_reg[A_LOADS];
-  u4_t b_reg[GPK];
-  uint32_t m_reg[GPK * (SMALL_BS ? 2 : 1)];
+  // two register sets for the global prefetch (distance: two k-steps), two fragment sets for the LDS prefetch
+  struct Stage {
+    u4_t a[A_LOADS];
+    u4_t b[GPK];
+    uint32_t m[GPK * (SMALL_BS ? 2 : 1)];
+  };
+  Stage R0, R1;
+  struct Frags {
+    h8_t a[4], b[4];
+  };
+  Frags F0, F1;
 
   const int a_row = tid >> 3, a_kc = tid & 7;  // thread's first A chunk: row a_row (+32 per load), k chunk a_kc
   const _Float16* a_ptr[A_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
+    // rows beyond M re-read row M-1 and are never stored (a predicated load would serialise the loop)
     int m = m0 + a_row + i * 32;
     m = m < p.M ? m : p.M - 1;
     a_ptr[i] = p.A + (int64_t)m * p.lda + a_kc * 8;
   }
   const int64_t bcol = n0 + tid;
   const int64_t mcol = mnb_meta_col(bcol);
+  const int last_step = p.ksteps - 1;
 
   auto meta_at = [&](int64_t idx) -> uint32_t {
     if constexpr (HAS_ZP)
@@ -79,23 +107,21 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
       return reinterpret_cast<const uint16_t*>(p.meta)[idx];
   };
 
-  auto load_global = [&](int ks) {
+  // k-steps past the end are clamped to the last one: the loop body stays branch free, the data is never used
+  auto load_global = [&](int ks_raw, Stage& R) {
+    const int ks = ks_raw < last_step ? ks_raw : last_step;
     const int k0 = ks * BK;
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      // unconditional loads (a predicated load serialises on its own zero fill): rows beyond M re-read row M-1
-      // and are never stored; K is a multiple of BK for this kernel
-      a_reg[i] = *reinterpret_cast<const u4_t*>(a_ptr[i] + k0);
-    }
+    for (int i = 0; i < A_LOADS; ++i) R.a[i] = *reinterpret_cast<const u4_t*>(a_ptr[i] + k0);
 #pragma unroll
     for (int g = 0; g < GPK; ++g) {
       const int64_t kg = (int64_t)ks * GPK + g;
-      b_reg[g] = *reinterpret_cast<const u4_t*>(p.W + kg * p.Npad + bcol);
+      R.b[g] = *reinterpret_cast<const u4_t*>(p.W + kg * p.Npad + bcol);
       if constexpr (SMALL_BS) {
-        m_reg[2 * g] = meta_at((kg * 2) * p.Npad + mcol);
-        m_reg[2 * g + 1] = meta_at((kg * 2 + 1) * p.Npad + mcol);
+        R.m[2 * g] = meta_at((kg * 2) * p.Npad + mcol);
+        R.m[2 * g + 1] = meta_at((kg * 2 + 1) * p.Npad + mcol);
       } else {
-        m_reg[g] = meta_at(((kg * GK) >> p.bs_shift) * p.Npad + mcol);
+        R.m[g] = meta_at(((kg * GK) >> p.bs_shift) * p.Npad + mcol);
       }
     }
   };
@@ -112,16 +138,16 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
   };
 
   // dequantise group g of this thread's column and write its GK halves to buffer `buf`
-  auto store_b_group = [&](int buf, int g) {
+  auto store_b_group = [&](int buf, int g, const Stage& R) {
     _Float16* brow = lds + buf * STAGE_HALVES + (BM + tid) * LDS_STRIDE + g * GK;
-    const uint32_t wd[4] = {b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]};
+    const uint32_t wd[4] = {R.b[g][0], R.b[g][1], R.b[g][2], R.b[g][3]};
     h2_t s2a, s2b;
     ZpH za, zb;
     if constexpr (SMALL_BS) {
-      decode(m_reg[2 * g], s2a, za);
-      decode(m_reg[2 * g + 1], s2b, zb);
+      decode(R.m[2 * g], s2a, za);
+      decode(R.m[2 * g + 1], s2b, zb);
     } else {
-      decode(m_reg[g], s2a, za);
+      decode(R.m[g], s2a, za);
       s2b = s2a;
       zb = za;
     }
@@ -147,60 +173,82 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
     }
   };
 
-  auto store_a = [&](int buf, int i) {
-    *reinterpret_cast<u4_t*>(lds + buf * STAGE_HALVES + (a_row + i * 32) * LDS_STRIDE + a_kc * 8) = a_reg[i];
+  auto store_a = [&](int buf, int i, const Stage& R) {
+    *reinterpret_cast<u4_t*>(lds + buf * STAGE_HALVES + (a_row + i * 32) * LDS_STRIDE + a_kc * 8) = R.a[i];
   };
 
-  auto mfma_slab = [&](int buf, int kk) {
+  auto read_frags = [&](int buf, int kk, Frags& F) {
     const _Float16* As = lds + buf * STAGE_HALVES;
     const _Float16* Bs = As + BM * LDS_STRIDE;
-    h8_t af[4], bf[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      af[t] = *reinterpret_cast<const h8_t*>(As + (wm * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
-      bf[t] = *reinterpret_cast<const h8_t*>(Bs + (wn * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
+      F.a[t] = *reinterpret_cast<const h8_t*>(As + (wm * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
+      F.b[t] = *reinterpret_cast<const h8_t*>(Bs + (wn * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
     }
+  };
+
+  auto mfma_slab = [&](const Frags& F) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(F.a[i], F.b[j], acc[i][j], 0, 0, 0);
   };
 
-  // ---- prologue: stage k-step 0 into buffer 0
-  load_global(0);
+  // staging work of one k-step in three parts (one per MFMA slab it hides behind)
+  auto store_third = [&](int buf, int q, const Stage& R) {
+    if (q == 0) {
 #pragma unroll
-  for (int i = 0; i < A_LOADS; ++i) store_a(0, i);
-#pragma unroll
-  for (int g = 0; g < GPK; ++g) store_b_group(0, g);
-  __syncthreads();
+      for (int i = 0; i < A_LOADS; ++i) store_a(buf, i, R);
+    } else if constexpr (GPK == 2) {
+      store_b_group(buf, q - 1, R);
+    } else {
+      store_b_group(buf, 2 * (q - 1), R);
+      store_b_group(buf, 2 * (q - 1) + 1, R);
+    }
+  };
 
-  for (int ks = 0; ks < p.ksteps; ++ks) {
+  // One k-step.  On entry: LDS buffer `cur` holds step ks, F0 holds its slab 0, Rn holds (or is receiving) step
+  // ks+1.  Slabs 0-2: MFMAs with, in their shadow, the global loads of step ks+2 (into Rf), the fragment reads of
+  // the following slab and the staging of step ks+1 into the other buffer.  Then the barrier: every wavefront has
+  // finished writing the other buffer and has its slab-3 fragments in registers, so buffer `cur` is free again.
+  // Slab 3 runs after the barrier, with the first fragments of step ks+1 fetched in its shadow.
+  auto k_step = [&](int ks, Stage& Rf, Stage& Rn) {
     const int cur = ks & 1, nxt = cur ^ 1;
-    const bool more = ks + 1 < p.ksteps;
-    if (more) load_global(ks + 1);
-    // four k-slabs of MFMAs; the staging of the next step is spread between them
-    mfma_slab(cur, 0);
-    if (more) {
-#pragma unroll
-      for (int i = 0; i < A_LOADS / 2; ++i) store_a(nxt, i);
-    }
-    mfma_slab(cur, 1);
-    if (more) {
-#pragma unroll
-      for (int i = A_LOADS / 2; i < A_LOADS; ++i) store_a(nxt, i);
-    }
-    mfma_slab(cur, 2);
-    if (more) {
-#pragma unroll
-      for (int g = 0; g < GPK / 2; ++g) store_b_group(nxt, g);
-    }
-    mfma_slab(cur, 3);
-    if (more) {
-#pragma unroll
-      for (int g = GPK / 2; g < GPK; ++g) store_b_group(nxt, g);
-    }
+    // slab 0: global loads of step ks+2, fragments of slab 1, the 8 A vectors of step ks+1 into the other buffer
+    load_global(ks + 2, Rf);
+    read_frags(cur, 1, F1);
+    mfma_slab(F0);
+    store_third(nxt, 0, Rn);
+    slab_pipeline<true, 3, 2>();
+    // slab 1: fragments of slab 2, first half of the weights of step ks+1
+    read_frags(cur, 2, F0);
+    mfma_slab(F1);
+    store_third(nxt, 1, Rn);
+    slab_pipeline<false, 6, 4>();
+    // slab 2: fragments of slab 3, second half of the weights
+    read_frags(cur, 3, F1);
+    mfma_slab(F0);
+    store_third(nxt, 2, Rn);
+    slab_pipeline<false, 6, 4>();
     __syncthreads();
+    // slab 3, behind the barrier: first fragments of step ks+1
+    read_frags(nxt, 0, F0);
+    mfma_slab(F1);
+    slab_pipeline<false, 0, 0>();
+  };
+
+  // ---- prologue: steps 0 and 1 in flight, step 0 staged
+  load_global(0, R0);
+  load_global(1, R1);
+#pragma unroll
+  for (int q = 0; q < 3; ++q) store_third(0, q, R0);
+  __syncthreads();
+  read_frags(0, 0, F0);
+
+  for (int ks = 0; ks < p.ksteps; ks += 2) {  // ksteps is even
+    k_step(ks, R0, R1);
+    k_step(ks + 1, R1, R0);
   }
 
   // ---- epilogue: D[i][j] of a 32x32 tile: lane holds column j = lane % 32, rows 8*(r/4) + 4*(lane/32) + r%4
@@ -258,7 +306,7 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.N = (int)a.L.N;
   p.K = (int)a.L.K;
   p.bs_shift = log2i(a.L.bs);
-  p.ksteps = (int)((a.L.K + BK - 1) / BK);
+  p.ksteps = (int)(a.L.K / BK);  // K is a multiple of 2 * BK
   if (a.L.bits == 4) {
     if (a.L.bs == 16) return a.L.has_zp ? launch<4, true, true>(p, s) : launch<4, false, true>(p, s);
     return a.L.has_zp ? launch<4, true, false>(p, s) : launch<4, false, false>(p, s);
