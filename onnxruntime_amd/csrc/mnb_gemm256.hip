@@ -1,9 +1,10 @@
 // Dequant-in-LDS MFMA GEMM for fp16 models and large M: 256 x 256 output tile per workgroup.
 //
 // Device counterpart of the reference's prefill loop (SQ4BitGemm_CompFp32, onnxruntime/core/mlas/lib/qnbitgemm.cpp:
-// 563-732).  Four wavefronts (2 x 2), each owning a 128 x 128 block of the tile as 4 x 4 v_mfma_f32_32x32x16_f16
-// accumulators (256 accumulator registers per lane).  Per k-step of 64:
-//   * every thread fetches 8 x 16 B of A and 2 (4-bit) or 4 (8-bit) x 16 B of packed weights for the NEXT step
+// 563-732).  Eight wavefronts (4 x 2, two per SIMD so that one can issue its staging work while the other owns the
+// matrix core), each owning a 64 x 128 block of the tile as 2 x 4 v_mfma_f32_32x32x16_f16 accumulators (128
+// accumulator registers per lane).  Per k-step of 64:
+//   * every thread fetches 4 x 16 B of A and 1 (4-bit) or 2 (8-bit) x 16 B of packed weights two steps ahead
 //     into registers while the matrix cores work on the current one;
 //   * the weights are dequantised to fp16 in registers (exact (q - zp), one rounding by the scale: bit-identical
 //     to the reference's fp16 dequantisation) and written, with the A rows, into the other LDS buffer;
@@ -19,7 +20,7 @@ typedef uint32_t u4_t __attribute__((ext_vector_type(4)));  // plain register qu
 
 constexpr int BM = 256, BN = 256, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // halves per staged row
-constexpr int THREADS = 256;
+constexpr int THREADS = 512;
 constexpr int STAGE_HALVES = (BM + BN) * LDS_STRIDE;  // one buffer: A rows then B rows
 
 struct Gemm256Params {
@@ -33,16 +34,16 @@ struct Gemm256Params {
   int ksteps;
 };
 
-// Scheduling pipeline of one slab section (16 MFMAs): after every MFMA a few of the other instructions of the
-// section, so they run in the MFMA's shadow; the 8 fragment reads go behind the first 8 MFMAs.  The closing
+// Scheduling pipeline of one slab section (8 MFMAs): after every MFMA a few of the other instructions of the
+// section, so they run in the MFMA's shadow; the 6 fragment reads go behind the first 6 MFMAs.  The closing
 // sched_barrier keeps the scheduler from mixing the MFMAs of different slabs (they reuse the same accumulators).
 template <bool VMEM, int VALU, int LDS_WRITE_EVERY>
 __device__ __forceinline__ void slab_pipeline() {
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
+  for (int i = 0; i < 8; ++i) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // 1 MFMA
-    if (i < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // 1 LDS read
-    if (VMEM && i < 12) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // 1 VMEM read
+    if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // 1 LDS read
+    if (VMEM && i < 7) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);     // 1 VMEM read
     if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
     if constexpr (LDS_WRITE_EVERY > 0) {
       if (i % LDS_WRITE_EVERY == LDS_WRITE_EVERY - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // 1 LDS write
@@ -52,24 +53,24 @@ __device__ __forceinline__ void slab_pipeline() {
 }
 
 template <int BITS, bool HAS_ZP, bool SMALL_BS>
-__global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p) {
+__global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int GK = 128 / BITS;                    // k per 16-byte group
   constexpr int GPK = BK / GK;                      // groups per column per k-step: 2 or 4
-  constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 8
+  constexpr int B_LOADS = BN * GPK / THREADS;       // 16-byte weight loads per thread per k-step: 1 or 2
+  constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 4
   extern __shared__ __align__(16) _Float16 lds[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  // XCD-aware tile order: consecutive workgroups go to different XCDs, so give each XCD a contiguous band of rows
+  const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 wavefronts: rows wm*64, columns wn*128
   const int m0 = blockIdx.y * BM;
   const int n0 = blockIdx.x * BN;
   const int li = lane & 31, kq = lane >> 5;
 
-  f16_t acc[4][4];
+  f16_t acc[2][4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -78,25 +79,26 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
   // two register sets for the global prefetch (distance: two k-steps), two fragment sets for the LDS prefetch
   struct Stage {
     u4_t a[A_LOADS];
-    u4_t b[GPK];
-    uint32_t m[GPK * (SMALL_BS ? 2 : 1)];
+    u4_t b[B_LOADS];
+    uint32_t m[B_LOADS * (SMALL_BS ? 2 : 1)];
   };
   Stage R0, R1;
   struct Frags {
-    h8_t a[4], b[4];
+    h8_t a[2], b[4];
   };
   Frags F0, F1;
 
-  const int a_row = tid >> 3, a_kc = tid & 7;  // thread's first A chunk: row a_row (+32 per load), k chunk a_kc
+  const int a_row = tid >> 3, a_kc = tid & 7;  // thread's first A chunk: row a_row (+64 per load), k chunk a_kc
   const _Float16* a_ptr[A_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
     // rows beyond M re-read row M-1 and are never stored (a predicated load would serialise the loop)
-    int m = m0 + a_row + i * 32;
+    int m = m0 + a_row + i * 64;
     m = m < p.M ? m : p.M - 1;
     a_ptr[i] = p.A + (int64_t)m * p.lda + a_kc * 8;
   }
-  const int64_t bcol = n0 + tid;
+  const int b_col = tid & (BN - 1), b_g0 = tid >> 8;  // thread's weight column and first group (+2 per load)
+  const int64_t bcol = n0 + b_col;
   const int64_t mcol = mnb_meta_col(bcol);
   const int last_step = p.ksteps - 1;
 
@@ -114,8 +116,8 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) R.a[i] = *reinterpret_cast<const u4_t*>(a_ptr[i] + k0);
 #pragma unroll
-    for (int g = 0; g < GPK; ++g) {
-      const int64_t kg = (int64_t)ks * GPK + g;
+    for (int g = 0; g < B_LOADS; ++g) {
+      const int64_t kg = (int64_t)ks * GPK + b_g0 + 2 * g;
       R.b[g] = *reinterpret_cast<const u4_t*>(p.W + kg * p.Npad + bcol);
       if constexpr (SMALL_BS) {
         R.m[2 * g] = meta_at((kg * 2) * p.Npad + mcol);
@@ -137,9 +139,9 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
     }
   };
 
-  // dequantise group g of this thread's column and write its GK halves to buffer `buf`
+  // dequantise the thread's g-th group and write its GK halves to buffer `buf`
   auto store_b_group = [&](int buf, int g, const Stage& R) {
-    _Float16* brow = lds + buf * STAGE_HALVES + (BM + tid) * LDS_STRIDE + g * GK;
+    _Float16* brow = lds + buf * STAGE_HALVES + (BM + b_col) * LDS_STRIDE + (b_g0 + 2 * g) * GK;
     const uint32_t wd[4] = {R.b[g][0], R.b[g][1], R.b[g][2], R.b[g][3]};
     h2_t s2a, s2b;
     ZpH za, zb;
@@ -174,22 +176,23 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
   };
 
   auto store_a = [&](int buf, int i, const Stage& R) {
-    *reinterpret_cast<u4_t*>(lds + buf * STAGE_HALVES + (a_row + i * 32) * LDS_STRIDE + a_kc * 8) = R.a[i];
+    *reinterpret_cast<u4_t*>(lds + buf * STAGE_HALVES + (a_row + i * 64) * LDS_STRIDE + a_kc * 8) = R.a[i];
   };
 
   auto read_frags = [&](int buf, int kk, Frags& F) {
     const _Float16* As = lds + buf * STAGE_HALVES;
     const _Float16* Bs = As + BM * LDS_STRIDE;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      F.a[t] = *reinterpret_cast<const h8_t*>(As + (wm * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
+    for (int t = 0; t < 2; ++t)
+      F.a[t] = *reinterpret_cast<const h8_t*>(As + (wm * 64 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
       F.b[t] = *reinterpret_cast<const h8_t*>(Bs + (wn * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
-    }
   };
 
   auto mfma_slab = [&](const Frags& F) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(F.a[i], F.b[j], acc[i][j], 0, 0, 0);
@@ -200,11 +203,8 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
     if (q == 0) {
 #pragma unroll
       for (int i = 0; i < A_LOADS; ++i) store_a(buf, i, R);
-    } else if constexpr (GPK == 2) {
+    } else if (q - 1 < B_LOADS) {
       store_b_group(buf, q - 1, R);
-    } else {
-      store_b_group(buf, 2 * (q - 1), R);
-      store_b_group(buf, 2 * (q - 1) + 1, R);
     }
   };
 
@@ -215,7 +215,7 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
   // Slab 3 runs after the barrier, with the first fragments of step ks+1 fetched in its shadow.
   auto k_step = [&](int ks, Stage& Rf, Stage& Rn) {
     const int cur = ks & 1, nxt = cur ^ 1;
-    // slab 0: global loads of step ks+2, fragments of slab 1, the 8 A vectors of step ks+1 into the other buffer
+    // slab 0: global loads of step ks+2, fragments of slab 1, the A vectors of step ks+1 into the other buffer
     load_global(ks + 2, Rf);
     read_frags(cur, 1, F1);
     mfma_slab(F0);
@@ -225,12 +225,12 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
     read_frags(cur, 2, F0);
     mfma_slab(F1);
     store_third(nxt, 1, Rn);
-    slab_pipeline<false, 6, 4>();
+    slab_pipeline<false, 9, 2>();
     // slab 2: fragments of slab 3, second half of the weights
     read_frags(cur, 3, F1);
     mfma_slab(F0);
     store_third(nxt, 2, Rn);
-    slab_pipeline<false, 6, 4>();
+    slab_pipeline<false, 9, 2>();
     __syncthreads();
     // slab 3, behind the barrier: first fragments of step ks+1
     read_frags(nxt, 0, F0);
@@ -258,10 +258,10 @@ __global__ void __launch_bounds__(THREADS, 1) mnb_gemm256_kernel(Gemm256Params p
     if (n >= p.N) continue;
     const float b = p.bias ? (float)p.bias[n] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < 2; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
+        const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
         if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + b);
       }
     }
