@@ -1,50 +1,99 @@
-// Dequant-in-LDS MFMA GEMM for fp16 models and large M: 256 x 256 output tile per workgroup.
+// MFMA GEMM for fp16 models and large M: 256 x 256 output tile per workgroup, weights dequantised in registers.
 //
 // Device counterpart of the reference's prefill loop (SQ4BitGemm_CompFp32, onnxruntime/core/mlas/lib/qnbitgemm.cpp:
-// 563-732).  Eight wavefronts (4 x 2, two per SIMD so that one can issue its staging work while the other owns the
-// matrix core), each owning a 64 x 128 block of the tile as 2 x 4 v_mfma_f32_32x32x16_f16 accumulators (128
-// accumulator registers per lane).  Per k-step of 64:
-//   * every thread fetches 4 x 16 B of A and 1 (4-bit) or 2 (8-bit) x 16 B of packed weights two steps ahead
-//     into registers while the matrix cores work on the current one;
-//   * the weights are dequantised to fp16 in registers (exact (q - zp), one rounding by the scale: bit-identical
-//     to the reference's fp16 dequantisation) and written, with the A rows, into the other LDS buffer;
-//   * one barrier per step.
-// LDS rows are padded by 16 bytes so both the 16-byte staging writes and the ds_read_b128 operand fetches are
-// bank-conflict free.  Bias add and the single fp32 -> fp16 narrowing happen in the epilogue.
+// 563-732: dequantise a strip of B, then run the float GEMM kernel over it).
+//
+// Eight wavefronts (2 x 4, two per SIMD), each owning a 128 x 64 block of the tile as 4 x 2
+// v_mfma_f32_32x32x16_f16 accumulators.  Per k-step of 64:
+//   * A (activations): every thread fetches 4 x 16 B two steps ahead into registers and writes them to the other
+//     LDS buffer; wavefronts read their A operands with ds_read_b128 (rows padded by 16 B: conflict free).
+//   * B (weights) never touches LDS.  Lane (column j = lane%32, half kq = lane/32) of a wavefront loads, two steps
+//     ahead, exactly the 8 bytes of packed weights it will feed to the matrix core: the two 32-bit words of its
+//     column's 16-byte vector that belong to its half.  Each word is dequantised in registers to 8 halves -- exact
+//     (q - zp), one rounding by the scale, bit-identical to the reference's fp16 dequantisation -- and IS the MFMA
+//     B operand of one k-slab.  (The contraction index of an MFMA may be permuted freely as long as A uses the same
+//     permutation: for 4-bit weights slab 2g takes k = 32g + 16kq + [0,8) and slab 2g+1 takes 32g + 16kq + [8,16).)
+//     LDS traffic is what bounded the design that staged a dequantised B tile in LDS (every wavefront re-read it);
+//     the price here is that the two wavefront rows dequantise the same columns.
+//   * one barrier per step; the dequantisation of slab s+1 and the A staging run in the shadow of slab s's MFMAs.
+// Bias add and the single fp32 -> fp16 narrowing happen in the epilogue.
 #include "mnb_device.cuh"
 #include "mnb_internal.h"
 
 namespace {
 
 typedef uint32_t u4_t __attribute__((ext_vector_type(4)));  // plain register quad (HIP's uint4 struct resists SROA)
+typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int LDS_STRIDE = BK + 8;  // halves per staged row
+constexpr int LDS_STRIDE = BK + 8;  // halves per staged A row
 constexpr int THREADS = 512;
-constexpr int STAGE_HALVES = (BM + BN) * LDS_STRIDE;  // one buffer: A rows then B rows
+constexpr int STAGE_HALVES = BM * LDS_STRIDE;  // one A buffer
 
 struct Gemm256Params {
   const _Float16* A;
-  const uint4* W;
+  const uint8_t* W;  // packed weights, byte addressed
   const uint8_t* meta;
   const _Float16* bias;
   _Float16* C;
   int64_t lda, ldc, Npad;
   int M, N, K, bs_shift;
   int ksteps;
+  int tiles_m, tiles_n;
+  uint32_t uc[4];  // unpack constants (see UnpackConsts)
 };
 
+// The constants of the nibble unpack, passed as kernel arguments: with literals the compiler emits
+// v_and_b32 + v_or_b32 (VOP3 takes no literal on this ISA family); with register operands, one v_and_or_b32.
+struct UnpackConsts {
+  uint32_t mask_lo, mask_hi, magic;  // 0x000F000F, 0x00F000F0, 0x64006400 (two halves of 1024)
+};
+
+__device__ __forceinline__ UnpackConsts make_unpack_consts(const uint32_t* k) {
+  UnpackConsts u;
+  u.mask_lo = k[0];
+  u.mask_hi = k[1];
+  // one SGPR operand per VALU instruction: the magic lives in a VGPR (an opaque move, so it is not folded back)
+  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic) : "s"(k[2]));
+  return u;
+}
+
+// Packed weights of one lane and slab -> 8 dequantised halves in k order: the B operand of one MFMA.
+// 4-bit: one word (w1 unused); 8-bit: two words.
+template <int BITS>
+__device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const UnpackConsts& uc, const ZpH& z,
+                                             h2_t s2) {
+  h2_t d[4];
+  if constexpr (BITS == 4) {
+    const h2_t sixteenth = mnb_h2((_Float16)0.0625f);
+    const uint32_t w8 = w0 >> 8;
+    const h2_t p0 = mnb_as_h2((w0 & uc.mask_lo) | uc.magic);
+    const h2_t p1 = mnb_as_h2((w0 & uc.mask_hi) | uc.magic);
+    const h2_t p2 = mnb_as_h2((w8 & uc.mask_lo) | uc.magic);
+    const h2_t p3 = mnb_as_h2((w8 & uc.mask_hi) | uc.magic);
+    d[0] = p0 + z.lo;
+    d[1] = __builtin_elementwise_fma(p1, sixteenth, z.hi);
+    d[2] = p2 + z.lo;
+    d[3] = __builtin_elementwise_fma(p3, sixteenth, z.hi);
+  } else {
+    mnb_unpack8_h(w0, z, d);
+    mnb_unpack8_h(w1, z, d + 2);
+  }
+  const u4_t o = {mnb_as_u32(d[0] * s2), mnb_as_u32(d[1] * s2), mnb_as_u32(d[2] * s2), mnb_as_u32(d[3] * s2)};
+  return __builtin_bit_cast(h8_t, o);
+}
+
 // Scheduling pipeline of one slab section (8 MFMAs): after every MFMA a few of the other instructions of the
-// section, so they run in the MFMA's shadow; the 6 fragment reads go behind the first 6 MFMAs.  The closing
-// sched_barrier keeps the scheduler from mixing the MFMAs of different slabs (they reuse the same accumulators).
-template <bool VMEM, int VALU, int LDS_WRITE_EVERY>
+// section, so they run in the MFMA's shadow.  The closing sched_barrier keeps the scheduler from mixing the MFMAs
+// of different slabs (they reuse the same accumulators).
+template <int LDS_READS, int VMEM, int VALU, int LDS_WRITE_EVERY>
 __device__ __forceinline__ void slab_pipeline() {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                        // 1 MFMA
-    if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // 1 LDS read
-    if (VMEM && i < 7) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);     // 1 VMEM read
-    if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                             // 1 MFMA
+    if (i < LDS_READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);          // 1 LDS read
+    if (i < VMEM) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);               // 2 VMEM reads
+    if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);  // VALU
     if constexpr (LDS_WRITE_EVERY > 0) {
       if (i % LDS_WRITE_EVERY == LDS_WRITE_EVERY - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // 1 LDS write
     }
@@ -52,78 +101,91 @@ __device__ __forceinline__ void slab_pipeline() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-template <int BITS, bool HAS_ZP, bool SMALL_BS>
+template <int BITS, bool HAS_ZP>
 __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
-  constexpr int GK = 128 / BITS;                    // k per 16-byte group
-  constexpr int GPK = BK / GK;                      // groups per column per k-step: 2 or 4
-  constexpr int B_LOADS = BN * GPK / THREADS;       // 16-byte weight loads per thread per k-step: 1 or 2
-  constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 4
+  constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 16-byte activation loads per thread per k-step: 4
+  // 4-bit: a 16-byte vector spans two slabs (one word each per lane); 8-bit: one slab (two words per lane)
+  constexpr int VEC_PER_STEP = (BITS == 4) ? 2 : 4;  // 8-byte weight loads per lane, column tile and k-step
+  constexpr int GK = 128 / BITS;
   extern __shared__ __align__(16) _Float16 lds[];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 wavefronts: rows wm*64, columns wn*128
-  const int m0 = blockIdx.y * BM;
-  const int n0 = blockIdx.x * BN;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts: rows wm*128, columns wn*64
+  // column-fastest tile order: the workgroups resident at one time share a few 256-row slabs of A
+  const int m0 = (blockIdx.x / p.tiles_n) * BM;
+  const int n0 = (blockIdx.x % p.tiles_n) * BN;
   const int li = lane & 31, kq = lane >> 5;
 
-  f16_t acc[2][4];
+  f16_t acc[4][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // two register sets for the global prefetch (distance: two k-steps), two fragment sets for the LDS prefetch
+  // two register sets for the global prefetch (distance: two k-steps)
   struct Stage {
     u4_t a[A_LOADS];
-    u4_t b[B_LOADS];
-    uint32_t m[B_LOADS * (SMALL_BS ? 2 : 1)];
+    u2_t b[VEC_PER_STEP][2];      // [vector of the k-step][column tile]
+    uint32_t m[VEC_PER_STEP][2];  // meta entry of the block the vector's half belongs to
   };
   Stage R0, R1;
-  struct Frags {
-    h8_t a[2], b[4];
-  };
-  Frags F0, F1;
+  h8_t FA0[4], FA1[4];  // A operands, double buffered over slabs
+  h8_t FB0[2], FB1[2];  // B operands, double buffered over slabs
 
+  const UnpackConsts uc = make_unpack_consts(p.uc);
+
+  // Addressing: every global access is  uniform base (SGPRs, advanced per k-step)  +  32-bit per-lane offset (a VGPR
+  // computed once), so the loads cost no VALU work inside the loop.
   const int a_row = tid >> 3, a_kc = tid & 7;  // thread's first A chunk: row a_row (+64 per load), k chunk a_kc
-  const _Float16* a_ptr[A_LOADS];
+  uint32_t a_off[A_LOADS];                     // byte offsets from p.A + k0
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
     // rows beyond M re-read row M-1 and are never stored (a predicated load would serialise the loop)
     int m = m0 + a_row + i * 64;
     m = m < p.M ? m : p.M - 1;
-    a_ptr[i] = p.A + (int64_t)m * p.lda + a_kc * 8;
+    a_off[i] = (uint32_t)(((int64_t)m * p.lda + a_kc * 8) * 2);
   }
-  const int b_col = tid & (BN - 1), b_g0 = tid >> 8;  // thread's weight column and first group (+2 per load)
-  const int64_t bcol = n0 + b_col;
-  const int64_t mcol = mnb_meta_col(bcol);
+  // this lane's weight columns (one per column tile): its 8 bytes inside each 16-byte vector, and its meta entries.
+  // The block of a lane's half vector is (k-group base >> bs_shift), plus kq when 4-bit blocks are 16 wide.
+  constexpr int META_BYTES = HAS_ZP ? 4 : 2;
+  const bool small_bs = (BITS == 4) && p.bs_shift == 4;
+  uint32_t w_off[2], m_off[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int64_t col = n0 + wn * 64 + j * 32 + li;
+    w_off[j] = (uint32_t)(col * 16 + kq * 8);
+    m_off[j] = (uint32_t)((mnb_meta_col(col) + (small_bs ? kq * p.Npad : 0)) * META_BYTES);
+  }
   const int last_step = p.ksteps - 1;
-
-  auto meta_at = [&](int64_t idx) -> uint32_t {
-    if constexpr (HAS_ZP)
-      return reinterpret_cast<const uint32_t*>(p.meta)[idx];
-    else
-      return reinterpret_cast<const uint16_t*>(p.meta)[idx];
-  };
+  const int64_t vec_pitch = p.Npad * 16;               // bytes between consecutive k-groups
+  const int64_t meta_pitch = p.Npad * META_BYTES;      // bytes between consecutive blocks
 
   // k-steps past the end are clamped to the last one: the loop body stays branch free, the data is never used
-  auto load_global = [&](int ks_raw, Stage& R) {
+  auto load_a = [&](int ks_raw, Stage& R) {
     const int ks = ks_raw < last_step ? ks_raw : last_step;
-    const int k0 = ks * BK;
+    const uint8_t* base = reinterpret_cast<const uint8_t*>(p.A + (int64_t)ks * BK);
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) R.a[i] = *reinterpret_cast<const u4_t*>(a_ptr[i] + k0);
+    for (int i = 0; i < A_LOADS; ++i) R.a[i] = *reinterpret_cast<const u4_t*>(base + a_off[i]);
+  };
+  auto load_b = [&](int ks_raw, Stage& R) {
+    const int ks = ks_raw < last_step ? ks_raw : last_step;
 #pragma unroll
-    for (int g = 0; g < B_LOADS; ++g) {
-      const int64_t kg = (int64_t)ks * GPK + b_g0 + 2 * g;
-      R.b[g] = *reinterpret_cast<const u4_t*>(p.W + kg * p.Npad + bcol);
-      if constexpr (SMALL_BS) {
-        R.m[2 * g] = meta_at((kg * 2) * p.Npad + mcol);
-        R.m[2 * g + 1] = meta_at((kg * 2 + 1) * p.Npad + mcol);
-      } else {
-        R.m[g] = meta_at(((kg * GK) >> p.bs_shift) * p.Npad + mcol);
+    for (int v = 0; v < VEC_PER_STEP; ++v) {
+      const int64_t kg = (int64_t)ks * VEC_PER_STEP + v;  // k-group of the vector
+      const int64_t kb = (kg * GK) >> p.bs_shift;         // block of the vector's first element
+      const uint8_t* wbase = p.W + kg * vec_pitch;
+      const uint8_t* mbase = p.meta + kb * meta_pitch;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        R.b[v][j] = *reinterpret_cast<const u2_t*>(wbase + w_off[j]);
+        if constexpr (HAS_ZP)
+          R.m[v][j] = *reinterpret_cast<const uint32_t*>(mbase + m_off[j]);
+        else
+          R.m[v][j] = *reinterpret_cast<const uint16_t*>(mbase + m_off[j]);
       }
     }
   };
@@ -139,38 +201,19 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     }
   };
 
-  // dequantise the thread's g-th group and write its GK halves to buffer `buf`
-  auto store_b_group = [&](int buf, int g, const Stage& R) {
-    _Float16* brow = lds + buf * STAGE_HALVES + (BM + b_col) * LDS_STRIDE + (b_g0 + 2 * g) * GK;
-    const uint32_t wd[4] = {R.b[g][0], R.b[g][1], R.b[g][2], R.b[g][3]};
-    h2_t s2a, s2b;
-    ZpH za, zb;
-    if constexpr (SMALL_BS) {
-      decode(R.m[2 * g], s2a, za);
-      decode(R.m[2 * g + 1], s2b, zb);
-    } else {
-      decode(R.m[g], s2a, za);
-      s2b = s2a;
-      zb = za;
-    }
-    if constexpr (BITS == 4) {
+  // B operands of slab kk (0..3) of the k-step held in R
+  auto make_b = [&](int kk, const Stage& R, h8_t* FB) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        h2_t d[4];
-        mnb_unpack4_h(wd[i], i < 2 ? za : zb, d);
-        const h2_t s2 = i < 2 ? s2a : s2b;
-        const u4_t o = {mnb_as_u32(d[0] * s2), mnb_as_u32(d[1] * s2), mnb_as_u32(d[2] * s2), mnb_as_u32(d[3] * s2)};
-        *reinterpret_cast<u4_t*>(brow + i * 8) = o;
-      }
-    } else {
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        h2_t d[4];
-        mnb_unpack8_h(wd[2 * i], za, d);
-        mnb_unpack8_h(wd[2 * i + 1], za, d + 2);
-        const u4_t o = {mnb_as_u32(d[0] * s2a), mnb_as_u32(d[1] * s2a), mnb_as_u32(d[2] * s2a),
-                        mnb_as_u32(d[3] * s2a)};
-        *reinterpret_cast<u4_t*>(brow + i * 8) = o;
+    for (int j = 0; j < 2; ++j) {
+      h2_t s2;
+      ZpH z;
+      if constexpr (BITS == 4) {
+        const int v = kk >> 1;
+        decode(R.m[v][j], s2, z);
+        FB[j] = dequant_word<4>(R.b[v][j][kk & 1], 0u, uc, z, s2);
+      } else {
+        decode(R.m[kk][j], s2, z);
+        FB[j] = dequant_word<8>(R.b[kk][j][0], R.b[kk][j][1], uc, z, s2);
       }
     }
   };
@@ -179,72 +222,64 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     *reinterpret_cast<u4_t*>(lds + buf * STAGE_HALVES + (a_row + i * 64) * LDS_STRIDE + a_kc * 8) = R.a[i];
   };
 
-  auto read_frags = [&](int buf, int kk, Frags& F) {
-    const _Float16* As = lds + buf * STAGE_HALVES;
-    const _Float16* Bs = As + BM * LDS_STRIDE;
+  // A operands of slab kk: lane (row li, half kq).  The k permutation matches the weights' (see the file header).
+  auto read_a = [&](int buf, int kk, h8_t* FA) {
+    const int koff = (BITS == 4) ? 32 * (kk >> 1) + 16 * kq + 8 * (kk & 1) : 16 * kk + 8 * kq;
+    const _Float16* As = lds + buf * STAGE_HALVES + (wm * 128 + li) * LDS_STRIDE + koff;
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-      F.a[t] = *reinterpret_cast<const h8_t*>(As + (wm * 64 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-      F.b[t] = *reinterpret_cast<const h8_t*>(Bs + (wn * 128 + t * 32 + li) * LDS_STRIDE + kk * 16 + kq * 8);
+    for (int t = 0; t < 4; ++t) FA[t] = *reinterpret_cast<const h8_t*>(As + t * 32 * LDS_STRIDE);
   };
 
-  auto mfma_slab = [&](const Frags& F) {
+  auto mfma_slab = [&](const h8_t* FA, const h8_t* FB) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(F.a[i], F.b[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(FA[i], FB[j], acc[i][j], 0, 0, 0);
   };
 
-  // staging work of one k-step in three parts (one per MFMA slab it hides behind)
-  auto store_third = [&](int buf, int q, const Stage& R) {
-    if (q == 0) {
-#pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) store_a(buf, i, R);
-    } else if (q - 1 < B_LOADS) {
-      store_b_group(buf, q - 1, R);
-    }
-  };
-
-  // One k-step.  On entry: LDS buffer `cur` holds step ks, F0 holds its slab 0, Rn holds (or is receiving) step
-  // ks+1.  Slabs 0-2: MFMAs with, in their shadow, the global loads of step ks+2 (into Rf), the fragment reads of
-  // the following slab and the staging of step ks+1 into the other buffer.  Then the barrier: every wavefront has
-  // finished writing the other buffer and has its slab-3 fragments in registers, so buffer `cur` is free again.
-  // Slab 3 runs after the barrier, with the first fragments of step ks+1 fetched in its shadow.
-  auto k_step = [&](int ks, Stage& Rf, Stage& Rn) {
+  // One k-step.  On entry: LDS buffer `cur` holds the A tile of step ks, FA0/FB0 hold the operands of its slab 0,
+  // Rc holds the weights of step ks (its A registers are already staged, hence free), Rn holds (or is receiving)
+  // A and weights of step ks+1.
+  auto k_step = [&](int ks, Stage& Rc, Stage& Rn) {
     const int cur = ks & 1, nxt = cur ^ 1;
-    // slab 0: global loads of step ks+2, fragments of slab 1, the A vectors of step ks+1 into the other buffer
-    load_global(ks + 2, Rf);
-    read_frags(cur, 1, F1);
-    mfma_slab(F0);
-    store_third(nxt, 0, Rn);
-    slab_pipeline<true, 3, 2>();
-    // slab 1: fragments of slab 2, first half of the weights of step ks+1
-    read_frags(cur, 2, F0);
-    mfma_slab(F1);
-    store_third(nxt, 1, Rn);
-    slab_pipeline<false, 9, 2>();
-    // slab 2: fragments of slab 3, second half of the weights
-    read_frags(cur, 3, F1);
-    mfma_slab(F0);
-    store_third(nxt, 2, Rn);
-    slab_pipeline<false, 9, 2>();
+    // slab 0: operands of slab 1; global loads of A for step ks+2; A of step ks+1 into the other buffer
+    load_a(ks + 2, Rc);
+    read_a(cur, 1, FA1);
+    make_b(1, Rc, FB1);
+    mfma_slab(FA0, FB0);
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) store_a(nxt, i, Rn);
+    slab_pipeline<4, 2, 4, 2>();
+    // slab 1: operands of slab 2
+    read_a(cur, 2, FA0);
+    make_b(2, Rc, FB0);
+    mfma_slab(FA1, FB1);
+    slab_pipeline<4, 0, 4, 0>();
+    // slab 2: operands of slab 3; after that the weight registers of Rc are free: weights of step ks+2
+    read_a(cur, 3, FA1);
+    make_b(3, Rc, FB1);
+    mfma_slab(FA0, FB0);
+    load_b(ks + 2, Rc);
+    slab_pipeline<4, 4, 4, 0>();
     __syncthreads();
-    // slab 3, behind the barrier: first fragments of step ks+1
-    read_frags(nxt, 0, F0);
-    mfma_slab(F1);
-    slab_pipeline<false, 0, 0>();
+    // slab 3, behind the barrier: operands of slab 0 of step ks+1
+    read_a(nxt, 0, FA0);
+    make_b(0, Rn, FB0);
+    mfma_slab(FA1, FB1);
+    slab_pipeline<4, 0, 4, 0>();
   };
 
-  // ---- prologue: steps 0 and 1 in flight, step 0 staged
-  load_global(0, R0);
-  load_global(1, R1);
+  // ---- prologue: steps 0 and 1 in flight, A of step 0 staged, operands of slab 0 ready
+  load_a(0, R0);
+  load_b(0, R0);
+  load_a(1, R1);
+  load_b(1, R1);
 #pragma unroll
-  for (int q = 0; q < 3; ++q) store_third(0, q, R0);
+  for (int i = 0; i < A_LOADS; ++i) store_a(0, i, R0);
   __syncthreads();
-  read_frags(0, 0, F0);
+  read_a(0, 0, FA0);
+  make_b(0, R0, FB0);
 
   for (int ks = 0; ks < p.ksteps; ks += 2) {  // ksteps is even
     k_step(ks, R0, R1);
@@ -253,15 +288,15 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 
   // ---- epilogue: D[i][j] of a 32x32 tile: lane holds column j = lane % 32, rows 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int n = n0 + wn * 128 + j * 32 + li;
+  for (int j = 0; j < 2; ++j) {
+    const int n = n0 + wn * 64 + j * 32 + li;
     if (n >= p.N) continue;
     const float b = p.bias ? (float)p.bias[n] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < 4; ++i) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
+        const int m = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
         if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + b);
       }
     }
@@ -274,18 +309,18 @@ int log2i(int v) {
   return s;
 }
 
-template <int BITS, bool HAS_ZP, bool SMALL_BS>
+template <int BITS, bool HAS_ZP>
 hipError_t launch(const Gemm256Params& p, hipStream_t s) {
-  const size_t smem = (size_t)2 * STAGE_HALVES * sizeof(_Float16);  // 147456 bytes
+  const size_t smem = (size_t)2 * STAGE_HALVES * sizeof(_Float16);  // 73728 bytes
   static bool configured = false;  // per instantiation; the attribute is sticky for the function
-  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, SMALL_BS>;
+  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return e;
     configured = true;
   }
-  dim3 grid((unsigned)((p.N + BN - 1) / BN), (unsigned)((p.M + BM - 1) / BM)), blk(THREADS);
+  dim3 grid((unsigned)(p.tiles_n * p.tiles_m)), blk(THREADS);
   kernel<<<grid, blk, smem, s>>>(p);
   return hipGetLastError();
 }
@@ -295,7 +330,7 @@ hipError_t launch(const Gemm256Params& p, hipStream_t s) {
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   Gemm256Params p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
-  p.W = reinterpret_cast<const uint4*>(a.packed);
+  p.W = reinterpret_cast<const uint8_t*>(a.packed);
   p.meta = reinterpret_cast<const uint8_t*>(a.packed) + a.L.meta_off;
   p.bias = reinterpret_cast<const _Float16*>(a.bias);
   p.C = reinterpret_cast<_Float16*>(a.C);
@@ -307,9 +342,12 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.K = (int)a.L.K;
   p.bs_shift = log2i(a.L.bs);
   p.ksteps = (int)(a.L.K / BK);  // K is a multiple of 2 * BK
-  if (a.L.bits == 4) {
-    if (a.L.bs == 16) return a.L.has_zp ? launch<4, true, true>(p, s) : launch<4, false, true>(p, s);
-    return a.L.has_zp ? launch<4, true, false>(p, s) : launch<4, false, false>(p, s);
-  }
-  return a.L.has_zp ? launch<8, true, false>(p, s) : launch<8, false, false>(p, s);
+  p.tiles_m = (int)((a.M + BM - 1) / BM);
+  p.tiles_n = (int)((a.L.N + BN - 1) / BN);
+  p.uc[0] = 0x000F000Fu;
+  p.uc[1] = 0x00F000F0u;
+  p.uc[2] = 0x64006400u;
+  p.uc[3] = 0;
+  if (a.L.bits == 4) return a.L.has_zp ? launch<4, true>(p, s) : launch<4, false>(p, s);
+  return a.L.has_zp ? launch<8, true>(p, s) : launch<8, false>(p, s);
 }
