@@ -25,6 +25,10 @@ import numpy as np
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
+# for a plain copy of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs are summarised in
+# profiles/hbm_traffic_skinny_c2_gemm256_c4.md.  They are properties of the kernels, not of one run.
+MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14847.3 * 2.0 + 28.0) * 1024), "c4_prefill": int((109728.5 * 2.0 + 83294.5) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
 LAYERS = 32
@@ -136,6 +140,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 GEMM")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies (a kernel of known traffic, for scaling the "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters); nothing else changes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the op shards along N without communication; nothing "
@@ -148,6 +155,15 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
     _lib.load()
+
+    if args.calibrate_copy:
+        src = torch.full((256 << 20,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     # ---- decode GEMV (headline) ------------------------------------------------------------------------------
     c2 = synthetic.config_c2(seed=0)
@@ -189,7 +205,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES["c2_decode"],
             "kernel": p2.kernel,
             "us_per_launch": round(us_per_launch, 3),
         },
@@ -211,7 +227,8 @@ def main() -> int:
             "ms_per_launch": round(ms4, 4),
             "kernel": p4.kernel,
             "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
-                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4), "traffic": None},
+                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4),
+                         "traffic": MEASURED_TRAFFIC_BYTES["c4_prefill"]},
         }
         del p4
         torch.cuda.empty_cache()
