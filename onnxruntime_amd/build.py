@@ -1,6 +1,10 @@
-"""Builds libmnb_mi355x.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+"""Builds, in-tree and with hipcc:
+  libmnb_mi355x.so            HIP kernels + C ABI for gfx950
+  libonnxruntime_mi355x_ep.so the ONNX Runtime plugin execution provider above that C ABI (needs the ONNX Runtime
+                              C API headers: directory given by ORT_INCLUDE_DIR, or an onnxruntime checkout at
+                              ORT_SOURCE_DIR / /root/reference)
 
-Usage: python -m onnxruntime_amd.build [--force]
+Usage: python -m onnxruntime_amd.build
 """
 from __future__ import annotations
 
@@ -60,5 +64,54 @@ def build(force: bool = True, jobs: int = 4) -> Path:
     return LIB
 
 
+EP_LIB = PKG / "libonnxruntime_mi355x_ep.so"
+EP_SOURCES = ["ep_lib_entry.cc", "ep_factory.cc", "ep.cc", "ep_kernels.cc", "ep_device_runtime.cc"]
+
+
+def ort_include_dir() -> Path | None:
+    """Directory that holds onnxruntime_c_api.h, or None when no ONNX Runtime headers are installed."""
+    cands = []
+    if os.environ.get("ORT_INCLUDE_DIR"):
+        cands.append(Path(os.environ["ORT_INCLUDE_DIR"]))
+    src = Path(os.environ.get("ORT_SOURCE_DIR", "/root/reference"))
+    cands.append(src / "include" / "onnxruntime" / "core" / "session")
+    for c in cands:
+        if (c / "onnxruntime_c_api.h").exists() and (c / "onnxruntime_ep_c_api.h").exists():
+            return c
+    return None
+
+
+def _compile_ep(src: str, inc: Path) -> Path:
+    out_dir = OBJ_DIR / "ep"
+    out_dir.mkdir(parents=True, exist_ok=True)
+    obj = out_dir / (src + ".o")
+    cmd = [hipcc(), "-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
+           "-I", str(inc), "-I", str(PKG.parent / "include"), "-c", str(CSRC / "ep" / src), "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on ep/{src}:\n{r.stderr}")
+    if r.stderr.strip():
+        print(r.stderr, file=sys.stderr)
+    return obj
+
+
+def build_ep(jobs: int = 4) -> Path | None:
+    """Compiles the plugin EP against the ONNX Runtime headers found by ort_include_dir(). Returns None (and keeps a
+    previously built library) when no headers are available."""
+    inc = ort_include_dir()
+    if inc is None:
+        print("onnxruntime_amd.build: ONNX Runtime headers not found, plugin EP not rebuilt", file=sys.stderr)
+        return EP_LIB if EP_LIB.exists() else None
+    if not LIB.exists():
+        build()
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda s: _compile_ep(s, inc), EP_SOURCES))
+    cmd = [hipcc(), "-shared", "-fPIC", "-o", str(EP_LIB), *map(str, objs), "-L", str(PKG), "-lmnb_mi355x",
+           "-Wl,-rpath,$ORIGIN", "-Wl,--no-undefined"]
+    subprocess.check_call(cmd)
+    return EP_LIB
+
+
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv or True))
+    print(build(force=True))
+    print(build_ep())

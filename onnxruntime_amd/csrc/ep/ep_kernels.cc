@@ -1,0 +1,494 @@
+// Kernels the MI355X plugin EP registers with ONNX Runtime
+// (OrtKernelImpl, include/onnxruntime/core/session/onnxruntime_ep_c_api.h:730-862):
+//   com.microsoft::MatMulNBits (opset 1, fp32 and fp16 activations)  -- the operator this provider exists for
+//   MemcpyFromHost / MemcpyToHost (onnx domain)                        -- the copies ONNX Runtime inserts around nodes
+//                                                                          of a provider with its own memory
+// The MatMulNBits kernel mirrors contrib::MatMulNBits<T1> of the reference
+// (onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc): attribute checks in the constructor (:100-138),
+// PrePack of B together with constant scales / zero points (:252-724), Compute = CheckInputs, output shape, early
+// return on an empty output, then the packed or the unpacked route (:1513-1570).
+#include "ep_common.h"
+
+namespace mi355x_ep {
+
+namespace {
+
+enum InputIndex : size_t { kA = 0, kB = 1, kScales = 2, kZeroPoints = 3, kGIdx = 4, kBias = 5 };
+
+// Shape and element type of a tensor value.
+struct TensorDesc {
+  std::vector<int64_t> dims;
+  ONNXTensorElementDataType type = ONNX_TENSOR_ELEMENT_DATA_TYPE_UNDEFINED;
+  int64_t count() const {
+    int64_t c = 1;
+    for (int64_t d : dims) c *= d;
+    return c;
+  }
+};
+
+OrtStatus* Describe(const Apis& a, const OrtValue* value, TensorDesc* out) {
+  OrtTensorTypeAndShapeInfo* info = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->GetTensorTypeAndShape(value, &info));
+  size_t rank = 0;
+  OrtStatus* st = a.ort->GetDimensionsCount(info, &rank);
+  if (st == nullptr) {
+    out->dims.assign(rank, 0);
+    if (rank > 0) st = a.ort->GetDimensions(info, out->dims.data(), rank);
+  }
+  if (st == nullptr) st = a.ort->GetTensorElementType(info, &out->type);
+  a.ort->ReleaseTensorTypeAndShapeInfo(info);
+  return st;
+}
+
+MnbTensorInfo ToMnb(const TensorDesc* d) {
+  MnbTensorInfo t{};
+  if (d == nullptr) return t;  // absent optional input
+  static const int64_t kNoDims = 0;
+  t.dims = d->dims.empty() ? &kNoDims : d->dims.data();
+  t.rank = d->dims.size();
+  t.dtype = static_cast<int>(d->type);
+  return t;
+}
+
+bool OnHost(const Apis& a, const OrtValue* v) {
+  return a.ep->MemoryDevice_GetDeviceType(a.ep->Value_GetMemoryDevice(v)) == OrtMemoryInfoDeviceType_CPU;
+}
+
+// A device view of a constant tensor: the tensor's own storage when it already lives on the GPU, otherwise a
+// temporary device copy that is freed with the object.
+class DeviceView {
+ public:
+  DeviceView() = default;
+  DeviceView(const DeviceView&) = delete;
+  DeviceView& operator=(const DeviceView&) = delete;
+  ~DeviceView() {
+    if (owned_ != nullptr) (void)hipFree(owned_);
+  }
+  OrtStatus* Init(const Apis& a, const OrtValue* v) {
+    const void* p = nullptr;
+    MI_RETURN_IF_ERROR(a.ort->GetTensorData(v, &p));
+    if (!OnHost(a, v)) {
+      ptr_ = p;
+      return nullptr;
+    }
+    size_t bytes = 0;
+    MI_RETURN_IF_ERROR(a.ort->GetTensorSizeInBytes(v, &bytes));
+    if (bytes == 0) return nullptr;
+    MI_RETURN_IF_HIP(a, hipMalloc(&owned_, bytes));
+    MI_RETURN_IF_HIP(a, hipMemcpy(owned_, p, bytes, hipMemcpyHostToDevice));
+    ptr_ = owned_;
+    return nullptr;
+  }
+  const void* get() const { return ptr_; }
+
+ private:
+  const void* ptr_ = nullptr;
+  void* owned_ = nullptr;
+};
+
+// =========================================================================================== MatMulNBits
+struct MatMulNBitsKernel : OrtKernelImpl {
+  Apis apis;
+  int64_t K = 0, N = 0, block_size = 0, bits = 4, accuracy_level = 0;
+  // constant initializers seen at kernel creation (owned by the session; valid until they are reported packed)
+  const OrtValue* const_scales = nullptr;
+  const OrtValue* const_zero_points = nullptr;
+  bool has_zp_arg = false;    // the node has a zero_points input, constant or not
+  bool has_g_idx = false;
+  // packed weights (weights + scales + zero points in the device layout)
+  void* packed = nullptr;
+  OrtAllocator* packed_allocator = nullptr;
+  int packed_dtype = 0;
+  bool packed_has_zp = false;
+};
+
+MatMulNBitsKernel* Self(OrtKernelImpl* p) { return static_cast<MatMulNBitsKernel*>(p); }
+
+void ORT_API_CALL MatMulNBitsRelease(OrtKernelImpl* this_ptr) noexcept {
+  MatMulNBitsKernel* k = Self(this_ptr);
+  if (k->packed != nullptr) {
+    if (k->packed_allocator != nullptr)
+      k->packed_allocator->Free(k->packed_allocator, k->packed);
+    else
+      (void)hipFree(k->packed);
+  }
+  delete k;
+}
+
+// PrePack(B) folds the constant scales and zero points into one device buffer in the gfx950 layout, the way the
+// reference folds them into its packed buffer on the B call (matmul_nbits.cc:252-330).  The later calls for scales
+// and zero points then only report those inputs as consumed.
+OrtStatus* ORT_API_CALL MatMulNBitsPrePack(OrtKernelImpl* this_ptr, const OrtValue* tensor, int input_index,
+                                           OrtAllocator* allocator, OrtSharedPrePackedWeightCache* /*cache*/,
+                                           bool* is_packed) noexcept {
+  MatMulNBitsKernel& k = *Self(this_ptr);
+  const Apis& a = k.apis;
+  *is_packed = false;
+  if (k.has_g_idx) return nullptr;  // no packed kernel with a group index (matmul_nbits.cc:258-262)
+
+  if (input_index == static_cast<int>(kScales) || input_index == static_cast<int>(kZeroPoints)) {
+    // consumed by the B call: ONNX Runtime may drop the initializer
+    *is_packed = k.packed != nullptr;
+    return nullptr;
+  }
+  if (input_index != static_cast<int>(kB)) return nullptr;
+  // Packing needs the scales now; zero points must be constant as well, or absent.
+  if (k.const_scales == nullptr) return nullptr;
+  if (k.has_zp_arg && k.const_zero_points == nullptr) return nullptr;
+
+  TensorDesc b_desc, s_desc, z_desc;
+  MI_RETURN_IF_ERROR(Describe(a, tensor, &b_desc));
+  MI_RETURN_IF_ERROR(Describe(a, k.const_scales, &s_desc));
+  if (k.const_zero_points != nullptr) MI_RETURN_IF_ERROR(Describe(a, k.const_zero_points, &z_desc));
+  if (z_desc.type != ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8 && k.const_zero_points != nullptr) return nullptr;
+  const int dtype = static_cast<int>(s_desc.type);
+  if (!MnbIsAvailable(static_cast<int>(k.bits), static_cast<int>(k.block_size), dtype)) return nullptr;
+
+  MnbTensorInfo bi = ToMnb(&b_desc), si = ToMnb(&s_desc), zi = ToMnb(k.const_zero_points ? &z_desc : nullptr),
+                none = ToMnb(nullptr);
+  MI_RETURN_IF_ERROR(StatusFromMnb(a, MnbCheckInputs(&bi, &si, &zi, &none, &none, k.N, k.K, k.block_size, k.bits)));
+
+  const size_t bytes = MnbPackQuantBDataSize(static_cast<size_t>(k.N), static_cast<size_t>(k.K),
+                                             static_cast<int>(k.bits), static_cast<int>(k.block_size),
+                                             k.const_zero_points != nullptr, dtype);
+  if (bytes == 0) return nullptr;
+  DeviceView b_dev, s_dev, z_dev;
+  MI_RETURN_IF_ERROR(b_dev.Init(a, tensor));
+  MI_RETURN_IF_ERROR(s_dev.Init(a, k.const_scales));
+  if (k.const_zero_points != nullptr) MI_RETURN_IF_ERROR(z_dev.Init(a, k.const_zero_points));
+
+  void* buffer = allocator != nullptr ? allocator->Alloc(allocator, bytes) : nullptr;
+  OrtAllocator* owner = allocator;
+  if (buffer == nullptr) {
+    owner = nullptr;
+    MI_RETURN_IF_HIP(a, hipMalloc(&buffer, bytes));
+  }
+  int rc = MnbPackQuantBData(static_cast<size_t>(k.N), static_cast<size_t>(k.K), static_cast<int>(k.bits),
+                             static_cast<int>(k.block_size), dtype, b_dev.get(), s_dev.get(), z_dev.get(), buffer,
+                             /*stream*/ nullptr);
+  hipError_t sync = rc == MNB_OK ? hipStreamSynchronize(nullptr) : hipSuccess;  // inputs may be freed on return
+  if (rc != MNB_OK || sync != hipSuccess) {
+    if (owner != nullptr)
+      owner->Free(owner, buffer);
+    else
+      (void)hipFree(buffer);
+    if (rc != MNB_OK) return StatusFromMnb(a, rc);
+    return a.ort->CreateStatus(ORT_EP_FAIL, hipGetErrorString(sync));
+  }
+  k.packed = buffer;
+  k.packed_allocator = owner;
+  k.packed_dtype = dtype;
+  k.packed_has_zp = k.const_zero_points != nullptr;
+  *is_packed = true;
+  return nullptr;
+}
+
+OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelContext* ctx) noexcept {
+  MatMulNBitsKernel& k = *Self(this_ptr);
+  const Apis& a = k.apis;
+  size_t num_inputs = 0;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetInputCount(ctx, &num_inputs));
+  const OrtValue* in[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  for (size_t i = 0; i < 6 && i < num_inputs; ++i) {
+    // inputs that PrePack consumed are gone from the context
+    if (k.packed != nullptr && (i == kB || i == kScales || i == kZeroPoints)) continue;
+    MI_RETURN_IF_ERROR(a.ort->KernelContext_GetInput(ctx, i, &in[i]));
+  }
+  if (in[kA] == nullptr) return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: input A is missing");
+
+  TensorDesc d[6];
+  const TensorDesc* present[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  for (size_t i = 0; i < 6; ++i) {
+    if (in[i] == nullptr) continue;
+    MI_RETURN_IF_ERROR(Describe(a, in[i], &d[i]));
+    present[i] = &d[i];
+  }
+  MnbTensorInfo bi = ToMnb(present[kB]), si = ToMnb(present[kScales]), zi = ToMnb(present[kZeroPoints]),
+                gi = ToMnb(present[kGIdx]), biasi = ToMnb(present[kBias]);
+  if (k.packed == nullptr && present[kScales] == nullptr) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: scales are required when B was not prepacked");
+  }
+  // With packed weights the scales / zero points were validated at PrePack time and are no longer inputs.
+  if (k.packed == nullptr) {
+    MI_RETURN_IF_ERROR(StatusFromMnb(a, MnbCheckInputs(&bi, &si, &zi, &gi, &biasi, k.N, k.K, k.block_size, k.bits)));
+  } else if (present[kBias] != nullptr) {
+    if (d[kBias].dims.size() != 1 || d[kBias].dims[0] != k.N) {
+      return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "bias must be a 1D tensor with shape [N]");
+    }
+  }
+  if (present[kGIdx] != nullptr) {
+    return a.ort->CreateStatus(ORT_NOT_IMPLEMENTED, "MatMulNBits with g_idx has no MI355X kernel");
+  }
+
+  const TensorDesc& ad = d[kA];
+  const int dtype = static_cast<int>(ad.type);
+  if (dtype != MNB_DTYPE_FLOAT && dtype != MNB_DTYPE_FLOAT16) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A must be float or float16");
+  }
+  if (ad.dims.empty() || ad.dims.back() != k.K) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMul dimension mismatch");  // MatMulComputeHelper
+  }
+  std::vector<int64_t> y_dims(ad.dims.begin(), ad.dims.end() - 1);
+  y_dims.push_back(k.N);
+  int64_t M = 1;
+  for (size_t i = 0; i + 1 < ad.dims.size(); ++i) M *= ad.dims[i];
+
+  OrtValue* y = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetOutput(ctx, 0, y_dims.data(), y_dims.size(), &y));
+  if (M == 0 || k.N == 0) return nullptr;  // empty output (matmul_nbits.cc:1533-1536)
+
+  const void* a_ptr = nullptr;
+  const void* bias_ptr = nullptr;
+  void* y_ptr = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->GetTensorData(in[kA], &a_ptr));
+  if (in[kBias] != nullptr) MI_RETURN_IF_ERROR(a.ort->GetTensorData(in[kBias], &bias_ptr));
+  MI_RETURN_IF_ERROR(a.ort->GetTensorMutableData(y, &y_ptr));
+  void* stream = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetGPUComputeStream(ctx, &stream));
+
+  const size_t Mz = static_cast<size_t>(M), Nz = static_cast<size_t>(k.N), Kz = static_cast<size_t>(k.K);
+  const int bits = static_cast<int>(k.bits), bs = static_cast<int>(k.block_size);
+  if (k.packed != nullptr) {
+    if (dtype != k.packed_dtype) {
+      return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A and scales must have the same element type");
+    }
+    return StatusFromMnb(a, MnbGemm(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr,
+                                    Nz, nullptr, 0, stream));
+  }
+
+  // B was not packed at session initialisation (prepacking disabled, or B / scales / zero points are not constant
+  // initializers): pack into stream-ordered scratch memory, then run the same kernels (matmul_nbits.cc:1184-1333).
+  if (in[kB] == nullptr) return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: input B is missing");
+  if (static_cast<int>(d[kScales].type) != dtype) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A and scales must have the same element type");
+  }
+  if (present[kZeroPoints] != nullptr && d[kZeroPoints].type != ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8) {
+    return a.ort->CreateStatus(ORT_NOT_IMPLEMENTED, "MatMulNBits: only uint8 zero points have an MI355X kernel");
+  }
+  const void* b_ptr = nullptr;
+  const void* s_ptr = nullptr;
+  const void* z_ptr = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->GetTensorData(in[kB], &b_ptr));
+  MI_RETURN_IF_ERROR(a.ort->GetTensorData(in[kScales], &s_ptr));
+  if (in[kZeroPoints] != nullptr) MI_RETURN_IF_ERROR(a.ort->GetTensorData(in[kZeroPoints], &z_ptr));
+  const size_t ws_bytes = MnbGemmUnpackedWorkspaceSize(Mz, Nz, Kz, bits, bs, z_ptr != nullptr, dtype);
+  if (ws_bytes == 0) return a.ort->CreateStatus(ORT_NOT_IMPLEMENTED, "MatMulNBits: configuration has no MI355X kernel");
+  void* ws = nullptr;
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  MI_RETURN_IF_HIP(a, hipMallocAsync(&ws, ws_bytes, hs));
+  int rc = MnbGemmUnpacked(Mz, Nz, Kz, bits, bs, dtype, a_ptr, Kz, b_ptr, s_ptr, z_ptr, bias_ptr, y_ptr, Nz, ws,
+                           ws_bytes, stream);
+  hipError_t free_err = hipFreeAsync(ws, hs);
+  MI_RETURN_IF_ERROR(StatusFromMnb(a, rc));
+  MI_RETURN_IF_HIP(a, free_err);
+  return nullptr;
+}
+
+bool InputExists(const Apis& a, const OrtKernelInfo* info, size_t index, size_t count) {
+  if (index >= count) return false;
+  size_t size = 0;
+  OrtStatus* st = a.ort->KernelInfo_GetInputName(info, index, nullptr, &size);
+  if (st != nullptr) {
+    a.ort->ReleaseStatus(st);
+    return false;
+  }
+  return size > 1;  // an omitted optional input has the empty name
+}
+
+OrtStatus* ORT_API_CALL CreateMatMulNBits(void* state, const OrtKernelInfo* info, OrtKernelImpl** kernel_out) noexcept {
+  const Apis& a = *static_cast<const Apis*>(state);
+  *kernel_out = nullptr;
+  std::unique_ptr<MatMulNBitsKernel> k(new (std::nothrow) MatMulNBitsKernel{});
+  if (!k) return a.ort->CreateStatus(ORT_FAIL, "out of memory creating the MatMulNBits kernel");
+  k->ort_version_supported = ORT_API_VERSION;
+  k->flags = 0;
+  k->Compute = MatMulNBitsCompute;
+  k->Release = MatMulNBitsRelease;
+  k->PrePackWeight = MatMulNBitsPrePack;
+  k->SetSharedPrePackedWeight = nullptr;  // device buffers are never shared through the host-side cache
+  k->apis = a;
+  MI_RETURN_IF_ERROR(a.ort->KernelInfoGetAttribute_int64(info, "K", &k->K));
+  MI_RETURN_IF_ERROR(a.ort->KernelInfoGetAttribute_int64(info, "N", &k->N));
+  MI_RETURN_IF_ERROR(a.ort->KernelInfoGetAttribute_int64(info, "block_size", &k->block_size));
+  if (OrtStatus* st = a.ort->KernelInfoGetAttribute_int64(info, "bits", &k->bits)) {
+    a.ort->ReleaseStatus(st);
+    k->bits = 4;  // schema default
+  }
+  if (OrtStatus* st = a.ort->KernelInfoGetAttribute_int64(info, "accuracy_level", &k->accuracy_level)) {
+    a.ort->ReleaseStatus(st);
+    k->accuracy_level = 0;
+  }
+  if (k->bits != 2 && k->bits != 4 && k->bits != 8) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT,
+                               "Only 2b, 4b and 8b quantization is supported for MatMulNBits op, additional bits "
+                               "support is planned.");
+  }
+  if (k->block_size != 16 && k->block_size != 32 && k->block_size != 64 && k->block_size != 128 &&
+      k->block_size != 256) {
+    std::string msg = "Only block sizes 16, 32, 64, 128, and 256 are supported for MatMulNBits op, got: " +
+                      std::to_string(k->block_size);
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, msg.c_str());
+  }
+  size_t count = 0;
+  MI_RETURN_IF_ERROR(a.ort->KernelInfo_GetInputCount(info, &count));
+  k->has_zp_arg = InputExists(a, info, kZeroPoints, count);
+  k->has_g_idx = InputExists(a, info, kGIdx, count);
+  int is_constant = 0;
+  const OrtValue* value = nullptr;
+  if (count > kScales) {
+    MI_RETURN_IF_ERROR(a.ort->KernelInfoGetConstantInput_tensor(info, kScales, &is_constant, &value));
+    if (is_constant) k->const_scales = value;
+  }
+  if (k->has_zp_arg) {
+    is_constant = 0;
+    value = nullptr;
+    MI_RETURN_IF_ERROR(a.ort->KernelInfoGetConstantInput_tensor(info, kZeroPoints, &is_constant, &value));
+    if (is_constant) k->const_zero_points = value;
+  }
+  *kernel_out = k.release();
+  return nullptr;
+}
+
+// =========================================================================================== Memcpy
+struct MemcpyKernel : OrtKernelImpl {
+  Apis apis;
+};
+
+void ORT_API_CALL MemcpyRelease(OrtKernelImpl* this_ptr) noexcept { delete static_cast<MemcpyKernel*>(this_ptr); }
+
+OrtStatus* ORT_API_CALL MemcpyCompute(OrtKernelImpl* this_ptr, OrtKernelContext* ctx) noexcept {
+  const Apis& a = static_cast<MemcpyKernel*>(this_ptr)->apis;
+  const OrtValue* x = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetInput(ctx, 0, &x));
+  if (x == nullptr) return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "Memcpy: input tensor is missing");
+  TensorDesc xd;
+  MI_RETURN_IF_ERROR(Describe(a, x, &xd));
+  OrtValue* y = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetOutput(ctx, 0, xd.dims.data(), xd.dims.size(), &y));
+  size_t bytes = 0;
+  MI_RETURN_IF_ERROR(a.ort->GetTensorSizeInBytes(x, &bytes));
+  if (bytes == 0) return nullptr;
+  const void* src = nullptr;
+  void* dst = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->GetTensorData(x, &src));
+  MI_RETURN_IF_ERROR(a.ort->GetTensorMutableData(y, &dst));
+  if (src == dst) return nullptr;
+  const bool src_host = OnHost(a, x), dst_host = OnHost(a, y);
+  hipMemcpyKind kind = src_host ? (dst_host ? hipMemcpyHostToHost : hipMemcpyHostToDevice)
+                                : (dst_host ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice);
+  void* stream = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetGPUComputeStream(ctx, &stream));
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+  MI_RETURN_IF_HIP(a, hipMemcpyAsync(dst, src, bytes, kind, hs));
+  // The consumer of a MemcpyToHost output is a CPU kernel that reads the bytes as soon as this returns.
+  if (dst_host) MI_RETURN_IF_HIP(a, hipStreamSynchronize(hs));
+  return nullptr;
+}
+
+OrtStatus* ORT_API_CALL CreateMemcpy(void* state, const OrtKernelInfo*, OrtKernelImpl** kernel_out) noexcept {
+  const Apis& a = *static_cast<const Apis*>(state);
+  auto* k = new (std::nothrow) MemcpyKernel{};
+  *kernel_out = k;
+  if (k == nullptr) return a.ort->CreateStatus(ORT_FAIL, "out of memory creating a Memcpy kernel");
+  k->ort_version_supported = ORT_API_VERSION;
+  k->flags = 0;
+  k->Compute = MemcpyCompute;
+  k->Release = MemcpyRelease;
+  k->PrePackWeight = nullptr;
+  k->SetSharedPrePackedWeight = nullptr;
+  k->apis = a;
+  return nullptr;
+}
+
+// =========================================================================================== registration
+struct DefBuilder {
+  const Apis& a;
+  OrtKernelDefBuilder* b = nullptr;
+  explicit DefBuilder(const Apis& apis) : a(apis) {}
+  ~DefBuilder() {
+    if (b != nullptr) a.ep->ReleaseKernelDefBuilder(b);
+  }
+};
+
+OrtStatus* TypeList(const Apis& a, const std::vector<ONNXTensorElementDataType>& elems,
+                    std::vector<const OrtDataType*>* out) {
+  out->clear();
+  for (auto e : elems) {
+    const OrtDataType* t = nullptr;
+    MI_RETURN_IF_ERROR(a.ep->GetTensorDataType(e, &t));
+    out->push_back(t);
+  }
+  return nullptr;
+}
+
+OrtStatus* AddMatMulNBits(const Apis& a, const Apis* state, const char* ep_name, OrtKernelRegistry* registry,
+                          ONNXTensorElementDataType t1) {
+  DefBuilder db(a);
+  MI_RETURN_IF_ERROR(a.ep->CreateKernelDefBuilder(&db.b));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetOperatorType(db.b, "MatMulNBits"));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetDomain(db.b, kMsDomain));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetSinceVersion(db.b, 1, 1));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetExecutionProvider(db.b, ep_name));
+  std::vector<const OrtDataType*> types;
+  MI_RETURN_IF_ERROR(TypeList(a, {t1}, &types));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T1", types.data(), types.size()));
+  MI_RETURN_IF_ERROR(TypeList(a, {ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8}, &types));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T2", types.data(), types.size()));
+  // Zero points in the activation type (the reference's "unquantized zero point" route) stay on the CPU provider.
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T3", types.data(), types.size()));
+  MI_RETURN_IF_ERROR(TypeList(a, {ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32}, &types));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T4", types.data(), types.size()));
+  OrtKernelDef* def = nullptr;
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_Build(db.b, &def));
+  OrtStatus* st = a.ep->KernelRegistry_AddKernel(registry, def, CreateMatMulNBits, const_cast<Apis*>(state));
+  a.ep->ReleaseKernelDef(def);
+  return st;
+}
+
+OrtStatus* AddMemcpy(const Apis& a, const Apis* state, const char* ep_name, OrtKernelRegistry* registry,
+                     bool from_host) {
+  DefBuilder db(a);
+  MI_RETURN_IF_ERROR(a.ep->CreateKernelDefBuilder(&db.b));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetOperatorType(db.b, from_host ? "MemcpyFromHost" : "MemcpyToHost"));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetDomain(db.b, kOnnxDomain));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetSinceVersion(db.b, 1, 1));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetExecutionProvider(db.b, ep_name));
+  if (from_host)
+    MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetInputMemType(db.b, 0, OrtMemTypeCPUInput));
+  else
+    MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetOutputMemType(db.b, 0, OrtMemTypeCPUOutput));
+  // Only the tensor types that can reach or leave a MatMulNBits node cross the boundary of this provider.
+  std::vector<const OrtDataType*> types;
+  MI_RETURN_IF_ERROR(TypeList(a,
+                              {ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16,
+                               ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8, ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32},
+                              &types));
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T", types.data(), types.size()));
+  OrtKernelDef* def = nullptr;
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_Build(db.b, &def));
+  OrtStatus* st = a.ep->KernelRegistry_AddKernel(registry, def, CreateMemcpy, const_cast<Apis*>(state));
+  a.ep->ReleaseKernelDef(def);
+  return st;
+}
+
+}  // namespace
+
+OrtStatus* CreateKernelRegistry(const Apis& apis, const char* ep_name, OrtKernelRegistry** out) {
+  *out = nullptr;
+  // Kernel create functions receive this pointer as their state; it outlives every session of the process.
+  static const Apis* state = new Apis(apis);
+  OrtKernelRegistry* registry = nullptr;
+  MI_RETURN_IF_ERROR(apis.ep->CreateKernelRegistry(&registry));
+  OrtStatus* st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT);
+  if (st == nullptr) st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16);
+  if (st == nullptr) st = AddMemcpy(apis, state, ep_name, registry, /*from_host*/ true);
+  if (st == nullptr) st = AddMemcpy(apis, state, ep_name, registry, /*from_host*/ false);
+  if (st != nullptr) {
+    apis.ep->ReleaseKernelRegistry(registry);
+    return st;
+  }
+  *out = registry;
+  return nullptr;
+}
+
+}  // namespace mi355x_ep

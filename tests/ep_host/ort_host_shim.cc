@@ -1,0 +1,792 @@
+// Test double of the ONNX Runtime side of the plugin-EP C ABI.
+//
+// No ONNX Runtime binary exists in the build image, so the tests load libonnxruntime_mi355x_ep.so into this host
+// instead.  It is compiled against the same public headers as the plugin (onnxruntime_c_api.h /
+// onnxruntime_ep_c_api.h, found on the include path), defines the opaque Ort* types itself, fills the OrtApi /
+// OrtEpApi tables with the entries the plugin uses (every other entry stays NULL, so a call the host does not model
+// crashes the test instead of passing silently) and then walks a session's life the way ONNX Runtime does:
+//   CreateEpFactories -> GetSupportedDevices -> CreateEp -> GetKernelRegistry -> GetCapability on a one-node graph
+//   -> allocator / data transfer / stream from the factory -> initializers copied to the device -> kernel creation
+//   -> PrePackWeight per constant input (packed initializers are freed) -> MemcpyFromHost -> Compute ->
+//   MemcpyToHost -> release of everything.
+// It is test infrastructure only; nothing in the product links to it.
+#include <dlfcn.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "onnxruntime_c_api.h"
+
+// ------------------------------------------------------------------------------------------- opaque types
+struct OrtStatus {
+  OrtErrorCode code;
+  std::string msg;
+};
+struct OrtMemoryDevice {
+  OrtMemoryInfoDeviceType type;
+  OrtDeviceMemoryType mem_type;
+  uint32_t vendor;
+  uint32_t device_id;
+};
+struct OrtMemoryInfo {
+  std::string name;
+  OrtMemoryDevice dev;
+  size_t alignment;
+  OrtAllocatorType alloc_type;
+};
+struct OrtValue {
+  std::vector<int64_t> dims;
+  ONNXTensorElementDataType type = ONNX_TENSOR_ELEMENT_DATA_TYPE_UNDEFINED;
+  void* data = nullptr;
+  size_t bytes = 0;
+  const OrtMemoryInfo* mem = nullptr;
+  OrtAllocator* owner = nullptr;  // frees `data`; NULL = borrowed or malloc'ed host memory
+  bool host_owned = false;
+  ~OrtValue() {
+    if (data == nullptr) return;
+    if (owner != nullptr)
+      owner->Free(owner, data);
+    else if (host_owned)
+      free(data);
+  }
+};
+struct OrtTensorTypeAndShapeInfo {
+  std::vector<int64_t> dims;
+  ONNXTensorElementDataType type;
+};
+struct OrtHardwareDevice {
+  OrtHardwareDeviceType type;
+  uint32_t vendor_id;
+  uint32_t device_id;
+};
+struct OrtEpDevice {
+  OrtEpFactory* factory;
+  const OrtHardwareDevice* hw;
+  std::vector<const OrtMemoryInfo*> mem_infos;
+};
+struct OrtDataType {
+  ONNXTensorElementDataType elem;
+};
+struct OrtKernelDef {
+  std::string op, domain, ep;
+  int start = 1, end = 1;
+  std::map<std::string, std::vector<ONNXTensorElementDataType>> constraints;
+  std::map<size_t, OrtMemType> input_mem, output_mem;
+};
+struct OrtKernelDefBuilder {
+  OrtKernelDef def;
+};
+struct OrtKernelRegistry {
+  struct Entry {
+    OrtKernelDef def;
+    OrtKernelCreateFunc fn;
+    void* state;
+  };
+  std::vector<Entry> entries;
+};
+struct OrtOpAttr {
+  std::string name;
+  int64_t value;
+};
+struct OrtValueInfo {
+  std::string name;
+};
+struct OrtNode {
+  std::string op, domain, name;
+  int since_version = 1;
+  std::vector<std::unique_ptr<OrtValueInfo>> inputs;  // NULL entry = omitted optional input
+  std::vector<OrtOpAttr> attrs;
+  std::vector<std::string> schema_attrs;                     // attribute names the operator schema knows
+  std::map<std::string, ONNXTensorElementDataType> types;    // type-constraint name -> bound element type
+};
+struct OrtGraph {
+  std::vector<const OrtNode*> nodes;
+};
+struct OrtEpGraphSupportInfo {
+  const OrtKernelRegistry* registry;
+  std::string ep_name;
+  std::vector<const OrtNode*> claimed;
+};
+struct OrtKernelInfo {
+  const OrtNode* node;
+  std::map<size_t, const OrtValue*> constants;
+};
+struct OrtSyncStream {
+  OrtSyncStreamImpl* impl;
+};
+struct OrtKernelContext {
+  std::vector<const OrtValue*> inputs;
+  std::vector<std::unique_ptr<OrtValue>> outputs;
+  std::vector<bool> output_on_host;
+  OrtAllocator* device_allocator;
+  const OrtMemoryInfo* cpu_mem;
+  OrtSyncStream* stream;
+};
+
+namespace {
+
+size_t ElemSize(ONNXTensorElementDataType t) {
+  switch (t) {
+    case ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT:
+    case ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32:
+      return 4;
+    case ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16:
+      return 2;
+    case ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8:
+      return 1;
+    default:
+      return 0;
+  }
+}
+
+size_t ByteSize(const std::vector<int64_t>& dims, ONNXTensorElementDataType t) {
+  size_t n = ElemSize(t);
+  for (int64_t d : dims) n *= static_cast<size_t>(d);
+  return n;
+}
+
+OrtStatus* MakeStatus(OrtErrorCode code, const char* msg) { return new OrtStatus{code, msg ? msg : ""}; }
+
+const OrtKernelRegistry::Entry* LookUp(const OrtKernelRegistry& reg, const std::string& ep, const OrtNode& node) {
+  for (const auto& e : reg.entries) {
+    const OrtKernelDef& d = e.def;
+    if (d.op != node.op || d.domain != node.domain || d.ep != ep) continue;
+    if (node.since_version < d.start || node.since_version > d.end) continue;
+    bool ok = true;
+    for (const auto& c : d.constraints) {
+      auto it = node.types.find(c.first);
+      if (it == node.types.end()) continue;  // the node does not use that formal parameter
+      bool found = false;
+      for (auto t : c.second) found = found || t == it->second;
+      ok = ok && found;
+    }
+    if (ok) return &e;
+  }
+  return nullptr;
+}
+
+// ------------------------------------------------------------------------------------------- API tables
+OrtApi g_ort{};
+OrtEpApi g_ep{};
+OrtDataType g_types[32];
+
+void FillApis() {
+  static bool done = false;
+  if (done) return;
+  done = true;
+  for (int i = 0; i < 32; ++i) g_types[i].elem = static_cast<ONNXTensorElementDataType>(i);
+
+  // ---- OrtApi
+  g_ort.CreateStatus = [](OrtErrorCode code, const char* msg) noexcept -> OrtStatus* { return MakeStatus(code, msg); };
+  g_ort.GetErrorCode = [](const OrtStatus* s) noexcept { return s->code; };
+  g_ort.GetErrorMessage = [](const OrtStatus* s) noexcept { return s->msg.c_str(); };
+  g_ort.ReleaseStatus = [](OrtStatus* s) noexcept { delete s; };
+  g_ort.GetEpApi = []() noexcept -> const OrtEpApi* { return &g_ep; };
+  g_ort.HardwareDevice_Type = [](const OrtHardwareDevice* d) noexcept { return d->type; };
+  g_ort.HardwareDevice_VendorId = [](const OrtHardwareDevice* d) noexcept { return d->vendor_id; };
+  g_ort.HardwareDevice_DeviceId = [](const OrtHardwareDevice* d) noexcept { return d->device_id; };
+  g_ort.CreateMemoryInfo_V2 = [](const char* name, OrtMemoryInfoDeviceType type, uint32_t vendor, int32_t device_id,
+                                 OrtDeviceMemoryType mem_type, size_t alignment, OrtAllocatorType alloc_type,
+                                 OrtMemoryInfo** out) noexcept -> OrtStatus* {
+    *out = new OrtMemoryInfo{name, {type, mem_type, vendor, static_cast<uint32_t>(device_id)}, alignment, alloc_type};
+    return nullptr;
+  };
+  g_ort.ReleaseMemoryInfo = [](OrtMemoryInfo* m) noexcept { delete m; };
+  g_ort.KernelInfoGetAttribute_int64 = [](const OrtKernelInfo* info, const char* name, int64_t* out) noexcept
+      -> OrtStatus* {
+    for (const auto& a : info->node->attrs)
+      if (a.name == name) {
+        *out = a.value;
+        return nullptr;
+      }
+    return MakeStatus(ORT_FAIL, (std::string("No attribute with name:'") + name + "'is defined.").c_str());
+  };
+  g_ort.KernelInfo_GetInputCount = [](const OrtKernelInfo* info, size_t* out) noexcept -> OrtStatus* {
+    *out = info->node->inputs.size();
+    return nullptr;
+  };
+  g_ort.KernelInfo_GetInputName = [](const OrtKernelInfo* info, size_t index, char* out, size_t* size) noexcept
+      -> OrtStatus* {
+    if (index >= info->node->inputs.size())
+      return MakeStatus(ORT_INVALID_ARGUMENT, "::OrtKernelInfo input index is out of bounds");
+    const std::string name = info->node->inputs[index] ? info->node->inputs[index]->name : std::string();
+    const size_t need = name.size() + 1;
+    if (out == nullptr) {
+      *size = need;
+      return nullptr;
+    }
+    if (*size < need) {
+      *size = need;
+      return MakeStatus(ORT_INVALID_ARGUMENT, "Output buffer is not large enough for ::OrtKernelInfo input name");
+    }
+    std::memcpy(out, name.c_str(), need);
+    *size = need;
+    return nullptr;
+  };
+  g_ort.KernelInfoGetConstantInput_tensor = [](const OrtKernelInfo* info, size_t index, int* is_constant,
+                                               const OrtValue** out) noexcept -> OrtStatus* {
+    auto it = info->constants.find(index);
+    *is_constant = it != info->constants.end();
+    *out = *is_constant ? it->second : nullptr;
+    return nullptr;
+  };
+  g_ort.GetTensorTypeAndShape = [](const OrtValue* v, OrtTensorTypeAndShapeInfo** out) noexcept -> OrtStatus* {
+    *out = new OrtTensorTypeAndShapeInfo{v->dims, v->type};
+    return nullptr;
+  };
+  g_ort.ReleaseTensorTypeAndShapeInfo = [](OrtTensorTypeAndShapeInfo* i) noexcept { delete i; };
+  g_ort.GetDimensionsCount = [](const OrtTensorTypeAndShapeInfo* i, size_t* out) noexcept -> OrtStatus* {
+    *out = i->dims.size();
+    return nullptr;
+  };
+  g_ort.GetDimensions = [](const OrtTensorTypeAndShapeInfo* i, int64_t* dims, size_t n) noexcept -> OrtStatus* {
+    for (size_t k = 0; k < n && k < i->dims.size(); ++k) dims[k] = i->dims[k];
+    return nullptr;
+  };
+  g_ort.GetTensorElementType = [](const OrtTensorTypeAndShapeInfo* i, ONNXTensorElementDataType* out) noexcept
+      -> OrtStatus* {
+    *out = i->type;
+    return nullptr;
+  };
+  g_ort.GetTensorData = [](const OrtValue* v, const void** out) noexcept -> OrtStatus* {
+    *out = v->data;
+    return nullptr;
+  };
+  g_ort.GetTensorMutableData = [](OrtValue* v, void** out) noexcept -> OrtStatus* {
+    *out = v->data;
+    return nullptr;
+  };
+  g_ort.GetTensorSizeInBytes = [](const OrtValue* v, size_t* out) noexcept -> OrtStatus* {
+    *out = v->bytes;
+    return nullptr;
+  };
+  g_ort.KernelContext_GetInputCount = [](const OrtKernelContext* c, size_t* out) noexcept -> OrtStatus* {
+    *out = c->inputs.size();
+    return nullptr;
+  };
+  g_ort.KernelContext_GetInput = [](const OrtKernelContext* c, size_t index, const OrtValue** out) noexcept
+      -> OrtStatus* {
+    *out = index < c->inputs.size() ? c->inputs[index] : nullptr;
+    return nullptr;
+  };
+  g_ort.KernelContext_GetOutput = [](OrtKernelContext* c, size_t index, const int64_t* dims, size_t rank,
+                                     OrtValue** out) noexcept -> OrtStatus* {
+    if (index >= c->outputs.size()) return MakeStatus(ORT_INVALID_ARGUMENT, "output index out of range");
+    if (!c->outputs[index]) {
+      auto v = std::make_unique<OrtValue>();
+      v->dims.assign(dims, dims + rank);
+      v->type = c->inputs[0]->type;  // every kernel modelled here produces the type of its first input
+      v->bytes = ByteSize(v->dims, v->type);
+      if (c->output_on_host[index]) {
+        v->mem = c->cpu_mem;
+        v->data = v->bytes ? malloc(v->bytes) : nullptr;
+        v->host_owned = true;
+      } else {
+        v->mem = c->device_allocator->Info(c->device_allocator);
+        v->owner = c->device_allocator;
+        v->data = v->bytes ? c->device_allocator->Alloc(c->device_allocator, v->bytes) : nullptr;
+        if (v->bytes && v->data == nullptr) return MakeStatus(ORT_FAIL, "device allocation of an output failed");
+      }
+      c->outputs[index] = std::move(v);
+    }
+    *out = c->outputs[index].get();
+    return nullptr;
+  };
+  g_ort.KernelContext_GetGPUComputeStream = [](const OrtKernelContext* c, void** out) noexcept -> OrtStatus* {
+    *out = c->stream ? c->stream->impl->GetHandle(c->stream->impl) : nullptr;
+    return nullptr;
+  };
+  g_ort.SyncStream_GetHandle = [](OrtSyncStream* s) noexcept -> void* { return s->impl->GetHandle(s->impl); };
+  g_ort.Graph_GetNumNodes = [](const OrtGraph* g, size_t* n) noexcept -> OrtStatus* {
+    *n = g->nodes.size();
+    return nullptr;
+  };
+  g_ort.Graph_GetNodes = [](const OrtGraph* g, const OrtNode** nodes, size_t n) noexcept -> OrtStatus* {
+    for (size_t i = 0; i < n && i < g->nodes.size(); ++i) nodes[i] = g->nodes[i];
+    return nullptr;
+  };
+  g_ort.Node_GetOperatorType = [](const OrtNode* n, const char** out) noexcept -> OrtStatus* {
+    *out = n->op.c_str();
+    return nullptr;
+  };
+  g_ort.Node_GetDomain = [](const OrtNode* n, const char** out) noexcept -> OrtStatus* {
+    *out = n->domain.c_str();
+    return nullptr;
+  };
+  g_ort.Node_GetName = [](const OrtNode* n, const char** out) noexcept -> OrtStatus* {
+    *out = n->name.c_str();
+    return nullptr;
+  };
+  g_ort.Node_GetNumInputs = [](const OrtNode* n, size_t* out) noexcept -> OrtStatus* {
+    *out = n->inputs.size();
+    return nullptr;
+  };
+  g_ort.Node_GetInputs = [](const OrtNode* n, const OrtValueInfo** inputs, size_t count) noexcept -> OrtStatus* {
+    for (size_t i = 0; i < count && i < n->inputs.size(); ++i) inputs[i] = n->inputs[i].get();
+    return nullptr;
+  };
+  g_ort.Node_GetAttributeByName = [](const OrtNode* n, const char* name, const OrtOpAttr** out) noexcept
+      -> OrtStatus* {
+    *out = nullptr;
+    for (const auto& a : n->attrs)
+      if (a.name == name) {
+        *out = &a;
+        return nullptr;
+      }
+    for (const auto& s : n->schema_attrs)
+      if (s == name) return nullptr;  // optional attribute left unset
+    return MakeStatus(ORT_NOT_FOUND, "attribute not found");
+  };
+  g_ort.ReadOpAttr = [](const OrtOpAttr* a, OrtOpAttrType type, void* data, size_t len, size_t* out) noexcept
+      -> OrtStatus* {
+    if (type != ORT_OP_ATTR_INT || len < sizeof(int64_t)) return MakeStatus(ORT_INVALID_ARGUMENT, "bad ReadOpAttr");
+    *static_cast<int64_t*>(data) = a->value;
+    *out = sizeof(int64_t);
+    return nullptr;
+  };
+
+  // ---- OrtEpApi
+  g_ep.CreateEpDevice = [](OrtEpFactory* f, const OrtHardwareDevice* hw, const OrtKeyValuePairs*,
+                           const OrtKeyValuePairs*, OrtEpDevice** out) noexcept -> OrtStatus* {
+    *out = new OrtEpDevice{f, hw, {}};
+    return nullptr;
+  };
+  g_ep.ReleaseEpDevice = [](OrtEpDevice* d) noexcept { delete d; };
+  g_ep.EpDevice_AddAllocatorInfo = [](OrtEpDevice* d, const OrtMemoryInfo* m) noexcept -> OrtStatus* {
+    d->mem_infos.push_back(m);
+    return nullptr;
+  };
+  g_ep.EpGraphSupportInfo_AddSingleNode = [](OrtEpGraphSupportInfo* g, const OrtNode* n) noexcept -> OrtStatus* {
+    g->claimed.push_back(n);
+    return nullptr;
+  };
+  g_ep.EpGraphSupportInfo_LookUpKernel = [](OrtEpGraphSupportInfo* g, const OrtNode* n,
+                                            const OrtKernelDef** out) noexcept -> OrtStatus* {
+    const auto* e = LookUp(*g->registry, g->ep_name, *n);
+    *out = e ? &e->def : nullptr;
+    return nullptr;
+  };
+  g_ep.MemoryInfo_GetMemoryDevice = [](const OrtMemoryInfo* m) noexcept -> const OrtMemoryDevice* { return &m->dev; };
+  g_ep.Value_GetMemoryDevice = [](const OrtValue* v) noexcept -> const OrtMemoryDevice* { return &v->mem->dev; };
+  g_ep.MemoryDevice_AreEqual = [](const OrtMemoryDevice* a, const OrtMemoryDevice* b) noexcept {
+    return a->type == b->type && a->mem_type == b->mem_type && a->vendor == b->vendor &&
+           a->device_id == b->device_id;
+  };
+  g_ep.MemoryDevice_GetDeviceType = [](const OrtMemoryDevice* d) noexcept { return d->type; };
+  g_ep.MemoryDevice_GetMemoryType = [](const OrtMemoryDevice* d) noexcept { return d->mem_type; };
+  g_ep.MemoryDevice_GetVendorId = [](const OrtMemoryDevice* d) noexcept { return d->vendor; };
+  g_ep.MemoryDevice_GetDeviceId = [](const OrtMemoryDevice* d) noexcept { return d->device_id; };
+  g_ep.CreateKernelRegistry = [](OrtKernelRegistry** out) noexcept -> OrtStatus* {
+    *out = new OrtKernelRegistry{};
+    return nullptr;
+  };
+  g_ep.ReleaseKernelRegistry = [](OrtKernelRegistry* r) noexcept { delete r; };
+  g_ep.KernelRegistry_AddKernel = [](OrtKernelRegistry* r, const OrtKernelDef* def, OrtKernelCreateFunc fn,
+                                     void* state) noexcept -> OrtStatus* {
+    r->entries.push_back({*def, fn, state});
+    return nullptr;
+  };
+  g_ep.CreateKernelDefBuilder = [](OrtKernelDefBuilder** out) noexcept -> OrtStatus* {
+    *out = new OrtKernelDefBuilder{};
+    return nullptr;
+  };
+  g_ep.ReleaseKernelDefBuilder = [](OrtKernelDefBuilder* b) noexcept { delete b; };
+  g_ep.KernelDefBuilder_SetOperatorType = [](OrtKernelDefBuilder* b, const char* v) noexcept -> OrtStatus* {
+    b->def.op = v;
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_SetDomain = [](OrtKernelDefBuilder* b, const char* v) noexcept -> OrtStatus* {
+    b->def.domain = v;
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_SetSinceVersion = [](OrtKernelDefBuilder* b, int s, int e) noexcept -> OrtStatus* {
+    if (s < 1) return MakeStatus(ORT_INVALID_ARGUMENT, "Start version must be >= 1");
+    if (e < s) return MakeStatus(ORT_INVALID_ARGUMENT, "End version must be >= to the start version");
+    b->def.start = s;
+    b->def.end = e;
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_SetExecutionProvider = [](OrtKernelDefBuilder* b, const char* v) noexcept -> OrtStatus* {
+    b->def.ep = v;
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_SetInputMemType = [](OrtKernelDefBuilder* b, size_t i, OrtMemType t) noexcept -> OrtStatus* {
+    b->def.input_mem[i] = t;
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_SetOutputMemType = [](OrtKernelDefBuilder* b, size_t i, OrtMemType t) noexcept
+      -> OrtStatus* {
+    b->def.output_mem[i] = t;
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_AddTypeConstraint = [](OrtKernelDefBuilder* b, const char* name,
+                                               const OrtDataType* const* types, size_t n) noexcept -> OrtStatus* {
+    auto& v = b->def.constraints[name];
+    v.clear();
+    for (size_t i = 0; i < n; ++i) v.push_back(types[i]->elem);
+    return nullptr;
+  };
+  g_ep.KernelDefBuilder_Build = [](OrtKernelDefBuilder* b, OrtKernelDef** out) noexcept -> OrtStatus* {
+    if (b->def.op.empty() || b->def.ep.empty())
+      return MakeStatus(ORT_INVALID_ARGUMENT, "kernel def needs an operator type and an execution provider");
+    *out = new OrtKernelDef(b->def);
+    return nullptr;
+  };
+  g_ep.ReleaseKernelDef = [](OrtKernelDef* d) noexcept { delete d; };
+  g_ep.GetTensorDataType = [](ONNXTensorElementDataType t, const OrtDataType** out) noexcept -> OrtStatus* {
+    if (static_cast<int>(t) < 0 || static_cast<int>(t) >= 32) return MakeStatus(ORT_INVALID_ARGUMENT, "bad type");
+    *out = &g_types[static_cast<int>(t)];
+    return nullptr;
+  };
+}
+
+const OrtApi* ORT_API_CALL GetApi(uint32_t version) NO_EXCEPTION {
+  return version <= ORT_API_VERSION ? &g_ort : nullptr;
+}
+const char* ORT_API_CALL GetVersionString(void) NO_EXCEPTION { return "ort-host-shim"; }
+const OrtApiBase g_base{GetApi, GetVersionString};
+
+// ------------------------------------------------------------------------------------------- session walk
+struct Trace {
+  char* buf;
+  size_t len;
+  size_t used = 0;
+  void add(const char* fmt, ...) {
+    if (buf == nullptr || used >= len) return;
+    va_list ap;
+    va_start(ap, fmt);
+    int n = vsnprintf(buf + used, len - used, fmt, ap);
+    va_end(ap);
+    if (n > 0) used += static_cast<size_t>(n) < len - used ? static_cast<size_t>(n) : len - used - 1;
+  }
+};
+
+struct Plugin {
+  void* handle = nullptr;
+  CreateEpApiFactoriesFn create = nullptr;
+  ReleaseEpApiFactoryFn release = nullptr;
+};
+
+Plugin* LoadPlugin(const char* path, std::string* error) {
+  static std::map<std::string, Plugin> loaded;
+  auto it = loaded.find(path);
+  if (it != loaded.end()) return &it->second;
+  Plugin p;
+  p.handle = dlopen(path, RTLD_NOW | RTLD_LOCAL);
+  if (p.handle == nullptr) {
+    *error = std::string("dlopen failed: ") + dlerror();
+    return nullptr;
+  }
+  p.create = reinterpret_cast<CreateEpApiFactoriesFn>(dlsym(p.handle, "CreateEpFactories"));
+  p.release = reinterpret_cast<ReleaseEpApiFactoryFn>(dlsym(p.handle, "ReleaseEpFactory"));
+  if (p.create == nullptr || p.release == nullptr) {
+    *error = "the library does not export CreateEpFactories / ReleaseEpFactory";
+    return nullptr;
+  }
+  return &(loaded[path] = p);
+}
+
+int Fail(OrtStatus* st, const char* where, char* err, size_t err_len) {
+  int code = st->code == ORT_OK ? ORT_FAIL : static_cast<int>(st->code);
+  if (err != nullptr && err_len > 0) snprintf(err, err_len, "%s: %s", where, st->msg.c_str());
+  delete st;
+  return code;
+}
+
+int HostFail(int code, const std::string& msg, char* err, size_t err_len) {
+  if (err != nullptr && err_len > 0) snprintf(err, err_len, "%s", msg.c_str());
+  return code;
+}
+
+}  // namespace
+
+extern "C" {
+
+// One operator input handed in by the test: host data + shape. data == NULL: the optional input is absent.
+struct EpHostTensor {
+  const void* data;
+  const int64_t* dims;
+  size_t rank;
+  int dtype;  // ONNXTensorElementDataType
+};
+
+enum {
+  EP_HOST_NOT_CLAIMED = -1,   // GetCapability left the node to the CPU provider
+  EP_HOST_LOAD_FAILED = -2,
+  EP_HOST_NO_DEVICE = -3,     // the factory offered no OrtEpDevice
+  EP_HOST_PROTOCOL = -4       // the plugin broke an expectation of the host
+};
+
+// Factory-level queries that need no GPU. Writes "name|vendor|vendor_id|version|num_ep_devices" into `out`.
+__attribute__((visibility("default"))) int EpHostProbeFactory(const char* plugin_path, int offer_amd_gpu, char* out,
+                                                             size_t out_len, char* err, size_t err_len) {
+  FillApis();
+  std::string error;
+  Plugin* plugin = LoadPlugin(plugin_path, &error);
+  if (plugin == nullptr) return HostFail(EP_HOST_LOAD_FAILED, error, err, err_len);
+  OrtEpFactory* factory = nullptr;
+  size_t n = 0;
+  if (OrtStatus* st = plugin->create("mi355x", &g_base, nullptr, &factory, 1, &n))
+    return Fail(st, "CreateEpFactories", err, err_len);
+  if (n != 1 || factory == nullptr) return HostFail(EP_HOST_PROTOCOL, "expected exactly one factory", err, err_len);
+  OrtHardwareDevice cpu{OrtHardwareDeviceType_CPU, 0x8086, 0};
+  OrtHardwareDevice nv{OrtHardwareDeviceType_GPU, 0x10DE, 1};
+  OrtHardwareDevice amd{OrtHardwareDeviceType_GPU, 0x1002, 0x75A3};
+  std::vector<const OrtHardwareDevice*> hw{&cpu, &nv};
+  if (offer_amd_gpu) hw.push_back(&amd);
+  OrtEpDevice* devs[4] = {nullptr, nullptr, nullptr, nullptr};
+  size_t num = 0;
+  if (OrtStatus* st = factory->GetSupportedDevices(factory, hw.data(), hw.size(), devs, 4, &num)) {
+    plugin->release(factory);
+    return Fail(st, "GetSupportedDevices", err, err_len);
+  }
+  snprintf(out, out_len, "%s|%s|0x%04x|%s|%zu|%d", factory->GetName(factory), factory->GetVendor(factory),
+           factory->GetVendorId(factory), factory->GetVersion(factory), num,
+           static_cast<int>(factory->IsStreamAware(factory)));
+  for (size_t i = 0; i < num; ++i) delete devs[i];
+  plugin->release(factory);
+  return 0;
+}
+
+// Runs one com.microsoft::MatMulNBits node through the plugin.  `inputs` has six entries in operator order
+// (A, B, scales, zero_points, g_idx, bias); bit i of `constant_mask` marks input i as a constant initializer (the
+// host then offers it to PrePackWeight), the other inputs are fed per run.  Compute is called `repeat` times; the
+// result of the last call is copied to `y` (y_bytes capacity) and its shape to y_dims / y_rank (capacity 8).
+// Returns 0, an OrtErrorCode reported by the plugin, or a negative EP_HOST_* code; `trace` receives a short log
+// ("claimed=1 prepacked=1,2,3 ...").
+__attribute__((visibility("default"))) int EpHostRunMatMulNBits(
+    const char* plugin_path, int64_t N, int64_t K, int64_t bits, int64_t block_size, int64_t accuracy_level,
+    const EpHostTensor* inputs, int constant_mask, void* y, size_t y_bytes, int64_t* y_dims, size_t* y_rank,
+    int repeat, char* trace_buf, size_t trace_len, char* err, size_t err_len) {
+  FillApis();
+  Trace trace{trace_buf, trace_len};
+  if (trace_buf && trace_len) trace_buf[0] = 0;
+  std::string error;
+  Plugin* plugin = LoadPlugin(plugin_path, &error);
+  if (plugin == nullptr) return HostFail(EP_HOST_LOAD_FAILED, error, err, err_len);
+
+  OrtEpFactory* factory = nullptr;
+  size_t num_factories = 0;
+  if (OrtStatus* st = plugin->create("mi355x", &g_base, nullptr, &factory, 1, &num_factories))
+    return Fail(st, "CreateEpFactories", err, err_len);
+  struct FactoryGuard {
+    Plugin* p;
+    OrtEpFactory* f;
+    ~FactoryGuard() { p->release(f); }
+  } factory_guard{plugin, factory};
+
+  OrtHardwareDevice cpu{OrtHardwareDeviceType_CPU, 0x8086, 0};
+  OrtHardwareDevice amd{OrtHardwareDeviceType_GPU, 0x1002, 0x75A3};
+  const OrtHardwareDevice* hw[2] = {&cpu, &amd};
+  OrtEpDevice* ep_devices[2] = {nullptr, nullptr};
+  size_t num_ep_devices = 0;
+  if (OrtStatus* st = factory->GetSupportedDevices(factory, hw, 2, ep_devices, 2, &num_ep_devices))
+    return Fail(st, "GetSupportedDevices", err, err_len);
+  if (num_ep_devices == 0) return HostFail(EP_HOST_NO_DEVICE, "the factory offered no device", err, err_len);
+  std::unique_ptr<OrtEpDevice> ep_device(ep_devices[0]);
+  const OrtMemoryInfo* device_mem = nullptr;
+  for (const OrtMemoryInfo* m : ep_device->mem_infos)
+    if (m->dev.mem_type == OrtDeviceMemoryType_DEFAULT) device_mem = m;
+  if (device_mem == nullptr) return HostFail(EP_HOST_PROTOCOL, "no default device memory info", err, err_len);
+  OrtMemoryInfo cpu_mem{"Cpu", {OrtMemoryInfoDeviceType_CPU, OrtDeviceMemoryType_DEFAULT, 0, 0}, 0, OrtDeviceAllocator};
+
+  OrtEp* ep = nullptr;
+  const OrtHardwareDevice* chosen = ep_device->hw;
+  const OrtKeyValuePairs* no_meta = nullptr;
+  if (OrtStatus* st = factory->CreateEp(factory, &chosen, &no_meta, 1, nullptr, nullptr, &ep))
+    return Fail(st, "CreateEp", err, err_len);
+  struct EpGuard {
+    OrtEpFactory* f;
+    OrtEp* e;
+    ~EpGuard() { f->ReleaseEp(f, e); }
+  } ep_guard{factory, ep};
+  const std::string ep_name = ep->GetName(ep);
+
+  const OrtKernelRegistry* registry = nullptr;
+  if (OrtStatus* st = ep->GetKernelRegistry(ep, &registry)) return Fail(st, "GetKernelRegistry", err, err_len);
+  if (registry == nullptr) return HostFail(EP_HOST_PROTOCOL, "GetKernelRegistry returned NULL", err, err_len);
+  trace.add("kernels=%zu ", registry->entries.size());
+
+  // ---- the graph: one MatMulNBits node
+  OrtNode node;
+  node.op = "MatMulNBits";
+  node.domain = "com.microsoft";
+  node.name = "node0";
+  node.since_version = 1;
+  node.schema_attrs = {"K", "N", "bits", "block_size", "accuracy_level"};
+  node.attrs = {{"K", K}, {"N", N}, {"bits", bits}, {"block_size", block_size}, {"accuracy_level", accuracy_level}};
+  static const char* kInputNames[6] = {"A", "B", "scales", "zero_points", "g_idx", "bias"};
+  static const char* kInputTypes[6] = {"T1", "T2", "T1", "T3", "T4", "T1"};
+  size_t last = 0;
+  for (size_t i = 0; i < 6; ++i)
+    if (inputs[i].data != nullptr || i == 0) last = i;
+  for (size_t i = 0; i <= last; ++i) {
+    if (inputs[i].data == nullptr && i != 0) {
+      node.inputs.emplace_back(nullptr);
+      continue;
+    }
+    node.inputs.emplace_back(new OrtValueInfo{kInputNames[i]});
+    auto t = static_cast<ONNXTensorElementDataType>(inputs[i].dtype);
+    auto it = node.types.find(kInputTypes[i]);
+    if (it == node.types.end()) node.types[kInputTypes[i]] = t;
+  }
+  OrtGraph graph;
+  graph.nodes.push_back(&node);
+  OrtEpGraphSupportInfo support{registry, ep_name, {}};
+  if (OrtStatus* st = ep->GetCapability(ep, &graph, &support)) return Fail(st, "GetCapability", err, err_len);
+  trace.add("claimed=%zu ", support.claimed.size());
+  if (support.claimed.empty()) return HostFail(EP_HOST_NOT_CLAIMED, "node not claimed", err, err_len);
+
+  // ---- session resources
+  OrtAllocator* allocator = nullptr;
+  if (OrtStatus* st = ep->CreateAllocator(ep, device_mem, &allocator)) return Fail(st, "CreateAllocator", err, err_len);
+  struct AllocGuard {
+    OrtEpFactory* f;
+    OrtAllocator* a;
+    ~AllocGuard() { f->ReleaseAllocator(f, a); }
+  } alloc_guard{factory, allocator};
+  OrtDataTransferImpl* transfer = nullptr;
+  if (OrtStatus* st = factory->CreateDataTransfer(factory, &transfer)) return Fail(st, "CreateDataTransfer", err, err_len);
+  struct TransferGuard {
+    OrtDataTransferImpl* t;
+    ~TransferGuard() { t->Release(t); }
+  } transfer_guard{transfer};
+  if (!transfer->CanCopy(transfer, &cpu_mem.dev, &device_mem->dev) ||
+      !transfer->CanCopy(transfer, &device_mem->dev, &cpu_mem.dev))
+    return HostFail(EP_HOST_PROTOCOL, "data transfer refuses host<->device copies", err, err_len);
+  OrtSyncStreamImpl* stream_impl = nullptr;
+  if (OrtStatus* st = ep->CreateSyncStreamForDevice(ep, &device_mem->dev, &stream_impl))
+    return Fail(st, "CreateSyncStreamForDevice", err, err_len);
+  struct StreamGuard {
+    OrtSyncStreamImpl* s;
+    ~StreamGuard() { s->Release(s); }
+  } stream_guard{stream_impl};
+  OrtSyncStream stream{stream_impl};
+
+  // ---- values. Host copies wrap the caller's memory; constants go to the device through the data transfer.
+  std::unique_ptr<OrtValue> host_values[6], device_values[6];
+  for (size_t i = 0; i < 6; ++i) {
+    if (inputs[i].data == nullptr) continue;
+    auto v = std::make_unique<OrtValue>();
+    v->dims.assign(inputs[i].dims, inputs[i].dims + inputs[i].rank);
+    v->type = static_cast<ONNXTensorElementDataType>(inputs[i].dtype);
+    v->bytes = ByteSize(v->dims, v->type);
+    v->data = const_cast<void*>(inputs[i].data);
+    v->mem = &cpu_mem;
+    host_values[i] = std::move(v);
+  }
+  auto to_device = [&](size_t i, bool with_stream) -> OrtStatus* {
+    auto d = std::make_unique<OrtValue>();
+    d->dims = host_values[i]->dims;
+    d->type = host_values[i]->type;
+    d->bytes = host_values[i]->bytes;
+    d->mem = device_mem;
+    d->owner = allocator;
+    d->data = d->bytes ? allocator->Alloc(allocator, d->bytes) : nullptr;
+    if (d->bytes && d->data == nullptr) return MakeStatus(ORT_FAIL, "device allocation failed");
+    const OrtValue* src = host_values[i].get();
+    OrtValue* dst = d.get();
+    OrtSyncStream* s = with_stream ? &stream : nullptr;
+    OrtStatus* st = transfer->CopyTensors(transfer, &src, &dst, &s, 1);
+    device_values[i] = std::move(d);
+    return st;
+  };
+  for (size_t i = 1; i < 6; ++i) {
+    if (!host_values[i]) continue;
+    // initializers are copied without a stream at session initialisation, run inputs on the run's stream
+    if (OrtStatus* st = to_device(i, !((constant_mask >> i) & 1))) return Fail(st, "CopyTensors", err, err_len);
+  }
+
+  // ---- kernel creation + PrePack
+  const auto* entry = LookUp(*registry, ep_name, node);
+  if (entry == nullptr) return HostFail(EP_HOST_PROTOCOL, "claimed node without a kernel", err, err_len);
+  OrtKernelInfo info{&node, {}};
+  for (size_t i = 1; i < 6; ++i)
+    if (device_values[i] && ((constant_mask >> i) & 1)) info.constants[i] = device_values[i].get();
+  OrtKernelImpl* kernel = nullptr;
+  if (OrtStatus* st = entry->fn(entry->state, &info, &kernel)) return Fail(st, "kernel creation", err, err_len);
+  if (kernel == nullptr) return HostFail(EP_HOST_PROTOCOL, "kernel creation returned NULL", err, err_len);
+  struct KernelGuard {
+    OrtKernelImpl* k;
+    ~KernelGuard() { k->Release(k); }
+  } kernel_guard{kernel};
+  if (kernel->flags != 0) return HostFail(EP_HOST_PROTOCOL, "OrtKernelImpl::flags must start as 0", err, err_len);
+  trace.add("prepacked=");
+  bool packed[6] = {false, false, false, false, false, false};
+  if (kernel->PrePackWeight != nullptr) {
+    for (size_t i = 1; i < 6; ++i) {
+      if (!info.constants.count(i)) continue;
+      bool is_packed = false;
+      if (OrtStatus* st = kernel->PrePackWeight(kernel, device_values[i].get(), static_cast<int>(i), allocator,
+                                                nullptr, &is_packed))
+        return Fail(st, "PrePackWeight", err, err_len);
+      packed[i] = is_packed;
+      if (is_packed) trace.add("%zu,", i);
+    }
+    // Like ONNX Runtime, drop the initializers the kernel took over - after all PrePack calls of the node.
+    for (size_t i = 1; i < 6; ++i)
+      if (packed[i]) device_values[i].reset();
+  }
+  trace.add(" ");
+
+  // ---- Memcpy kernels around the node
+  auto memcpy_kernel = [&](const char* op, ONNXTensorElementDataType t, OrtKernelImpl** out) -> OrtStatus* {
+    OrtNode n;
+    n.op = op;
+    n.domain = "";
+    n.since_version = 1;
+    n.inputs.emplace_back(new OrtValueInfo{"X"});
+    n.types["T"] = t;
+    const auto* e = LookUp(*registry, ep_name, n);
+    if (e == nullptr) return MakeStatus(ORT_FAIL, (std::string("no kernel registered for ") + op).c_str());
+    OrtKernelInfo ki{&n, {}};
+    return e->fn(e->state, &ki, out);
+  };
+
+  int rc = 0;
+  for (int r = 0; r < (repeat < 1 ? 1 : repeat) && rc == 0; ++r) {
+    // A: host -> device through MemcpyFromHost
+    OrtKernelImpl* from_host = nullptr;
+    if (OrtStatus* st = memcpy_kernel("MemcpyFromHost", host_values[0]->type, &from_host))
+      return Fail(st, "MemcpyFromHost creation", err, err_len);
+    KernelGuard from_guard{from_host};
+    OrtKernelContext copy_in{{host_values[0].get()}, {}, {false}, allocator, &cpu_mem, &stream};
+    copy_in.outputs.resize(1);
+    if (OrtStatus* st = from_host->Compute(from_host, &copy_in)) return Fail(st, "MemcpyFromHost", err, err_len);
+
+    OrtKernelContext ctx{{}, {}, {false}, allocator, &cpu_mem, &stream};
+    ctx.outputs.resize(1);
+    ctx.inputs.assign(node.inputs.size(), nullptr);
+    ctx.inputs[0] = copy_in.outputs[0].get();
+    for (size_t i = 1; i < node.inputs.size(); ++i)
+      if (!packed[i] && device_values[i]) ctx.inputs[i] = device_values[i].get();
+    if (OrtStatus* st = kernel->Compute(kernel, &ctx)) return Fail(st, "Compute", err, err_len);
+    if (!ctx.outputs[0]) return HostFail(EP_HOST_PROTOCOL, "Compute produced no output", err, err_len);
+
+    OrtKernelImpl* to_host = nullptr;
+    if (OrtStatus* st = memcpy_kernel("MemcpyToHost", ctx.outputs[0]->type, &to_host))
+      return Fail(st, "MemcpyToHost creation", err, err_len);
+    KernelGuard to_guard{to_host};
+    OrtKernelContext copy_out{{ctx.outputs[0].get()}, {}, {true}, allocator, &cpu_mem, &stream};
+    copy_out.outputs.resize(1);
+    if (OrtStatus* st = to_host->Compute(to_host, &copy_out)) return Fail(st, "MemcpyToHost", err, err_len);
+    if (OrtStatus* st = stream_impl->Flush(stream_impl)) return Fail(st, "stream Flush", err, err_len);
+    const OrtValue& out = *copy_out.outputs[0];
+    if (out.bytes > y_bytes) return HostFail(EP_HOST_PROTOCOL, "output larger than the caller's buffer", err, err_len);
+    if (out.bytes) std::memcpy(y, out.data, out.bytes);
+    *y_rank = out.dims.size() < 8 ? out.dims.size() : 8;
+    for (size_t i = 0; i < *y_rank; ++i) y_dims[i] = out.dims[i];
+  }
+  if (OrtStatus* st = ep->Sync(ep)) return Fail(st, "OrtEp::Sync", err, err_len);
+  bool concurrent = false;
+  if (OrtStatus* st = ep->IsConcurrentRunSupported(ep, &concurrent)) return Fail(st, "IsConcurrentRunSupported", err, err_len);
+  trace.add("concurrent=%d", static_cast<int>(concurrent));
+  return rc;
+}
+
+}  // extern "C"

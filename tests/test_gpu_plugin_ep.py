@@ -1,0 +1,92 @@
+"""MatMulNBits through the plugin execution provider: the ONNX Runtime host test double drives the plugin library
+through the plugin-EP C ABI (factory, capability, allocator, data transfer, PrePack, Memcpy kernels, Compute) and the
+output is compared with the oracle and the reference's own vectors."""
+import numpy as np
+import pytest
+
+from ep_host import host
+from golden_cases import load_js_cases
+from gpu_util import check_against_oracle
+from onnxruntime_amd.synthetic import make_case
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(not host.available(), reason="plugin EP or host shim not built")]
+
+JS = load_js_cases()
+
+
+def _run(c, A=None, **kw):
+    return host.run_matmul_nbits(c.N, c.K, c.bits, c.block_size, c.A if A is None else A, c.B, c.scales,
+                                 c.zero_points, None, c.bias, **kw)
+
+
+@pytest.mark.parametrize("case", JS[::3], ids=[f"{i}" for i in range(0, len(JS), 3)])
+def test_reference_vectors_through_plugin(case):
+    c = case
+    y, trace = host.run_matmul_nbits(c["N"], c["K"], c["bits"], c["block_size"], c["A"], c["B"], c["scales"],
+                                     c["zero_points"])
+    assert "claimed=1" in trace
+    assert np.array_equal(y, c["Y"]), c["name"]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits,bs,zp,bias", [(4, 32, True, True), (4, 128, False, False), (8, 64, True, False),
+                                             (8, 16, False, True)])
+@pytest.mark.parametrize("M", [1, 7, 200])
+def test_prepacked_route(oracle, dtype, bits, bs, zp, bias, M):
+    c = make_case(M, 320, 512, bits, bs, dtype, has_zp=zp, has_bias=bias, seed=M + bits + bs)
+    y, trace = _run(c)
+    want = "prepacked=1,2,3," if zp else "prepacked=1,2,"
+    assert want in trace, trace          # B, scales (and zero points) were taken over by PrePack
+    check_against_oracle(oracle, c, y)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_unpacked_route_matches_prepacked(oracle, dtype):
+    """Scales fed per run (not constant): no PrePack, Compute packs into stream-ordered scratch. Same bits out."""
+    c = make_case(5, 200, 384, 4, 32, dtype, has_zp=True, has_bias=True, seed=3)
+    y_packed, _ = _run(c)
+    y_unpacked, trace = _run(c, constant=("B",), repeat=3)
+    assert "prepacked= " in trace, trace
+    assert np.array_equal(y_packed.view(np.uint8), y_unpacked.view(np.uint8))
+    check_against_oracle(oracle, c, y_unpacked)
+
+
+def test_batched_activations_and_empty_output(oracle):
+    c = make_case(6, 96, 128, 4, 32, np.float16, has_zp=False, seed=11)
+    A3 = c.A.reshape(2, 3, c.K)
+    y, _ = _run(c, A=A3)
+    assert y.shape == (2, 3, c.N)
+    check_against_oracle(oracle, c, y.reshape(6, c.N))
+    y0, _ = _run(c, A=np.zeros((0, c.K), np.float16))
+    assert y0.shape == (0, c.N)
+
+
+def test_nodes_left_to_the_cpu_provider():
+    c = make_case(2, 64, 128, 4, 32, np.float32, has_zp=True, seed=5)
+    # g_idx present: not claimed
+    with pytest.raises(host.EpHostError) as e:
+        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A, c.B, c.scales, c.zero_points, np.zeros(c.K, np.int32), None)
+    assert e.value.code == host.NOT_CLAIMED
+    # zero points in the activation type: no kernel registered for T3 = float
+    with pytest.raises(host.EpHostError) as e:
+        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A, c.B, c.scales, c.scales.copy(), None, None)
+    assert e.value.code == host.NOT_CLAIMED
+    # 2-bit weights: the schema allows them, the device library has no kernel
+    with pytest.raises(host.EpHostError) as e:
+        host.run_matmul_nbits(c.N, c.K, 2, 32, c.A, c.B[:, :, :8], c.scales, None, None, None)
+    assert e.value.code == host.NOT_CLAIMED
+
+
+def test_shape_errors_carry_the_reference_messages():
+    c = make_case(2, 64, 128, 4, 32, np.float32, has_zp=True, seed=6)
+    INVALID_ARGUMENT = 2
+    with pytest.raises(host.EpHostError) as e:   # constant scales of the wrong size: caught in PrePack
+        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A, c.B, c.scales.reshape(-1)[:-1], c.zero_points)
+    assert e.value.code == INVALID_ARGUMENT and "scales" in e.value.message
+    with pytest.raises(host.EpHostError) as e:   # run-time scales of the wrong size: caught in Compute
+        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A, c.B, c.scales.reshape(-1)[:-1], c.zero_points, constant=("B",))
+    assert e.value.code == INVALID_ARGUMENT and "scales" in e.value.message
+    with pytest.raises(host.EpHostError) as e:   # A whose inner dimension is not K
+        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A[:, :-1], c.B, c.scales, c.zero_points)
+    assert e.value.code == INVALID_ARGUMENT and "dimension mismatch" in e.value.message
