@@ -91,15 +91,17 @@ MNB_API size_t MnbPackQuantBDataSize(size_t N, size_t K, int bits, int block_siz
 MNB_API int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype, const void* b_dev,
                               const void* scales_dev, const void* zero_points_dev, void* packed_dev, void* stream);
 
-/* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call scratch MnbGemm wants for
- * this problem. Currently always 0: no kernel needs scratch. */
+/* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call device scratch MnbGemm needs for
+ * this problem. Non-zero only for fp16 activations with M > 16 whose shape selects the weight-streaming kernel (a
+ * copy of A in matrix-core operand order, about M*K*2 bytes); 0 otherwise. */
 MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                     int a_dtype);
 
 /* Replaces MlasQNBitGemmBatch at SQNBIT_CompFp32 (mlas_qnbit.h:111-125) for one B matrix:
  *   C[M][N] (ldc) = A[M][K] (lda) x dequant(packed)^T (+ bias[N]).
  * a_dev, bias_dev (optional) and c_dev have element type a_dtype; lda and ldc count elements. M <= 16 runs the
- * dequantising GEMV, larger M the LDS-staged MFMA GEMM (fp16) or the fp32 tile kernel. M == 0 or N == 0 is a
+ * dequantising GEMV; larger M the weight-streaming matrix-core kernel or, once 256 x 256 tiles fill the chip, the
+ * tiled MFMA GEMM (fp16), or the fp32 tile kernel. M == 0 or N == 0 is a
  * no-op. workspace_dev / workspace_bytes: per-call scratch of MnbGemmWorkspaceSize bytes (may be NULL / 0 when
  * that size is 0); it must not be shared by calls that may overlap. */
 MNB_API int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,

@@ -252,8 +252,17 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
     if (dtype != k.packed_dtype) {
       return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A and scales must have the same element type");
     }
-    return StatusFromMnb(a, MnbGemm(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr,
-                                    Nz, nullptr, 0, stream));
+    // per-call scratch comes from the stream-ordered pool, so concurrent Run() calls never share it
+    const size_t gemm_ws = MnbGemmWorkspaceSize(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype);
+    void* gemm_scratch = nullptr;
+    hipStream_t gs = static_cast<hipStream_t>(stream);
+    if (gemm_ws > 0) MI_RETURN_IF_HIP(a, hipMallocAsync(&gemm_scratch, gemm_ws, gs));
+    const int gemm_rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr, Nz,
+                                gemm_scratch, gemm_ws, stream);
+    const hipError_t gemm_free = gemm_scratch != nullptr ? hipFreeAsync(gemm_scratch, gs) : hipSuccess;
+    MI_RETURN_IF_ERROR(StatusFromMnb(a, gemm_rc));
+    MI_RETURN_IF_HIP(a, gemm_free);
+    return nullptr;
   }
 
   // B was not packed at session initialisation (prepacking disabled, or B / scales / zero points are not constant

@@ -168,13 +168,32 @@ int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype,
 }  // extern "C"
 
 // ------------------------------------------------------------------------------------------------ kernel choice
+// fp16, M > 16: the weight-streaming kernel (mnb_mid.hip) takes any shape; the 256 x 256 tile GEMM wins once its tiles
+// fill the chip.  The estimate compares 2MNK at the streaming kernel's measured rate with whole rounds of 256 tiles
+// at the tile kernel's measured time per 64-deep k-step.
+static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
+  if (M <= 128 || L.K % 128 != 0) return false;
+  static const int64_t mid_max_m = [] {
+    const char* e = getenv("MNB_MID_MAX_M");  // tuning override: M up to this value always streams
+    return e ? (int64_t)atoll(e) : (int64_t)-1;
+  }();
+  if (mid_max_m >= 0) return M > mid_max_m;
+  const double t_mid = 2.0 * (double)M * (double)L.N * (double)L.K / 550e12;
+  const int64_t tiles = ((M + 255) / 256) * ((L.N + 255) / 256);
+  const double step = L.bits == 4 ? 1.45e-6 : 2.95e-6;
+  const double t_256 = (double)((tiles + 255) / 256) * (double)(L.K / 64) * step;
+  return t_256 < t_mid;
+}
+
 MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
   if (mnb_skinny_applicable(a)) return kMnbKernelSkinny;
   if (mnb_gemv_applicable(a)) return kMnbKernelGemv;
   if (a.L.dtype == kMnbDtypeFloat16) {
-    // 16-byte activation loads: base and row pitch aligned, no partial 8-element chunk at the end of a row
-    const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (a.L.K % 8 == 0);
-    if (aligned) return (a.M > 128 && a.L.K % 128 == 0) ? kMnbKernelGemm256 : kMnbKernelGemmMfma;
+    // the tile GEMM loads activations 16 bytes at a time: base and row pitch aligned
+    const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
+    if (aligned && mnb_prefer_gemm256(a.L, a.M)) return kMnbKernelGemm256;
+    // the workspace is sized for the streaming kernel only when the shape alone selects it
+    if (!mnb_prefer_gemm256(a.L, a.M) || a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;
   }
   return kMnbKernelGemmGeneric;
 }
@@ -183,7 +202,7 @@ const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout&) {
   switch (k) {
     case kMnbKernelSkinny: return "mnb_skinny_kernel";
     case kMnbKernelGemv: return "mnb_gemv_kernel";
-    case kMnbKernelGemmMfma: return "mnb_gemm_mfma_kernel";
+    case kMnbKernelMid: return "mnb_mid_kernel";
     case kMnbKernelGemm256: return "mnb_gemm256_kernel";
     case kMnbKernelGemmGeneric: return "mnb_gemm_generic_kernel";
     default: return "none";
@@ -195,7 +214,12 @@ extern "C" {
 size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                             int a_dtype) {
   if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0 || M == 0) return 0;
-  return 0;  // no kernel needs per-call scratch at present
+  // only the mid-M fp16 kernel needs scratch: a copy of A in matrix-core operand order
+  if (a_dtype == kMnbDtypeFloat16 && M > 16) {
+    const MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+    if (!mnb_prefer_gemm256(L, (int64_t)M)) return mnb_mid_workspace_bytes(L, (int64_t)M);
+  }
+  return 0;
 }
 
 int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
@@ -224,7 +248,14 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
   switch (mnb_select_kernel(a)) {
     case kMnbKernelSkinny: e = mnb_launch_skinny(a, s); break;
     case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
-    case kMnbKernelGemmMfma: e = mnb_launch_gemm_mfma(a, s); break;
+    case kMnbKernelMid: {
+      const size_t need = mnb_mid_workspace_bytes(a.L, a.M);
+      if (a.workspace_bytes < need)
+        return fail(MNB_INVALID_ARGUMENT, "MnbGemm: workspace of %zu bytes needed (MnbGemmWorkspaceSize), %zu given", need,
+                    a.workspace_bytes);
+      e = mnb_launch_mid(a, s);
+      break;
+    }
     case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }

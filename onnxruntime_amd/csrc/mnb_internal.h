@@ -21,8 +21,8 @@ enum MnbKernelKind {
   kMnbKernelNone = 0,
   kMnbKernelSkinny,     // fp16, M <= 16: dequantising skinny GEMM on the matrix cores
   kMnbKernelGemv,       // fp32, M <= 16: dequantising GEMV (VALU dot products, activations in SGPRs)
-  kMnbKernelGemmMfma,   // fp16, LDS-staged MFMA GEMM, 128 x 128 tiles (17 <= M <= 128)
-  kMnbKernelGemm256,    // fp16, LDS-staged MFMA GEMM, 256 x 256 tiles (M > 128)
+  kMnbKernelMid,        // fp16, M > 16: weights from registers to the matrix cores, K split over waves (any shape)
+  kMnbKernelGemm256,    // fp16, MFMA GEMM with 256 x 256 tiles: large M, enough tiles to fill the chip
   kMnbKernelGemmGeneric // any shape / fp32 large M: simple tile kernel
 };
 
@@ -37,8 +37,10 @@ hipError_t mnb_launch_dequant_packed(void* dst, const void* packed, const MnbLay
 
 bool mnb_skinny_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s);
+bool mnb_mid_applicable(const MnbGemmArgs& a);
+hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s);
+size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M);  // staged copy of A
 bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
-hipError_t mnb_launch_gemm_mfma(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);

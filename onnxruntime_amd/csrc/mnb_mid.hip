@@ -1,0 +1,302 @@
+// fp16 kernel for 16 < M <= a few hundred rows: the regime between decode and prefill, where the reference runs its
+// strip-wise dequantise + SGEMM loop (SQ4BitGemm_CompFp32, onnxruntime/core/mlas/lib/qnbitgemm.cpp:563-732) and the
+// work is still dominated by streaming the weights once.
+//
+// Same structure as the decode kernel (mnb_skinny.hip): a workgroup owns 16*T output columns and a block of 16*MT rows,
+// K is split over its wavefronts (reduced through LDS at the end, fixed order), and every lane feeds its own 16-byte
+// weight vector to v_mfma_f32_16x16x32_f16 as the B operand -- no LDS on the weight path.  The difference is that each
+// dequantised operand is used by MT row tiles, so the weights are dequantised exactly ((q - zp) * scale in fp16, the
+// reference's fp16 dequantisation bit for bit) and the matrix cores accumulate across blocks; the VALU cost of the
+// dequantisation is amortised over MT * 4 matrix instructions per word.
+//
+// The A operand of lane (j, kq) is 16 bytes of row j at a 64-byte stride between lanes -- read from the row-major
+// activations, one load instruction would touch 64 cache lines.  A small staging kernel therefore first rewrites A
+// into operand order in the caller's workspace, [chunk][word i][row tile][kq][j] in 16-byte units (zero-filled beyond
+// M and K, any alignment of the source), so that every operand load of a wavefront is 1 KiB contiguous.  The staged
+// copy is M x K halves (at most a few MB) and is re-read from L2 by every workgroup.
+#include "mnb_mfma16_common.cuh"
+
+namespace {
+
+struct MidParams {
+  SkinnyParams s;
+  const uint4* As;  // staged activations
+  int row_tiles;    // 16-row tiles in the staged copy (multiple of the kernel's MT)
+};
+
+// A (row-major, lda) -> operand order.  One thread per 16-byte unit.
+template <int BITS>
+__global__ void __launch_bounds__(256) mnb_mid_stage_a_kernel(const _Float16* __restrict__ A, int64_t lda, int M, int K,
+                                                              int chunks, int row_tiles, int vec_ok,
+                                                              uint4* __restrict__ As) {
+  constexpr int GK = 128 / BITS, NI = GK / 8, CK = 4 * GK;
+  const int64_t u = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)chunks * NI * row_tiles * 64;
+  if (u >= total) return;
+  const int j = (int)(u & 15), kq = (int)((u >> 4) & 3);
+  const int64_t v = u >> 6;
+  const int rt = (int)(v % row_tiles);
+  const int i = (int)((v / row_tiles) % NI);
+  const int c = (int)(v / ((int64_t)row_tiles * NI));
+  const int row = rt * 16 + j;
+  const int k0 = c * CK + kq * GK + 8 * i;
+  uint4 out = make_uint4(0u, 0u, 0u, 0u);
+  if (row < M && k0 < K) {
+    const _Float16* src = A + (int64_t)row * lda + k0;
+    if (vec_ok && k0 + 8 <= K) {
+      out = *reinterpret_cast<const uint4*>(src);
+    } else {
+      __align__(16) _Float16 tmp[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tmp[e] = (k0 + e < K) ? src[e] : (_Float16)0.0f;
+      out = *reinterpret_cast<const uint4*>(tmp);
+    }
+  }
+  As[u] = out;
+}
+
+// exact (q - zp) * scale for the 8 weights of one 4-bit word / the 8 weights of two 8-bit words
+template <int BITS>
+__device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const UnpackConsts& uc, h2_t z_lo, h2_t z_hi,
+                                             h2_t s2) {
+  uint4 r;
+  if constexpr (BITS == 4) {
+    const uint32_t w8 = w0 >> 8;
+    const h2_t p0 = mnb_as_h2((w0 & uc.mask_lo) | uc.magic_lo);  // 1024 + q
+    const h2_t p1 = mnb_as_h2((w0 & uc.mask_hi) | uc.magic_hi);  //   64 + q
+    const h2_t p2 = mnb_as_h2((w8 & uc.mask_lo) | uc.magic_lo);
+    const h2_t p3 = mnb_as_h2((w8 & uc.mask_hi) | uc.magic_hi);
+    r.x = mnb_as_u32((p0 + z_lo) * s2);
+    r.y = mnb_as_u32((p1 + z_hi) * s2);
+    r.z = mnb_as_u32((p2 + z_lo) * s2);
+    r.w = mnb_as_u32((p3 + z_hi) * s2);
+  } else {
+    const h2_t p0 = mnb_as_h2(__builtin_amdgcn_perm(kMagic, w0, 0x07010700u));
+    const h2_t p1 = mnb_as_h2(__builtin_amdgcn_perm(kMagic, w0, 0x07030702u));
+    const h2_t p2 = mnb_as_h2(__builtin_amdgcn_perm(kMagic, w1, 0x07010700u));
+    const h2_t p3 = mnb_as_h2(__builtin_amdgcn_perm(kMagic, w1, 0x07030702u));
+    r.x = mnb_as_u32((p0 + z_lo) * s2);
+    r.y = mnb_as_u32((p1 + z_lo) * s2);
+    r.z = mnb_as_u32((p2 + z_lo) * s2);
+    r.w = mnb_as_u32((p3 + z_lo) * s2);
+  }
+  return __builtin_bit_cast(h8_t, r);
+}
+
+template <int BITS, bool HAS_ZP, int T, int MT>
+__device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t (*af)[(128 / BITS) / 8],
+                                                  const UnpackConsts& uc, f4_t (*y)[T]) {
+  constexpr int NI = (128 / BITS) / 8;
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
+    _Float16 s0, s1, nz0, nz1;
+    decode_meta<BITS, HAS_ZP>(R.m0[t], s0, nz0);
+    if constexpr (BITS == 4) {
+      decode_meta<BITS, HAS_ZP>(R.m1[t], s1, nz1);
+    } else {
+      s1 = s0;
+      nz1 = nz0;
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const bool second = (BITS == 4) && i >= 2;  // words 2, 3 of a 4-bit vector may belong to the next block
+      const _Float16 nz = second ? nz1 : nz0;
+      const h2_t s2 = mnb_h2(second ? s1 : s0);
+      const h2_t z_lo = mnb_h2(nz);                        // -(1024 + zp)
+      const h2_t z_hi = mnb_h2(nz + (_Float16)960.0f);     // -(64 + zp), exact
+      const h8_t b = BITS == 4 ? dequant_word<4>(wd[i], 0u, uc, z_lo, z_hi, s2)
+                               : dequant_word<8>(wd[(2 * i) & 3], wd[(2 * i + 1) & 3], uc, z_lo, z_hi, s2);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) y[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][i], b, y[mt][t], 0, 0, 0);
+    }
+  }
+}
+
+template <int BITS, bool HAS_ZP, int T, int MT, int NW>
+__global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
+  const SkinnyParams& p = mp.s;
+  constexpr int GK = 128 / BITS;
+  constexpr int NI = GK / 8;
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* red = reinterpret_cast<float*>(smem);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, kq = lane >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
+  const int64_t col0 = n0 + j;
+  const int m0 = blockIdx.y * (16 * MT);
+
+  // staged A: unit index = (((c * NI + i) * row_tiles + rt) * 4 + kq) * 16 + j
+  const uint4* a_lane = mp.As + ((int64_t)blockIdx.y * MT * 4 + kq) * 16 + j;
+  const int64_t a_step = (int64_t)mp.row_tiles * 64;  // units between consecutive (c, i)
+  f4_t y[MT][T];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < T; ++t) y[mt][t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const UnpackConsts uc = make_unpack_consts(p.uc);
+
+  h8_t af[MT][NI];
+  auto load_a = [&](int c) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+        af[mt][i] = __builtin_bit_cast(h8_t, a_lane[((int64_t)c * NI + i) * a_step + mt * 64]);
+  };
+
+  // weights two chunks ahead (double buffer), activations one chunk ahead (single buffer, refilled right after the
+  // matrix instructions that read it have been issued); the second wavefront of the SIMD covers what is left
+  ChunkRegs<BITS, T> R0, R1;
+  int c = wave;
+  if (c < p.chunks) {
+    load_chunk<BITS, HAS_ZP, 1, T>(p, c, kq, col0, R0);
+    load_a(c);
+  }
+  if (c + NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + NW, kq, col0, R1);
+  for (; c < p.chunks; c += 2 * NW) {
+    mid_compute_chunk<BITS, HAS_ZP, T, MT>(R0, af, uc, y);
+    if (c + NW < p.chunks) load_a(c + NW);
+    if (c + 2 * NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + 2 * NW, kq, col0, R0);
+    if (c + NW < p.chunks) {
+      mid_compute_chunk<BITS, HAS_ZP, T, MT>(R1, af, uc, y);
+      if (c + 2 * NW < p.chunks) load_a(c + 2 * NW);
+      if (c + 3 * NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + 3 * NW, kq, col0, R1);
+    }
+  }
+
+  // reduce over the wavefronts, one row tile at a time: lane (j, kq), register r of y[mt][t] holds
+  // row m0 + 16 mt + 4 kq + r, column n0 + 16 t + j
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (mt > 0) __syncthreads();
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[(wave * T * 4 + t * 4 + r) * 64 + lane] = y[mt][t][r];
+    __syncthreads();
+    for (int i = threadIdx.x; i < T * 4 * 64; i += NW * 64) {
+      const int l = i & 63, tr = i >> 6;
+      const int t = tr >> 2, r = tr & 3;
+      const int m = m0 + mt * 16 + 4 * (l >> 4) + r;
+      const int64_t n = n0 + t * 16 + (l & 15);
+      if (m >= p.M || n >= p.N) continue;
+      float sum = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * T * 4 + tr) * 64 + l];
+      if (p.bias) sum += (float)p.bias[n];
+      p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
+    }
+  }
+}
+
+struct MidPlan {
+  int t, mt, nw;
+};
+
+MidPlan mid_plan(const MnbLayout& L, int64_t M) {
+  MidPlan pl;
+  const int CK = 4 * L.group_k;
+  const int chunks = (int)((L.K + CK - 1) / CK);
+  const int64_t tiles = (L.N + 15) / 16;
+  pl.mt = M <= 32 ? 2 : 4;
+  // the widest column slab (best reuse of the activations) that still leaves the chip enough workgroups
+  const int64_t row_blocks = (M + 16 * pl.mt - 1) / (16 * pl.mt);
+  pl.t = (tiles / 4) * row_blocks >= 192 ? 4 : (tiles / 2) * row_blocks >= 96 ? 2 : 1;
+  pl.nw = chunks >= 16 ? 8 : 4;
+  if (const char* e = getenv("MNB_MID_PLAN")) {  // tuning override "<T>,<MT>,<NW>"
+    int t = 0, mt = 0, nw = 0;
+    if (sscanf(e, "%d,%d,%d", &t, &mt, &nw) == 3 && (t == 1 || t == 2 || t == 4) && (mt == 2 || mt == 4) &&
+        (nw == 4 || nw == 8)) {
+      pl.t = t;
+      pl.mt = mt;
+      pl.nw = nw;
+    }
+  }
+  return pl;
+}
+
+template <int BITS, bool HAS_ZP, int T, int MT>
+hipError_t launch_nw(const MidParams& mp, const MidPlan& pl, hipStream_t s) {
+  const SkinnyParams& p = mp.s;
+  dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)));
+  const size_t smem = (size_t)pl.nw * T * 4 * 64 * sizeof(float);
+  if (pl.nw == 8)
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8><<<grid, dim3(512), smem, s>>>(mp);
+  else
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4><<<grid, dim3(256), smem, s>>>(mp);
+  return hipGetLastError();
+}
+
+template <int BITS, bool HAS_ZP, int T>
+hipError_t launch_mt(const MidParams& p, const MidPlan& pl, hipStream_t s) {
+  return pl.mt == 2 ? launch_nw<BITS, HAS_ZP, T, 2>(p, pl, s) : launch_nw<BITS, HAS_ZP, T, 4>(p, pl, s);
+}
+
+template <int BITS, bool HAS_ZP>
+hipError_t launch_t(const MidParams& p, const MidPlan& pl, hipStream_t s) {
+  switch (pl.t) {
+    case 4: return launch_mt<BITS, HAS_ZP, 4>(p, pl, s);
+    case 2: return launch_mt<BITS, HAS_ZP, 2>(p, pl, s);
+    default: return launch_mt<BITS, HAS_ZP, 1>(p, pl, s);
+  }
+}
+
+int log2i(int v) {
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+
+int mid_row_tiles(int64_t M, int mt) { return (int)((M + 16 * mt - 1) / (16 * mt)) * mt; }
+
+}  // namespace
+
+bool mnb_mid_applicable(const MnbGemmArgs& a) { return a.L.dtype == kMnbDtypeFloat16 && a.M > 16; }
+
+// bytes of the staged copy of A
+size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
+  const MidPlan pl = mid_plan(L, M);
+  const int CK = 4 * L.group_k;
+  const int64_t chunks = (L.K + CK - 1) / CK;
+  return (size_t)chunks * (L.group_k / 8) * mid_row_tiles(M, pl.mt) * 64 * 16;
+}
+
+hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
+  const MnbLayout& L = a.L;
+  const MidPlan pl = mid_plan(L, a.M);
+  const int CK = 4 * L.group_k;
+  MidParams mp{};
+  SkinnyParams& p = mp.s;
+  p.A = reinterpret_cast<const _Float16*>(a.A);
+  p.W = reinterpret_cast<const uint4*>(a.packed);
+  p.meta = reinterpret_cast<const uint8_t*>(a.packed) + L.meta_off;
+  p.bias = reinterpret_cast<const _Float16*>(a.bias);
+  p.C = reinterpret_cast<_Float16*>(a.C);
+  p.lda = a.lda;
+  p.ldc = a.ldc;
+  p.Npad = L.Npad;
+  p.M = (int)a.M;
+  p.N = (int)L.N;
+  p.K = (int)L.K;
+  p.bs_shift = log2i(L.bs);
+  p.chunks = (int)((L.K + CK - 1) / CK);
+  p.uc[0] = 0x000F000Fu;
+  p.uc[1] = 0x00F000F0u;
+  p.uc[2] = 0x64006400u;
+  p.uc[3] = 0x54005400u;
+  mp.As = reinterpret_cast<const uint4*>(a.workspace);
+  mp.row_tiles = mid_row_tiles(a.M, pl.mt);
+  const int vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
+  const int64_t units = (int64_t)p.chunks * (L.group_k / 8) * mp.row_tiles * 64;
+  const dim3 sgrid((unsigned)((units + 255) / 256));
+  uint4* staged = reinterpret_cast<uint4*>(a.workspace);
+  if (L.bits == 4)
+    mnb_mid_stage_a_kernel<4><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
+  else
+    mnb_mid_stage_a_kernel<8><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  if (L.bits == 4) return L.has_zp ? launch_t<4, true>(mp, pl, s) : launch_t<4, false>(mp, pl, s);
+  return L.has_zp ? launch_t<8, true>(mp, pl, s) : launch_t<8, false>(mp, pl, s);
+}

@@ -26,139 +26,9 @@
 #include <cstdio>
 #include <cstdlib>
 
-#include "mnb_device.cuh"
-#include "mnb_internal.h"
+#include "mnb_mfma16_common.cuh"
 
 namespace {
-
-struct SkinnyParams {
-  const _Float16* A;
-  const uint4* W;
-  const uint8_t* meta;
-  const _Float16* bias;
-  _Float16* C;
-  int64_t lda, ldc, Npad;
-  int M, N, K;
-  int bs_shift;
-  int chunks;       // chunks that hold elements below K
-  int phase_chunks; // chunks staged in LDS at a time
-  int mtr;          // rows of A staged (power of two >= M, <= 16)
-  int a_vec_ok;     // A allows 16-byte loads
-  uint32_t uc[4];   // UnpackConsts
-};
-
-constexpr int kLdsPad = 8;  // halves of padding per staged row
-
-// The four constants of the nibble unpack.  They are passed as kernel arguments rather than written as literals:
-// VOP3 encodings of this ISA family take no literal, so with literals the compiler emits v_and_b32 + v_or_b32
-// (two instructions); with register operands it selects the single v_and_or_b32.
-struct UnpackConsts {
-  uint32_t mask_lo, mask_hi, magic_lo, magic_hi;  // 0x000F000F, 0x00F000F0, 0x64006400 (1024), 0x54005400 (64)
-};
-
-// One SGPR operand per VALU instruction: the masks stay scalar, the magics are moved to VGPRs once per kernel.
-// The move is opaque to the optimiser so that it cannot fold the value back into a literal.
-__device__ __forceinline__ UnpackConsts make_unpack_consts(const uint32_t* k) {
-  UnpackConsts u;
-  u.mask_lo = k[0];
-  u.mask_hi = k[1];
-  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic_lo) : "s"(k[2]));
-  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic_hi) : "s"(k[3]));
-  return u;
-}
-
-// raw magic halves of one 32-bit word: 4-bit -> 8 halves {1024+e0,1024+e1,64+e2,64+e3,1024+e4,1024+e5,64+e6,64+e7}
-__device__ __forceinline__ h8_t raw4(uint32_t w, const UnpackConsts& u) {
-  const uint32_t w8 = w >> 8;
-  uint4 r;
-  r.x = (w & u.mask_lo) | u.magic_lo;
-  r.y = (w & u.mask_hi) | u.magic_hi;
-  r.z = (w8 & u.mask_lo) | u.magic_lo;
-  r.w = (w8 & u.mask_hi) | u.magic_hi;
-  return __builtin_bit_cast(h8_t, r);
-}
-// 8-bit: two words -> 8 halves 1024+b
-__device__ __forceinline__ h8_t raw8(uint32_t w0, uint32_t w1) {
-  uint4 r;
-  r.x = __builtin_amdgcn_perm(kMagic, w0, 0x07010700u);
-  r.y = __builtin_amdgcn_perm(kMagic, w0, 0x07030702u);
-  r.z = __builtin_amdgcn_perm(kMagic, w1, 0x07010700u);
-  r.w = __builtin_amdgcn_perm(kMagic, w1, 0x07030702u);
-  return __builtin_bit_cast(h8_t, r);
-}
-
-// ---- registers of one chunk: weights, meta and (direct variant) the A operands ---------------------------------
-template <int BITS, int T>
-struct ChunkRegs {
-  uint4 w[T];
-  uint32_t m0[T];  // meta entry of the lane's (first) block: raw bits (32 with zero points, else 16)
-  uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
-};
-
-// T adjacent meta entries (2 or 4 bytes each) with one load; dst holds the raw bits of each entry
-template <bool HAS_ZP, int T>
-__device__ __forceinline__ void load_meta_vec(const uint8_t* __restrict__ meta, int64_t first, uint32_t* dst) {
-  if constexpr (HAS_ZP) {
-    const uint32_t* q = reinterpret_cast<const uint32_t*>(meta) + first;
-    if constexpr (T == 4) {
-      const uint4 v = *reinterpret_cast<const uint4*>(q);
-      dst[0] = v.x, dst[1] = v.y, dst[2] = v.z, dst[3] = v.w;
-    } else if constexpr (T == 2) {
-      const uint2 v = *reinterpret_cast<const uint2*>(q);
-      dst[0] = v.x, dst[1] = v.y;
-    } else {
-      dst[0] = *q;
-    }
-  } else {
-    const uint16_t* q = reinterpret_cast<const uint16_t*>(meta) + first;
-    if constexpr (T == 4) {
-      const uint2 v = *reinterpret_cast<const uint2*>(q);
-      dst[0] = v.x & 0xFFFFu, dst[1] = v.x >> 16, dst[2] = v.y & 0xFFFFu, dst[3] = v.y >> 16;
-    } else if constexpr (T == 2) {
-      const uint32_t v = *reinterpret_cast<const uint32_t*>(q);
-      dst[0] = v & 0xFFFFu, dst[1] = v >> 16;
-    } else {
-      dst[0] = *q;
-    }
-  }
-}
-
-// col0 = first column of the workgroup + j; the T tiles of a lane are columns col0 + 16 t.
-template <int BITS, bool HAS_ZP, int MODE, int T>
-__device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq, int64_t col0, ChunkRegs<BITS, T>& R) {
-  constexpr int GK = 128 / BITS;
-  constexpr int CK = 4 * GK;
-  // small loads first: memory returns in issue order, and the weights are waited for tile by tile
-  const int64_t mcol = mnb_meta_col(col0);  // entries of columns col0 + 16 t follow at mcol + t
-  if constexpr (MODE == 0) {
-    const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
-    load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
-  } else {
-    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
-    load_meta_vec<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0);
-    if constexpr (BITS == 4) load_meta_vec<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1);
-  }
-#pragma unroll
-  for (int t = 0; t < T; ++t) R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + col0 + t * 16];
-}
-
-template <int BITS, bool HAS_ZP>
-__device__ __forceinline__ void decode_meta(uint32_t raw, _Float16& s, _Float16& neg_1024_plus_zp) {
-  if constexpr (HAS_ZP) {
-    const h2_t m = mnb_as_h2(raw);
-    s = m.x;
-    neg_1024_plus_zp = m.y;
-  } else {
-    s = __builtin_bit_cast(_Float16, (uint16_t)raw);
-    neg_1024_plus_zp = (_Float16)(-(1024.0f + (float)(1 << (BITS - 1))));
-  }
-}
-
-// constant MFMA B operands (identical in every lane) that turn the A operands into the correction terms
-struct BConst {
-  h8_t off;  // -(offset of the raw half at each of the 8 positions of a word [+ default zero point])
-  h8_t one;  // -1
-};
 
 // One chunk: T column tiles x (4 k-groups) against the 16-row A operands af[].
 template <int BITS, bool HAS_ZP, int MODE, int T>
@@ -243,20 +113,6 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
       }
     }
   }
-}
-
-template <int BITS, bool HAS_ZP>
-__device__ __forceinline__ BConst make_bconst() {
-  // offsets the raw halves carry: 1024 (low nibbles, bytes) and 64 (high nibbles); without zero points the
-  // default zero point 2^(bits-1) is folded in.  All values are integers below 2048: exact in fp16.
-  const float zp = HAS_ZP ? 0.f : (float)(1 << (BITS - 1));
-  const _Float16 lo = (_Float16)(-(1024.0f + zp));
-  const _Float16 hi = (_Float16)(-((BITS == 4 ? 64.0f : 1024.0f) + zp));
-  const _Float16 m1 = (_Float16)(-1.0f);
-  BConst bc;
-  bc.off = h8_t{lo, lo, hi, hi, lo, lo, hi, hi};
-  bc.one = h8_t{m1, m1, m1, m1, m1, m1, m1, m1};
-  return bc;
 }
 
 // Reduce the per-wavefront tiles through LDS in wavefront order and write Y.
