@@ -138,6 +138,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 GEMM")
+    ap.add_argument("--no-quantize", action="store_true", help="skip the blockwise quantiser (producer of the format)")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -231,6 +232,33 @@ def main() -> int:
                          "traffic": MEASURED_TRAFFIC_BYTES["c4_prefill"]},
         }
         del p4
+        torch.cuda.empty_cache()
+
+    # ---- blockwise quantiser: fp16 [K, N] weights -> the operands of configs[1] --------------------------------
+    if not args.no_quantize:
+        from onnxruntime_amd.matmul_nbits import quantize_blockwise
+        Kq, Nq, copies = c2.K, c2.N, 4
+        gen = torch.Generator(device="cuda").manual_seed(0)
+        ws = [torch.randn(Kq, Nq, generator=gen, device="cuda", dtype=torch.float16) * 0.05 for _ in range(copies)]
+
+        def qstep():
+            for w in ws:  # 4 x 117 MB of distinct sources: beyond the Infinity Cache
+                quantize_blockwise(w, c2.bits, c2.block_size, symmetric=True)
+
+        msq = time_steps(torch, qstep, max(4, args.steps // 5), 2) / copies
+        kbq = Kq // c2.block_size
+        qbytes = Kq * Nq * 2 + Nq * kbq * (c2.block_size * c2.bits // 8) + Nq * kbq * 2
+        out["quantize"] = {
+            "workload": "MlasQuantizeBlockwise semantics: fp16 [4096, 14336] -> int4 block_size=128 symmetric",
+            "value": round(qbytes / (msq * 1e-3) / 1e9, 1),
+            "unit": "GB/s",
+            "ms_per_launch": round(msq, 4),
+            "kernel": "mnb_quantize_kernel",
+            "roofline": {"bound": "hbm", "achieved": round(qbytes / (msq * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(qbytes / (msq * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "traffic": None},
+        }
+        del ws
         torch.cuda.empty_cache()
 
     # ---- the other configurations (not part of the JSON contract) ---------------------------------------------

@@ -132,6 +132,15 @@ MNB_API int MnbDequantizeBlockwise(void* dst_dev, const void* b_dev, const void*
 MNB_API int MnbDequantizePacked(void* dst_dev, const void* packed_dev, size_t N, size_t K, int bits, int block_size,
                                 int has_zero_points, int a_dtype, void* stream);
 
+/* Replaces MlasQuantizeBlockwise<T, bits> with column-wise blocks (onnxruntime/core/mlas/inc/mlas_q4.h:315-328,
+ * definition onnxruntime/core/mlas/lib/q4_dq.cpp:468-574): quantises src_dev, a row-major [K][leading_dimension]
+ * matrix of a_dtype elements of which the first N columns are used, into the canonical operands b_dev
+ * u8[N][k_blocks][block_size*bits/8] and scales_dev T[N][k_blocks], plus zero_points_dev u8[N][ceil(k_blocks*bits/8)]
+ * for asymmetric quantisation; zero_points_dev == NULL selects symmetric quantisation (zero point 2^(bits-1)).
+ * Every byte of the outputs is written. Elements k >= K of the last block are stored as the zero point. */
+MNB_API int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_points_dev, const void* src_dev,
+                                 int block_size, int bits, size_t K, size_t N, size_t leading_dimension, int a_dtype,
+                                 void* stream);
 /* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
 MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);
 

@@ -3,7 +3,7 @@ from ._lib import MnbError, LIB_PATH  # noqa: F401
 
 
 def __getattr__(name):
-    if name in ("MatMulNBits", "check_inputs", "dequantize_blockwise"):
+    if name in ("MatMulNBits", "check_inputs", "dequantize_blockwise", "quantize_blockwise"):
         from . import matmul_nbits
         return getattr(matmul_nbits, name)
     raise AttributeError(name)

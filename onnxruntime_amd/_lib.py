@@ -47,6 +47,8 @@ SIGNATURES = {
     "MnbGemmUnpackedWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
     "MnbGemmUnpacked": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "MnbQuantizeBlockwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_size_t, c_size_t,
+                                     c_int, c_void_p]),
     "MnbDequantizeBlockwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_size_t,
                                        c_int, c_void_p]),
     "MnbDequantizePacked": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),

@@ -286,6 +286,19 @@ int MnbGemmUnpacked(size_t M, size_t N, size_t K, int bits, int block_size, int 
                  static_cast<char*>(workspace_dev) + pack, workspace_bytes - pack, stream);
 }
 
+int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_points_dev, const void* src_dev, int block_size,
+                         int bits, size_t K, size_t N, size_t leading_dimension, int a_dtype, void* stream) {
+  if (int rc = check_config("MnbQuantizeBlockwise", bits, block_size, a_dtype)) return rc;
+  if (N == 0 || K == 0) return MNB_OK;
+  if (!b_dev || !scales_dev || !src_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbQuantizeBlockwise: B, scales and src must not be NULL");
+  if (leading_dimension < N)
+    return fail(MNB_INVALID_ARGUMENT, "MnbQuantizeBlockwise: leading_dimension (%zu) < N (%zu)", leading_dimension, N);
+  hipError_t e = mnb_launch_quantize(b_dev, scales_dev, zero_points_dev, src_dev, (int64_t)K, (int64_t)N,
+                                     (int64_t)leading_dimension, bits, block_size, a_dtype, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbQuantizeBlockwise");
+}
+
 int MnbDequantizeBlockwise(void* dst_dev, const void* b_dev, const void* scales_dev, const void* zero_points_dev,
                            int block_size, int bits, size_t K, size_t N, int a_dtype, void* stream) {
   if (int rc = check_config("MnbDequantizeBlockwise", bits, block_size, a_dtype)) return rc;

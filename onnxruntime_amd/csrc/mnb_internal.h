@@ -33,6 +33,8 @@ hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales
                            hipStream_t s);
 hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,
                                         int64_t K, int bits, int bs, int dtype, hipStream_t s);
+hipError_t mnb_launch_quantize(void* B, void* scales, void* zp, const void* src, int64_t K, int64_t N, int64_t ld,
+                               int bits, int bs, int dtype, hipStream_t s);
 hipError_t mnb_launch_dequant_packed(void* dst, const void* packed, const MnbLayout& L, hipStream_t s);
 
 bool mnb_skinny_applicable(const MnbGemmArgs& a);

@@ -204,3 +204,22 @@ def dequantize_blockwise(b: torch.Tensor, scales: torch.Tensor, zero_points: Opt
                                           _ptr(None if zero_points is None else zero_points.contiguous()), block_size,
                                           bits, K, N, _DTYPES[scales.dtype], _stream_ptr(b.device)))
     return w
+
+
+def quantize_blockwise(w: torch.Tensor, bits: int, block_size: int, symmetric: bool):
+    """MlasQuantizeBlockwise on the device (column-wise blocks): w is the [K, N] weight matrix of a MatMul in fp16 or
+    fp32 (row stride >= N allowed). Returns the operator's inputs (B u8 [N, k_blocks, block_size*bits/8],
+    scales [N, k_blocks] in w's dtype, zero_points u8 [N, ceil(k_blocks*bits/8)] or None when symmetric)."""
+    lib = _lib.load()
+    if w.dim() != 2 or w.dtype not in (torch.float16, torch.float32):
+        raise MnbError(_lib.INVALID_ARGUMENT, "quantize_blockwise: w must be a 2-D fp16 or fp32 tensor")
+    if w.stride(1) != 1:
+        w = w.contiguous()
+    K, N = w.shape
+    kb = (K + block_size - 1) // block_size
+    b = torch.empty(N, kb, block_size * bits // 8, dtype=torch.uint8, device=w.device)
+    scales = torch.empty(N, kb, dtype=w.dtype, device=w.device)
+    zp = None if symmetric else torch.empty(N, (kb * bits + 7) // 8, dtype=torch.uint8, device=w.device)
+    _lib.check(lib.MnbQuantizeBlockwise(_ptr(b), _ptr(scales), _ptr(zp), _ptr(w), block_size, bits, K, N,
+                                        w.stride(0) if K > 1 else N, _DTYPES[w.dtype], _stream_ptr(w.device)))
+    return b, scales, zp

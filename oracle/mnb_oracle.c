@@ -283,19 +283,23 @@ void mnbo_matmul_f16(const uint16_t* A, const uint8_t* B, const uint16_t* scales
  *               zp = clamp(round(-min / scale)) (0 when scale is 0); q = clamp(round(v / scale + zp))
  *   symmetric : s = max if |max| > |min| else min; scale = -s / 2^(bits-1);
  *               zp = 2^(bits-1); q = clamp(round(v / scale + zp))  (computed with the reciprocal of scale)
- * src is row-major [K][N].  Rounding is roundf (half away from zero), as in the reference.
+ * src is row-major [K][N].  Rounding is roundf (half away from zero), as in the reference.  fp16 models: elements
+ * are widened to fp32, the scale is computed in fp32 and stored as fp16 (RNE); the zero point comes from the
+ * unrounded scale, the reciprocal from the stored one.  Positions k >= K of the last block, which the reference
+ * leaves unwritten, hold the zero point here (they dequantise to 0).
  * Parity: pinned only by round-trip and closed-form properties (tests/test_oracle_quantize.py); tie-breaking
  * on exact .5 values is "parity unpinned" because the compiled reference is not available in this build.
  */
-void mnbo_quantize_f32(uint8_t* B, float* scales, uint8_t* zp, const float* src, int64_t K, int64_t N, int bits,
-                       int64_t bs, int symmetric) {
+static void quantize_core(uint8_t* B, float* scales, uint8_t* zp, const float* src, int64_t K, int64_t N, int bits,
+                          int64_t bs, int symmetric, int scale_is_f16) {
   int64_t kbc = k_blocks_of(K, bs);
   int64_t blob = blob_of(bs, bits);
   int64_t zrow = zp_row_of(kbc, bits);
   const int maxq = (1 << bits) - 1;
   const int mid = 1 << (bits - 1);
   memset(B, 0, (size_t)(N * kbc * blob));
-  if (zp) memset(zp, 0, (size_t)(N * zrow));
+  /* unused slots of the last zero-point byte keep the reference's filler, the default zero point (:493) */
+  if (zp) memset(zp, bits == 8 ? 0 : bits == 4 ? 0x88 : 0xAA, (size_t)(N * zrow));
   for (int64_t n = 0; n < N; ++n)
     for (int64_t kb = 0; kb < kbc; ++kb) {
       int64_t k0 = kb * bs, k1 = k0 + bs < K ? k0 + bs : K;
@@ -313,7 +317,6 @@ void mnbo_quantize_f32(uint8_t* B, float* scales, uint8_t* zp, const float* src,
         if (zf < 0.f) zf = 0.f;
         if (zf > (float)maxq) zf = (float)maxq;
         z = (int)roundf(zf);
-        rscale = scale == 0.f ? 0.f : 1.f / scale;
       } else {
         float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
         for (int64_t k = k0; k < k1; ++k) {
@@ -323,15 +326,17 @@ void mnbo_quantize_f32(uint8_t* B, float* scales, uint8_t* zp, const float* src,
         }
         float smax = fabsf(mx) > fabsf(mn) ? mx : mn; /* the larger half maps to [-2^(bits-1), 0] */
         scale = -smax / (float)mid;
-        rscale = scale == 0.f ? 0.f : 1.f / scale;
         z = mid;
       }
+      /* the scale is stored in the model's type; the reciprocal is taken from the stored value (:552-553) */
+      if (scale_is_f16) scale = mnbo_f16_to_f32(mnbo_f32_to_f16(scale));
+      rscale = scale == 0.f ? 0.f : 1.f / scale;
       scales[n * kbc + kb] = scale;
       if (zp) {
         uint8_t* row = zp + n * zrow;
         if (bits == 8) row[kb] = (uint8_t)z;
-        else if (bits == 4) row[kb >> 1] |= (uint8_t)(z << ((kb & 1) * 4));
-        else row[kb >> 2] |= (uint8_t)(z << ((kb & 3) * 2));
+        else if (bits == 4) row[kb >> 1] = (uint8_t)((row[kb >> 1] & ~(0xF << ((kb & 1) * 4))) | (z << ((kb & 1) * 4)));
+        else row[kb >> 2] = (uint8_t)((row[kb >> 2] & ~(0x3 << ((kb & 3) * 2))) | (z << ((kb & 3) * 2)));
       }
       uint8_t* out = B + (n * kbc + kb) * blob;
       for (int64_t k = k0; k < k0 + bs; ++k) {
@@ -346,4 +351,21 @@ void mnbo_quantize_f32(uint8_t* B, float* scales, uint8_t* zp, const float* src,
         else out[r >> 2] |= (uint8_t)(q << ((r & 3) * 2));
       }
     }
+}
+
+void mnbo_quantize_f32(uint8_t* B, float* scales, uint8_t* zp, const float* src, int64_t K, int64_t N, int bits,
+                       int64_t bs, int symmetric) {
+  quantize_core(B, scales, zp, src, K, N, bits, bs, symmetric, 0);
+}
+
+void mnbo_quantize_f16(uint8_t* B, uint16_t* scales, uint8_t* zp, const uint16_t* src, int64_t K, int64_t N, int bits,
+                       int64_t bs, int symmetric) {
+  int64_t kbc = k_blocks_of(K, bs);
+  float* src32 = (float*)malloc(sizeof(float) * (size_t)(K * N));
+  float* s32 = (float*)malloc(sizeof(float) * (size_t)(N * kbc));
+  mnbo_f16_to_f32_buffer(src, src32, (size_t)(K * N));
+  quantize_core(B, s32, zp, src32, K, N, bits, bs, symmetric, 1);
+  mnbo_f32_to_f16_buffer(s32, scales, (size_t)(N * kbc));
+  free(src32);
+  free(s32);
 }

@@ -75,6 +75,8 @@ class _C:
                                             _i64, _int]
             lib.mnbo_matmul_f16.argtypes = [_u16p, _u8p, _u16p, _u8p, _u16p, _u16p, _i64, _i64, _i64, _int, _i64, _int]
             lib.mnbo_quantize_f32.argtypes = [_u8p, _f32p, _u8p, _f32p, _i64, _i64, _int, _i64, _int]
+            lib.mnbo_quantize_f16.argtypes = [_u8p, _u16p, _u8p, _u16p, _i64, _i64, _int, _i64, _int]
+            lib.mnbo_quantize_f16.restype = None
             for f in (lib.mnbo_f16_to_f32_buffer, lib.mnbo_f32_to_f16_buffer, lib.mnbo_dequantize_f32,
                       lib.mnbo_dequantize_f16, lib.mnbo_matmul_f32, lib.mnbo_matmul_f64, lib.mnbo_matmul_f16,
                       lib.mnbo_quantize_f32):
@@ -153,13 +155,20 @@ class _C:
 
     # -- quantise -------------------------------------------------------------
     def quantize(self, W, bits, bs, symmetric):
-        """W is [K, N] fp32 row-major. Returns (B[N,kb,blob], scales[N,kb], zp[N,zrow] or None)."""
-        W = np.ascontiguousarray(W, np.float32)
+        """W is [K, N] row-major, fp32 or fp16 (the model's type; other types are taken as fp32).
+        Returns (B[N,kb,blob], scales[N,kb] in W's type, zp[N,zrow] or None)."""
         K, N = W.shape
         kb = (K + bs - 1) // bs
         Bq = np.empty((N, kb, bs * bits // 8), np.uint8)
-        sc = np.empty((N, kb), np.float32)
         zp = None if symmetric else np.empty((N, (kb * bits + 7) // 8), np.uint8)
+        if W.dtype == np.float16:
+            W = np.ascontiguousarray(W)
+            sc = np.empty((N, kb), np.float16)
+            self.lib.mnbo_quantize_f16(_ptr(Bq, _u8p), _ptr(sc, _u16p), _ptr(zp, _u8p), _ptr(W, _u16p), K, N, bits,
+                                       bs, 1 if symmetric else 0)
+            return Bq, sc, zp
+        W = np.ascontiguousarray(W, np.float32)
+        sc = np.empty((N, kb), np.float32)
         self.lib.mnbo_quantize_f32(_ptr(Bq, _u8p), _ptr(sc, _f32p), _ptr(zp, _u8p), _ptr(W, _f32p), K, N, bits, bs,
                                    1 if symmetric else 0)
         return Bq, sc, zp
