@@ -40,6 +40,7 @@ struct Gemm256Params {
   int M, N, K, bs_shift;
   int ksteps;
   int tiles_m, tiles_n;
+  int c_vec_ok;  // C allows 16-byte stores of 8 columns: aligned base and pitch, N a multiple of 8
   uint32_t uc[4];  // unpack constants (see UnpackConsts)
 };
 
@@ -286,18 +287,53 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     k_step(ks + 1, R1, R0);
   }
 
-  // ---- epilogue: D[i][j] of a 32x32 tile: lane holds column j = lane % 32, rows 8*(r/4) + 4*(lane/32) + r%4
+  // ---- epilogue.  D[i][j] of a 32x32 tile: lane holds column j = lane % 32, rows 8*(r/4) + 4*(lane/32) + r%4.
+  // Stored straight from the accumulators that is 2 bytes per lane and 64-byte row segments; instead each wavefront
+  // transposes its block through its own slice of the (now idle) A buffers, 64 rows at a time, and writes whole
+  // 128-byte rows with 16-byte stores.
+  float bcol[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int n = n0 + wn * 64 + j * 32 + li;
-    if (n >= p.N) continue;
-    const float b = p.bias ? (float)p.bias[n] : 0.f;
+    bcol[j] = (p.bias && n < p.N) ? (float)p.bias[n] : 0.f;
+  }
+  if (p.c_vec_ok) {
+    constexpr int EP_STRIDE = 72;  // halves per staged row: 16-byte aligned rows, conflict-free 16-byte reads
+    __syncthreads();               // every wavefront is done with the A tiles
+    _Float16* ep = lds + wave * (64 * EP_STRIDE);
+    const int erow = lane >> 3, ecol = (lane & 7) * 8;
+    const int n_out = n0 + wn * 64 + ecol;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int h = 0; h < 2; ++h) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
-        if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + b);
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            ep[(ii * 32 + (r >> 2) * 8 + kq * 4 + (r & 3)) * EP_STRIDE + j * 32 + li] =
+                (_Float16)(acc[2 * h + ii][j][r] + bcol[j]);
+      // LDS operations of one wavefront complete in issue order: the reads below see the writes above
+#pragma unroll
+      for (int ps = 0; ps < 8; ++ps) {
+        const int row = ps * 8 + erow;
+        const u4_t v = *reinterpret_cast<const u4_t*>(ep + row * EP_STRIDE + ecol);
+        const int m = m0 + wm * 128 + h * 64 + row;
+        if (m < p.M && n_out < p.N) *reinterpret_cast<u4_t*>(p.C + (int64_t)m * p.ldc + n_out) = v;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn * 64 + j * 32 + li;
+      if (n >= p.N) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
+          if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + bcol[j]);
+        }
       }
     }
   }
@@ -348,6 +384,7 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.uc[1] = 0x00F000F0u;
   p.uc[2] = 0x64006400u;
   p.uc[3] = 0;
+  p.c_vec_ok = (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.ldc % 8 == 0) && (a.L.N % 8 == 0);
   if (a.L.bits == 4) return a.L.has_zp ? launch<4, true>(p, s) : launch<4, false>(p, s);
   return a.L.has_zp ? launch<8, true>(p, s) : launch<8, false>(p, s);
 }
