@@ -138,6 +138,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 GEMM")
+    ap.add_argument("--no-ceilings", action="store_true",
+                    help="skip the read-only / MFMA-only probe kernels that report what the machine sustains")
     ap.add_argument("--no-quantize", action="store_true", help="skip the blockwise quantiser (producer of the format)")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
@@ -214,6 +216,21 @@ def main() -> int:
     del g2, g2hot, p2
     torch.cuda.empty_cache()
 
+    # ---- what this GPU sustains with the plainest kernels (context for the fractions above and below) ----------
+    if not args.no_ceilings:
+        import ctypes
+        lib = _lib.load()
+        v = ctypes.c_double(0.0)
+        _lib.check(lib.MnbMeasureReadBandwidth(bytes_per_launch, LAYERS, ctypes.byref(v)))
+        read_same = v.value
+        _lib.check(lib.MnbMeasureReadBandwidth(1 << 30, 2, ctypes.byref(v)))
+        read_big = v.value
+        out["roofline"]["measured_ceiling"] = {
+            "read_only_kernel_same_bytes_per_launch_GBs": round(read_same, 1),
+            "read_only_kernel_1GiB_per_launch_GBs": round(read_big, 1),
+            "frac_of_read_only_kernel": round(gbs / read_same, 4) if read_same > 0 else None,
+        }
+
     # ---- prefill GEMM ----------------------------------------------------------------------------------------
     if not args.no_prefill:
         c4 = synthetic.config_c4(seed=0)
@@ -231,6 +248,19 @@ def main() -> int:
                          "unit": "TFLOP/s", "frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4),
                          "traffic": MEASURED_TRAFFIC_BYTES["c4_prefill"]},
         }
+        if not args.no_ceilings:
+            import ctypes
+            lib = _lib.load()
+            v = ctypes.c_double(0.0)
+            _lib.check(lib.MnbMeasureMfmaRate(0, ctypes.byref(v)))
+            mfma_const = v.value
+            _lib.check(lib.MnbMeasureMfmaRate(1, ctypes.byref(v)))
+            mfma_rand = v.value
+            out["prefill"]["roofline"]["measured_ceiling"] = {
+                "mfma_only_loop_constant_operands_TFLOPs": round(mfma_const, 1),
+                "mfma_only_loop_random_operands_TFLOPs": round(mfma_rand, 1),
+                "frac_of_mfma_only_random": round(tflops / mfma_rand, 4) if mfma_rand > 0 else None,
+            }
         del p4
         torch.cuda.empty_cache()
 

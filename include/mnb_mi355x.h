@@ -144,6 +144,16 @@ MNB_API int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_point
 /* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
 MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);
 
+/* Diagnostics without a counterpart in the reference: ceilings of the machine the library runs on, measured with
+ * the plainest kernels, so that the throughput of the real kernels can be read against what the device sustains.
+ * Both calls allocate their own buffers, run for a few milliseconds and synchronise the device.
+ * MnbMeasureReadBandwidth: GB/s of `launches` back-to-back kernels (one HIP graph) that each only read their own
+ * `bytes_per_launch` bytes of device memory once.
+ * MnbMeasureMfmaRate: TFLOP/s of a loop of nothing but v_mfma_f32_32x32x16_f16 on every CU, with constant operands
+ * (random_operands = 0) or random fp16 operands (1): the sustained matrix-core clock depends on operand toggling. */
+MNB_API int MnbMeasureReadBandwidth(size_t bytes_per_launch, int launches, double* gb_per_s);
+MNB_API int MnbMeasureMfmaRate(int random_operands, double* tflops);
+
 #ifdef __cplusplus
 }
 #endif

@@ -52,6 +52,8 @@ SIGNATURES = {
     "MnbDequantizeBlockwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_size_t,
                                        c_int, c_void_p]),
     "MnbDequantizePacked": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
+    "MnbMeasureReadBandwidth": (c_int, [c_size_t, c_int, ctypes.POINTER(ctypes.c_double)]),
+    "MnbMeasureMfmaRate": (c_int, [c_int, ctypes.POINTER(ctypes.c_double)]),
     "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
 }
 

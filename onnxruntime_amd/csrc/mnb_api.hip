@@ -299,6 +299,19 @@ int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_points_dev, c
   return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbQuantizeBlockwise");
 }
 
+int MnbMeasureReadBandwidth(size_t bytes_per_launch, int launches, double* gb_per_s) {
+  if (!gb_per_s || bytes_per_launch < 16 || launches < 1 || (double)bytes_per_launch * launches > 8e9)
+    return fail(MNB_INVALID_ARGUMENT, "MnbMeasureReadBandwidth: need gb_per_s, >= 16 bytes, >= 1 launch, <= 8 GB in total");
+  hipError_t e = mnb_probe_read(bytes_per_launch, launches, gb_per_s);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbMeasureReadBandwidth");
+}
+
+int MnbMeasureMfmaRate(int random_operands, double* tflops) {
+  if (!tflops) return fail(MNB_INVALID_ARGUMENT, "MnbMeasureMfmaRate: tflops must not be NULL");
+  hipError_t e = mnb_probe_mfma(random_operands, tflops);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbMeasureMfmaRate");
+}
+
 int MnbDequantizeBlockwise(void* dst_dev, const void* b_dev, const void* scales_dev, const void* zero_points_dev,
                            int block_size, int bits, size_t K, size_t N, int a_dtype, void* stream) {
   if (int rc = check_config("MnbDequantizeBlockwise", bits, block_size, a_dtype)) return rc;

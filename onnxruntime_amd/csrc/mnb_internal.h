@@ -46,3 +46,7 @@ bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
+
+// machine ceilings (mnb_probe.hip); diagnostics, synchronous
+hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s);
+hipError_t mnb_probe_mfma(int random_operands, double* tflops);
