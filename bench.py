@@ -28,7 +28,8 @@ sys.path.insert(0, str(ROOT))
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
 # for a plain copy of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs are summarised in
 # profiles/hbm_traffic_skinny_c2_gemm256_c4.md.  They are properties of the kernels, not of one run.
-MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14847.3 * 2.0 + 28.0) * 1024), "c4_prefill": int((109728.5 * 2.0 + 83294.5) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14847.3 * 2.0 + 28.0) * 1024), "c4_prefill": int((109683.5 * 2.0 + 57344.0) * 1024),
+                          "quantize": int((57409.6 * 2.0 + 41462.0) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
 LAYERS = 32
@@ -286,7 +287,7 @@ def main() -> int:
             "kernel": "mnb_quantize_kernel",
             "roofline": {"bound": "hbm", "achieved": round(qbytes / (msq * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(qbytes / (msq * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                         "traffic": None},
+                         "traffic": MEASURED_TRAFFIC_BYTES["quantize"]},
         }
         del ws
         torch.cuda.empty_cache()
