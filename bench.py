@@ -27,7 +27,7 @@ sys.path.insert(0, str(ROOT))
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
 # for a plain copy of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs are summarised in
-# profiles/hbm_traffic_skinny_c2_gemm256_c4.md.  They are properties of the kernels, not of one run.
+# profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md.  They are properties of the kernels, not of one run.
 MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14847.3 * 2.0 + 28.0) * 1024), "c4_prefill": int((109683.5 * 2.0 + 57344.0) * 1024),
                           "quantize": int((57409.6 * 2.0 + 41462.0) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
