@@ -165,6 +165,123 @@ __global__ void __launch_bounds__(NW * 64) mnb_gemv_kernel(GemvParams p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------ fp32, few rows
+// fp32 models with M <= 4.  The kernel above gives every workgroup 64 columns, i.e. N / 64 workgroups: a K = N = 4096
+// projection occupies a quarter of the chip.  Here a workgroup owns 16 columns: lane (j = lane % 16, kq = lane / 16)
+// takes k-group 4c + kq of chunk c for column j, so a wavefront still reads four 256-byte runs of the packed weights
+// per load.  The activations are no longer wave-uniform; they are staged once per workgroup in LDS (fp32, one
+// padded row of 36 floats per k-group of 32: the four kq segments of a ds_read_b128 hit different banks) and read as
+// 16-byte broadcasts.  Arithmetic per weight is that of the kernel above: float(q) - zp, fused multiply-add with the
+// activation, the block sum times the scale.  The four kq partial sums meet through two cross-lane exchanges, the
+// wavefronts (K split) through LDS in a fixed order.
+constexpr int kG16Pad = 4;         // floats of padding per staged k-group
+constexpr int kG16PhaseK = 2048;   // k staged at a time (x MT rows x 4 B <= 36 KiB)
+
+template <int BITS, bool HAS_ZP, bool SMALL_BS, int MT, int NW>
+__global__ void __launch_bounds__(NW * 64) mnb_gemv16_kernel(GemvParams p) {
+  constexpr int GK = 128 / BITS;                // k per 16-byte vector
+  constexpr int GS = GK + kG16Pad;              // staged floats per k-group
+  constexpr int PH_GROUPS = kG16PhaseK / GK;    // k-groups per phase
+  constexpr int NBLK = SMALL_BS ? 2 : 1;
+  constexpr int WORDS = 4 / NBLK;
+  constexpr int EPW = (BITS == 4) ? 8 : 4;
+  __shared__ __align__(16) float As[MT * PH_GROUPS * GS];
+  __shared__ float red[NW * MT * 16];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, kq = lane >> 4;
+  const int64_t n = (int64_t)blockIdx.x * 16 + j;  // < Npad always
+  const float* __restrict__ A = reinterpret_cast<const float*>(p.A);
+  const int64_t mcol = mnb_meta_col(n);
+
+  float acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) acc[m] = 0.f;
+
+  for (int g0 = 0; g0 < p.KG; g0 += PH_GROUPS) {
+    const int g1 = g0 + PH_GROUPS < p.KG ? g0 + PH_GROUPS : p.KG;
+    const int groups = g1 - g0;
+    // chunks of 4 k-groups; wavefront w takes chunks w, w + NW, ...; two vectors in flight per lane.  The first
+    // weight loads go out before the activations are staged, so the two latencies overlap.
+    const int chunks = (groups + 3) / 4;
+    int c = wave;
+    uint4 w0 = make_uint4(0, 0, 0, 0), w1 = w0;
+    auto gl = [&](int cc) { return g0 + cc * 4 + kq; };
+    if (c < chunks && gl(c) < g1) w0 = p.W[(int64_t)gl(c) * p.Npad + n];
+    if (c + NW < chunks && gl(c + NW) < g1) w1 = p.W[(int64_t)gl(c + NW) * p.Npad + n];
+    __syncthreads();  // the previous phase is no longer read
+    for (int i = threadIdx.x; i < MT * groups * (GK / 4); i += NW * 64) {
+      const int q4 = i % (GK / 4), g = (i / (GK / 4)) % groups, m = i / ((GK / 4) * groups);
+      const int mm = m < p.M ? m : p.M - 1;  // rows >= M repeat the last row and are never stored
+      const float4 v = *reinterpret_cast<const float4*>(A + (int64_t)mm * p.lda + (int64_t)(g0 + g) * GK + q4 * 4);
+      *reinterpret_cast<float4*>(&As[(m * PH_GROUPS + g) * GS + q4 * 4]) = v;
+    }
+    __syncthreads();
+    for (; c < chunks; c += NW) {
+      const uint4 wv = w0;
+      w0 = w1;
+      if (c + 2 * NW < chunks && gl(c + 2 * NW) < g1) w1 = p.W[(int64_t)gl(c + 2 * NW) * p.Npad + n];
+      const int g = gl(c);
+      if (g >= g1) continue;  // ragged last chunk of the phase
+      const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};
+      const int64_t kb = SMALL_BS ? (int64_t)g * 2 : (((int64_t)g * GK) >> p.bs_shift);
+      const float* a_grp = &As[(g - g0) * GS];
+#pragma unroll
+      for (int b = 0; b < NBLK; ++b) {
+        float sc, zp;
+        mnb_load_meta_f<HAS_ZP, BITS>(p.meta, (kb + b) * p.Npad + mcol, sc, zp);
+        float part[MT];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) part[m] = 0.f;
+#pragma unroll
+        for (int i = 0; i < WORDS; ++i) {
+          float d[EPW];
+          if constexpr (BITS == 4)
+            mnb_unpack4_f(wd[b * WORDS + i], zp, d);
+          else
+            mnb_unpack8_f(wd[b * WORDS + i], zp, d);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) {
+            const float* a = a_grp + m * PH_GROUPS * GS + (b * WORDS + i) * EPW;
+#pragma unroll
+            for (int e4 = 0; e4 < EPW / 4; ++e4) {
+              const float4 av = *reinterpret_cast<const float4*>(a + e4 * 4);
+              part[m] = __builtin_fmaf(av.x, d[e4 * 4 + 0], part[m]);
+              part[m] = __builtin_fmaf(av.y, d[e4 * 4 + 1], part[m]);
+              part[m] = __builtin_fmaf(av.z, d[e4 * 4 + 2], part[m]);
+              part[m] = __builtin_fmaf(av.w, d[e4 * 4 + 3], part[m]);
+            }
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) acc[m] = __builtin_fmaf(part[m], sc, acc[m]);
+      }
+    }
+  }
+  // the four kq partial sums of a column, then the wavefronts
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    acc[m] += __shfl_xor(acc[m], 16, 64);
+    acc[m] += __shfl_xor(acc[m], 32, 64);
+  }
+  if (kq == 0) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) red[(wave * MT + m) * 16 + j] = acc[m];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < MT * 16; i += NW * 64) {
+    const int m = i >> 4, l = i & 15;
+    const int64_t nn = (int64_t)blockIdx.x * 16 + l;
+    if (m >= p.M || nn >= p.N) continue;
+    float sum = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * MT + m) * 16 + l];
+    if (p.bias) sum += reinterpret_cast<const float*>(p.bias)[nn];
+    reinterpret_cast<float*>(p.C)[(int64_t)m * p.ldc + nn] = sum;
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ generic
 // Any M, N, K, lda, alignment.  One wavefront per 64 columns x MT rows; sequential k, fp32 accumulation of
 // a * (d * scale) exactly as the reference's scalar definition.  Slow; used when the fast kernels' alignment
@@ -314,6 +431,30 @@ hipError_t launch_generic_zp(const GemvParams& p, hipStream_t s) {
   return hipGetLastError();
 }
 
+template <int BITS, bool HAS_ZP, bool SMALL_BS, int MT>
+hipError_t launch_gemv16_nw(const GemvParams& p, hipStream_t s) {
+  dim3 grid((unsigned)((p.N + 15) / 16));
+  const int chunks = (p.KG + 3) / 4;
+  if (chunks >= 32) {
+    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 8><<<grid, dim3(512), 0, s>>>(p);
+  } else {
+    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 4><<<grid, dim3(256), 0, s>>>(p);
+  }
+  return hipGetLastError();
+}
+
+template <int BITS, bool HAS_ZP>
+hipError_t launch_gemv16(const GemvParams& p, hipStream_t s) {
+  const bool small = (BITS == 4) && p.bs == 16;
+#define MNB_G16(MT_)                                                                         \
+  return small ? launch_gemv16_nw<BITS, HAS_ZP, (BITS == 4), MT_>(p, s)                      \
+               : launch_gemv16_nw<BITS, HAS_ZP, false, MT_>(p, s)
+  if (p.M <= 1) { MNB_G16(1); }
+  if (p.M <= 2) { MNB_G16(2); }
+  MNB_G16(4);
+#undef MNB_G16
+}
+
 int log2i(int v) {
   int s = 0;
   while ((1 << s) < v) ++s;
@@ -355,6 +496,11 @@ bool mnb_gemv_applicable(const MnbGemmArgs& a) {
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s) {
   GemvParams p = make_params(a);
   const int64_t col_groups = (a.L.N + 63) / 64;
+  // few rows and too few 64-column slabs to fill the chip: 16-column workgroups
+  if (a.M <= 4 && col_groups < 192) {
+    if (a.L.bits == 4) return a.L.has_zp ? launch_gemv16<4, true>(p, s) : launch_gemv16<4, false>(p, s);
+    return a.L.has_zp ? launch_gemv16<8, true>(p, s) : launch_gemv16<8, false>(p, s);
+  }
   const int mt = gemv_mt(a.M), nw = gemv_nw(a.L);
   if (a.L.bits == 4)
     return a.L.has_zp ? launch_gemv_zp<float, 4, true>(p, mt, nw, col_groups, s)

@@ -84,12 +84,12 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
 }
 
 // One chunk: word step i of every column tile against the MT row tiles, then -- the A operands of step i being dead --
-// their reload for the wavefront's next chunk (a_next, or NULL at the end).  The activations are thus prefetched
+// their reload for the wavefront's next chunk (a_next, when has_next).  The activations are thus prefetched
 // three quarters of a chunk ahead without a second register set.
 template <int BITS, bool HAS_ZP, int T, int MT>
 __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h8_t (*af)[(128 / BITS) / 8],
-                                                  const uint4* a_next, int64_t a_step, const UnpackConsts& uc,
-                                                  f4_t (*y)[T]) {
+                                                  const uint4* a_next, bool has_next, int64_t a_step,
+                                                  const UnpackConsts& uc, f4_t (*y)[T]) {
   constexpr int NI = (128 / BITS) / 8;
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
@@ -107,7 +107,7 @@ __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) y[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][i], b, y[mt][t], 0, 0, 0);
     }
-    if (a_next != nullptr) {
+    if (has_next) {  // wave-uniform: no divergent branch inside the chunk
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) af[mt][i] = __builtin_bit_cast(h8_t, a_next[i * a_step + mt * 64]);
     }
@@ -148,7 +148,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
   };
 
   // weights two chunks ahead (double buffer); activations reloaded word step by word step inside the chunk
-  auto a_of = [&](int c) -> const uint4* { return c < p.chunks ? a_lane + (int64_t)c * NI * a_step : nullptr; };
+  auto a_of = [&](int c) -> const uint4* { return a_lane + (int64_t)c * NI * a_step; };
   ChunkRegs<BITS, T> R0, R1;
   int c = wave;
   if (c < p.chunks) {
@@ -157,10 +157,10 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
   }
   if (c + NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + NW, kq, col0, R1);
   for (; c < p.chunks; c += 2 * NW) {
-    mid_compute_chunk<BITS, HAS_ZP, T, MT>(R0, af, a_of(c + NW), a_step, uc, y);
+    mid_compute_chunk<BITS, HAS_ZP, T, MT>(R0, af, a_of(c + NW), c + NW < p.chunks, a_step, uc, y);
     if (c + 2 * NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + 2 * NW, kq, col0, R0);
     if (c + NW < p.chunks) {
-      mid_compute_chunk<BITS, HAS_ZP, T, MT>(R1, af, a_of(c + 2 * NW), a_step, uc, y);
+      mid_compute_chunk<BITS, HAS_ZP, T, MT>(R1, af, a_of(c + 2 * NW), c + 2 * NW < p.chunks, a_step, uc, y);
       if (c + 3 * NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + 3 * NW, kq, col0, R1);
     }
   }
