@@ -17,6 +17,7 @@
 #include <cstring>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -175,10 +176,7 @@ OrtApi g_ort{};
 OrtEpApi g_ep{};
 OrtDataType g_types[32];
 
-void FillApis() {
-  static bool done = false;
-  if (done) return;
-  done = true;
+void FillApisOnce() {
   for (int i = 0; i < 32; ++i) g_types[i].elem = static_cast<ONNXTensorElementDataType>(i);
 
   // ---- OrtApi
@@ -445,6 +443,11 @@ void FillApis() {
   };
 }
 
+void FillApis() {
+  static std::once_flag once;
+  std::call_once(once, FillApisOnce);
+}
+
 const OrtApi* ORT_API_CALL GetApi(uint32_t version) NO_EXCEPTION {
   return version <= ORT_API_VERSION ? &g_ort : nullptr;
 }
@@ -473,6 +476,8 @@ struct Plugin {
 };
 
 Plugin* LoadPlugin(const char* path, std::string* error) {
+  static std::mutex mutex;  // sessions may be driven from several test threads
+  std::lock_guard<std::mutex> lock(mutex);
   static std::map<std::string, Plugin> loaded;
   auto it = loaded.find(path);
   if (it != loaded.end()) return &it->second;

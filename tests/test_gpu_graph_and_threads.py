@@ -1,0 +1,73 @@
+"""The C ABI under HIP graph capture (every kernel family, replayed with eager work in between) and the plugin EP
+driven from several host threads at once."""
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+from ep_host import host
+from gpu_util import check_against_oracle, dev, make_op
+from onnxruntime_amd.synthetic import make_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,N,K,bits,bs,dtype", [
+    (1, 512, 1024, 4, 128, np.float16),     # matrix-core decode kernel
+    (3, 300, 520, 8, 32, np.float32),       # fp32 GEMV
+    (40, 384, 1024, 4, 32, np.float16),     # weight-streaming kernel (staging kernel + main kernel, workspace)
+    (300, 512, 1024, 4, 64, np.float16),    # tile GEMM or streaming kernel, by the cost estimate
+    (20, 100, 200, 4, 16, np.float32),      # generic kernel
+])
+def test_gemm_replays_from_a_hip_graph(M, N, K, bits, bs, dtype):
+    c = make_case(M, N, K, bits, bs, dtype, has_zp=True, has_bias=True, seed=M + N)
+    op = make_op(c)
+    bias = dev(c.bias)
+    a1, a2 = dev(c.A), dev(c.A[::-1].copy())
+    a = a1.clone()
+    y = op.Compute(a, bias=bias)                      # eager: also sizes the workspace outside the capture
+    want1 = y.clone()
+    want2 = op.Compute(a2, bias=bias).clone()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            op.Compute(a, bias=bias, out=y)
+    for rep in range(4):                              # replays, with eager work and new inputs in between
+        src, want = (a1, want1) if rep % 2 == 0 else (a2, want2)
+        a.copy_(src)
+        y.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), f"replay {rep}"
+        _ = op.Compute(a2, bias=bias)                 # eager call of the same op between replays
+        torch.cuda.synchronize()
+
+
+@pytest.mark.skipif(not host.available(), reason="plugin EP or host shim not built")
+def test_plugin_sessions_on_concurrent_threads(oracle):
+    cases = [make_case(M, 192, 256, bits, 32, dt, has_zp=True, has_bias=bool(M % 2), seed=M)
+             for M, bits, dt in [(1, 4, np.float16), (5, 8, np.float32), (33, 4, np.float16), (2, 4, np.float32)]]
+    results, errors = [None] * len(cases), []
+
+    def work(i):
+        try:
+            c = cases[i]
+            for _ in range(5):
+                y, _ = host.run_matmul_nbits(c.N, c.K, c.bits, c.block_size, c.A, c.B, c.scales, c.zero_points,
+                                             None, c.bias, repeat=2)
+            results[i] = y
+        except Exception as e:  # noqa: BLE001
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for c, y in zip(cases, results):
+        check_against_oracle(oracle, c, y)
