@@ -290,7 +290,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct) {
   pl.mtr = pow2_ceil((int)M);
   // workgroups: as many column slabs as fill the chip; wide slabs (T = 4) amortise the A operands best
   const int64_t tiles = (L.N + 15) / 16;
-  pl.t = tiles >= 4 * 200 ? 4 : tiles >= 2 * 200 ? 2 : 1;
+  pl.t = tiles >= 800 ? 4 : tiles >= 320 ? 2 : 1;  // measured: N = 6144 prefers 2 (192 workgroups), N = 4096 prefers 1
   // wavefronts per workgroup: aim for >= 2 chunks per wavefront
   pl.nw = chunks >= 32 ? 16 : chunks >= 16 ? 8 : 4;
   if (const char* e = getenv("MNB_SKINNY_PLAN")) {  // tuning override "<T>,<NW>"
