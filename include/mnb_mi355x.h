@@ -92,8 +92,9 @@ MNB_API int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int 
                               const void* scales_dev, const void* zero_points_dev, void* packed_dev, void* stream);
 
 /* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call device scratch MnbGemm needs for
- * this problem. Non-zero only for fp16 activations with M > 16 whose shape selects the weight-streaming kernel (a
- * copy of A in matrix-core operand order, about M*K*2 bytes); 0 otherwise. */
+ * this problem. Non-zero only for fp16 activations whose shape selects the weight-streaming kernel (M > 16 below the
+ * tile GEMM's range, or M <= 16 with K not a multiple of 128 (4-bit) / 64 (8-bit)): a copy of A in matrix-core
+ * operand order, about M*K*2 bytes; 0 otherwise. */
 MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                     int a_dtype);
 

@@ -186,7 +186,15 @@ static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
 }
 
 MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
-  if (mnb_skinny_applicable(a)) return kMnbKernelSkinny;
+  if (mnb_skinny_applicable(a)) {
+    // The decode kernel reads activations 16 bytes at a time; when K is not a whole number of its chunks (or A is
+    // misaligned) its fallback stages A element by element.  The streaming kernel's staged copy of A (zero-padded,
+    // any alignment) is the faster route whenever the caller's workspace allows it.
+    const bool direct = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) &&
+                        (a.L.K % (4 * a.L.group_k) == 0);
+    if (!direct && a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;
+    return kMnbKernelSkinny;
+  }
   if (mnb_gemv_applicable(a)) return kMnbKernelGemv;
   if (a.L.dtype == kMnbDtypeFloat16) {
     // the tile GEMM loads activations 16 bytes at a time: base and row pitch aligned
@@ -215,9 +223,11 @@ size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_si
                             int a_dtype) {
   if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0 || M == 0) return 0;
   // only the mid-M fp16 kernel needs scratch: a copy of A in matrix-core operand order
-  if (a_dtype == kMnbDtypeFloat16 && M > 16) {
+  if (a_dtype == kMnbDtypeFloat16) {
     const MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
-    if (!mnb_prefer_gemm256(L, (int64_t)M)) return mnb_mid_workspace_bytes(L, (int64_t)M);
+    // M <= 16 needs it only when K is not a whole number of the decode kernel's chunks
+    const bool wants = M > 16 ? !mnb_prefer_gemm256(L, (int64_t)M) : (K % (size_t)(4 * L.group_k) != 0);
+    if (wants) return mnb_mid_workspace_bytes(L, (int64_t)M);
   }
   return 0;
 }
@@ -340,6 +350,7 @@ const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_
   a.M = (int64_t)M;
   a.lda = (int64_t)((K + 7) / 8 * 8);  // assume the usual aligned activations
   a.A = nullptr;
+  a.workspace_bytes = ~(size_t)0;  // a caller that follows MnbGemmWorkspaceSize
   return mnb_kernel_name(mnb_select_kernel(a), a.L);
 }
 

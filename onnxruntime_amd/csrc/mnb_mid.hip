@@ -252,7 +252,7 @@ int mid_row_tiles(int64_t M, int mt) { return (int)((M + 16 * mt - 1) / (16 * mt
 
 }  // namespace
 
-bool mnb_mid_applicable(const MnbGemmArgs& a) { return a.L.dtype == kMnbDtypeFloat16 && a.M > 16; }
+bool mnb_mid_applicable(const MnbGemmArgs& a) { return a.L.dtype == kMnbDtypeFloat16 && a.M >= 1; }
 
 // bytes of the staged copy of A
 size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
