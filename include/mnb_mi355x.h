@@ -142,6 +142,58 @@ MNB_API int MnbDequantizePacked(void* dst_dev, const void* packed_dev, size_t N,
 MNB_API int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_points_dev, const void* src_dev,
                                  int block_size, int bits, size_t K, size_t N, size_t leading_dimension, int a_dtype,
                                  void* stream);
+
+/* ---- several projections behind one activation ------------------------------------------------------------------
+ * com.microsoft::MatMulNBitsMlp and MatMulNBitsQkv (onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3851-3975 and
+ * :3977-4090; the reference's only kernels for them are the WebGPU ones,
+ * onnxruntime/contrib_ops/webgpu/quantization/matmul_nbits_mlp.cc:241-543 and matmul_nbits_qkv.cc:150-392).
+ * The weight matrices share K, bits and block_size, have no zero points, and are packed into ONE buffer so that one
+ * launch streams all of them; the biases (NULL = absent) are folded into that buffer at pack time. */
+
+/* Optional prologue of both operators: SimplifiedLayerNormalization (skip_dev == NULL) or
+ * SkipSimplifiedLayerNormalization of the activation
+ * (onnxruntime/contrib_ops/cpu/skip_layer_norm.cc:44-97): x = A + skip, A_norm = x / sqrt(mean_k(x^2) + epsilon) *
+ * norm_scale, computed in fp32 and narrowed once.  norm_scale_dev == NULL: no prologue (skip must be NULL too). */
+typedef struct MnbNormPrologue {
+  const void* norm_scale_dev; /* T[K] */
+  const void* skip_dev;       /* optional T[skip_rows][ld_skip]; row m of A is added to skip row m % skip_rows */
+  size_t ld_skip;
+  size_t skip_rows;           /* 0 = one skip row per row of A */
+  void* skip_sum_dev;         /* optional output T[M][ld_skip_sum]: A + skip (the operators' input_skip_bias_sum) */
+  size_t ld_skip_sum;
+  float epsilon;
+} MnbNormPrologue;
+
+#define MNB_ACTIVATION_SILU 0 /* the only activation the operator defines (matmul_nbits_mlp.cc:24-31) */
+
+/* MatMulNBitsMlp: Y[M][N] = silu(A' x gate^T + gate_bias) * (A' x up^T + up_bias), A' = A or its normalisation.
+ * Gate/up products and the activation are evaluated in fp32; Y is narrowed once. */
+MNB_API size_t MnbMlpPackSize(size_t N, size_t K, int bits, int block_size, int a_dtype);
+MNB_API int MnbMlpPack(size_t N, size_t K, int bits, int block_size, int a_dtype, const void* gate_b_dev,
+                       const void* gate_scales_dev, const void* gate_bias_dev, const void* up_b_dev,
+                       const void* up_scales_dev, const void* up_bias_dev, void* packed_dev, void* stream);
+MNB_API size_t MnbMlpWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, int has_norm);
+MNB_API int MnbMlpGemm(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, const void* a_dev,
+                       size_t lda, const MnbNormPrologue* norm, const void* packed_dev, int activation, void* y_dev,
+                       size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* MatMulNBitsQkv: Q[M][Nq], K[M][Nkv], V[M][Nkv] = A' x {q,k,v}^T + bias. */
+MNB_API size_t MnbQkvPackSize(size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype);
+MNB_API int MnbQkvPack(size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype, const void* q_b_dev,
+                       const void* q_scales_dev, const void* q_bias_dev, const void* k_b_dev,
+                       const void* k_scales_dev, const void* k_bias_dev, const void* v_b_dev,
+                       const void* v_scales_dev, const void* v_bias_dev, void* packed_dev, void* stream);
+MNB_API size_t MnbQkvWorkspaceSize(size_t M, size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype,
+                                   int has_norm);
+MNB_API int MnbQkvGemm(size_t M, size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype,
+                       const void* a_dev, size_t lda, const MnbNormPrologue* norm, const void* packed_dev, void* q_dev,
+                       size_t ldq, void* k_dev, size_t ldk, void* v_dev, size_t ldv, void* workspace_dev,
+                       size_t workspace_bytes, void* stream);
+
+/* The prologue alone (what the fused calls run first): a_norm_dev T[M][K], dense. */
+MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* a_dev, size_t lda,
+                                   const MnbNormPrologue* norm, void* a_norm_dev, void* stream);
+
 /* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
 MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);
 

@@ -31,6 +31,13 @@ class MnbTensorInfo(ctypes.Structure):
     _fields_ = [("dims", ctypes.POINTER(c_int64)), ("rank", c_size_t), ("dtype", c_int)]
 
 
+class MnbNormPrologue(ctypes.Structure):
+    _fields_ = [("norm_scale_dev", c_void_p), ("skip_dev", c_void_p), ("ld_skip", c_size_t), ("skip_rows", c_size_t),
+                ("skip_sum_dev", c_void_p), ("ld_skip_sum", c_size_t), ("epsilon", ctypes.c_float)]
+
+
+_NORM_P = ctypes.POINTER(MnbNormPrologue)
+
 # name -> (restype, argtypes); every symbol include/mnb_mi355x.h declares
 SIGNATURES = {
     "MnbGetLastErrorMessage": (c_char_p, []),
@@ -52,6 +59,18 @@ SIGNATURES = {
     "MnbDequantizeBlockwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_size_t, c_size_t,
                                        c_int, c_void_p]),
     "MnbDequantizePacked": (c_int, [c_void_p, c_void_p, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p]),
+    "MnbMlpPackSize": (c_size_t, [c_size_t, c_size_t, c_int, c_int, c_int]),
+    "MnbMlpPack": (c_int, [c_size_t, c_size_t, c_int, c_int, c_int] + [c_void_p] * 8),
+    "MnbMlpWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
+    "MnbMlpGemm": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_void_p, c_size_t, _NORM_P, c_void_p,
+                           c_int, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "MnbQkvPackSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
+    "MnbQkvPack": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int] + [c_void_p] * 11),
+    "MnbQkvWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
+    "MnbQkvGemm": (c_int, [c_size_t, c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_void_p, c_size_t, _NORM_P,
+                           c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t,
+                           c_void_p]),
+    "MnbSimplifiedLayerNorm": (c_int, [c_size_t, c_size_t, c_int, c_void_p, c_size_t, _NORM_P, c_void_p, c_void_p]),
     "MnbMeasureReadBandwidth": (c_int, [c_size_t, c_int, ctypes.POINTER(ctypes.c_double)]),
     "MnbMeasureMfmaRate": (c_int, [c_int, ctypes.POINTER(ctypes.c_double)]),
     "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),

@@ -242,7 +242,7 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
   if (lda < K || ldc < N) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: lda (%zu) < K (%zu) or ldc (%zu) < N (%zu)", lda, K, ldc, N);
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff)
     return fail(MNB_INVALID_ARGUMENT, "MnbGemm: M, N and K must fit in 31 bits");
-  MnbGemmArgs a;
+  MnbGemmArgs a{};  // epi: plain output
   a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
   a.M = (int64_t)M;
   a.A = a_dev;
@@ -294,6 +294,241 @@ int MnbGemmUnpacked(size_t M, size_t N, size_t K, int bits, int block_size, int 
     return rc;
   return MnbGemm(M, N, K, bits, block_size, has_zp, a_dtype, a_dev, lda, workspace_dev, bias_dev, c_dev, ldc,
                  static_cast<char*>(workspace_dev) + pack, workspace_bytes - pack, stream);
+}
+
+// ---------------------------------------------------------------------------------------- fused projections
+}  // extern "C"
+
+bool mnb_kernel_has_fused_epilogue(MnbKernelKind k) { return k == kMnbKernelSkinny || k == kMnbKernelMid; }
+
+namespace {
+
+size_t round256(size_t v) { return (v + 255) / 256 * 256; }
+size_t elem_size(int dtype) { return dtype == kMnbDtypeFloat16 ? 2 : 4; }
+
+// bytes of [normalised A][plain product over the packed columns][workspace of the GEMM kernel]
+struct FusedWorkspace {
+  size_t a_norm, tmp, inner;
+  size_t total() const { return a_norm + tmp + inner; }
+};
+
+FusedWorkspace fused_workspace(const MnbFusedLayout& F, size_t M, int has_norm) {
+  FusedWorkspace w{};
+  const MnbLayout& L = F.L;
+  w.a_norm = has_norm ? round256(M * (size_t)L.K * elem_size(L.dtype)) : 0;
+  w.inner = MnbGemmWorkspaceSize(M, (size_t)L.N, (size_t)L.K, L.bits, L.bs, 0, L.dtype);
+  // the decode and streaming kernels write the operator's outputs themselves; they are chosen by shape alone when
+  // the workspace above is there (fp16: M <= 16, or the streaming kernel's regime)
+  const bool fused = L.dtype == kMnbDtypeFloat16 && (M <= 16 || w.inner > 0);
+  w.tmp = fused ? 0 : round256(M * (size_t)L.N * elem_size(L.dtype));
+  return w;
+}
+
+int check_norm(const char* fn, const MnbNormPrologue* norm, size_t K) {
+  if (!norm) return MNB_OK;
+  if (!norm->norm_scale_dev) {
+    if (norm->skip_dev || norm->skip_sum_dev)
+      return fail(MNB_INVALID_ARGUMENT, "%s: norm_scale input must be present when skip input is provided", fn);
+    return MNB_OK;
+  }
+  if (norm->skip_dev && norm->ld_skip < K) return fail(MNB_INVALID_ARGUMENT, "%s: ld_skip (%zu) < K (%zu)", fn, norm->ld_skip, K);
+  if (norm->skip_sum_dev && !norm->skip_dev)
+    return fail(MNB_INVALID_ARGUMENT, "%s: skip input must be present when input_skip_bias_sum output is requested", fn);
+  if (norm->skip_sum_dev && norm->ld_skip_sum < K)
+    return fail(MNB_INVALID_ARGUMENT, "%s: ld_skip_sum (%zu) < K (%zu)", fn, norm->ld_skip_sum, K);
+  if (!(norm->epsilon >= 0.f)) return fail(MNB_INVALID_ARGUMENT, "%s: epsilon must not be negative", fn);
+  return MNB_OK;
+}
+
+hipError_t run_norm(const MnbNormPrologue* n, const void* a, size_t lda, void* a_norm, size_t M, size_t K, int dtype,
+                    hipStream_t s) {
+  return mnb_launch_rmsnorm(a_norm, n->skip_sum_dev, (int64_t)n->ld_skip_sum, a, (int64_t)lda, n->skip_dev,
+                            (int64_t)n->ld_skip, (int64_t)n->skip_rows, n->norm_scale_dev, n->epsilon, (int64_t)M,
+                            (int64_t)K, dtype, s);
+}
+
+// One GEMM over the packed matrices of F, outputs as epi describes.
+int fused_gemm(const char* fn, const MnbFusedLayout& F, size_t M, const void* a_dev, size_t lda,
+               const MnbNormPrologue* norm, const void* packed_dev, MnbEpilogue epi, void* workspace_dev,
+               size_t workspace_bytes, hipStream_t s) {
+  const MnbLayout& L = F.L;
+  const bool has_norm = norm && norm->norm_scale_dev;
+  if (int rc = check_norm(fn, norm, (size_t)L.K)) return rc;
+  if (lda < (size_t)L.K) return fail(MNB_INVALID_ARGUMENT, "%s: lda (%zu) < K (%lld)", fn, lda, (long long)L.K);
+  if (M > 0x7fffffff || L.N > 0x7fffffff || L.K > 0x7fffffff)
+    return fail(MNB_INVALID_ARGUMENT, "%s: M, N and K must fit in 31 bits", fn);
+  if (!workspace_dev) workspace_bytes = 0;
+  if (reinterpret_cast<uintptr_t>(workspace_dev) % 256 != 0)
+    return fail(MNB_INVALID_ARGUMENT, "%s: the workspace must be 256-byte aligned", fn);
+  const FusedWorkspace w = fused_workspace(F, M, has_norm);
+  if (workspace_bytes < w.total())
+    return fail(MNB_INVALID_ARGUMENT, "%s: workspace of %zu bytes needed, %zu given", fn, w.total(), workspace_bytes);
+  char* ws = static_cast<char*>(workspace_dev);
+  const void* act = a_dev;
+  size_t ld_act = lda;
+  if (has_norm) {
+    hipError_t e = run_norm(norm, a_dev, lda, ws, M, (size_t)L.K, L.dtype, s);
+    if (e != hipSuccess) return hip_fail(e, fn);
+    act = ws;
+    ld_act = (size_t)L.K;
+  }
+  MnbGemmArgs a{};
+  a.L = L;
+  a.M = (int64_t)M;
+  a.A = act;
+  a.lda = (int64_t)ld_act;
+  a.packed = packed_dev;
+  a.bias = static_cast<const char*>(packed_dev) + F.bias_off;
+  a.workspace = w.inner ? ws + w.a_norm + w.tmp : nullptr;
+  a.workspace_bytes = w.inner ? workspace_bytes - w.a_norm - w.tmp : 0;
+  MnbKernelKind k = mnb_select_kernel(a);
+  const bool direct = mnb_kernel_has_fused_epilogue(k);
+  if (direct) {
+    a.epi = epi;
+  } else {
+    // plain product over the packed columns, then the finishing pass
+    if (w.tmp == 0) return fail(MNB_FAIL, "%s: no scratch for the product planned for this shape", fn);
+    a.C = ws + w.a_norm;
+    a.ldc = L.N;
+  }
+  hipError_t e;
+  switch (k) {
+    case kMnbKernelSkinny: e = mnb_launch_skinny(a, s); break;
+    case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
+    case kMnbKernelMid: e = mnb_launch_mid(a, s); break;
+    case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
+    default: e = mnb_launch_gemm_generic(a, s); break;
+  }
+  if (e != hipSuccess) return hip_fail(e, fn);
+  if (!direct) {
+    e = mnb_launch_fused_finish(epi, a.C, a.ldc, (int64_t)M, L.dtype, s);
+    if (e != hipSuccess) return hip_fail(e, fn);
+  }
+  return MNB_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t MnbMlpPackSize(size_t N, size_t K, int bits, int block_size, int a_dtype) {
+  if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0) return 0;
+  return (size_t)mnb_make_fused_layout(kMnbFusedMlp, (int64_t)N, 0, (int64_t)K, bits, block_size, a_dtype).total_bytes;
+}
+
+int MnbMlpPack(size_t N, size_t K, int bits, int block_size, int a_dtype, const void* gate_b_dev,
+               const void* gate_scales_dev, const void* gate_bias_dev, const void* up_b_dev, const void* up_scales_dev,
+               const void* up_bias_dev, void* packed_dev, void* stream) {
+  if (int rc = check_config("MnbMlpPack", bits, block_size, a_dtype)) return rc;
+  if (N == 0 || K == 0) return MNB_OK;
+  if (!gate_b_dev || !gate_scales_dev || !up_b_dev || !up_scales_dev || !packed_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbMlpPack: B and scales of both projections and the packed buffer must not be NULL");
+  if (reinterpret_cast<uintptr_t>(packed_dev) % 256 != 0)
+    return fail(MNB_INVALID_ARGUMENT, "MnbMlpPack: the packed buffer must be 256-byte aligned");
+  const MnbFusedLayout F = mnb_make_fused_layout(kMnbFusedMlp, (int64_t)N, 0, (int64_t)K, bits, block_size, a_dtype);
+  const void* B[3] = {gate_b_dev, up_b_dev, nullptr};
+  const void* S[3] = {gate_scales_dev, up_scales_dev, nullptr};
+  const void* bias[3] = {gate_bias_dev, up_bias_dev, nullptr};
+  hipError_t e = mnb_launch_pack_fused(F, B, S, bias, packed_dev, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbMlpPack");
+}
+
+size_t MnbMlpWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, int has_norm) {
+  if (!supported(bits, block_size, a_dtype) || N == 0 || K == 0 || M == 0) return 0;
+  const MnbFusedLayout F = mnb_make_fused_layout(kMnbFusedMlp, (int64_t)N, 0, (int64_t)K, bits, block_size, a_dtype);
+  return fused_workspace(F, M, has_norm).total();
+}
+
+int MnbMlpGemm(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, const void* a_dev, size_t lda,
+               const MnbNormPrologue* norm, const void* packed_dev, int activation, void* y_dev, size_t ldc,
+               void* workspace_dev, size_t workspace_bytes, void* stream) {
+  if (int rc = check_config("MnbMlpGemm", bits, block_size, a_dtype)) return rc;
+  if (activation != MNB_ACTIVATION_SILU)
+    return fail(MNB_INVALID_ARGUMENT, "MatMulNBitsMlp: activation %d is not supported.", activation);
+  if (M == 0 || N == 0) return MNB_OK;
+  if (K == 0) return fail(MNB_INVALID_ARGUMENT, "MnbMlpGemm: K must be positive");
+  if (!a_dev || !packed_dev || !y_dev) return fail(MNB_INVALID_ARGUMENT, "MnbMlpGemm: A, the packed weights and Y must not be NULL");
+  if (ldc < N) return fail(MNB_INVALID_ARGUMENT, "MnbMlpGemm: ldc (%zu) < N (%zu)", ldc, N);
+  const MnbFusedLayout F = mnb_make_fused_layout(kMnbFusedMlp, (int64_t)N, 0, (int64_t)K, bits, block_size, a_dtype);
+  MnbEpilogue epi{};
+  epi.kind = kMnbFusedMlp;
+  epi.n[0] = (int64_t)N;
+  epi.out[0] = y_dev;
+  epi.ld[0] = (int64_t)ldc;
+  return fused_gemm("MnbMlpGemm", F, M, a_dev, lda, norm, packed_dev, epi, workspace_dev, workspace_bytes,
+                    (hipStream_t)stream);
+}
+
+size_t MnbQkvPackSize(size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype) {
+  if (!supported(bits, block_size, a_dtype) || Nq == 0 || Nkv == 0 || K == 0) return 0;
+  return (size_t)mnb_make_fused_layout(kMnbFusedQkv, (int64_t)Nq, (int64_t)Nkv, (int64_t)K, bits, block_size, a_dtype)
+      .total_bytes;
+}
+
+int MnbQkvPack(size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype, const void* q_b_dev,
+               const void* q_scales_dev, const void* q_bias_dev, const void* k_b_dev, const void* k_scales_dev,
+               const void* k_bias_dev, const void* v_b_dev, const void* v_scales_dev, const void* v_bias_dev,
+               void* packed_dev, void* stream) {
+  if (int rc = check_config("MnbQkvPack", bits, block_size, a_dtype)) return rc;
+  if (Nq == 0 || Nkv == 0 || K == 0) return MNB_OK;
+  if (!q_b_dev || !q_scales_dev || !k_b_dev || !k_scales_dev || !v_b_dev || !v_scales_dev || !packed_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbQkvPack: B and scales of the three projections and the packed buffer must not be NULL");
+  if (reinterpret_cast<uintptr_t>(packed_dev) % 256 != 0)
+    return fail(MNB_INVALID_ARGUMENT, "MnbQkvPack: the packed buffer must be 256-byte aligned");
+  const MnbFusedLayout F =
+      mnb_make_fused_layout(kMnbFusedQkv, (int64_t)Nq, (int64_t)Nkv, (int64_t)K, bits, block_size, a_dtype);
+  const void* B[3] = {q_b_dev, k_b_dev, v_b_dev};
+  const void* S[3] = {q_scales_dev, k_scales_dev, v_scales_dev};
+  const void* bias[3] = {q_bias_dev, k_bias_dev, v_bias_dev};
+  hipError_t e = mnb_launch_pack_fused(F, B, S, bias, packed_dev, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbQkvPack");
+}
+
+size_t MnbQkvWorkspaceSize(size_t M, size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype,
+                           int has_norm) {
+  if (!supported(bits, block_size, a_dtype) || Nq == 0 || Nkv == 0 || K == 0 || M == 0) return 0;
+  const MnbFusedLayout F =
+      mnb_make_fused_layout(kMnbFusedQkv, (int64_t)Nq, (int64_t)Nkv, (int64_t)K, bits, block_size, a_dtype);
+  return fused_workspace(F, M, has_norm).total();
+}
+
+int MnbQkvGemm(size_t M, size_t Nq, size_t Nkv, size_t K, int bits, int block_size, int a_dtype, const void* a_dev,
+               size_t lda, const MnbNormPrologue* norm, const void* packed_dev, void* q_dev, size_t ldq, void* k_dev,
+               size_t ldk, void* v_dev, size_t ldv, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  if (int rc = check_config("MnbQkvGemm", bits, block_size, a_dtype)) return rc;
+  if (M == 0) return MNB_OK;
+  if (Nq == 0 || Nkv == 0 || K == 0) return fail(MNB_INVALID_ARGUMENT, "MnbQkvGemm: Nq, Nkv and K must be positive");
+  if (!a_dev || !packed_dev || !q_dev || !k_dev || !v_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbQkvGemm: A, the packed weights and the three outputs must not be NULL");
+  if (ldq < Nq || ldk < Nkv || ldv < Nkv)
+    return fail(MNB_INVALID_ARGUMENT, "MnbQkvGemm: an output pitch is smaller than its width");
+  const MnbFusedLayout F =
+      mnb_make_fused_layout(kMnbFusedQkv, (int64_t)Nq, (int64_t)Nkv, (int64_t)K, bits, block_size, a_dtype);
+  MnbEpilogue epi{};
+  epi.kind = kMnbFusedQkv;
+  void* outs[3] = {q_dev, k_dev, v_dev};
+  const size_t lds[3] = {ldq, ldk, ldv};
+  for (int i = 0; i < 3; ++i) {
+    epi.start[i] = F.map.start[i];
+    epi.n[i] = F.map.n[i];
+    epi.out[i] = outs[i];
+    epi.ld[i] = (int64_t)lds[i];
+  }
+  return fused_gemm("MnbQkvGemm", F, M, a_dev, lda, norm, packed_dev, epi, workspace_dev, workspace_bytes,
+                    (hipStream_t)stream);
+}
+
+int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* a_dev, size_t lda, const MnbNormPrologue* norm,
+                           void* a_norm_dev, void* stream) {
+  if (a_dtype != MNB_DTYPE_FLOAT && a_dtype != MNB_DTYPE_FLOAT16)
+    return fail(MNB_NOT_IMPLEMENTED, "MnbSimplifiedLayerNorm: element type %d has no MI355X kernel", a_dtype);
+  if (M == 0 || K == 0) return MNB_OK;
+  if (!norm || !norm->norm_scale_dev || !a_dev || !a_norm_dev)
+    return fail(MNB_INVALID_ARGUMENT, "MnbSimplifiedLayerNorm: A, norm_scale and the output must not be NULL");
+  if (int rc = check_norm("MnbSimplifiedLayerNorm", norm, K)) return rc;
+  if (lda < K) return fail(MNB_INVALID_ARGUMENT, "MnbSimplifiedLayerNorm: lda (%zu) < K (%zu)", lda, K);
+  hipError_t e = run_norm(norm, a_dev, lda, a_norm_dev, M, K, a_dtype, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbSimplifiedLayerNorm");
 }
 
 int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_points_dev, const void* src_dev, int block_size,

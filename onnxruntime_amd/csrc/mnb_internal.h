@@ -4,6 +4,15 @@
 
 #include "mnb_layout.h"
 
+// Destination of a GEMM over several matrices packed as one (mnb_layout.h): kMnbFusedNone writes C / ldc.
+struct MnbEpilogue {
+  int kind;          // kMnbFused*
+  int64_t start[3];  // qkv: first packed column of each output
+  int64_t n[3];      // columns of each output (mlp: n[0])
+  void* out[3];      // qkv: the three outputs; mlp: out[0]
+  int64_t ld[3];
+};
+
 struct MnbGemmArgs {
   MnbLayout L;
   int64_t M;
@@ -15,6 +24,7 @@ struct MnbGemmArgs {
   int64_t ldc;
   void* workspace;
   size_t workspace_bytes;
+  MnbEpilogue epi;  // kind != kMnbFusedNone: C / ldc are unused, bias is indexed by packed column
 };
 
 enum MnbKernelKind {
@@ -31,6 +41,8 @@ const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout& L);
 
 hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
                            hipStream_t s);
+hipError_t mnb_launch_pack_fused(const MnbFusedLayout& F, const void* const* B, const void* const* scales,
+                                 const void* const* bias, void* packed, hipStream_t s);
 hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,
                                         int64_t K, int bits, int bs, int dtype, hipStream_t s);
 hipError_t mnb_launch_quantize(void* B, void* scales, void* zp, const void* src, int64_t K, int64_t N, int64_t ld,
@@ -46,6 +58,17 @@ bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
+
+// kernels around the fused operators (mnb_fused.hip)
+// A (+ skip) -> A_norm = x / sqrt(mean(x^2) + eps) * scale per row; sum_out (optional) = A + skip
+hipError_t mnb_launch_rmsnorm(void* a_norm, void* sum_out, int64_t ld_sum, const void* A, int64_t lda, const void* skip,
+                              int64_t ld_skip, int64_t skip_rows, const void* scale, float epsilon, int64_t M, int64_t K,
+                              int dtype, hipStream_t s);
+// tmp[M][Np] (plain GEMM over the packed matrix, bias included) -> the operator's outputs
+hipError_t mnb_launch_fused_finish(const MnbEpilogue& epi, const void* tmp, int64_t ld_tmp, int64_t M, int dtype,
+                                   hipStream_t s);
+// true when the kernel mnb_select_kernel picks writes the fused outputs itself
+bool mnb_kernel_has_fused_epilogue(MnbKernelKind k);
 
 // machine ceilings (mnb_probe.hip); diagnostics, synchronous
 hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s);

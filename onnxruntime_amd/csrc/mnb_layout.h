@@ -70,3 +70,75 @@ MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dty
   L.total_bytes = mnb_round_up(L.meta_off + L.KBp * L.Npad * L.meta_bytes, 256);
   return L;
 }
+
+// ---- several weight matrices behind one activation (MatMulNBitsMlp, MatMulNBitsQkv; contrib_defs.cc:3851-4090) ----
+// The matrices share K, bits and block size and have no zero points.  They are packed as ONE matrix of Np columns so
+// that a single launch streams all of them:
+//   kMnbFusedMlp  gate and up interleaved by 16-column tiles: packed tile 2u = gate columns [16u, 16u+16), packed
+//                 tile 2u+1 = the same columns of up.  A workgroup that owns an even number of adjacent tiles holds
+//                 both operands of  silu(gate) * up  for its columns.
+//   kMnbFusedQkv  Q, K and V side by side, each segment padded to a multiple of 16 columns, so that a 16-column tile
+//                 never straddles two outputs.
+// Behind the packed matrix the buffer holds one bias value per packed column (zero where the operator has no bias).
+constexpr int kMnbFusedNone = 0;
+constexpr int kMnbFusedMlp = 1;
+constexpr int kMnbFusedQkv = 2;
+
+struct MnbColMap {
+  int kind;          // kMnbFused*
+  int nsrc;          // matrices: 2 (mlp) or 3 (qkv)
+  int64_t n[3];      // columns of each matrix
+  int64_t start[3];  // qkv: first packed column of each segment
+  int64_t Np;        // packed columns
+};
+
+struct MnbFusedLayout {
+  MnbLayout L;  // the packed matrix: N = Np
+  MnbColMap map;
+  int64_t bias_off;
+  int64_t total_bytes;
+};
+
+// packed column -> (matrix, column); false for padding columns
+MNB_HD bool mnb_map_col(const MnbColMap& m, int64_t np, int* src, int64_t* col) {
+  if (m.kind == kMnbFusedMlp) {
+    const int64_t tile = np >> 4;
+    *src = (int)(tile & 1);
+    *col = (tile >> 1) * 16 + (np & 15);
+    return np < m.Np && *col < m.n[0];
+  }
+  if (m.kind == kMnbFusedQkv) {
+    const int s = np >= m.start[2] ? 2 : np >= m.start[1] ? 1 : 0;
+    *src = s;
+    *col = np - m.start[s];
+    return np < m.Np && *col < m.n[s];
+  }
+  *src = 0;
+  *col = np;
+  return np < m.n[0];
+}
+
+MNB_HD MnbFusedLayout mnb_make_fused_layout(int kind, int64_t n0, int64_t n1, int64_t K, int bits, int bs, int dtype) {
+  MnbFusedLayout F;
+  MnbColMap& m = F.map;
+  m.kind = kind;
+  if (kind == kMnbFusedMlp) {  // n0 = N of gate and up
+    m.nsrc = 2;
+    m.n[0] = m.n[1] = n0;
+    m.n[2] = 0;
+    m.start[0] = m.start[1] = m.start[2] = 0;
+    m.Np = 2 * mnb_round_up(n0, 16);
+  } else {  // n0 = Nq, n1 = Nkv
+    m.nsrc = 3;
+    m.n[0] = n0;
+    m.n[1] = m.n[2] = n1;
+    m.start[0] = 0;
+    m.start[1] = mnb_round_up(n0, 16);
+    m.start[2] = m.start[1] + mnb_round_up(n1, 16);
+    m.Np = m.start[2] + mnb_round_up(n1, 16);
+  }
+  F.L = mnb_make_layout(m.Np, K, bits, bs, dtype, 0);
+  F.bias_off = F.L.total_bytes;
+  F.total_bytes = F.bias_off + mnb_round_up(m.Np * (dtype == kMnbDtypeFloat16 ? 2 : 4), 256);
+  return F;
+}

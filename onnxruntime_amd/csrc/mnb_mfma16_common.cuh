@@ -7,6 +7,16 @@
 
 namespace {
 
+// Where the finished tiles go (wave-uniform, evaluated once per workgroup at the very end).
+struct EpiParams {
+  int kind;                // kMnbFusedNone: C[m * ldc + n];  kMnbFusedMlp: silu(gate) * up;  kMnbFusedQkv: three outputs
+  int start1, start2;      // qkv: first packed column of the second and third output
+  int n0, n1, n2;          // columns of each output (mlp: n0)
+  _Float16* out1;          // qkv: second and third output (the first is C / ldc)
+  _Float16* out2;
+  int64_t ld1, ld2;
+};
+
 struct SkinnyParams {
   const _Float16* A;
   const uint4* W;
@@ -21,6 +31,7 @@ struct SkinnyParams {
   int mtr;          // rows of A staged (power of two >= M, <= 16)
   int a_vec_ok;     // A allows 16-byte loads
   uint32_t uc[4];   // UnpackConsts
+  EpiParams epi;
 };
 
 constexpr int kLdsPad = 8;  // halves of padding per staged row
@@ -148,6 +159,57 @@ __device__ __forceinline__ BConst make_bconst() {
   bc.off = h8_t{lo, lo, hi, hi, lo, lo, hi, hi};
   bc.one = h8_t{m1, m1, m1, m1, m1, m1, m1, m1};
   return bc;
+}
+
+// Sum the per-wavefront partial tiles (red[(w * T * 4 + t * 4 + r) * 64 + lane], written by NW wavefronts) in
+// wavefront order and write the result.  Lane l, register r of tile t is row m_base + 4 * (l / 16) + r, packed column
+// n0 + 16 t + l % 16.  bias is indexed by packed column.
+template <int T, int NW>
+__device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, const float* red, int m_base,
+                                                       int64_t n0) {
+  auto total = [&](int tr, int l) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * T * 4 + tr) * 64 + l];
+    return sum;
+  };
+  if (p.epi.kind == kMnbFusedMlp) {
+    // adjacent tiles (2u, 2u + 1) are gate and up of output columns [n0 / 2 + 16 u, +16)
+    if constexpr (T >= 2) {
+      for (int i = threadIdx.x; i < (T / 2) * 4 * 64; i += NW * 64) {
+        const int l = i & 63, ur = i >> 6;
+        const int u = ur >> 2, r = ur & 3;
+        const int m = m_base + 4 * (l >> 4) + r;
+        const int64_t n_out = (n0 >> 1) + u * 16 + (l & 15);
+        if (m >= p.M || n_out >= p.epi.n0) continue;
+        const int64_t ng = n0 + u * 32 + (l & 15);
+        const float g = total((2 * u) * 4 + r, l) + (float)p.bias[ng];
+        const float up = total((2 * u + 1) * 4 + r, l) + (float)p.bias[ng + 16];
+        p.C[(int64_t)m * p.ldc + n_out] = (_Float16)(g / (1.0f + __expf(-g)) * up);
+      }
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < T * 4 * 64; i += NW * 64) {
+    const int l = i & 63, tr = i >> 6;
+    const int t = tr >> 2, r = tr & 3;
+    const int m = m_base + 4 * (l >> 4) + r;
+    const int64_t n = n0 + t * 16 + (l & 15);
+    if (m >= p.M || n >= p.N) continue;
+    float sum = total(tr, l);
+    if (p.bias) sum += (float)p.bias[n];
+    if (p.epi.kind == kMnbFusedQkv) {
+      if (n >= p.epi.start2) {
+        if (n - p.epi.start2 < p.epi.n2) p.epi.out2[(int64_t)m * p.epi.ld2 + (n - p.epi.start2)] = (_Float16)sum;
+      } else if (n >= p.epi.start1) {
+        if (n - p.epi.start1 < p.epi.n1) p.epi.out1[(int64_t)m * p.epi.ld1 + (n - p.epi.start1)] = (_Float16)sum;
+      } else if (n < p.epi.n0) {
+        p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
+      }
+    } else {
+      p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
+    }
+  }
 }
 
 }  // namespace

@@ -175,18 +175,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[(wave * T * 4 + t * 4 + r) * 64 + lane] = y[mt][t][r];
     __syncthreads();
-    for (int i = threadIdx.x; i < T * 4 * 64; i += NW * 64) {
-      const int l = i & 63, tr = i >> 6;
-      const int t = tr >> 2, r = tr & 3;
-      const int m = m0 + mt * 16 + 4 * (l >> 4) + r;
-      const int64_t n = n0 + t * 16 + (l & 15);
-      if (m >= p.M || n >= p.N) continue;
-      float sum = 0.f;
-#pragma unroll
-      for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * T * 4 + tr) * 64 + l];
-      if (p.bias) sum += (float)p.bias[n];
-      p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
-    }
+    reduce_and_store_tiles<T, NW>(p, red, m0 + mt * 16, n0);
   }
 }
 
@@ -194,7 +183,7 @@ struct MidPlan {
   int t, mt, nw;
 };
 
-MidPlan mid_plan(const MnbLayout& L, int64_t M) {
+MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   MidPlan pl;
   const int CK = 4 * L.group_k;
   const int chunks = (int)((L.K + CK - 1) / CK);
@@ -213,6 +202,7 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M) {
       pl.nw = nw;
     }
   }
+  if (pl.t < min_t) pl.t = min_t;  // gate/up pairs live in one workgroup
   return pl;
 }
 
@@ -264,7 +254,7 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
 
 hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
-  const MidPlan pl = mid_plan(L, a.M);
+  const MidPlan pl = mid_plan(L, a.M, a.epi.kind == kMnbFusedMlp ? 2 : 1);
   const int CK = 4 * L.group_k;
   MidParams mp{};
   SkinnyParams& p = mp.s;
@@ -281,6 +271,20 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   p.K = (int)L.K;
   p.bs_shift = log2i(L.bs);
   p.chunks = (int)((L.K + CK - 1) / CK);
+  p.epi.kind = a.epi.kind;
+  if (a.epi.kind != kMnbFusedNone) {
+    p.C = reinterpret_cast<_Float16*>(a.epi.out[0]);
+    p.ldc = a.epi.ld[0];
+    p.epi.start1 = (int)a.epi.start[1];
+    p.epi.start2 = (int)a.epi.start[2];
+    p.epi.n0 = (int)a.epi.n[0];
+    p.epi.n1 = (int)a.epi.n[1];
+    p.epi.n2 = (int)a.epi.n[2];
+    p.epi.out1 = reinterpret_cast<_Float16*>(a.epi.out[1]);
+    p.epi.out2 = reinterpret_cast<_Float16*>(a.epi.out[2]);
+    p.epi.ld1 = a.epi.ld[1];
+    p.epi.ld2 = a.epi.ld[2];
+  }
   p.uc[0] = 0x000F000Fu;
   p.uc[1] = 0x00F000F0u;
   p.uc[2] = 0x64006400u;

@@ -10,17 +10,26 @@
 // ------------------------------------------------------------------------------------------------ pack weights
 // One thread per (column n, group g).  Consecutive threads take consecutive groups of one column, so the reads of
 // the canonical matrix are contiguous; the 16-byte writes are strided by Npad.
+// The canonical operands of up to three matrices that share one packed buffer (one matrix for MatMulNBits itself).
+struct MnbPackSrc {
+  const uint8_t* B[3];
+  const void* scales[3];
+  const void* bias[3];
+  MnbColMap map;  // packed column -> (matrix, column)
+};
+
 template <int BITS>
-__global__ void __launch_bounds__(256) mnb_pack_weights_kernel(const uint8_t* __restrict__ B, uint4* __restrict__ W,
-                                                               MnbLayout L) {
+__global__ void __launch_bounds__(256) mnb_pack_weights_kernel(MnbPackSrc S, uint4* __restrict__ W, MnbLayout L) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t n = idx / L.KG;
   const int64_t g = idx % L.KG;
   if (n >= L.Npad) return;
   uint32_t w[4] = {0, 0, 0, 0};
   const int64_t col_bytes = L.k_blocks * L.bs * BITS / 8;  // bytes of one canonical column
-  if (n < L.N) {
-    const uint8_t* src = B + n * col_bytes + g * 16;
+  int m;
+  int64_t col;
+  if (mnb_map_col(S.map, n, &m, &col)) {
+    const uint8_t* src = S.B[m] + col * col_bytes + g * 16;
     for (int i = 0; i < 4; ++i) {
       uint32_t v = 0;
       for (int b = 0; b < 4; ++b) {
@@ -47,24 +56,25 @@ __global__ void __launch_bounds__(256) mnb_pack_weights_kernel(const uint8_t* __
 // ------------------------------------------------------------------------------------------------ pack meta
 // One thread per (block kb, column n).
 template <typename T, int BITS, bool HAS_ZP>
-__global__ void __launch_bounds__(256) mnb_pack_meta_kernel(const T* __restrict__ scales,
-                                                            const uint8_t* __restrict__ zp, uint8_t* __restrict__ meta,
-                                                            MnbLayout L) {
+__global__ void __launch_bounds__(256) mnb_pack_meta_kernel(MnbPackSrc S, const uint8_t* __restrict__ zp,
+                                                            uint8_t* __restrict__ meta, MnbLayout L) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= L.KBp * L.Npad) return;
   const int64_t kb = idx / L.Npad;
   const int64_t n = idx % L.Npad;
   const int64_t dst = kb * L.Npad + mnb_meta_col(n);
-  const bool valid = n < L.N && kb < L.k_blocks;
-  T s = valid ? scales[n * L.k_blocks + kb] : (T)0;
+  int m;
+  int64_t col;
+  const bool valid = mnb_map_col(S.map, n, &m, &col) && kb < L.k_blocks;
+  T s = valid ? reinterpret_cast<const T*>(S.scales[m])[col * L.k_blocks + kb] : (T)0;
   int z = 0;
-  if constexpr (HAS_ZP) {
+  if constexpr (HAS_ZP) {  // zero points exist only for a single matrix: col == n
     if (valid) {
       const int64_t row = (L.k_blocks * BITS + 7) / 8;
       if constexpr (BITS == 8) {
-        z = zp[n * row + kb];
+        z = zp[col * row + kb];
       } else {
-        z = (zp[n * row + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
+        z = (zp[col * row + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
       }
     }
   }
@@ -84,6 +94,18 @@ __global__ void __launch_bounds__(256) mnb_pack_meta_kernel(const T* __restrict_
       reinterpret_cast<float*>(meta)[dst] = s;
     }
   }
+}
+
+// One bias value per packed column (zero for padding columns and absent biases).
+template <typename T>
+__global__ void __launch_bounds__(256) mnb_pack_bias_kernel(MnbPackSrc S, T* __restrict__ dst) {
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= S.map.Np) return;
+  int m;
+  int64_t col;
+  T v = (T)0;
+  if (mnb_map_col(S.map, n, &m, &col) && S.bias[m]) v = reinterpret_cast<const T*>(S.bias[m])[col];
+  dst[n] = v;
 }
 
 // ------------------------------------------------------------------------------------------------ dequantise
@@ -140,37 +162,59 @@ __global__ void __launch_bounds__(256) mnb_dequant_packed_kernel(T* __restrict__
 
 // ------------------------------------------------------------------------------------------------ launchers
 template <typename T>
-static hipError_t pack_t(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
-                         hipStream_t s) {
+static hipError_t pack_t(const MnbLayout& L, const MnbPackSrc& S, const void* zp, void* packed, hipStream_t s) {
   uint4* W = reinterpret_cast<uint4*>(packed);
   uint8_t* meta = reinterpret_cast<uint8_t*>(packed) + L.meta_off;
   const int64_t wn = L.Npad * L.KG;
   const int64_t mn = L.KBp * L.Npad;
   dim3 blk(256);
   if (L.bits == 4) {
-    mnb_pack_weights_kernel<4><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>((const uint8_t*)B, W, L);
+    mnb_pack_weights_kernel<4><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>(S, W, L);
     if (zp)
-      mnb_pack_meta_kernel<T, 4, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales,
-                                                                                         (const uint8_t*)zp, meta, L);
+      mnb_pack_meta_kernel<T, 4, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, (const uint8_t*)zp, meta, L);
     else
-      mnb_pack_meta_kernel<T, 4, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales, nullptr,
-                                                                                          meta, L);
+      mnb_pack_meta_kernel<T, 4, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, nullptr, meta, L);
   } else {
-    mnb_pack_weights_kernel<8><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>((const uint8_t*)B, W, L);
+    mnb_pack_weights_kernel<8><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>(S, W, L);
     if (zp)
-      mnb_pack_meta_kernel<T, 8, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales,
-                                                                                         (const uint8_t*)zp, meta, L);
+      mnb_pack_meta_kernel<T, 8, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, (const uint8_t*)zp, meta, L);
     else
-      mnb_pack_meta_kernel<T, 8, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>((const T*)scales, nullptr,
-                                                                                          meta, L);
+      mnb_pack_meta_kernel<T, 8, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, nullptr, meta, L);
   }
   return hipGetLastError();
 }
 
 hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
                            hipStream_t s) {
-  return L.dtype == kMnbDtypeFloat16 ? pack_t<_Float16>(L, B, scales, zp, packed, s)
-                                     : pack_t<float>(L, B, scales, zp, packed, s);
+  MnbPackSrc S{};
+  S.B[0] = reinterpret_cast<const uint8_t*>(B);
+  S.scales[0] = scales;
+  S.map.kind = kMnbFusedNone;
+  S.map.nsrc = 1;
+  S.map.n[0] = L.N;
+  S.map.Np = L.N;
+  return L.dtype == kMnbDtypeFloat16 ? pack_t<_Float16>(L, S, zp, packed, s) : pack_t<float>(L, S, zp, packed, s);
+}
+
+hipError_t mnb_launch_pack_fused(const MnbFusedLayout& F, const void* const* B, const void* const* scales,
+                                 const void* const* bias, void* packed, hipStream_t s) {
+  MnbPackSrc S{};
+  for (int i = 0; i < F.map.nsrc; ++i) {
+    S.B[i] = reinterpret_cast<const uint8_t*>(B[i]);
+    S.scales[i] = scales[i];
+    S.bias[i] = bias[i];
+  }
+  S.map = F.map;
+  hipError_t e = F.L.dtype == kMnbDtypeFloat16 ? pack_t<_Float16>(F.L, S, nullptr, packed, s)
+                                               : pack_t<float>(F.L, S, nullptr, packed, s);
+  if (e != hipSuccess) return e;
+  uint8_t* bias_dst = reinterpret_cast<uint8_t*>(packed) + F.bias_off;
+  const dim3 grid((unsigned)((F.map.Np + 255) / 256)), blk(256);
+  if (F.L.dtype == kMnbDtypeFloat16)
+    mnb_pack_bias_kernel<_Float16><<<grid, blk, 0, s>>>(S, reinterpret_cast<_Float16*>(bias_dst));
+  else
+    mnb_pack_bias_kernel<float><<<grid, blk, 0, s>>>(S, reinterpret_cast<float*>(bias_dst));
+  return hipGetLastError();
 }
 
 hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,

@@ -121,30 +121,13 @@ template <int T, int NW>
 __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* red, const f4_t* y, int wave, int lane,
                                                 int64_t n0) {
   const int kq = lane >> 4;
-  if constexpr (NW > 1) {
 #pragma unroll
-    for (int t = 0; t < T; ++t)
+  for (int t = 0; t < T; ++t)
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (4 * kq + r < p.M) red[(wave * T * 4 + t * 4 + r) * 64 + lane] = y[t][r];
-    __syncthreads();
-  }
-  for (int i = threadIdx.x; i < T * 4 * 64; i += NW * 64) {
-    const int l = i & 63, tr = i >> 6;
-    const int t = tr >> 2, r = tr & 3;
-    const int m = 4 * (l >> 4) + r;
-    const int64_t n = n0 + t * 16 + (l & 15);
-    if (m >= p.M || n >= p.N) continue;
-    float sum = 0.f;
-    if constexpr (NW > 1) {
-#pragma unroll
-      for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * T * 4 + tr) * 64 + l];
-    } else {
-      sum = y[t][r];
-    }
-    if (p.bias) sum += (float)p.bias[n];
-    p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
-  }
+    for (int r = 0; r < 4; ++r)
+      if (4 * kq + r < p.M) red[(wave * T * 4 + t * 4 + r) * 64 + lane] = y[t][r];
+  __syncthreads();
+  reduce_and_store_tiles<T, NW>(p, red, 0, n0);
 }
 
 // ---- direct variant: A operands straight from global memory (16-byte aligned rows), no barrier before the end ----
@@ -282,7 +265,7 @@ int pow2_ceil(int v) {
   return r;
 }
 
-SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct) {
+SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   SkinnyPlan pl;
   const int GK = L.group_k, CK = 4 * GK;
   const int chunks = (int)((L.K + CK - 1) / CK);
@@ -300,6 +283,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct) {
       pl.nw = nw;
     }
   }
+  if (pl.t < min_t) pl.t = min_t;  // gate/up pairs live in one workgroup
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
   pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
@@ -370,7 +354,7 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
   // direct variant: 16-byte loads of whole chunks of A
   const bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
-  SkinnyPlan pl = skinny_plan(L, a.M, a_vec_ok);
+  SkinnyPlan pl = skinny_plan(L, a.M, a_vec_ok, a.epi.kind == kMnbFusedMlp ? 2 : 1);
   SkinnyParams p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
   p.W = reinterpret_cast<const uint4*>(a.packed);
@@ -389,6 +373,20 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   p.phase_chunks = pl.phase_chunks;
   p.mtr = pl.mtr;
   p.a_vec_ok = a_vec_ok;
+  p.epi.kind = a.epi.kind;
+  if (a.epi.kind != kMnbFusedNone) {
+    p.C = reinterpret_cast<_Float16*>(a.epi.out[0]);
+    p.ldc = a.epi.ld[0];
+    p.epi.start1 = (int)a.epi.start[1];
+    p.epi.start2 = (int)a.epi.start[2];
+    p.epi.n0 = (int)a.epi.n[0];
+    p.epi.n1 = (int)a.epi.n[1];
+    p.epi.n2 = (int)a.epi.n[2];
+    p.epi.out1 = reinterpret_cast<_Float16*>(a.epi.out[1]);
+    p.epi.out2 = reinterpret_cast<_Float16*>(a.epi.out[2]);
+    p.epi.ld1 = a.epi.ld[1];
+    p.epi.ld2 = a.epi.ld[2];
+  }
   p.uc[0] = 0x000F000Fu;
   p.uc[1] = 0x00F000F0u;
   p.uc[2] = 0x64006400u;

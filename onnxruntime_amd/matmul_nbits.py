@@ -195,6 +195,200 @@ class MatMulNBits:
         return w
 
 
+class _FusedProjections:
+    """Shared host side of MatMulNBitsMlp / MatMulNBitsQkv: attribute checks, the optional
+    (Skip)SimplifiedLayerNormalization prologue and the workspace."""
+
+    OP = ""
+
+    def __init__(self, K: int, bits: int, block_size: int, accuracy_level: int, epsilon: float, dtype: torch.dtype):
+        if bits not in (2, 4, 8):
+            raise MnbError(_lib.INVALID_ARGUMENT, "Only 2b, 4b and 8b quantization is supported for MatMulNBits op, "
+                                                  "additional bits support is planned.")
+        if block_size not in (16, 32, 64, 128, 256):
+            raise MnbError(_lib.INVALID_ARGUMENT, "Only block sizes 16, 32, 64, 128, and 256 are supported for "
+                                                  f"MatMulNBits op, got: {block_size}")
+        self.K, self.bits, self.block_size = int(K), int(bits), int(block_size)
+        self.accuracy_level, self.epsilon, self.dtype = int(accuracy_level), float(epsilon), dtype
+        self.k_blocks = (self.K + self.block_size - 1) // self.block_size
+        self.blob_size = self.block_size * self.bits // 8
+        self.lib = _lib.load()
+        self.supported = (dtype in (torch.float16, torch.float32) and bits in (4, 8)
+                          and bool(self.lib.MnbIsAvailable(bits, block_size, _DTYPES[dtype])))
+        self.packed: Optional[torch.Tensor] = None
+        self._workspace = {}
+
+    def _check_projection(self, name: str, n: int, b, scales, bias) -> None:
+        kb, blob = self.k_blocks, self.blob_size
+        check_inputs(tuple(b.shape), tuple(scales.shape), None, None, None if bias is None else tuple(bias.shape),
+                     n, self.K, self.block_size, self.bits, scales_dtype=self.dtype)
+        if scales.dtype != self.dtype or (bias is not None and bias.dtype != self.dtype):
+            raise MnbError(_lib.INVALID_ARGUMENT, f"{self.OP}: {name} scales and bias must have the type of A")
+
+    _get_workspace = MatMulNBits._get_workspace
+
+    def _prologue(self, a2: torch.Tensor, skip, norm_scale, want_sum: bool):
+        """Returns (MnbNormPrologue or None, skip-sum tensor or None, tensors to keep alive)."""
+        if norm_scale is None:
+            if skip is not None:
+                raise MnbError(_lib.INVALID_ARGUMENT, "norm_scale input must be present when skip input is provided")
+            return None, None, ()
+        if tuple(norm_scale.shape) != (self.K,):
+            raise MnbError(_lib.INVALID_ARGUMENT, f"norm_scale shape must be [K] where K = {self.K}")
+        M = a2.shape[0]
+        n = _lib.MnbNormPrologue()
+        n.norm_scale_dev = norm_scale.contiguous().data_ptr()
+        n.epsilon = self.epsilon
+        keep = [norm_scale]
+        sm = None
+        if skip is not None:
+            if skip.shape[-1] != self.K or skip.numel() == 0 or a2.numel() % skip.numel() != 0:
+                raise MnbError(_lib.INVALID_ARGUMENT, f"{self.OP}: skip must broadcast over the rows of A")
+            s2 = skip.reshape(-1, self.K).contiguous()
+            n.skip_dev, n.ld_skip, n.skip_rows = s2.data_ptr(), self.K, s2.shape[0]
+            keep.append(s2)
+            if want_sum:
+                sm = torch.empty(M, self.K, dtype=self.dtype, device=a2.device)
+                n.skip_sum_dev, n.ld_skip_sum = sm.data_ptr(), self.K
+        elif want_sum:
+            raise MnbError(_lib.INVALID_ARGUMENT,
+                           "skip input must be present when input_skip_bias_sum output is requested")
+        return n, sm, tuple(keep)
+
+    def _rows(self, a: torch.Tensor) -> torch.Tensor:
+        if not self.supported:
+            raise MnbError(_lib.NOT_IMPLEMENTED, f"this {self.OP} configuration has no MI355X kernel")
+        if self.packed is None:
+            raise MnbError(_lib.INVALID_ARGUMENT, f"{self.OP}: PrePack has not run")
+        if a.dtype != self.dtype:
+            raise MnbError(_lib.INVALID_ARGUMENT, f"A has dtype {a.dtype}, the node was built for {self.dtype}")
+        if a.shape[-1] != self.K:
+            raise MnbError(_lib.INVALID_ARGUMENT,
+                           f"{self.OP}: the last dimension of A ({a.shape[-1]}) must equal K ({self.K})")
+        a2 = a.reshape(-1, self.K)
+        return a2 if a2.stride(-1) == 1 else a2.contiguous()
+
+
+class MatMulNBitsMlp(_FusedProjections):
+    """com.microsoft::MatMulNBitsMlp (contrib_defs.cc:3851-3975) bound to the MI355X kernels:
+    Y = silu(A' gate^T + gate_bias) * (A' up^T + up_bias), A' = A or its (skip) simplified layer normalisation."""
+
+    OP = "MatMulNBitsMlp"
+
+    def __init__(self, K: int, N: int, bits: int = 4, block_size: int = 32, accuracy_level: int = 0,
+                 activation: str = "silu", epsilon: float = 1e-5, dtype: torch.dtype = torch.float16):
+        super().__init__(K, bits, block_size, accuracy_level, epsilon, dtype)
+        if activation != "silu":  # matmul_nbits_mlp.cc:24-31
+            raise MnbError(_lib.INVALID_ARGUMENT, f"MatMulNBitsMlp: activation '{activation}' is not supported.")
+        self.N = int(N)
+
+    def PrePack(self, gate_b, gate_scales, gate_bias, up_b, up_scales, up_bias) -> bool:
+        self._check_projection("gate", self.N, gate_b, gate_scales, gate_bias)
+        self._check_projection("up", self.N, up_b, up_scales, up_bias)
+        if not self.supported:
+            return False
+        dt = _DTYPES[self.dtype]
+        size = self.lib.MnbMlpPackSize(self.N, self.K, self.bits, self.block_size, dt)
+        packed = torch.empty(size, dtype=torch.uint8, device=gate_b.device)
+        c = lambda t: None if t is None else t.contiguous()  # noqa: E731
+        ts = [c(gate_b), c(gate_scales), c(gate_bias), c(up_b), c(up_scales), c(up_bias)]
+        _lib.check(self.lib.MnbMlpPack(self.N, self.K, self.bits, self.block_size, dt, *[_ptr(t) for t in ts],
+                                       _ptr(packed), _stream_ptr(gate_b.device)))
+        self.packed = packed
+        return True
+
+    def Compute(self, a: torch.Tensor, skip: Optional[torch.Tensor] = None, norm_scale: Optional[torch.Tensor] = None,
+                want_skip_sum: bool = False):
+        """Returns Y, or (Y, input_skip_bias_sum) when ``want_skip_sum``."""
+        a2 = self._rows(a)
+        lead, M = tuple(a.shape[:-1]), a2.shape[0]
+        y = torch.empty(*lead, self.N, dtype=self.dtype, device=a.device)
+        norm, sm, keep = self._prologue(a2, skip, norm_scale, want_skip_sum)
+        if y.numel():
+            dt = _DTYPES[self.dtype]
+            wsz = self.lib.MnbMlpWorkspaceSize(M, self.N, self.K, self.bits, self.block_size, dt, int(norm is not None))
+            ws = self._get_workspace(a.device, wsz)
+            _lib.check(self.lib.MnbMlpGemm(M, self.N, self.K, self.bits, self.block_size, dt, _ptr(a2),
+                                           a2.stride(0) if M > 1 else self.K,
+                                           None if norm is None else ctypes.byref(norm), _ptr(self.packed), 0,
+                                           _ptr(y), self.N, _ptr(ws), wsz, _stream_ptr(a.device)))
+        del keep
+        return (y, sm.view(*lead, self.K)) if want_skip_sum else y
+
+
+class MatMulNBitsQkv(_FusedProjections):
+    """com.microsoft::MatMulNBitsQkv (contrib_defs.cc:3977-4090): Q, K, V = A' x {q, k, v}^T + bias."""
+
+    OP = "MatMulNBitsQkv"
+
+    def __init__(self, K: int, Nq: int, Nkv: int, bits: int = 4, block_size: int = 32, accuracy_level: int = 0,
+                 epsilon: float = 1e-6, dtype: torch.dtype = torch.float16):
+        super().__init__(K, bits, block_size, accuracy_level, epsilon, dtype)
+        self.Nq, self.Nkv = int(Nq), int(Nkv)
+
+    def PrePack(self, q_b, q_scales, q_bias, k_b, k_scales, k_bias, v_b, v_scales, v_bias) -> bool:
+        self._check_projection("q", self.Nq, q_b, q_scales, q_bias)
+        self._check_projection("k", self.Nkv, k_b, k_scales, k_bias)
+        self._check_projection("v", self.Nkv, v_b, v_scales, v_bias)
+        if not self.supported:
+            return False
+        dt = _DTYPES[self.dtype]
+        size = self.lib.MnbQkvPackSize(self.Nq, self.Nkv, self.K, self.bits, self.block_size, dt)
+        packed = torch.empty(size, dtype=torch.uint8, device=q_b.device)
+        ts = [None if t is None else t.contiguous()
+              for t in (q_b, q_scales, q_bias, k_b, k_scales, k_bias, v_b, v_scales, v_bias)]
+        _lib.check(self.lib.MnbQkvPack(self.Nq, self.Nkv, self.K, self.bits, self.block_size, dt,
+                                       *[_ptr(t) for t in ts], _ptr(packed), _stream_ptr(q_b.device)))
+        self.packed = packed
+        return True
+
+    def Compute(self, a: torch.Tensor, skip: Optional[torch.Tensor] = None, norm_scale: Optional[torch.Tensor] = None,
+                want_skip_sum: bool = False):
+        """Returns (Q, K, V) or (Q, K, V, input_skip_bias_sum).  The operator requires norm_scale; it is optional
+        here so that the projections can be used on their own."""
+        a2 = self._rows(a)
+        lead, M = tuple(a.shape[:-1]), a2.shape[0]
+        outs = [torch.empty(*lead, n, dtype=self.dtype, device=a.device) for n in (self.Nq, self.Nkv, self.Nkv)]
+        norm, sm, keep = self._prologue(a2, skip, norm_scale, want_skip_sum)
+        if M:
+            dt = _DTYPES[self.dtype]
+            wsz = self.lib.MnbQkvWorkspaceSize(M, self.Nq, self.Nkv, self.K, self.bits, self.block_size, dt,
+                                               int(norm is not None))
+            ws = self._get_workspace(a.device, wsz)
+            _lib.check(self.lib.MnbQkvGemm(M, self.Nq, self.Nkv, self.K, self.bits, self.block_size, dt, _ptr(a2),
+                                           a2.stride(0) if M > 1 else self.K,
+                                           None if norm is None else ctypes.byref(norm), _ptr(self.packed),
+                                           _ptr(outs[0]), self.Nq, _ptr(outs[1]), self.Nkv, _ptr(outs[2]), self.Nkv,
+                                           _ptr(ws), wsz, _stream_ptr(a.device)))
+        del keep
+        return tuple(outs) + ((sm.view(*lead, self.K),) if want_skip_sum else ())
+
+
+def simplified_layer_norm(a: torch.Tensor, norm_scale: torch.Tensor, epsilon: float,
+                          skip: Optional[torch.Tensor] = None, want_skip_sum: bool = False):
+    """(Skip)SimplifiedLayerNormalization over the last axis on the device (the prologue of the fused operators)."""
+    lib = _lib.load()
+    K = a.shape[-1]
+    a2 = a.reshape(-1, K)
+    a2 = a2 if a2.stride(-1) == 1 else a2.contiguous()
+    M = a2.shape[0]
+    out = torch.empty(M, K, dtype=a.dtype, device=a.device)
+    n = _lib.MnbNormPrologue()
+    g = norm_scale.contiguous()
+    n.norm_scale_dev, n.epsilon = g.data_ptr(), float(epsilon)
+    sm = None
+    if skip is not None:
+        s2 = skip.reshape(-1, K).contiguous()
+        n.skip_dev, n.ld_skip, n.skip_rows = s2.data_ptr(), K, s2.shape[0]
+        if want_skip_sum:
+            sm = torch.empty(M, K, dtype=a.dtype, device=a.device)
+            n.skip_sum_dev, n.ld_skip_sum = sm.data_ptr(), K
+    _lib.check(lib.MnbSimplifiedLayerNorm(M, K, _DTYPES[a.dtype], _ptr(a2), a2.stride(0) if M > 1 else K,
+                                          ctypes.byref(n), _ptr(out), _stream_ptr(a.device)))
+    out = out.view(a.shape)
+    return (out, sm.view(a.shape)) if want_skip_sum else out
+
+
 def dequantize_blockwise(b: torch.Tensor, scales: torch.Tensor, zero_points: Optional[torch.Tensor], N: int, K: int,
                          bits: int, block_size: int) -> torch.Tensor:
     """MlasDequantizeBlockwise on the device: W [N, K] in the dtype of scales."""

@@ -369,3 +369,66 @@ void mnbo_quantize_f16(uint8_t* B, uint16_t* scales, uint8_t* zp, const uint16_t
   free(src32);
   free(s32);
 }
+
+/* ------------------------------------------------------------------ prologue of the fused projections
+ *
+ * SimplifiedLayerNormalization / SkipSimplifiedLayerNormalization of the activation, the optional first stage of
+ * com.microsoft::MatMulNBitsMlp and MatMulNBitsQkv (onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3851-3877).
+ * Follows the CPU kernel, onnxruntime/contrib_ops/cpu/skip_layer_norm.cc:44-97 (fp32 job; the fp16 job widens
+ * input, skip, gamma and bias to fp32, runs the same arithmetic and narrows both outputs once):
+ *   val = input + skip (+ bias);  sum_out = val;  out = val / sqrt(sum(val^2) / K + epsilon) * gamma
+ * with fp32 accumulation in k order; row m of the input uses skip row m % skip_rows (:56, offset % skip_size).
+ * skip == NULL gives SimplifiedLayerNormalization (onnxruntime/core/providers/cpu/nn/layer_norm_impl.cc:65-73,87-89:
+ * the same formula without the addition).  `bias` exists only so that the reference's own test vector with a bias
+ * (onnxruntime/test/contrib_ops/skiplayernorm_op_test.cc:996-1048) can be replayed; the fused operators have none.
+ * Parity: pinned by that vector and by :954-993 of the same file (tests/test_oracle_fused.py), plus closed forms.
+ */
+void mnbo_skip_simplified_layer_norm_f32(float* out, float* sum_out, const float* input, const float* skip,
+                                         int64_t skip_rows, const float* gamma, const float* bias, float epsilon,
+                                         int64_t M, int64_t K) {
+  for (int64_t m = 0; m < M; ++m) {
+    const float* x = input + m * K;
+    const float* s = skip ? skip + (m % (skip_rows > 0 ? skip_rows : M)) * K : NULL;
+    float* o = out + m * K;
+    float mean_square = 0.0f;
+    for (int64_t h = 0; h < K; ++h) {
+      float val = x[h];
+      if (s) val = val + s[h];
+      if (bias) val = val + bias[h];
+      if (sum_out) sum_out[m * K + h] = val;
+      o[h] = val;
+      float sq = val * val;
+      mean_square = mean_square + sq;
+    }
+    float denom = sqrtf(mean_square / (float)K + epsilon);
+    for (int64_t h = 0; h < K; ++h) {
+      float q = o[h] / denom;
+      o[h] = q * gamma[h];
+    }
+  }
+}
+
+void mnbo_skip_simplified_layer_norm_f16(uint16_t* out, uint16_t* sum_out, const uint16_t* input, const uint16_t* skip,
+                                         int64_t skip_rows, const uint16_t* gamma, const uint16_t* bias, float epsilon,
+                                         int64_t M, int64_t K) {
+  int64_t srows = skip_rows > 0 ? skip_rows : M;
+  float* in32 = (float*)malloc(sizeof(float) * (size_t)(M * K));
+  float* sk32 = skip ? (float*)malloc(sizeof(float) * (size_t)(srows * K)) : NULL;
+  float* g32 = (float*)malloc(sizeof(float) * (size_t)K);
+  float* b32 = bias ? (float*)malloc(sizeof(float) * (size_t)K) : NULL;
+  float* o32 = (float*)malloc(sizeof(float) * (size_t)(M * K));
+  float* s32 = sum_out ? (float*)malloc(sizeof(float) * (size_t)(M * K)) : NULL;
+  mnbo_f16_to_f32_buffer(input, in32, (size_t)(M * K));
+  if (skip) mnbo_f16_to_f32_buffer(skip, sk32, (size_t)(srows * K));
+  mnbo_f16_to_f32_buffer(gamma, g32, (size_t)K);
+  if (bias) mnbo_f16_to_f32_buffer(bias, b32, (size_t)K);
+  mnbo_skip_simplified_layer_norm_f32(o32, s32, in32, sk32, srows, g32, b32, epsilon, M, K);
+  mnbo_f32_to_f16_buffer(o32, out, (size_t)(M * K));
+  if (sum_out) mnbo_f32_to_f16_buffer(s32, sum_out, (size_t)(M * K));
+  free(in32);
+  free(sk32);
+  free(g32);
+  free(b32);
+  free(o32);
+  free(s32);
+}

@@ -77,6 +77,12 @@ class _C:
             lib.mnbo_quantize_f32.argtypes = [_u8p, _f32p, _u8p, _f32p, _i64, _i64, _int, _i64, _int]
             lib.mnbo_quantize_f16.argtypes = [_u8p, _u16p, _u8p, _u16p, _i64, _i64, _int, _i64, _int]
             lib.mnbo_quantize_f16.restype = None
+            lib.mnbo_skip_simplified_layer_norm_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _i64, _f32p, _f32p,
+                                                                ctypes.c_float, _i64, _i64]
+            lib.mnbo_skip_simplified_layer_norm_f32.restype = None
+            lib.mnbo_skip_simplified_layer_norm_f16.argtypes = [_u16p, _u16p, _u16p, _u16p, _i64, _u16p, _u16p,
+                                                                ctypes.c_float, _i64, _i64]
+            lib.mnbo_skip_simplified_layer_norm_f16.restype = None
             for f in (lib.mnbo_f16_to_f32_buffer, lib.mnbo_f32_to_f16_buffer, lib.mnbo_dequantize_f32,
                       lib.mnbo_dequantize_f16, lib.mnbo_matmul_f32, lib.mnbo_matmul_f64, lib.mnbo_matmul_f16,
                       lib.mnbo_quantize_f32):
@@ -152,6 +158,77 @@ class _C:
         self.lib.mnbo_matmul_f64(_ptr(a, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), _ptr(b, _f32p),
                                  _ptr(y, _f64p), _ptr(bound, _f64p), M, N, K, bits, bs, nthreads)
         return y.reshape(*lead, N), bound.reshape(*lead, N)
+
+    # -- fused projections ----------------------------------------------------
+    def simplified_layer_norm(self, A, skip, gamma, epsilon, bias=None, want_sum=False):
+        """(Skip)SimplifiedLayerNormalization over the last axis in the dtype of ``A`` (fp16 or fp32).
+
+        ``skip`` may have fewer leading rows than ``A`` (row m uses skip row m % rows).  Returns out, or
+        (out, input + skip [+ bias]) when ``want_sum``."""
+        K = A.shape[-1]
+        M = A.size // K
+        f16 = A.dtype == np.float16
+        ptr_t, np_t = (_u16p, np.uint16) if f16 else (_f32p, np.float32)
+
+        def arr(x):
+            if x is None:
+                return None
+            x = np.ascontiguousarray(x, np.float16 if f16 else np.float32)
+            return x.view(np_t) if f16 else x
+
+        a, sk, g, b = arr(A), arr(skip), arr(gamma), arr(bias)
+        srows = 0 if sk is None else sk.size // K
+        out = np.empty((M, K), np_t)
+        sm = np.empty((M, K), np_t) if want_sum else None
+        fn = self.lib.mnbo_skip_simplified_layer_norm_f16 if f16 else self.lib.mnbo_skip_simplified_layer_norm_f32
+        fn(_ptr(out, ptr_t), _ptr(sm, ptr_t), _ptr(a, ptr_t), _ptr(sk, ptr_t), srows, _ptr(g, ptr_t), _ptr(b, ptr_t),
+           float(epsilon), M, K)
+        view = (lambda x: x.view(np.float16).reshape(A.shape)) if f16 else (lambda x: x.reshape(A.shape))
+        return (view(out), view(sm)) if want_sum else view(out)
+
+    def projections_f32(self, A, mats, N_each, K, bits, bs, nthreads=1):
+        """fp32 result (before the narrowing of an fp16 model) of A x dequant(B_i)^T + bias_i for every
+        (B, scales, bias) in ``mats``: operands widened exactly, fp32 accumulation in k order."""
+        outs = []
+        a32 = np.ascontiguousarray(A.astype(np.float32))
+        for (B, scales, bias), N in zip(mats, N_each):
+            b32 = None if bias is None else bias.astype(np.float32)
+            outs.append(self.matmul(a32, B, scales.astype(np.float32), None, b32, N, K, bits, bs, nthreads))
+        return outs
+
+    def mlp(self, A, gate, up, N, K, bits, bs, norm=None, nthreads=1):
+        """com.microsoft::MatMulNBitsMlp (contrib_defs.cc:3851-3975): Y = silu(gate(A')) * up(A'), A' = A or its
+        (skip) simplified layer normalisation ``norm = (skip or None, gamma, epsilon)``.  gate / up are
+        (B, scales, bias or None).  The projections are the fp32 results of :meth:`projections_f32`; the activation
+        and the product are evaluated in fp64 and narrowed once to the dtype of A.
+        Returns Y, or (Y, input + skip) when ``norm`` has a skip input."""
+        act, sm = A, None
+        if norm is not None:
+            skip, gamma, eps = norm
+            if skip is not None:
+                act, sm = self.simplified_layer_norm(A, skip, gamma, eps, want_sum=True)
+            else:
+                act = self.simplified_layer_norm(A, None, gamma, eps)
+        g, u = self.projections_f32(act, (gate, up), (N, N), K, bits, bs, nthreads)
+        g = g.astype(np.float64)
+        with np.errstate(over="ignore"):
+            y = g / (1.0 + np.exp(-g)) * u.astype(np.float64)
+        y = self.f32_to_f16(y.astype(np.float32)) if A.dtype == np.float16 else y.astype(np.float32)
+        return y if sm is None else (y, sm)
+
+    def qkv(self, A, q, k, v, Nq, Nkv, K, bits, bs, norm=None, nthreads=1):
+        """com.microsoft::MatMulNBitsQkv (contrib_defs.cc:3977-4090): the three projections of A' (see :meth:`mlp`).
+        Returns (Q, K, V) or (Q, K, V, input + skip)."""
+        act, sm = A, None
+        if norm is not None:
+            skip, gamma, eps = norm
+            if skip is not None:
+                act, sm = self.simplified_layer_norm(A, skip, gamma, eps, want_sum=True)
+            else:
+                act = self.simplified_layer_norm(A, None, gamma, eps)
+        outs = [self.matmul(act, B, s, None, b, n, K, bits, bs, nthreads) for (B, s, b), n in
+                zip((q, k, v), (Nq, Nkv, Nkv))]
+        return tuple(outs) if sm is None else tuple(outs) + (sm,)
 
     # -- quantise -------------------------------------------------------------
     def quantize(self, W, bits, bs, symmetric):
