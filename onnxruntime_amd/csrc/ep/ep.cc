@@ -58,6 +58,35 @@ OrtStatus* MatMulNBitsNodeSupported(const Apis& a, const OrtNode* node, bool* su
   return nullptr;
 }
 
+// MatMulNBitsMlp / MatMulNBitsQkv: the same (bits, block_size) support as MatMulNBits, and the one activation the
+// operator defines (onnxruntime/contrib_ops/webgpu/quantization/matmul_nbits_mlp.cc:24-31).
+OrtStatus* FusedProjectionNodeSupported(const Apis& a, const OrtNode* node, bool is_mlp, bool* supported) {
+  *supported = false;
+  int64_t bits = 4, block_size = 0;
+  bool found = false;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, node, "bits", &bits, &found));
+  if (!found) bits = 4;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, node, "block_size", &block_size, &found));
+  if (!found) return nullptr;
+  if (is_mlp) {
+    const OrtOpAttr* attr = nullptr;
+    if (OrtStatus* st = a.ort->Node_GetAttributeByName(node, "activation", &attr)) {
+      a.ort->ReleaseStatus(st);
+      return nullptr;
+    }
+    if (attr == nullptr) return nullptr;
+    char act[16] = {};
+    size_t used = 0;
+    if (OrtStatus* st = a.ort->ReadOpAttr(attr, ORT_OP_ATTR_STRING, act, sizeof(act) - 1, &used)) {
+      a.ort->ReleaseStatus(st);  // longer than any supported name
+      return nullptr;
+    }
+    if (std::strncmp(act, "silu", sizeof(act)) != 0) return nullptr;
+  }
+  *supported = MnbIsAvailable(static_cast<int>(bits), static_cast<int>(block_size), MNB_DTYPE_FLOAT16) != 0;
+  return nullptr;
+}
+
 OrtStatus* ORT_API_CALL GetCapabilityImpl(OrtEp* this_ptr, const OrtGraph* graph,
                                           OrtEpGraphSupportInfo* graph_support_info) noexcept {
   Ep& ep = *Self(this_ptr);
@@ -76,6 +105,10 @@ OrtStatus* ORT_API_CALL GetCapabilityImpl(OrtEp* this_ptr, const OrtGraph* graph
     if (std::strcmp(op_type, "MatMulNBits") == 0) {
       bool ok = false;
       MI_RETURN_IF_ERROR(MatMulNBitsNodeSupported(a, node, &ok));
+      if (!ok) continue;
+    } else if (std::strcmp(op_type, "MatMulNBitsMlp") == 0 || std::strcmp(op_type, "MatMulNBitsQkv") == 0) {
+      bool ok = false;
+      MI_RETURN_IF_ERROR(FusedProjectionNodeSupported(a, node, op_type[11] == 'M', &ok));
       if (!ok) continue;
     }
     MI_RETURN_IF_ERROR(a.ep->EpGraphSupportInfo_AddSingleNode(graph_support_info, node));

@@ -7,84 +7,13 @@
 // (onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc): attribute checks in the constructor (:100-138),
 // PrePack of B together with constant scales / zero points (:252-724), Compute = CheckInputs, output shape, early
 // return on an empty output, then the packed or the unpacked route (:1513-1570).
-#include "ep_common.h"
+#include "ep_kernel_util.h"
 
 namespace mi355x_ep {
 
 namespace {
 
 enum InputIndex : size_t { kA = 0, kB = 1, kScales = 2, kZeroPoints = 3, kGIdx = 4, kBias = 5 };
-
-// Shape and element type of a tensor value.
-struct TensorDesc {
-  std::vector<int64_t> dims;
-  ONNXTensorElementDataType type = ONNX_TENSOR_ELEMENT_DATA_TYPE_UNDEFINED;
-  int64_t count() const {
-    int64_t c = 1;
-    for (int64_t d : dims) c *= d;
-    return c;
-  }
-};
-
-OrtStatus* Describe(const Apis& a, const OrtValue* value, TensorDesc* out) {
-  OrtTensorTypeAndShapeInfo* info = nullptr;
-  MI_RETURN_IF_ERROR(a.ort->GetTensorTypeAndShape(value, &info));
-  size_t rank = 0;
-  OrtStatus* st = a.ort->GetDimensionsCount(info, &rank);
-  if (st == nullptr) {
-    out->dims.assign(rank, 0);
-    if (rank > 0) st = a.ort->GetDimensions(info, out->dims.data(), rank);
-  }
-  if (st == nullptr) st = a.ort->GetTensorElementType(info, &out->type);
-  a.ort->ReleaseTensorTypeAndShapeInfo(info);
-  return st;
-}
-
-MnbTensorInfo ToMnb(const TensorDesc* d) {
-  MnbTensorInfo t{};
-  if (d == nullptr) return t;  // absent optional input
-  static const int64_t kNoDims = 0;
-  t.dims = d->dims.empty() ? &kNoDims : d->dims.data();
-  t.rank = d->dims.size();
-  t.dtype = static_cast<int>(d->type);
-  return t;
-}
-
-bool OnHost(const Apis& a, const OrtValue* v) {
-  return a.ep->MemoryDevice_GetDeviceType(a.ep->Value_GetMemoryDevice(v)) == OrtMemoryInfoDeviceType_CPU;
-}
-
-// A device view of a constant tensor: the tensor's own storage when it already lives on the GPU, otherwise a
-// temporary device copy that is freed with the object.
-class DeviceView {
- public:
-  DeviceView() = default;
-  DeviceView(const DeviceView&) = delete;
-  DeviceView& operator=(const DeviceView&) = delete;
-  ~DeviceView() {
-    if (owned_ != nullptr) (void)hipFree(owned_);
-  }
-  OrtStatus* Init(const Apis& a, const OrtValue* v) {
-    const void* p = nullptr;
-    MI_RETURN_IF_ERROR(a.ort->GetTensorData(v, &p));
-    if (!OnHost(a, v)) {
-      ptr_ = p;
-      return nullptr;
-    }
-    size_t bytes = 0;
-    MI_RETURN_IF_ERROR(a.ort->GetTensorSizeInBytes(v, &bytes));
-    if (bytes == 0) return nullptr;
-    MI_RETURN_IF_HIP(a, hipMalloc(&owned_, bytes));
-    MI_RETURN_IF_HIP(a, hipMemcpy(owned_, p, bytes, hipMemcpyHostToDevice));
-    ptr_ = owned_;
-    return nullptr;
-  }
-  const void* get() const { return ptr_; }
-
- private:
-  const void* ptr_ = nullptr;
-  void* owned_ = nullptr;
-};
 
 // =========================================================================================== MatMulNBits
 struct MatMulNBitsKernel : OrtKernelImpl {
@@ -293,17 +222,6 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
   return nullptr;
 }
 
-bool InputExists(const Apis& a, const OrtKernelInfo* info, size_t index, size_t count) {
-  if (index >= count) return false;
-  size_t size = 0;
-  OrtStatus* st = a.ort->KernelInfo_GetInputName(info, index, nullptr, &size);
-  if (st != nullptr) {
-    a.ort->ReleaseStatus(st);
-    return false;
-  }
-  return size > 1;  // an omitted optional input has the empty name
-}
-
 OrtStatus* ORT_API_CALL CreateMatMulNBits(void* state, const OrtKernelInfo* info, OrtKernelImpl** kernel_out) noexcept {
   const Apis& a = *static_cast<const Apis*>(state);
   *kernel_out = nullptr;
@@ -410,26 +328,6 @@ OrtStatus* ORT_API_CALL CreateMemcpy(void* state, const OrtKernelInfo*, OrtKerne
 }
 
 // =========================================================================================== registration
-struct DefBuilder {
-  const Apis& a;
-  OrtKernelDefBuilder* b = nullptr;
-  explicit DefBuilder(const Apis& apis) : a(apis) {}
-  ~DefBuilder() {
-    if (b != nullptr) a.ep->ReleaseKernelDefBuilder(b);
-  }
-};
-
-OrtStatus* TypeList(const Apis& a, const std::vector<ONNXTensorElementDataType>& elems,
-                    std::vector<const OrtDataType*>* out) {
-  out->clear();
-  for (auto e : elems) {
-    const OrtDataType* t = nullptr;
-    MI_RETURN_IF_ERROR(a.ep->GetTensorDataType(e, &t));
-    out->push_back(t);
-  }
-  return nullptr;
-}
-
 OrtStatus* AddMatMulNBits(const Apis& a, const Apis* state, const char* ep_name, OrtKernelRegistry* registry,
                           ONNXTensorElementDataType t1) {
   DefBuilder db(a);
@@ -490,6 +388,7 @@ OrtStatus* CreateKernelRegistry(const Apis& apis, const char* ep_name, OrtKernel
   MI_RETURN_IF_ERROR(apis.ep->CreateKernelRegistry(&registry));
   OrtStatus* st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT);
   if (st == nullptr) st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16);
+  if (st == nullptr) st = AddFusedProjectionKernels(apis, state, ep_name, registry);
   if (st == nullptr) st = AddMemcpy(apis, state, ep_name, registry, /*from_host*/ true);
   if (st == nullptr) st = AddMemcpy(apis, state, ep_name, registry, /*from_host*/ false);
   if (st != nullptr) {

@@ -19,6 +19,24 @@ class EpHostTensor(ctypes.Structure):
                 ("dtype", ctypes.c_int)]
 
 
+class EpHostAttr(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char_p), ("kind", ctypes.c_int), ("i", ctypes.c_int64), ("f", ctypes.c_float),
+                ("s", ctypes.c_char_p)]
+
+
+class EpHostNodeSpec(ctypes.Structure):
+    _fields_ = [("op_type", ctypes.c_char_p), ("attrs", ctypes.POINTER(EpHostAttr)), ("num_attrs", ctypes.c_size_t),
+                ("schema_attrs", ctypes.POINTER(ctypes.c_char_p)), ("num_schema_attrs", ctypes.c_size_t),
+                ("input_names", ctypes.POINTER(ctypes.c_char_p)), ("input_types", ctypes.POINTER(ctypes.c_char_p)),
+                ("num_inputs", ctypes.c_size_t), ("num_outputs", ctypes.c_size_t),
+                ("skipped_output_mask", ctypes.c_int)]
+
+
+class EpHostOutput(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("capacity", ctypes.c_size_t), ("dims", ctypes.c_int64 * 8),
+                ("rank", ctypes.c_size_t), ("produced", ctypes.c_int)]
+
+
 class EpHostError(RuntimeError):
     def __init__(self, code, message, trace=""):
         super().__init__(f"[{code}] {message}")
@@ -40,7 +58,116 @@ def _load():
         ctypes.POINTER(EpHostTensor), ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int64),
         ctypes.POINTER(ctypes.c_size_t), ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t, ctypes.c_char_p,
         ctypes.c_size_t]
+    lib.EpHostRunNode.restype = ctypes.c_int
+    lib.EpHostRunNode.argtypes = [ctypes.c_char_p, ctypes.POINTER(EpHostNodeSpec), ctypes.POINTER(EpHostTensor),
+                                  ctypes.c_int, ctypes.POINTER(EpHostOutput), ctypes.c_int, ctypes.c_char_p,
+                                  ctypes.c_size_t, ctypes.c_char_p, ctypes.c_size_t]
     return lib
+
+
+def _tensors(arrays, names, constant):
+    tensors = (EpHostTensor * len(arrays))()
+    keep, mask = [], 0
+    for i, (nm, arr) in enumerate(zip(names, arrays)):
+        if arr is None:
+            tensors[i] = EpHostTensor(None, None, 0, 0)
+            continue
+        arr = np.ascontiguousarray(arr)
+        dims = (ctypes.c_int64 * max(arr.ndim, 1))(*arr.shape)
+        keep += [arr, dims]
+        ptr = arr.ctypes.data if arr.size else ctypes.addressof(dims)
+        tensors[i] = EpHostTensor(ptr, ctypes.cast(dims, ctypes.POINTER(ctypes.c_int64)), arr.ndim,
+                                  _ONNX_TYPE[arr.dtype])
+        if nm in constant and i > 0:
+            mask |= 1 << i
+    return tensors, mask, keep
+
+
+def run_node(op_type, attrs, schema_attrs, input_names, input_types, arrays, constant, out_shapes, skipped=(),
+             repeat=1):
+    """One node of the com.microsoft domain through the plugin EP.
+
+    ``attrs``: dict name -> int | float | str.  ``arrays``: inputs in operator order (None = omitted).
+    ``out_shapes``: expected shape of every schema output; outputs whose index is in ``skipped`` are optional outputs
+    the graph does not use.  Returns ([outputs or None], trace)."""
+    lib = _load()
+    cattrs = (EpHostAttr * len(attrs))()
+    for j, (k, v) in enumerate(attrs.items()):
+        if isinstance(v, str):
+            cattrs[j] = EpHostAttr(k.encode(), 2, 0, 0.0, v.encode())
+        elif isinstance(v, float):
+            cattrs[j] = EpHostAttr(k.encode(), 1, 0, v, None)
+        else:
+            cattrs[j] = EpHostAttr(k.encode(), 0, int(v), 0.0, None)
+    sa = (ctypes.c_char_p * len(schema_attrs))(*[x.encode() for x in schema_attrs])
+    inn = (ctypes.c_char_p * len(input_names))(*[x.encode() for x in input_names])
+    itt = (ctypes.c_char_p * len(input_types))(*[x.encode() for x in input_types])
+    tensors, mask, keep = _tensors(arrays, input_names, constant)
+    dtype = arrays[0].dtype
+    outs = (EpHostOutput * len(out_shapes))()
+    bufs = []
+    skip_mask = 0
+    for o, shape in enumerate(out_shapes):
+        if o in skipped:
+            skip_mask |= 1 << o
+            bufs.append(None)
+            continue
+        buf = np.empty(shape, dtype)
+        bufs.append(buf)
+        outs[o].data = buf.ctypes.data if buf.size else None
+        outs[o].capacity = buf.nbytes
+    spec = EpHostNodeSpec(op_type.encode(), cattrs, len(attrs), sa, len(schema_attrs), inn, itt, len(input_names),
+                          len(out_shapes), skip_mask)
+    trace, err = ctypes.create_string_buffer(512), ctypes.create_string_buffer(2048)
+    rc = lib.EpHostRunNode(str(PLUGIN).encode(), ctypes.byref(spec), tensors, mask, outs, repeat, trace, len(trace),
+                           err, len(err))
+    if rc != 0:
+        raise EpHostError(rc, err.value.decode(), trace.value.decode())
+    for o, buf in enumerate(bufs):
+        if buf is None:
+            assert not outs[o].produced
+            continue
+        assert outs[o].produced
+        assert tuple(outs[o].dims[i] for i in range(outs[o].rank)) == buf.shape
+    del keep
+    return bufs, trace.value.decode()
+
+
+_MLP_INPUTS = ["A", "skip", "norm_scale", "gate_B", "gate_scales", "gate_bias", "up_B", "up_scales", "up_bias"]
+_MLP_TYPES = ["T1", "T1", "T1", "T2", "T1", "T1", "T2", "T1", "T1"]
+_QKV_INPUTS = ["A", "skip", "norm_scale", "q_B", "q_scales", "q_bias", "k_B", "k_scales", "k_bias", "v_B", "v_scales",
+               "v_bias"]
+_QKV_TYPES = ["T1", "T1", "T1", "T2", "T1", "T1", "T2", "T1", "T1", "T2", "T1", "T1"]
+
+
+def run_mlp(N, K, bits, block_size, A, gate, up, skip=None, norm_scale=None, want_sum=False, activation="silu",
+            epsilon=None, constant=None, repeat=1):
+    """One MatMulNBitsMlp node; gate / up are (B, scales, bias or None).  Returns (Y, sum or None, trace)."""
+    attrs = {"K": K, "N": N, "bits": bits, "block_size": block_size, "accuracy_level": 0, "activation": activation}
+    if epsilon is not None:
+        attrs["epsilon"] = float(epsilon)
+    arrays = [A, skip, norm_scale, *gate, *up]
+    constant = _MLP_INPUTS[2:] if constant is None else constant
+    outs, trace = run_node("MatMulNBitsMlp", attrs, ["K", "N", "bits", "block_size", "accuracy_level", "activation",
+                                                     "epsilon"], _MLP_INPUTS, _MLP_TYPES, arrays, constant,
+                           [A.shape[:-1] + (N,), A.shape], skipped=() if want_sum else (1,), repeat=repeat)
+    return outs[0], outs[1], trace
+
+
+def run_qkv(Nq, Nkv, K, bits, block_size, A, q, k, v, skip=None, norm_scale=None, want_sum=False, epsilon=None,
+            constant=None, repeat=1):
+    """One MatMulNBitsQkv node.  Returns (Q, K, V, sum or None, trace)."""
+    attrs = {"K": K, "Nq": Nq, "Nkv": Nkv, "bits": bits, "block_size": block_size, "accuracy_level": 0}
+    if epsilon is not None:
+        attrs["epsilon"] = float(epsilon)
+    arrays = [A, skip, norm_scale, *q, *k, *v]
+    constant = _QKV_INPUTS[2:] if constant is None else constant
+    lead = A.shape[:-1]
+    outs, trace = run_node("MatMulNBitsQkv", attrs, ["K", "Nq", "Nkv", "bits", "block_size", "accuracy_level",
+                                                     "epsilon"], _QKV_INPUTS, _QKV_TYPES, arrays, constant,
+                           [lead + (Nq,), lead + (Nkv,), lead + (Nkv,), A.shape], skipped=() if want_sum else (3,),
+                           repeat=repeat)
+    return outs[0], outs[1], outs[2], outs[3], trace
 
 
 def probe_factory(offer_amd_gpu: bool = True) -> dict:

@@ -93,6 +93,9 @@ struct OrtKernelRegistry {
 struct OrtOpAttr {
   std::string name;
   int64_t value;
+  int kind = 0;  // 0 int, 1 float, 2 string
+  float f = 0.f;
+  std::string s;
 };
 struct OrtValueInfo {
   std::string name;
@@ -127,6 +130,7 @@ struct OrtKernelContext {
   OrtAllocator* device_allocator;
   const OrtMemoryInfo* cpu_mem;
   OrtSyncStream* stream;
+  std::vector<bool> output_skipped = {};  // optional outputs the graph does not use: GetOutput yields NULL
 };
 
 namespace {
@@ -204,6 +208,38 @@ void FillApisOnce() {
       }
     return MakeStatus(ORT_FAIL, (std::string("No attribute with name:'") + name + "'is defined.").c_str());
   };
+  g_ort.KernelInfoGetAttribute_float = [](const OrtKernelInfo* info, const char* name, float* out) noexcept
+      -> OrtStatus* {
+    for (const auto& a : info->node->attrs)
+      if (a.name == name && a.kind == 1) {
+        *out = a.f;
+        return nullptr;
+      }
+    return MakeStatus(ORT_FAIL, (std::string("No attribute with name:'") + name + "'is defined.").c_str());
+  };
+  g_ort.KernelInfoGetAttribute_string = [](const OrtKernelInfo* info, const char* name, char* out,
+                                           size_t* size) noexcept -> OrtStatus* {
+    for (const auto& a : info->node->attrs)
+      if (a.name == name && a.kind == 2) {
+        const size_t need = a.s.size() + 1;
+        if (out == nullptr) {
+          *size = need;
+          return nullptr;
+        }
+        if (*size < need) {
+          *size = need;
+          return MakeStatus(ORT_INVALID_ARGUMENT, "Result buffer is not large enough");
+        }
+        std::memcpy(out, a.s.c_str(), need);
+        *size = need;
+        return nullptr;
+      }
+    return MakeStatus(ORT_FAIL, (std::string("No attribute with name:'") + name + "'is defined.").c_str());
+  };
+  g_ort.KernelContext_GetOutputCount = [](const OrtKernelContext* c, size_t* out) noexcept -> OrtStatus* {
+    *out = c->outputs.size();
+    return nullptr;
+  };
   g_ort.KernelInfo_GetInputCount = [](const OrtKernelInfo* info, size_t* out) noexcept -> OrtStatus* {
     *out = info->node->inputs.size();
     return nullptr;
@@ -275,6 +311,10 @@ void FillApisOnce() {
   g_ort.KernelContext_GetOutput = [](OrtKernelContext* c, size_t index, const int64_t* dims, size_t rank,
                                      OrtValue** out) noexcept -> OrtStatus* {
     if (index >= c->outputs.size()) return MakeStatus(ORT_INVALID_ARGUMENT, "output index out of range");
+    if (index < c->output_skipped.size() && c->output_skipped[index]) {
+      *out = nullptr;
+      return nullptr;
+    }
     if (!c->outputs[index]) {
       auto v = std::make_unique<OrtValue>();
       v->dims.assign(dims, dims + rank);
@@ -342,10 +382,23 @@ void FillApisOnce() {
   };
   g_ort.ReadOpAttr = [](const OrtOpAttr* a, OrtOpAttrType type, void* data, size_t len, size_t* out) noexcept
       -> OrtStatus* {
-    if (type != ORT_OP_ATTR_INT || len < sizeof(int64_t)) return MakeStatus(ORT_INVALID_ARGUMENT, "bad ReadOpAttr");
-    *static_cast<int64_t*>(data) = a->value;
-    *out = sizeof(int64_t);
-    return nullptr;
+    if (type == ORT_OP_ATTR_INT && a->kind == 0 && len >= sizeof(int64_t)) {
+      *static_cast<int64_t*>(data) = a->value;
+      *out = sizeof(int64_t);
+      return nullptr;
+    }
+    if (type == ORT_OP_ATTR_FLOAT && a->kind == 1 && len >= sizeof(float)) {
+      *static_cast<float*>(data) = a->f;
+      *out = sizeof(float);
+      return nullptr;
+    }
+    if (type == ORT_OP_ATTR_STRING && a->kind == 2) {
+      *out = a->s.size();
+      if (len < a->s.size()) return MakeStatus(ORT_INVALID_ARGUMENT, "Size of data not large enough to hold the string");
+      std::memcpy(data, a->s.data(), a->s.size());  // not NUL-terminated, like the real call
+      return nullptr;
+    }
+    return MakeStatus(ORT_INVALID_ARGUMENT, "bad ReadOpAttr");
   };
 
   // ---- OrtEpApi
@@ -558,16 +611,51 @@ __attribute__((visibility("default"))) int EpHostProbeFactory(const char* plugin
   return 0;
 }
 
-// Runs one com.microsoft::MatMulNBits node through the plugin.  `inputs` has six entries in operator order
-// (A, B, scales, zero_points, g_idx, bias); bit i of `constant_mask` marks input i as a constant initializer (the
-// host then offers it to PrePackWeight), the other inputs are fed per run.  Compute is called `repeat` times; the
-// result of the last call is copied to `y` (y_bytes capacity) and its shape to y_dims / y_rank (capacity 8).
+// One attribute of the node under test.
+struct EpHostAttr {
+  const char* name;
+  int kind;  // 0 int, 1 float, 2 string
+  int64_t i;
+  float f;
+  const char* s;
+};
+
+// Description of the node under test: operator, attributes, and for each input its name and type-constraint name.
+struct EpHostNodeSpec {
+  const char* op_type;
+  const EpHostAttr* attrs;
+  size_t num_attrs;
+  const char* const* schema_attrs;  // every attribute name the operator schema defines
+  size_t num_schema_attrs;
+  const char* const* input_names;
+  const char* const* input_types;
+  size_t num_inputs;
+  size_t num_outputs;               // outputs of the schema
+  int skipped_output_mask;          // bit o: optional output o is not used by the graph
+};
+
+// One output buffer of the caller.
+struct EpHostOutput {
+  void* data;
+  size_t capacity;
+  int64_t dims[8];
+  size_t rank;
+  int produced;
+};
+
+}  // extern "C"
+
+namespace {
+
+// Runs one node through the plugin.  `inputs` has spec.num_inputs entries in operator order; input 0 is the
+// activation and is fed per run from host memory through MemcpyFromHost.  Bit i of `constant_mask` marks input i as
+// a constant initializer (the host then offers it to PrePackWeight), the other inputs are fed per run as device
+// tensors.  Compute is called `repeat` times; the outputs of the last call are copied to `outs`.
 // Returns 0, an OrtErrorCode reported by the plugin, or a negative EP_HOST_* code; `trace` receives a short log
 // ("claimed=1 prepacked=1,2,3 ...").
-__attribute__((visibility("default"))) int EpHostRunMatMulNBits(
-    const char* plugin_path, int64_t N, int64_t K, int64_t bits, int64_t block_size, int64_t accuracy_level,
-    const EpHostTensor* inputs, int constant_mask, void* y, size_t y_bytes, int64_t* y_dims, size_t* y_rank,
-    int repeat, char* trace_buf, size_t trace_len, char* err, size_t err_len) {
+int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTensor* inputs, int constant_mask,
+            EpHostOutput* outs, int repeat, char* trace_buf, size_t trace_len, char* err, size_t err_len) {
+  const size_t NI = spec.num_inputs;
   FillApis();
   Trace trace{trace_buf, trace_len};
   if (trace_buf && trace_len) trace_buf[0] = 0;
@@ -617,18 +705,26 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
   if (registry == nullptr) return HostFail(EP_HOST_PROTOCOL, "GetKernelRegistry returned NULL", err, err_len);
   trace.add("kernels=%zu ", registry->entries.size());
 
-  // ---- the graph: one MatMulNBits node
+  // ---- the graph: one node
   OrtNode node;
-  node.op = "MatMulNBits";
+  node.op = spec.op_type;
   node.domain = "com.microsoft";
   node.name = "node0";
   node.since_version = 1;
-  node.schema_attrs = {"K", "N", "bits", "block_size", "accuracy_level"};
-  node.attrs = {{"K", K}, {"N", N}, {"bits", bits}, {"block_size", block_size}, {"accuracy_level", accuracy_level}};
-  static const char* kInputNames[6] = {"A", "B", "scales", "zero_points", "g_idx", "bias"};
-  static const char* kInputTypes[6] = {"T1", "T2", "T1", "T3", "T4", "T1"};
+  for (size_t i = 0; i < spec.num_schema_attrs; ++i) node.schema_attrs.push_back(spec.schema_attrs[i]);
+  for (size_t i = 0; i < spec.num_attrs; ++i) {
+    OrtOpAttr at;
+    at.name = spec.attrs[i].name;
+    at.value = spec.attrs[i].i;
+    at.kind = spec.attrs[i].kind;
+    at.f = spec.attrs[i].f;
+    at.s = spec.attrs[i].s ? spec.attrs[i].s : "";
+    node.attrs.push_back(at);
+  }
+  const char* const* kInputNames = spec.input_names;
+  const char* const* kInputTypes = spec.input_types;
   size_t last = 0;
-  for (size_t i = 0; i < 6; ++i)
+  for (size_t i = 0; i < NI; ++i)
     if (inputs[i].data != nullptr || i == 0) last = i;
   for (size_t i = 0; i <= last; ++i) {
     if (inputs[i].data == nullptr && i != 0) {
@@ -674,8 +770,8 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
   OrtSyncStream stream{stream_impl};
 
   // ---- values. Host copies wrap the caller's memory; constants go to the device through the data transfer.
-  std::unique_ptr<OrtValue> host_values[6], device_values[6];
-  for (size_t i = 0; i < 6; ++i) {
+  std::vector<std::unique_ptr<OrtValue>> host_values(NI), device_values(NI);
+  for (size_t i = 0; i < NI; ++i) {
     if (inputs[i].data == nullptr) continue;
     auto v = std::make_unique<OrtValue>();
     v->dims.assign(inputs[i].dims, inputs[i].dims + inputs[i].rank);
@@ -701,7 +797,7 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
     device_values[i] = std::move(d);
     return st;
   };
-  for (size_t i = 1; i < 6; ++i) {
+  for (size_t i = 1; i < NI; ++i) {
     if (!host_values[i]) continue;
     // initializers are copied without a stream at session initialisation, run inputs on the run's stream
     if (OrtStatus* st = to_device(i, !((constant_mask >> i) & 1))) return Fail(st, "CopyTensors", err, err_len);
@@ -711,7 +807,7 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
   const auto* entry = LookUp(*registry, ep_name, node);
   if (entry == nullptr) return HostFail(EP_HOST_PROTOCOL, "claimed node without a kernel", err, err_len);
   OrtKernelInfo info{&node, {}};
-  for (size_t i = 1; i < 6; ++i)
+  for (size_t i = 1; i < NI; ++i)
     if (device_values[i] && ((constant_mask >> i) & 1)) info.constants[i] = device_values[i].get();
   OrtKernelImpl* kernel = nullptr;
   if (OrtStatus* st = entry->fn(entry->state, &info, &kernel)) return Fail(st, "kernel creation", err, err_len);
@@ -722,9 +818,9 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
   } kernel_guard{kernel};
   if (kernel->flags != 0) return HostFail(EP_HOST_PROTOCOL, "OrtKernelImpl::flags must start as 0", err, err_len);
   trace.add("prepacked=");
-  bool packed[6] = {false, false, false, false, false, false};
+  std::vector<bool> packed(NI, false);
   if (kernel->PrePackWeight != nullptr) {
-    for (size_t i = 1; i < 6; ++i) {
+    for (size_t i = 1; i < NI; ++i) {
       if (!info.constants.count(i)) continue;
       bool is_packed = false;
       if (OrtStatus* st = kernel->PrePackWeight(kernel, device_values[i].get(), static_cast<int>(i), allocator,
@@ -734,7 +830,7 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
       if (is_packed) trace.add("%zu,", i);
     }
     // Like ONNX Runtime, drop the initializers the kernel took over - after all PrePack calls of the node.
-    for (size_t i = 1; i < 6; ++i)
+    for (size_t i = 1; i < NI; ++i)
       if (packed[i]) device_values[i].reset();
   }
   trace.add(" ");
@@ -764,33 +860,79 @@ __attribute__((visibility("default"))) int EpHostRunMatMulNBits(
     copy_in.outputs.resize(1);
     if (OrtStatus* st = from_host->Compute(from_host, &copy_in)) return Fail(st, "MemcpyFromHost", err, err_len);
 
-    OrtKernelContext ctx{{}, {}, {false}, allocator, &cpu_mem, &stream};
-    ctx.outputs.resize(1);
+    OrtKernelContext ctx{{}, {}, {}, allocator, &cpu_mem, &stream};
+    ctx.outputs.resize(spec.num_outputs);
+    ctx.output_on_host.assign(spec.num_outputs, false);
+    ctx.output_skipped.assign(spec.num_outputs, false);
+    for (size_t o = 0; o < spec.num_outputs; ++o) ctx.output_skipped[o] = (spec.skipped_output_mask >> o) & 1;
     ctx.inputs.assign(node.inputs.size(), nullptr);
     ctx.inputs[0] = copy_in.outputs[0].get();
     for (size_t i = 1; i < node.inputs.size(); ++i)
       if (!packed[i] && device_values[i]) ctx.inputs[i] = device_values[i].get();
     if (OrtStatus* st = kernel->Compute(kernel, &ctx)) return Fail(st, "Compute", err, err_len);
-    if (!ctx.outputs[0]) return HostFail(EP_HOST_PROTOCOL, "Compute produced no output", err, err_len);
-
-    OrtKernelImpl* to_host = nullptr;
-    if (OrtStatus* st = memcpy_kernel("MemcpyToHost", ctx.outputs[0]->type, &to_host))
-      return Fail(st, "MemcpyToHost creation", err, err_len);
-    KernelGuard to_guard{to_host};
-    OrtKernelContext copy_out{{ctx.outputs[0].get()}, {}, {true}, allocator, &cpu_mem, &stream};
-    copy_out.outputs.resize(1);
-    if (OrtStatus* st = to_host->Compute(to_host, &copy_out)) return Fail(st, "MemcpyToHost", err, err_len);
-    if (OrtStatus* st = stream_impl->Flush(stream_impl)) return Fail(st, "stream Flush", err, err_len);
-    const OrtValue& out = *copy_out.outputs[0];
-    if (out.bytes > y_bytes) return HostFail(EP_HOST_PROTOCOL, "output larger than the caller's buffer", err, err_len);
-    if (out.bytes) std::memcpy(y, out.data, out.bytes);
-    *y_rank = out.dims.size() < 8 ? out.dims.size() : 8;
-    for (size_t i = 0; i < *y_rank; ++i) y_dims[i] = out.dims[i];
+    for (size_t o = 0; o < spec.num_outputs; ++o) {
+      outs[o].produced = 0;
+      if (ctx.output_skipped[o]) continue;
+      if (!ctx.outputs[o]) return HostFail(EP_HOST_PROTOCOL, "Compute produced no output", err, err_len);
+      OrtKernelImpl* to_host = nullptr;
+      if (OrtStatus* st = memcpy_kernel("MemcpyToHost", ctx.outputs[o]->type, &to_host))
+        return Fail(st, "MemcpyToHost creation", err, err_len);
+      KernelGuard to_guard{to_host};
+      OrtKernelContext copy_out{{ctx.outputs[o].get()}, {}, {true}, allocator, &cpu_mem, &stream};
+      copy_out.outputs.resize(1);
+      if (OrtStatus* st = to_host->Compute(to_host, &copy_out)) return Fail(st, "MemcpyToHost", err, err_len);
+      if (OrtStatus* st = stream_impl->Flush(stream_impl)) return Fail(st, "stream Flush", err, err_len);
+      const OrtValue& out = *copy_out.outputs[0];
+      if (out.bytes > outs[o].capacity)
+        return HostFail(EP_HOST_PROTOCOL, "output larger than the caller's buffer", err, err_len);
+      if (out.bytes) std::memcpy(outs[o].data, out.data, out.bytes);
+      outs[o].rank = out.dims.size() < 8 ? out.dims.size() : 8;
+      for (size_t i = 0; i < outs[o].rank; ++i) outs[o].dims[i] = out.dims[i];
+      outs[o].produced = 1;
+    }
   }
   if (OrtStatus* st = ep->Sync(ep)) return Fail(st, "OrtEp::Sync", err, err_len);
   bool concurrent = false;
   if (OrtStatus* st = ep->IsConcurrentRunSupported(ep, &concurrent)) return Fail(st, "IsConcurrentRunSupported", err, err_len);
   trace.add("concurrent=%d", static_cast<int>(concurrent));
+  return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+// Any operator of the com.microsoft domain the plugin registers (MatMulNBitsMlp, MatMulNBitsQkv, ...).
+__attribute__((visibility("default"))) int EpHostRunNode(const char* plugin_path, const EpHostNodeSpec* spec,
+                                                        const EpHostTensor* inputs, int constant_mask,
+                                                        EpHostOutput* outs, int repeat, char* trace_buf,
+                                                        size_t trace_len, char* err, size_t err_len) {
+  return RunNode(plugin_path, *spec, inputs, constant_mask, outs, repeat, trace_buf, trace_len, err, err_len);
+}
+
+// One com.microsoft::MatMulNBits node; `inputs` has six entries (A, B, scales, zero_points, g_idx, bias).  The result
+// of the last Compute call is copied to `y` (y_bytes capacity) and its shape to y_dims / y_rank (capacity 8).
+__attribute__((visibility("default"))) int EpHostRunMatMulNBits(
+    const char* plugin_path, int64_t N, int64_t K, int64_t bits, int64_t block_size, int64_t accuracy_level,
+    const EpHostTensor* inputs, int constant_mask, void* y, size_t y_bytes, int64_t* y_dims, size_t* y_rank,
+    int repeat, char* trace_buf, size_t trace_len, char* err, size_t err_len) {
+  const EpHostAttr attrs[5] = {{"K", 0, K, 0.f, nullptr},
+                               {"N", 0, N, 0.f, nullptr},
+                               {"bits", 0, bits, 0.f, nullptr},
+                               {"block_size", 0, block_size, 0.f, nullptr},
+                               {"accuracy_level", 0, accuracy_level, 0.f, nullptr}};
+  static const char* kSchemaAttrs[5] = {"K", "N", "bits", "block_size", "accuracy_level"};
+  static const char* kInputNames[6] = {"A", "B", "scales", "zero_points", "g_idx", "bias"};
+  static const char* kInputTypes[6] = {"T1", "T2", "T1", "T3", "T4", "T1"};
+  const EpHostNodeSpec spec{"MatMulNBits", attrs, 5, kSchemaAttrs, 5, kInputNames, kInputTypes, 6, 1, 0};
+  EpHostOutput out{};
+  out.data = y;
+  out.capacity = y_bytes;
+  const int rc = RunNode(plugin_path, spec, inputs, constant_mask, &out, repeat, trace_buf, trace_len, err, err_len);
+  if (rc == 0) {
+    *y_rank = out.rank;
+    for (size_t i = 0; i < out.rank; ++i) y_dims[i] = out.dims[i];
+  }
   return rc;
 }
 

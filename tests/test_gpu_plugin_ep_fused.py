@@ -1,0 +1,106 @@
+"""MatMulNBitsMlp / MatMulNBitsQkv through the plugin execution provider: the ONNX Runtime host test double drives
+kernel creation (attributes incl. the string `activation` and float `epsilon`), PrePack of all projections into one
+buffer, Compute with optional skip / norm_scale inputs and the optional input_skip_bias_sum output."""
+import numpy as np
+import pytest
+
+from ep_host import host
+from gpu_util import FP16_GATE, FP32_GATE
+from onnxruntime_amd.synthetic import make_case
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(not host.available(), reason="plugin EP or host shim not built")]
+
+
+def _proj(M, N, K, bits, bs, dtype, bias, seed):
+    c = make_case(M, N, K, bits, bs, dtype, has_bias=bias, seed=seed)
+    return c, (c.B, c.scales, c.bias)
+
+
+def _close(oracle, got, act, c, n, K, bits, bs, dtype):
+    y64, bound = oracle.C.matmul_f64(act, c.B, c.scales, None, c.bias, n, K, bits, bs, nthreads=8)
+    err = np.abs(got.astype(np.float64) - y64)
+    if dtype == np.float32:
+        assert float(np.max(err / (bound + 1e-30))) <= FP32_GATE
+    else:
+        assert float(np.linalg.norm(err) / max(np.linalg.norm(y64), 1e-30)) <= FP16_GATE
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("M,prologue", [(1, None), (1, "skip"), (5, "simplified"), (40, "skip"), (300, None)])
+def test_mlp_through_plugin(oracle, dtype, M, prologue):
+    N, K, bits, bs = 200, 256, 4, 32
+    g, gm = _proj(M, N, K, bits, bs, dtype, True, 1)
+    u, um = _proj(M, N, K, bits, bs, dtype, False, 2)
+    rng = np.random.default_rng(3)
+    gamma = rng.uniform(0.5, 1.5, K).astype(dtype) if prologue else None
+    skip = rng.standard_normal((M, K)).astype(dtype) if prologue == "skip" else None
+    y, sm, trace = host.run_mlp(N, K, bits, bs, g.A, gm, um, skip=skip, norm_scale=gamma,
+                                want_sum=prologue == "skip", epsilon=1e-5)
+    assert "claimed=1" in trace and "prepacked=3,4,5,6,7," in trace, trace  # up_bias is absent: input 8 omitted
+    want = oracle.C.mlp(g.A, gm, um, N, K, bits, bs, norm=None if not prologue else (skip, gamma, 1e-5), nthreads=8)
+    if prologue == "skip":
+        want, want_sum = want
+        assert np.array_equal(sm, want_sum)
+    w64 = want.astype(np.float64)
+    rel = float(np.linalg.norm(y.astype(np.float64) - w64) / max(np.linalg.norm(w64), 1e-30))
+    assert rel <= (FP16_GATE if dtype == np.float16 else 1e-5), rel
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_mlp_unpacked_route_matches_prepacked(dtype):
+    """Scales fed per run: no PrePack, Compute packs into stream-ordered scratch.  Same bits out."""
+    M, N, K, bits, bs = 3, 72, 128, 8, 64
+    g, gm = _proj(M, N, K, bits, bs, dtype, True, 4)
+    u, um = _proj(M, N, K, bits, bs, dtype, True, 5)
+    y1, _, t1 = host.run_mlp(N, K, bits, bs, g.A, gm, um)
+    y2, _, t2 = host.run_mlp(N, K, bits, bs, g.A, gm, um, constant=("gate_B", "up_B"), repeat=3)
+    assert "prepacked=3,4,5,6,7,8," in t1 and "prepacked= " in t2, (t1, t2)
+    assert np.array_equal(y1.view(np.uint8), y2.view(np.uint8))
+
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("M,skip", [(1, True), (6, False), (130, True)])
+def test_qkv_through_plugin(oracle, dtype, M, skip):
+    Nq, Nkv, K, bits, bs = 256, 72, 320, 4, 32
+    q, qm = _proj(M, Nq, K, bits, bs, dtype, True, 6)
+    k, km = _proj(M, Nkv, K, bits, bs, dtype, False, 7)
+    v, vm = _proj(M, Nkv, K, bits, bs, dtype, True, 8)
+    rng = np.random.default_rng(9)
+    gamma = rng.uniform(0.5, 1.5, K).astype(dtype)
+    sk = rng.standard_normal((M, K)).astype(dtype) if skip else None
+    A3 = q.A.reshape(1, M, K)
+    sk3 = None if sk is None else sk.reshape(1, M, K)
+    Q, Kk, V, sm, trace = host.run_qkv(Nq, Nkv, K, bits, bs, A3, qm, km, vm, skip=sk3, norm_scale=gamma,
+                                       want_sum=skip)
+    assert "claimed=1" in trace and "prepacked=3,4,5,6,7,9,10,11," in trace, trace
+    assert Q.shape == (1, M, Nq) and Kk.shape == (1, M, Nkv) and V.shape == (1, M, Nkv)
+    if skip:
+        act, want_sum = oracle.C.simplified_layer_norm(q.A, sk, gamma, 1e-6, want_sum=True)
+        assert np.array_equal(sm.reshape(M, K), want_sum)
+    else:
+        act = oracle.C.simplified_layer_norm(q.A, None, gamma, 1e-6)   # schema default epsilon
+    for got, c, n in ((Q, q, Nq), (Kk, k, Nkv), (V, v, Nkv)):
+        _close(oracle, got.reshape(M, n), act, c, n, K, bits, bs, dtype)
+
+
+def test_fused_nodes_left_to_the_cpu_provider_or_rejected():
+    M, N, K = 1, 64, 128
+    g, gm = _proj(M, N, K, 4, 32, np.float16, False, 1)
+    with pytest.raises(host.EpHostError) as e:
+        host.run_mlp(N, K, 4, 32, g.A, gm, gm, activation="gelu")
+    assert e.value.code == host.NOT_CLAIMED
+    with pytest.raises(host.EpHostError) as e:   # 2-bit weights have no device kernel
+        c2 = make_case(M, N, K, 2, 32, np.float16, seed=1)
+        host.run_mlp(N, K, 2, 32, c2.A, (c2.B, c2.scales, None), (c2.B, c2.scales, None))
+    assert e.value.code == host.NOT_CLAIMED
+    # input errors surface as the operator's own messages
+    with pytest.raises(host.EpHostError, match="requires norm_scale when skip is present"):
+        host.run_mlp(N, K, 4, 32, g.A, gm, gm, skip=g.A)
+    with pytest.raises(host.EpHostError, match="norm_scale must have shape"):
+        host.run_mlp(N, K, 4, 32, g.A, gm, gm, norm_scale=np.ones(K - 1, np.float16))
+    with pytest.raises(host.EpHostError, match="skip input must be present when input_skip_bias_sum output is requested"):
+        host.run_mlp(N, K, 4, 32, g.A, gm, gm, norm_scale=np.ones(K, np.float16), want_sum=True)
+    bad = (g.B[:, :-1], g.scales, None)
+    with pytest.raises(host.EpHostError, match="quantized_weight"):
+        host.run_mlp(N, K, 4, 32, g.A, gm, bad)
