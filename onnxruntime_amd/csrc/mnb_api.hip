@@ -299,8 +299,6 @@ int MnbGemmUnpacked(size_t M, size_t N, size_t K, int bits, int block_size, int 
 // ---------------------------------------------------------------------------------------- fused projections
 }  // extern "C"
 
-bool mnb_kernel_has_fused_epilogue(MnbKernelKind k) { return k == kMnbKernelSkinny || k == kMnbKernelMid; }
-
 namespace {
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -312,15 +310,28 @@ struct FusedWorkspace {
   size_t total() const { return a_norm + tmp + inner; }
 };
 
+// true when every output of the operator is a multiple of 8 columns wide (the tile GEMM's 16-byte stores)
+bool widths_allow_vector_stores(const MnbFusedLayout& F) {
+  for (int i = 0; i < F.map.nsrc; ++i)
+    if (F.map.n[i] % 8 != 0) return false;
+  return true;
+}
+
 FusedWorkspace fused_workspace(const MnbFusedLayout& F, size_t M, int has_norm) {
   FusedWorkspace w{};
   const MnbLayout& L = F.L;
   w.a_norm = has_norm ? round256(M * (size_t)L.K * elem_size(L.dtype)) : 0;
   w.inner = MnbGemmWorkspaceSize(M, (size_t)L.N, (size_t)L.K, L.bits, L.bs, 0, L.dtype);
-  // the decode and streaming kernels write the operator's outputs themselves; they are chosen by shape alone when
-  // the workspace above is there (fp16: M <= 16, or the streaming kernel's regime)
-  const bool fused = L.dtype == kMnbDtypeFloat16 && (M <= 16 || w.inner > 0);
-  w.tmp = fused ? 0 : round256(M * (size_t)L.N * elem_size(L.dtype));
+  if (L.dtype == kMnbDtypeFloat16) {
+    // fp16: the decode and streaming kernels write the operator's outputs themselves, and so does the tile GEMM when
+    // the outputs allow 16-byte stores.  Where the shape selects the tile GEMM, the streaming kernel's scratch is
+    // reserved as well: it takes over when the caller's pointers turn out not to be aligned.
+    const bool tile_gemm = M > 16 && w.inner == 0;
+    if (tile_gemm && widths_allow_vector_stores(F)) w.inner = mnb_mid_workspace_bytes(L, (int64_t)M);
+    w.tmp = (tile_gemm && w.inner == 0) ? round256(M * (size_t)L.N * elem_size(L.dtype)) : 0;
+  } else {
+    w.tmp = round256(M * (size_t)L.N * elem_size(L.dtype));
+  }
   return w;
 }
 
@@ -382,7 +393,8 @@ int fused_gemm(const char* fn, const MnbFusedLayout& F, size_t M, const void* a_
   a.workspace = w.inner ? ws + w.a_norm + w.tmp : nullptr;
   a.workspace_bytes = w.inner ? workspace_bytes - w.a_norm - w.tmp : 0;
   MnbKernelKind k = mnb_select_kernel(a);
-  const bool direct = mnb_kernel_has_fused_epilogue(k);
+  if (k == kMnbKernelGemm256 && w.tmp == 0 && !mnb_gemm256_fused_ok(epi)) k = kMnbKernelMid;  // scratch reserved above
+  const bool direct = k == kMnbKernelSkinny || k == kMnbKernelMid || (k == kMnbKernelGemm256 && w.tmp == 0);
   if (direct) {
     a.epi = epi;
   } else {

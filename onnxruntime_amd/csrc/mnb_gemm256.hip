@@ -42,6 +42,13 @@ struct Gemm256Params {
   int tiles_m, tiles_n;
   int c_vec_ok;  // C allows 16-byte stores of 8 columns: aligned base and pitch, N a multiple of 8
   uint32_t uc[4];  // unpack constants (see UnpackConsts)
+  // several matrices packed as one (mnb_layout.h); these kinds always take the 16-byte store path
+  int epi_kind;            // kMnbFusedNone / kMnbFusedMlp: C[M][n_out0] = silu(gate) * up / kMnbFusedQkv: three outputs
+  int start1, start2;      // qkv: first packed column of the second and third output
+  int n_out0, n_out1, n_out2;
+  _Float16* out1;
+  _Float16* out2;
+  int64_t ld1, ld2;
 };
 
 // The constants of the nibble unpack, passed as kernel arguments: with literals the compiler emits
@@ -314,12 +321,46 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
             ep[(ii * 32 + (r >> 2) * 8 + kq * 4 + (r & 3)) * EP_STRIDE + j * 32 + li] =
                 (_Float16)(acc[2 * h + ii][j][r] + bcol[j]);
       // LDS operations of one wavefront complete in issue order: the reads below see the writes above
+      if (p.epi_kind == kMnbFusedMlp) {
+        // a staged row is gate0 up0 gate1 up1 (16 columns each) = 32 output columns: four lanes per row, each reads
+        // its 8 gate and 8 up values (narrowed to fp16, as the two separate products would be) and writes 8 outputs
+        const int grow = lane >> 2, q = lane & 3;
+        const int gcol = (q >> 1) * 32 + (q & 1) * 8;
+        const int n_glu = ((n0 + wn * 64) >> 1) + q * 8;
 #pragma unroll
-      for (int ps = 0; ps < 8; ++ps) {
-        const int row = ps * 8 + erow;
-        const u4_t v = *reinterpret_cast<const u4_t*>(ep + row * EP_STRIDE + ecol);
-        const int m = m0 + wm * 128 + h * 64 + row;
-        if (m < p.M && n_out < p.N) *reinterpret_cast<u4_t*>(p.C + (int64_t)m * p.ldc + n_out) = v;
+        for (int ps = 0; ps < 4; ++ps) {
+          const int row = ps * 16 + grow;
+          const h8_t g = *reinterpret_cast<const h8_t*>(ep + row * EP_STRIDE + gcol);
+          const h8_t u = *reinterpret_cast<const h8_t*>(ep + row * EP_STRIDE + gcol + 16);
+          h8_t y;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float gf = (float)g[e];
+            y[e] = (_Float16)(gf / (1.0f + __expf(-gf)) * (float)u[e]);
+          }
+          const int m = m0 + wm * 128 + h * 64 + row;
+          if (m < p.M && n_glu < p.n_out0) *reinterpret_cast<h8_t*>(p.C + (int64_t)m * p.ldc + n_glu) = y;
+        }
+      } else {
+        // the 8 columns of a lane lie inside one 16-column tile, hence inside one output
+        _Float16* dst = p.C;
+        int64_t ld = p.ldc;
+        int n_loc = n_out, n_lim = p.N;
+        if (p.epi_kind == kMnbFusedQkv) {
+          n_lim = p.n_out0;
+          if (n_out >= p.start2) {
+            dst = p.out2, ld = p.ld2, n_loc = n_out - p.start2, n_lim = p.n_out2;
+          } else if (n_out >= p.start1) {
+            dst = p.out1, ld = p.ld1, n_loc = n_out - p.start1, n_lim = p.n_out1;
+          }
+        }
+#pragma unroll
+        for (int ps = 0; ps < 8; ++ps) {
+          const int row = ps * 8 + erow;
+          const u4_t v = *reinterpret_cast<const u4_t*>(ep + row * EP_STRIDE + ecol);
+          const int m = m0 + wm * 128 + h * 64 + row;
+          if (m < p.M && n_loc < n_lim) *reinterpret_cast<u4_t*>(dst + (int64_t)m * ld + n_loc) = v;
+        }
       }
     }
   } else {
@@ -363,6 +404,15 @@ hipError_t launch(const Gemm256Params& p, hipStream_t s) {
 
 }  // namespace
 
+// The fused outputs are written with 16-byte stores of 8 columns: every output 16-byte aligned, with a pitch and a
+// width that are multiples of 8 elements.
+bool mnb_gemm256_fused_ok(const MnbEpilogue& e) {
+  const int nout = e.kind == kMnbFusedQkv ? 3 : 1;
+  for (int i = 0; i < nout; ++i)
+    if (reinterpret_cast<uintptr_t>(e.out[i]) % 16 != 0 || e.ld[i] % 8 != 0 || e.n[i] % 8 != 0) return false;
+  return true;
+}
+
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   Gemm256Params p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
@@ -385,6 +435,22 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.uc[2] = 0x64006400u;
   p.uc[3] = 0;
   p.c_vec_ok = (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.ldc % 8 == 0) && (a.L.N % 8 == 0);
+  p.epi_kind = a.epi.kind;
+  if (a.epi.kind != kMnbFusedNone) {
+    if (!mnb_gemm256_fused_ok(a.epi)) return hipErrorInvalidValue;  // the caller checks before choosing this kernel
+    p.C = reinterpret_cast<_Float16*>(a.epi.out[0]);
+    p.ldc = a.epi.ld[0];
+    p.c_vec_ok = 1;
+    p.start1 = (int)a.epi.start[1];
+    p.start2 = (int)a.epi.start[2];
+    p.n_out0 = (int)a.epi.n[0];
+    p.n_out1 = (int)a.epi.n[1];
+    p.n_out2 = (int)a.epi.n[2];
+    p.out1 = reinterpret_cast<_Float16*>(a.epi.out[1]);
+    p.out2 = reinterpret_cast<_Float16*>(a.epi.out[2]);
+    p.ld1 = a.epi.ld[1];
+    p.ld2 = a.epi.ld[2];
+  }
   if (a.L.bits == 4) return a.L.has_zp ? launch<4, true>(p, s) : launch<4, false>(p, s);
   return a.L.has_zp ? launch<8, true>(p, s) : launch<8, false>(p, s);
 }

@@ -57,6 +57,7 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M);  // staged copy o
 bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
+bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
 
 // kernels around the fused operators (mnb_fused.hip)
@@ -67,8 +68,6 @@ hipError_t mnb_launch_rmsnorm(void* a_norm, void* sum_out, int64_t ld_sum, const
 // tmp[M][Np] (plain GEMM over the packed matrix, bias included) -> the operator's outputs
 hipError_t mnb_launch_fused_finish(const MnbEpilogue& epi, const void* tmp, int64_t ld_tmp, int64_t M, int dtype,
                                    hipStream_t s);
-// true when the kernel mnb_select_kernel picks writes the fused outputs itself
-bool mnb_kernel_has_fused_epilogue(MnbKernelKind k);
 
 // machine ceilings (mnb_probe.hip); diagnostics, synchronous
 hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s);

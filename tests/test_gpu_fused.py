@@ -89,7 +89,7 @@ MLP_CASES = [
     # M, N, K, bits, bs: decode kernel (aligned / ragged K), streaming kernel, tile GEMM, odd widths
     (1, 64, 128, 4, 32), (1, 1000, 512, 4, 128), (4, 40, 96, 4, 16), (16, 333, 256, 8, 64), (2, 48, 100, 4, 32),
     (17, 100, 256, 4, 32), (64, 512, 512, 4, 128), (100, 72, 320, 8, 32), (300, 520, 256, 4, 64),
-    (512, 1024, 1024, 4, 32), (2048, 2048, 1024, 4, 32),
+    (512, 1024, 1024, 4, 32), (2048, 2048, 1024, 4, 32), (2048, 2040, 1024, 4, 128), (2048, 2044, 1024, 4, 32),
 ]
 
 
@@ -170,6 +170,7 @@ QKV_CASES = [
     # M, Nq, Nkv, K, bits, bs
     (1, 64, 16, 128, 4, 32), (1, 4096, 1024, 4096, 4, 32), (5, 100, 24, 96, 4, 16), (16, 48, 40, 256, 8, 64),
     (33, 128, 32, 512, 4, 128), (100, 72, 8, 200, 4, 32), (300, 512, 128, 256, 4, 32), (600, 768, 256, 512, 8, 32),
+    (1024, 4000, 2040, 1024, 4, 32),   # tile GEMM; outputs begin inside a wavefront's 64-column block
 ]
 
 
@@ -210,6 +211,32 @@ def test_qkv_parity(oracle, dtype, norm, M, Nq, Nkv, K, bits, bs):
             want = oracle.C.matmul(act, c.B, c.scales, None, c.bias, n, K, bits, bs, nthreads=8)
             assert float(np.linalg.norm(got.astype(np.float64) - want.astype(np.float64)) /
                          max(np.linalg.norm(want.astype(np.float64)), 1e-30)) <= 1e-3
+
+
+def test_tile_gemm_shape_with_unaligned_output_takes_the_streaming_kernel(oracle):
+    """Where the shape selects the tile GEMM but Y does not allow 16-byte stores, the streaming kernel (whose scratch
+    the workspace contract reserves) writes the outputs: same result, up to the narrowing of gate / up."""
+    import ctypes
+    lib = _lib.load()
+    M, N, K, bits, bs = 2048, 2048, 1024, 4, 32
+    g, _ = _mats(M, N, K, bits, bs, np.float16, True, 51)
+    u, _ = _mats(M, N, K, bits, bs, np.float16, False, 52)
+    op = MatMulNBitsMlp(K, N, bits, bs)
+    op.PrePack(dev(g.B), dev(g.scales), dev(g.bias), dev(u.B), dev(u.scales), None)
+    a = dev(g.A)
+    y_ref = op.Compute(a)
+    wsz = lib.MnbMlpWorkspaceSize(M, N, K, bits, bs, _lib.DTYPE_FLOAT16, 0)
+    assert wsz > 0
+    ws = torch.empty(wsz, dtype=torch.uint8, device="cuda")
+    raw = torch.zeros(M * N + 4, dtype=torch.float16, device="cuda")
+    y = raw[4:].view(M, N)   # 8 bytes off a 16-byte boundary
+    _lib.check(lib.MnbMlpGemm(M, N, K, bits, bs, _lib.DTYPE_FLOAT16, a.data_ptr(), K, None, op.packed.data_ptr(), 0,
+                              y.data_ptr(), N, ws.data_ptr(), wsz, None))
+    torch.cuda.synchronize()
+    assert not raw[:4].any()
+    d = (y.float() - y_ref.float()).abs()
+    assert float(d.max()) <= 4e-3 * float(y_ref.float().abs().max())
+    _check_mlp(oracle, y.cpu().numpy(), g.A, g, u, N, K, bits, bs, np.float16)
 
 
 # ------------------------------------------------------------------------------------------------ contract
