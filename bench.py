@@ -142,6 +142,7 @@ def main() -> int:
     ap.add_argument("--no-ceilings", action="store_true",
                     help="skip the read-only / MFMA-only probe kernels that report what the machine sustains")
     ap.add_argument("--no-quantize", action="store_true", help="skip the blockwise quantiser (producer of the format)")
+    ap.add_argument("--no-fused", action="store_true", help="skip the fused gate/up projection (MatMulNBitsMlp)")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -290,6 +291,46 @@ def main() -> int:
                          "traffic": MEASURED_TRAFFIC_BYTES["quantize"]},
         }
         del ws
+        torch.cuda.empty_cache()
+
+    # ---- MatMulNBitsMlp: the gate and up projections of configs[1]'s shape in one launch ------------------------
+    if not args.no_fused:
+        from onnxruntime_amd.matmul_nbits import MatMulNBitsMlp
+        copies = 6   # 6 x 60 MB of distinct weights: beyond the Infinity Cache
+        dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()
+        up = synthetic.make_case(1, c2.N, c2.K, c2.bits, c2.block_size, np.float16, seed=1)
+        gb, gs, ub, us = dev(c2.B), dev(c2.scales), dev(up.B), dev(up.scales)
+        ops = []
+        for i in range(copies):
+            op = MatMulNBitsMlp(c2.K, c2.N, c2.bits, c2.block_size)
+            assert op.PrePack(torch.roll(gb, i, 0), gs, None, torch.roll(ub, i, 0), us, None)
+            ops.append(op)
+        a1 = dev(c2.A.reshape(1, c2.K))
+        skip1 = dev(up.A.reshape(1, c2.K))
+        gamma = torch.ones(c2.K, dtype=torch.float16, device="cuda")
+        fbytes = 2 * (c2.N * c2.k_blocks * (c2.block_size * c2.bits // 8) + c2.N * c2.k_blocks * 2) + \
+            c2.K * 2 + c2.N * 2
+        legs = {}
+        for name, kw in (("plain", {}), ("skip_norm", dict(skip=skip1, norm_scale=gamma, want_skip_sum=True))):
+            def fstep():
+                for op in ops:
+                    op.Compute(a1, **kw)
+            g = graph_of(torch, fstep)
+            msf = time_steps(torch, g.replay, max(4, args.steps // 2), 2) / copies
+            legs[name] = msf
+        gbs_f = fbytes / (legs["plain"] * 1e-3) / 1e9
+        out["mlp_decode"] = {
+            "workload": "MatMulNBitsMlp M=1 K=4096 N=14336 bits=4 block_size=128 fp16: silu(A gate^T) * (A up^T), "
+                        "gate and up packed as one matrix",
+            "value": round(gbs_f, 1),
+            "unit": "GB/s",
+            "ms_per_launch": round(legs["plain"], 5),
+            "ms_per_launch_with_skip_layer_norm_prologue": round(legs["skip_norm"], 5),
+            "kernel": "mnb_skinny_kernel",
+            "roofline": {"bound": "hbm", "achieved": round(gbs_f, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs_f / HBM_PEAK_GBS, 4), "traffic": None},
+        }
+        del ops
         torch.cuda.empty_cache()
 
     # ---- the other configurations (not part of the JSON contract) ---------------------------------------------
