@@ -113,6 +113,15 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
       }
     }
   }
+  if constexpr (T == 1) {
+    // With a single tile nothing separates the last matrix instruction from the first read of its result, and the
+    // compiler sinks that read behind the branches of the chunk loop, where its hazard handling loses track of the
+    // matrix instruction (seen as wrong rows 4 kq + 3).  Eight idle issue cycles cover the result latency
+    // (the check in tests/test_isa_hazards.py scans the generated code for reads that come too early).
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 7");
+    __builtin_amdgcn_sched_barrier(0);
+  }
 }
 
 // Reduce the per-wavefront tiles through LDS in wavefront order and write Y.
