@@ -11,7 +11,8 @@
  * Canonical (on-disk) operand layout, as defined by the operator schema
  * (onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3782-3849):
  *   k_blocks = ceil(K / block_size)
- *   B           u8 [N][k_blocks][block_size*bits/8]   4-bit: low nibble = even k;  8-bit: one byte per element
+ *   B           u8 [N][k_blocks][block_size*bits/8]   2-bit: element e of a byte in bits 2e..2e+1;  4-bit: low nibble =
+ *                                                     even k;  8-bit: one byte per element
  *   scales      T  [N][k_blocks]                       T = fp32 or fp16, same as A
  *   zero_points u8 [N][ceil(k_blocks*bits/8)]          packed like B; absent -> 2^(bits-1)
  *   bias        T  [N]
@@ -67,7 +68,7 @@ MNB_API int MnbGetVersion(void);
 MNB_API int MnbGetDeviceCount(void);
 
 /* Replaces MlasIsQNBitGemmAvailable (onnxruntime/core/mlas/inc/mlas_qnbit.h:134-139).
- * 1 if (bits, block_size, a_dtype) has a device kernel: bits in {4, 8}, block_size in {16,32,64,128,256},
+ * 1 if (bits, block_size, a_dtype) has a device kernel: bits in {2, 4, 8}, block_size in {16,32,64,128,256},
  * a_dtype in {MNB_DTYPE_FLOAT, MNB_DTYPE_FLOAT16}; else 0. */
 MNB_API int MnbIsAvailable(int bits, int block_size, int a_dtype);
 

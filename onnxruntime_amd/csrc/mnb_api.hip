@@ -29,7 +29,7 @@ int hip_fail(hipError_t e, const char* what) {
 }
 
 bool supported(int bits, int bs, int dtype) {
-  const bool b = bits == 4 || bits == 8;
+  const bool b = bits == 2 || bits == 4 || bits == 8;
   const bool s = bs == 16 || bs == 32 || bs == 64 || bs == 128 || bs == 256;
   const bool d = dtype == MNB_DTYPE_FLOAT || dtype == MNB_DTYPE_FLOAT16;
   return b && s && d;
@@ -44,7 +44,6 @@ int check_config(const char* fn, int bits, int bs, int dtype) {
   if (!(bs == 16 || bs == 32 || bs == 64 || bs == 128 || bs == 256))
     return fail(MNB_INVALID_ARGUMENT,
                 "%s: Only block sizes 16, 32, 64, 128, and 256 are supported for MatMulNBits op, got: %d", fn, bs);
-  if (bits == 2) return fail(MNB_NOT_IMPLEMENTED, "%s: 2-bit weights have no MI355X kernel", fn);
   if (dtype != MNB_DTYPE_FLOAT && dtype != MNB_DTYPE_FLOAT16)
     return fail(MNB_NOT_IMPLEMENTED, "%s: element type %d has no MI355X kernel (float and float16 only)", fn, dtype);
   return MNB_OK;

@@ -34,7 +34,8 @@ constexpr int kMnbKAlign = 128;
 
 struct MnbLayout {
   int64_t N, K;
-  int bits, bs, dtype, has_zp;
+  int bits, bs, dtype, has_zp;  // of the PACKED matrix (2-bit weights are stored as 4-bit ones with zero points)
+  int src_bits;                 // bits of the canonical operands
   int64_t k_blocks;   // ceil(K / bs)
   int64_t Npad, Kpad; // padded extents
   int64_t KG;         // 16-byte groups along k
@@ -53,6 +54,13 @@ MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dty
   MnbLayout L;
   L.N = N;
   L.K = K;
+  L.src_bits = bits;
+  if (bits == 2) {
+    // 2-bit weights are widened to nibbles when packed, so every 4-bit kernel runs them unchanged (at the 4-bit
+    // kernels' byte rate); their default zero point 2 is not the 4-bit kernels' 8, so it is always stored
+    bits = 4;
+    has_zp = 1;
+  }
   L.bits = bits;
   L.bs = bs;
   L.dtype = dtype;

@@ -28,6 +28,25 @@ __global__ void __launch_bounds__(256) mnb_pack_weights_kernel(MnbPackSrc S, uin
   const int64_t col_bytes = L.k_blocks * L.bs * BITS / 8;  // bytes of one canonical column
   int m;
   int64_t col;
+  if constexpr (BITS == 2) {
+    // 32 two-bit elements = 8 source bytes become one 16-byte vector of nibbles (same nibble order as below)
+    if (mnb_map_col(S.map, n, &m, &col)) {
+      const uint8_t* src = S.B[m] + col * col_bytes;
+      for (int i = 0; i < 4; ++i) {
+        uint32_t r = 0;
+        for (int e = 0; e < 8; ++e) {
+          const int64_t off = g * 8 + i * 2 + (e >> 2);
+          const uint32_t byte = off < col_bytes ? src[off] : 0u;
+          const uint32_t q = (byte >> (2 * (e & 3))) & 0x3u;
+          const int pos = (e & 1) ? 4 + (e >> 1) : (e >> 1);
+          r |= q << (4 * pos);
+        }
+        w[i] = r;
+      }
+    }
+    W[g * L.Npad + n] = make_uint4(w[0], w[1], w[2], w[3]);
+    return;
+  }
   if (mnb_map_col(S.map, n, &m, &col)) {
     const uint8_t* src = S.B[m] + col * col_bytes + g * 16;
     for (int i = 0; i < 4; ++i) {
@@ -71,10 +90,14 @@ __global__ void __launch_bounds__(256) mnb_pack_meta_kernel(MnbPackSrc S, const 
   if constexpr (HAS_ZP) {  // zero points exist only for a single matrix: col == n
     if (valid) {
       const int64_t row = (L.k_blocks * BITS + 7) / 8;
-      if constexpr (BITS == 8) {
+      if (zp == nullptr) {
+        z = 1 << (BITS - 1);  // 2-bit weights without zero points: the default is stored explicitly
+      } else if constexpr (BITS == 8) {
         z = zp[col * row + kb];
-      } else {
+      } else if constexpr (BITS == 4) {
         z = (zp[col * row + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
+      } else {
+        z = (zp[col * row + (kb >> 2)] >> ((kb & 3) * 2)) & 0x3;
       }
     }
   }
@@ -125,9 +148,12 @@ __global__ void __launch_bounds__(256) mnb_dequant_canonical_kernel(T* __restric
   if constexpr (BITS == 8) {
     q = blob[r];
     if (zp) z = zp[n * kbc + kb];
-  } else {
+  } else if constexpr (BITS == 4) {
     q = (blob[r >> 1] >> ((r & 1) * 4)) & 0xF;
     if (zp) z = (zp[n * ((kbc + 1) / 2) + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
+  } else {
+    q = (blob[r >> 2] >> ((r & 3) * 2)) & 0x3;
+    if (zp) z = (zp[n * ((kbc + 3) / 4) + (kb >> 2)] >> ((kb & 3) * 2)) & 0x3;
   }
   const T s = scales[n * kbc + kb];
   if constexpr (sizeof(T) == 2) {
@@ -168,18 +194,23 @@ static hipError_t pack_t(const MnbLayout& L, const MnbPackSrc& S, const void* zp
   const int64_t wn = L.Npad * L.KG;
   const int64_t mn = L.KBp * L.Npad;
   dim3 blk(256);
-  if (L.bits == 4) {
-    mnb_pack_weights_kernel<4><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>(S, W, L);
+  const dim3 wgrid((unsigned)((wn + 255) / 256)), mgrid((unsigned)((mn + 255) / 256));
+  const uint8_t* z = (const uint8_t*)zp;
+  if (L.src_bits == 2) {
+    mnb_pack_weights_kernel<2><<<wgrid, blk, 0, s>>>(S, W, L);
+    mnb_pack_meta_kernel<T, 2, true><<<mgrid, blk, 0, s>>>(S, z, meta, L);  // z may be NULL: default stored
+  } else if (L.bits == 4) {
+    mnb_pack_weights_kernel<4><<<wgrid, blk, 0, s>>>(S, W, L);
     if (zp)
-      mnb_pack_meta_kernel<T, 4, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, (const uint8_t*)zp, meta, L);
+      mnb_pack_meta_kernel<T, 4, true><<<mgrid, blk, 0, s>>>(S, z, meta, L);
     else
-      mnb_pack_meta_kernel<T, 4, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, nullptr, meta, L);
+      mnb_pack_meta_kernel<T, 4, false><<<mgrid, blk, 0, s>>>(S, nullptr, meta, L);
   } else {
-    mnb_pack_weights_kernel<8><<<dim3((unsigned)((wn + 255) / 256)), blk, 0, s>>>(S, W, L);
+    mnb_pack_weights_kernel<8><<<wgrid, blk, 0, s>>>(S, W, L);
     if (zp)
-      mnb_pack_meta_kernel<T, 8, true><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, (const uint8_t*)zp, meta, L);
+      mnb_pack_meta_kernel<T, 8, true><<<mgrid, blk, 0, s>>>(S, z, meta, L);
     else
-      mnb_pack_meta_kernel<T, 8, false><<<dim3((unsigned)((mn + 255) / 256)), blk, 0, s>>>(S, nullptr, meta, L);
+      mnb_pack_meta_kernel<T, 8, false><<<mgrid, blk, 0, s>>>(S, nullptr, meta, L);
   }
   return hipGetLastError();
 }
@@ -222,6 +253,16 @@ hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* sc
   const int64_t total = N * K;
   if (total == 0) return hipSuccess;
   dim3 grid((unsigned)((total + 255) / 256)), blk(256);
+  if (bits == 2) {
+    if (dtype == kMnbDtypeFloat16)
+      mnb_dequant_canonical_kernel<_Float16, 2><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,
+                                                                     (const _Float16*)scales, (const uint8_t*)zp, N, K,
+                                                                     bs);
+    else
+      mnb_dequant_canonical_kernel<float, 2><<<grid, blk, 0, s>>>((float*)dst, (const uint8_t*)B, (const float*)scales,
+                                                                  (const uint8_t*)zp, N, K, bs);
+    return hipGetLastError();
+  }
   if (dtype == kMnbDtypeFloat16) {
     if (bits == 4)
       mnb_dequant_canonical_kernel<_Float16, 4><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,

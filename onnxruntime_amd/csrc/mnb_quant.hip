@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
         return (uint32_t)(int)t;
       };
       uint8_t* out = B + (n * kbc + kb) * blob + (int64_t)r0 / PER_BYTE;
-      const int qbytes = qrows / PER_BYTE;  // 2 (4-bit, block 16) or a multiple of 4
+      const int qbytes = qrows / PER_BYTE;  // 1 (2-bit, block 16), 2 (4-bit block 16, 2-bit block 32) or a multiple of 4
       if (qbytes >= 4) {
         for (int w = 0; w < qbytes / 4; ++w) {
           uint32_t word = 0;
@@ -135,7 +135,10 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
       } else {
         uint32_t word = 0;
         for (int e = 0; e < qrows; ++e) word |= quant(r0 + e) << (e * BITS);
-        *reinterpret_cast<uint16_t*>(out) = (uint16_t)word;
+        if (qbytes == 1)
+          *out = (uint8_t)word;  // 2-bit, block 16: four elements per thread
+        else
+          *reinterpret_cast<uint16_t*>(out) = (uint16_t)word;
       }
     }
   }
@@ -160,6 +163,7 @@ hipError_t launch_t(void* B, void* scales, void* zp, const void* src, int64_t K,
     kernel<<<grid, blk, smem, s>>>((uint8_t*)B, (T*)scales, (uint8_t*)zp, (const T*)src, K, N, ld, bs, vec_ok);
     return hipGetLastError();
   };
+  if (bits == 2) return launch(mnb_quantize_kernel<T, 2>);
   return bits == 4 ? launch(mnb_quantize_kernel<T, 4>) : launch(mnb_quantize_kernel<T, 8>);
 }
 

@@ -71,7 +71,7 @@ class MatMulNBits:
         self.zp_row = (self.k_blocks * self.bits + 7) // 8
         self.lib = _lib.load()
         # what this device path takes; everything else stays with the CPU provider
-        self.supported = (dtype in (torch.float16, torch.float32) and bits in (4, 8) and not has_g_idx
+        self.supported = (dtype in (torch.float16, torch.float32) and bits in (2, 4, 8) and not has_g_idx
                           and zero_points_dtype == torch.uint8
                           and bool(self.lib.MnbIsAvailable(bits, block_size, _DTYPES[dtype])))
         self.packed: Optional[torch.Tensor] = None
@@ -213,7 +213,7 @@ class _FusedProjections:
         self.k_blocks = (self.K + self.block_size - 1) // self.block_size
         self.blob_size = self.block_size * self.bits // 8
         self.lib = _lib.load()
-        self.supported = (dtype in (torch.float16, torch.float32) and bits in (4, 8)
+        self.supported = (dtype in (torch.float16, torch.float32) and bits in (2, 4, 8)
                           and bool(self.lib.MnbIsAvailable(bits, block_size, _DTYPES[dtype])))
         self.packed: Optional[torch.Tensor] = None
         self._workspace = {}

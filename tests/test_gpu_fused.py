@@ -265,6 +265,6 @@ def test_fused_argument_errors():
     rc = lib.MnbMlpGemm(1, 64, 256, 4, 32, _lib.DTYPE_FLOAT16, dev(g.A).data_ptr(), 256, None, op.packed.data_ptr(), 7,
                         y.data_ptr(), 64, None, 0, None)
     assert rc == _lib.INVALID_ARGUMENT and "activation 7 is not supported" in _lib.last_error()
-    assert lib.MnbMlpPackSize(64, 256, 2, 32, _lib.DTYPE_FLOAT16) == 0  # 2-bit: no kernel
+    assert lib.MnbMlpPackSize(64, 256, 3, 32, _lib.DTYPE_FLOAT16) == 0  # 3-bit: no such format
     # empty batch
     assert tuple(op.Compute(torch.empty(0, 256, dtype=torch.float16, device="cuda")).shape) == (0, 64)

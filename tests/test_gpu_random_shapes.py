@@ -15,7 +15,7 @@ M_CHOICES = [1, 2, 3, 5, 8, 15, 16, 17, 31, 33, 64, 100, 129, 257]
 
 
 def _draw(rng):
-    bits = int(rng.choice([4, 8]))
+    bits = int(rng.choice([2, 4, 8]))
     bs = int(rng.choice([16, 32, 64, 128, 256]))
     dtype = np.float16 if rng.random() < 0.7 else np.float32
     M = int(rng.choice(M_CHOICES))

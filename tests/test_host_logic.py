@@ -24,15 +24,18 @@ def test_library_exports_every_declared_symbol():
 
 def test_availability_and_sizes():
     lib = _lib.load()
-    for bits in (4, 8):
+    for bits in (2, 4, 8):
         for bs in (16, 32, 64, 128, 256):
             for dt in (_lib.DTYPE_FLOAT, _lib.DTYPE_FLOAT16):
                 assert lib.MnbIsAvailable(bits, bs, dt) == 1
-    assert lib.MnbIsAvailable(2, 32, _lib.DTYPE_FLOAT16) == 0
+    assert lib.MnbIsAvailable(3, 32, _lib.DTYPE_FLOAT16) == 0
     assert lib.MnbIsAvailable(4, 512, _lib.DTYPE_FLOAT16) == 0
     assert lib.MnbIsAvailable(4, 32, 16) == 0  # bf16
     # packed size: weights (N*K/2) + fp16 scales for the headline decode shape, no padding needed
     assert lib.MnbPackQuantBDataSize(14336, 4096, 4, 128, 0, _lib.DTYPE_FLOAT16) == 14336 * 2048 + 14336 * 32 * 2
+    # 2-bit weights are stored as nibbles with explicit zero points: the 4-bit size with 4-byte meta entries
+    assert lib.MnbPackQuantBDataSize(14336, 4096, 2, 128, 0, _lib.DTYPE_FLOAT16) == \
+        lib.MnbPackQuantBDataSize(14336, 4096, 4, 128, 1, _lib.DTYPE_FLOAT16)
     assert lib.MnbPackQuantBDataSize(14336, 4096, 4, 32, 1, _lib.DTYPE_FLOAT16) == 14336 * 2048 + 14336 * 128 * 4
     assert lib.MnbPackQuantBDataSize(0, 4096, 4, 32, 1, _lib.DTYPE_FLOAT16) == 0
 
@@ -88,7 +91,7 @@ def test_constructor_and_prepack_guards():
     with pytest.raises(MnbError, match=r"MatMulNBits PrePack: zero_points initializer shape \{8,2\}"):
         op.PrePack(b, s, torch.zeros(8, 2, dtype=torch.uint8))
     # configurations the device path declines (they stay on the CPU provider)
-    assert not MatMulNBits(32, 8, bits=2, block_size=16).supported
+    assert MatMulNBits(32, 8, bits=2, block_size=16).supported
     assert not MatMulNBits(32, 8, has_g_idx=True).supported
     assert not MatMulNBits(32, 8, has_zero_points=True, zero_points_dtype=torch.float16).supported
     assert not MatMulNBits(32, 8, dtype=torch.bfloat16).supported
@@ -100,7 +103,7 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert rc == _lib.INVALID_ARGUMENT and "Only 2b, 4b and 8b" in _lib.last_error()
     rc = lib.MnbGemm(1, 8, 32, 4, 48, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
     assert rc == _lib.INVALID_ARGUMENT and "got: 48" in _lib.last_error()
-    rc = lib.MnbGemm(1, 8, 32, 2, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
+    rc = lib.MnbGemm(1, 8, 32, 4, 16, 0, 16, None, 32, None, None, None, 8, None, 0, None)   # bf16 activations
     assert rc == _lib.NOT_IMPLEMENTED
     rc = lib.MnbGemm(1, 8, 32, 4, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None)
     assert rc == _lib.INVALID_ARGUMENT and "must not be NULL" in _lib.last_error()
