@@ -2,7 +2,7 @@
 // (include/onnxruntime/core/session/onnxruntime_ep_c_api.h:2164-2550).  GetCapability claims every node for which
 // the registry holds a kernel and whose static attributes the device library supports; everything else stays with
 // ONNX Runtime's CPU provider, which is what makes the library a drop-in for the MatMulNBits path and nothing else.
-#include "ep_common.h"
+#include "ep_kernel_util.h"
 
 namespace mi355x_ep {
 
@@ -18,6 +18,8 @@ struct Ep : OrtEp {
 Ep* Self(OrtEp* p) { return static_cast<Ep*>(p); }
 
 const char* ORT_API_CALL GetNameImpl(const OrtEp*) noexcept { return kEpName; }
+
+}  // namespace
 
 // Reads an integer attribute of a node; `found` is false when the attribute is unset.
 OrtStatus* ReadIntAttr(const Apis& a, const OrtNode* node, const char* name, int64_t* value, bool* found) {
@@ -35,6 +37,8 @@ OrtStatus* ReadIntAttr(const Apis& a, const OrtNode* node, const char* name, int
   *found = true;
   return nullptr;
 }
+
+namespace {
 
 // Static screening of one MatMulNBits node: the conditions under which the reference kernel itself would not run
 // its fast path are kept on the CPU provider instead of failing at run time on the device
@@ -87,6 +91,99 @@ OrtStatus* FusedProjectionNodeSupported(const Apis& a, const OrtNode* node, bool
   return nullptr;
 }
 
+bool IsConstant(const Apis& a, const OrtValueInfo* v) {
+  bool c = false;
+  if (v == nullptr) return false;
+  if (OrtStatus* st = a.ort->ValueInfo_IsConstantInitializer(v, &c)) {
+    a.ort->ReleaseStatus(st);
+    return false;
+  }
+  return c;
+}
+
+// MatMulNBits -> Add(constant [N]) is the pair ONNX Runtime's MatMulNBitsFusion folds into the operator's bias input,
+// but only for its own CPU and CUDA providers (onnxruntime/core/optimizer/graph_transformer_utils.cc:343-344,459;
+// matmul_nbits_fusion.cc).  For this provider the Add would stay behind as a CPU node with a device-to-host copy in
+// front of it, so the pair is claimed as one fused node instead and compiled to a single GEMM launch with bias
+// (OrtEp::Compile, ep_compile.cc).  Conditions: the MatMulNBits node has no bias of its own, constant weights /
+// scales / zero points (they are packed at compile time), its output feeds this Add and nothing else, and the
+// other Add input is a constant 1-D tensor of N elements in the activation type.
+OrtStatus* FindBiasAdd(const Apis& a, const OrtNode* mm, const OrtNode** add_out) {
+  *add_out = nullptr;
+  int64_t N = 0;
+  bool found = false;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, mm, "N", &N, &found));
+  if (!found) return nullptr;
+  size_t num_inputs = 0, num_outputs = 0;
+  MI_RETURN_IF_ERROR(a.ort->Node_GetNumInputs(mm, &num_inputs));
+  std::vector<const OrtValueInfo*> in(num_inputs, nullptr);
+  MI_RETURN_IF_ERROR(a.ort->Node_GetInputs(mm, in.data(), num_inputs));
+  if (num_inputs > 5 && in[5] != nullptr) return nullptr;               // already has a bias
+  if (num_inputs < 3 || !IsConstant(a, in[1]) || !IsConstant(a, in[2])) return nullptr;
+  if (num_inputs > 3 && in[3] != nullptr && !IsConstant(a, in[3])) return nullptr;
+  MI_RETURN_IF_ERROR(a.ort->Node_GetNumOutputs(mm, &num_outputs));
+  if (num_outputs != 1) return nullptr;
+  const OrtValueInfo* y = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->Node_GetOutputs(mm, &y, 1));
+  bool is_graph_output = false;
+  MI_RETURN_IF_ERROR(a.ort->ValueInfo_IsGraphOutput(y, &is_graph_output));
+  size_t consumers = 0;
+  MI_RETURN_IF_ERROR(a.ort->ValueInfo_GetValueNumConsumers(y, &consumers));
+  if (is_graph_output || consumers != 1) return nullptr;
+  const OrtNode* add = nullptr;
+  int64_t index = -1;
+  MI_RETURN_IF_ERROR(a.ort->ValueInfo_GetValueConsumers(y, &add, &index, 1));
+  if (add == nullptr || (index != 0 && index != 1)) return nullptr;
+  const char* op = nullptr;
+  const char* domain = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->Node_GetOperatorType(add, &op));
+  MI_RETURN_IF_ERROR(a.ort->Node_GetDomain(add, &domain));
+  if (std::strcmp(op, "Add") != 0 || (domain[0] != 0 && std::strcmp(domain, "ai.onnx") != 0)) return nullptr;
+  size_t add_inputs = 0;
+  MI_RETURN_IF_ERROR(a.ort->Node_GetNumInputs(add, &add_inputs));
+  if (add_inputs != 2) return nullptr;
+  const OrtValueInfo* ain[2] = {nullptr, nullptr};
+  MI_RETURN_IF_ERROR(a.ort->Node_GetInputs(add, ain, 2));
+  const OrtValueInfo* bias = ain[1 - index];
+  if (!IsConstant(a, bias)) return nullptr;
+  const OrtValue* bias_value = nullptr;
+  const OrtValue* scales_value = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->ValueInfo_GetInitializerValue(bias, &bias_value));
+  MI_RETURN_IF_ERROR(a.ort->ValueInfo_GetInitializerValue(in[2], &scales_value));
+  if (bias_value == nullptr || scales_value == nullptr) return nullptr;
+  TensorDesc bd, sd;
+  MI_RETURN_IF_ERROR(Describe(a, bias_value, &bd));
+  MI_RETURN_IF_ERROR(Describe(a, scales_value, &sd));
+  if (bd.dims.size() != 1 || bd.dims[0] != N || bd.type != sd.type) return nullptr;
+  // Compile must not fail on this pair: screen here everything it validates.  A pair that does not pass stays
+  // un-fused, and the MatMulNBits kernel reports the problem at run time the way the reference kernel does.
+  int64_t K = 0, block_size = 0, bits = 4;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, mm, "K", &K, &found));
+  if (!found) return nullptr;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, mm, "block_size", &block_size, &found));
+  if (!found) return nullptr;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, mm, "bits", &bits, &found));
+  if (!found) bits = 4;
+  if (!MnbIsAvailable(static_cast<int>(bits), static_cast<int>(block_size), static_cast<int>(sd.type))) return nullptr;
+  const OrtValue* b_value = nullptr;
+  const OrtValue* zp_value = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->ValueInfo_GetInitializerValue(in[1], &b_value));
+  if (b_value == nullptr) return nullptr;
+  TensorDesc b_desc, z_desc;
+  MI_RETURN_IF_ERROR(Describe(a, b_value, &b_desc));
+  if (num_inputs > 3 && in[3] != nullptr) {
+    MI_RETURN_IF_ERROR(a.ort->ValueInfo_GetInitializerValue(in[3], &zp_value));
+    if (zp_value == nullptr) return nullptr;
+    MI_RETURN_IF_ERROR(Describe(a, zp_value, &z_desc));
+    if (z_desc.type != ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8) return nullptr;  // typed zero points: unpacked route only
+  }
+  MnbTensorInfo bi = ToMnb(&b_desc), si = ToMnb(&sd), zi = ToMnb(zp_value != nullptr ? &z_desc : nullptr),
+                none = ToMnb(nullptr), biasi = ToMnb(&bd);
+  if (MnbCheckInputs(&bi, &si, &zi, &none, &biasi, N, K, block_size, bits) != MNB_OK) return nullptr;
+  *add_out = add;
+  return nullptr;
+}
+
 OrtStatus* ORT_API_CALL GetCapabilityImpl(OrtEp* this_ptr, const OrtGraph* graph,
                                           OrtEpGraphSupportInfo* graph_support_info) noexcept {
   Ep& ep = *Self(this_ptr);
@@ -106,6 +203,16 @@ OrtStatus* ORT_API_CALL GetCapabilityImpl(OrtEp* this_ptr, const OrtGraph* graph
       bool ok = false;
       MI_RETURN_IF_ERROR(MatMulNBitsNodeSupported(a, node, &ok));
       if (!ok) continue;
+      const OrtNode* add = nullptr;
+      MI_RETURN_IF_ERROR(FindBiasAdd(a, node, &add));
+      if (add != nullptr) {
+        const OrtNode* pair[2] = {node, add};
+        OrtNodeFusionOptions options{};
+        options.ort_version_supported = ORT_API_VERSION;
+        options.drop_constant_initializers = true;  // everything constant is packed into device memory at Compile
+        MI_RETURN_IF_ERROR(a.ep->EpGraphSupportInfo_AddNodesToFuse(graph_support_info, pair, 2, &options));
+        continue;
+      }
     } else if (std::strcmp(op_type, "MatMulNBitsMlp") == 0 || std::strcmp(op_type, "MatMulNBitsQkv") == 0) {
       bool ok = false;
       MI_RETURN_IF_ERROR(FusedProjectionNodeSupported(a, node, op_type[11] == 'M', &ok));
@@ -140,6 +247,15 @@ OrtStatus* ORT_API_CALL IsConcurrentRunSupportedImpl(OrtEp*, bool* is_supported)
   return nullptr;
 }
 
+OrtStatus* ORT_API_CALL CompileImpl(OrtEp* this_ptr, const OrtGraph** graphs, const OrtNode** fused_nodes, size_t count,
+                                    OrtNodeComputeInfo** node_compute_infos, OrtNode** /*ep_context_nodes*/) noexcept {
+  return CompileFusedNodes(Self(this_ptr)->apis, graphs, fused_nodes, count, node_compute_infos);
+}
+
+void ORT_API_CALL ReleaseNodeComputeInfosImpl(OrtEp*, OrtNodeComputeInfo** infos, size_t count) noexcept {
+  for (size_t i = 0; i < count; ++i) ReleaseFusedNode(infos[i]);
+}
+
 OrtStatus* ORT_API_CALL SyncImpl(OrtEp* this_ptr) noexcept {
   Ep& ep = *Self(this_ptr);
   MI_RETURN_IF_HIP(ep.apis, hipSetDevice(ep.device));
@@ -160,7 +276,9 @@ OrtEp* CreateEp(Factory& factory, const Apis& apis, int device) {
   ep->CreateSyncStreamForDevice = CreateSyncStreamForDeviceImpl;
   ep->IsConcurrentRunSupported = IsConcurrentRunSupportedImpl;
   ep->Sync = SyncImpl;
-  // Compile / ReleaseNodeComputeInfos stay NULL: the provider registers kernels and never fuses subgraphs.
+  // the only subgraph the provider compiles is MatMulNBits + Add(bias); everything else runs registered kernels
+  ep->Compile = CompileImpl;
+  ep->ReleaseNodeComputeInfos = ReleaseNodeComputeInfosImpl;
   return ep;
 }
 

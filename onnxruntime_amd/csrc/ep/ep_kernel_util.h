@@ -107,6 +107,12 @@ inline OrtStatus* TypeList(const Apis& a, const std::vector<ONNXTensorElementDat
   return nullptr;
 }
 
+// ---- compiled subgraphs (ep_compile.cc): MatMulNBits + Add(bias) as one node
+OrtStatus* ReadIntAttr(const Apis& a, const OrtNode* node, const char* name, int64_t* value, bool* found);  // ep.cc
+OrtStatus* CompileFusedNodes(const Apis& a, const OrtGraph** graphs, const OrtNode** fused_nodes, size_t count,
+                             OrtNodeComputeInfo** node_compute_infos);
+void ReleaseFusedNode(OrtNodeComputeInfo* info);
+
 // ---- fused projections (ep_fused_kernels.cc): MatMulNBitsMlp and MatMulNBitsQkv for float and float16
 OrtStatus* AddFusedProjectionKernels(const Apis& a, const Apis* state, const char* ep_name, OrtKernelRegistry* registry);
 

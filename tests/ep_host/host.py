@@ -10,7 +10,7 @@ HERE = Path(__file__).resolve().parent
 SHIM = HERE / "libort_host_shim.so"
 PLUGIN = HERE.parent.parent / "onnxruntime_amd" / "libonnxruntime_mi355x_ep.so"
 
-NOT_CLAIMED, LOAD_FAILED, NO_DEVICE, PROTOCOL = -1, -2, -3, -4
+NOT_CLAIMED, LOAD_FAILED, NO_DEVICE, PROTOCOL, NOT_FUSED = -1, -2, -3, -4, -5
 _ONNX_TYPE = {np.dtype(np.float32): 1, np.dtype(np.uint8): 2, np.dtype(np.int32): 6, np.dtype(np.float16): 10}
 
 
@@ -30,6 +30,12 @@ class EpHostNodeSpec(ctypes.Structure):
                 ("input_names", ctypes.POINTER(ctypes.c_char_p)), ("input_types", ctypes.POINTER(ctypes.c_char_p)),
                 ("num_inputs", ctypes.c_size_t), ("num_outputs", ctypes.c_size_t),
                 ("skipped_output_mask", ctypes.c_int)]
+
+
+class EpHostAddSpec(ctypes.Structure):
+    _fields_ = [("operand", EpHostTensor), ("operand_is_constant", ctypes.c_int),
+                ("product_input_index", ctypes.c_int), ("product_is_graph_output", ctypes.c_int),
+                ("extra_consumer", ctypes.c_int)]
 
 
 class EpHostOutput(ctypes.Structure):
@@ -58,6 +64,12 @@ def _load():
         ctypes.POINTER(EpHostTensor), ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_int64),
         ctypes.POINTER(ctypes.c_size_t), ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t, ctypes.c_char_p,
         ctypes.c_size_t]
+    lib.EpHostRunMatMulNBitsAdd.restype = ctypes.c_int
+    lib.EpHostRunMatMulNBitsAdd.argtypes = [
+        ctypes.c_char_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+        ctypes.POINTER(EpHostTensor), ctypes.c_int, ctypes.POINTER(EpHostAddSpec), ctypes.c_void_p, ctypes.c_size_t,
+        ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_size_t), ctypes.c_int, ctypes.c_char_p,
+        ctypes.c_size_t, ctypes.c_char_p, ctypes.c_size_t]
     lib.EpHostRunNode.restype = ctypes.c_int
     lib.EpHostRunNode.argtypes = [ctypes.c_char_p, ctypes.POINTER(EpHostNodeSpec), ctypes.POINTER(EpHostTensor),
                                   ctypes.c_int, ctypes.POINTER(EpHostOutput), ctypes.c_int, ctypes.c_char_p,
@@ -215,4 +227,29 @@ def run_matmul_nbits(N, K, bits, block_size, A, B, scales, zero_points=None, g_i
         raise EpHostError(rc, err.value.decode(), trace.value.decode())
     shape = tuple(y_dims[i] for i in range(y_rank.value))
     assert shape == y.shape, (shape, y.shape)
+    return y, trace.value.decode()
+
+
+def run_matmul_nbits_add(N, K, bits, block_size, A, B, scales, operand, zero_points=None, bias=None,
+                         constant=("B", "scales", "zero_points", "bias"), operand_is_constant=True,
+                         product_input_index=0, product_is_graph_output=False, extra_consumer=False, repeat=1):
+    """MatMulNBits followed by Add(product, operand) through the plugin EP's compile path.  Returns (sum, trace);
+    raises EpHostError with code NOT_FUSED when the plugin leaves the pair un-fused."""
+    lib = _load()
+    names = ["A", "B", "scales", "zero_points", "g_idx", "bias"]
+    tensors, mask, keep = _tensors([A, B, scales, zero_points, None, bias], names, constant)
+    op_t, _, keep2 = _tensors([operand], ["operand"], ())
+    add = EpHostAddSpec(op_t[0], int(operand_is_constant), int(product_input_index), int(product_is_graph_output),
+                        int(extra_consumer))
+    y = np.empty(A.shape[:-1] + (N,), dtype=A.dtype)
+    y_dims = (ctypes.c_int64 * 8)()
+    y_rank = ctypes.c_size_t(0)
+    trace, err = ctypes.create_string_buffer(512), ctypes.create_string_buffer(2048)
+    rc = lib.EpHostRunMatMulNBitsAdd(str(PLUGIN).encode(), N, K, bits, block_size, tensors, mask, ctypes.byref(add),
+                                     y.ctypes.data if y.size else None, y.nbytes, y_dims, ctypes.byref(y_rank),
+                                     repeat, trace, len(trace), err, len(err))
+    del keep, keep2
+    if rc != 0:
+        raise EpHostError(rc, err.value.decode(), trace.value.decode())
+    assert tuple(y_dims[i] for i in range(y_rank.value)) == y.shape
     return y, trace.value.decode()

@@ -99,11 +99,15 @@ struct OrtOpAttr {
 };
 struct OrtValueInfo {
   std::string name;
+  const OrtValue* initializer = nullptr;  // host tensor of a constant initializer
+  bool is_graph_output = false;
+  std::vector<std::pair<const OrtNode*, int64_t>> consumers = {};  // (node, input index)
 };
 struct OrtNode {
   std::string op, domain, name;
   int since_version = 1;
   std::vector<std::unique_ptr<OrtValueInfo>> inputs;  // NULL entry = omitted optional input
+  std::vector<std::unique_ptr<OrtValueInfo>> outputs = {};
   std::vector<OrtOpAttr> attrs;
   std::vector<std::string> schema_attrs;                     // attribute names the operator schema knows
   std::map<std::string, ONNXTensorElementDataType> types;    // type-constraint name -> bound element type
@@ -115,6 +119,11 @@ struct OrtEpGraphSupportInfo {
   const OrtKernelRegistry* registry;
   std::string ep_name;
   std::vector<const OrtNode*> claimed;
+  std::vector<std::vector<const OrtNode*>> fused = {};  // groups handed to EpGraphSupportInfo_AddNodesToFuse
+  std::vector<bool> fused_drops_constants = {};
+};
+struct OrtNodeComputeContext {
+  std::string node_name;
 };
 struct OrtKernelInfo {
   const OrtNode* node;
@@ -368,6 +377,43 @@ void FillApisOnce() {
     for (size_t i = 0; i < count && i < n->inputs.size(); ++i) inputs[i] = n->inputs[i].get();
     return nullptr;
   };
+  g_ort.Node_GetNumOutputs = [](const OrtNode* n, size_t* out) noexcept -> OrtStatus* {
+    *out = n->outputs.size();
+    return nullptr;
+  };
+  g_ort.Node_GetOutputs = [](const OrtNode* n, const OrtValueInfo** outputs, size_t count) noexcept -> OrtStatus* {
+    for (size_t i = 0; i < count && i < n->outputs.size(); ++i) outputs[i] = n->outputs[i].get();
+    return nullptr;
+  };
+  g_ort.GetValueInfoName = [](const OrtValueInfo* v, const char** out) noexcept -> OrtStatus* {
+    *out = v->name.c_str();
+    return nullptr;
+  };
+  g_ort.ValueInfo_IsConstantInitializer = [](const OrtValueInfo* v, bool* out) noexcept -> OrtStatus* {
+    *out = v->initializer != nullptr;
+    return nullptr;
+  };
+  g_ort.ValueInfo_GetInitializerValue = [](const OrtValueInfo* v, const OrtValue** out) noexcept -> OrtStatus* {
+    *out = v->initializer;  // NULL when the value is not an initializer, like the real call
+    return nullptr;
+  };
+  g_ort.ValueInfo_IsGraphOutput = [](const OrtValueInfo* v, bool* out) noexcept -> OrtStatus* {
+    *out = v->is_graph_output;
+    return nullptr;
+  };
+  g_ort.ValueInfo_GetValueNumConsumers = [](const OrtValueInfo* v, size_t* out) noexcept -> OrtStatus* {
+    *out = v->consumers.size();
+    return nullptr;
+  };
+  g_ort.ValueInfo_GetValueConsumers = [](const OrtValueInfo* v, const OrtNode** nodes, int64_t* indices,
+                                         size_t count) noexcept -> OrtStatus* {
+    if (count < v->consumers.size()) return MakeStatus(ORT_INVALID_ARGUMENT, "consumer buffers are too small");
+    for (size_t i = 0; i < v->consumers.size(); ++i) {
+      nodes[i] = v->consumers[i].first;
+      indices[i] = v->consumers[i].second;
+    }
+    return nullptr;
+  };
   g_ort.Node_GetAttributeByName = [](const OrtNode* n, const char* name, const OrtOpAttr** out) noexcept
       -> OrtStatus* {
     *out = nullptr;
@@ -414,6 +460,13 @@ void FillApisOnce() {
   };
   g_ep.EpGraphSupportInfo_AddSingleNode = [](OrtEpGraphSupportInfo* g, const OrtNode* n) noexcept -> OrtStatus* {
     g->claimed.push_back(n);
+    return nullptr;
+  };
+  g_ep.EpGraphSupportInfo_AddNodesToFuse = [](OrtEpGraphSupportInfo* g, const OrtNode* const* nodes, size_t n,
+                                             const OrtNodeFusionOptions* options) noexcept -> OrtStatus* {
+    if (n == 0 || nodes == nullptr) return MakeStatus(ORT_INVALID_ARGUMENT, "Must specify a valid array of nodes");
+    g->fused.emplace_back(nodes, nodes + n);
+    g->fused_drops_constants.push_back(options != nullptr && options->drop_constant_initializers);
     return nullptr;
   };
   g_ep.EpGraphSupportInfo_LookUpKernel = [](OrtEpGraphSupportInfo* g, const OrtNode* n,
@@ -577,7 +630,8 @@ enum {
   EP_HOST_NOT_CLAIMED = -1,   // GetCapability left the node to the CPU provider
   EP_HOST_LOAD_FAILED = -2,
   EP_HOST_NO_DEVICE = -3,     // the factory offered no OrtEpDevice
-  EP_HOST_PROTOCOL = -4       // the plugin broke an expectation of the host
+  EP_HOST_PROTOCOL = -4,      // the plugin broke an expectation of the host
+  EP_HOST_NOT_FUSED = -5      // a MatMulNBits + Add pair was offered and the plugin did not ask to fuse it
 };
 
 // Factory-level queries that need no GPU. Writes "name|vendor|vendor_id|version|num_ep_devices" into `out`.
@@ -634,6 +688,15 @@ struct EpHostNodeSpec {
   int skipped_output_mask;          // bit o: optional output o is not used by the graph
 };
 
+// An Add node behind output 0 of the node under test (the graph ONNX Runtime's MatMulNBitsFusion would rewrite).
+struct EpHostAddSpec {
+  EpHostTensor operand;         // the other Add input
+  int operand_is_constant;      // it is a constant initializer
+  int product_input_index;      // which Add input (0 or 1) the product feeds
+  int product_is_graph_output;  // the product is also a graph output
+  int extra_consumer;           // a second node consumes the product as well
+};
+
 // One output buffer of the caller.
 struct EpHostOutput {
   void* data;
@@ -653,8 +716,14 @@ namespace {
 // tensors.  Compute is called `repeat` times; the outputs of the last call are copied to `outs`.
 // Returns 0, an OrtErrorCode reported by the plugin, or a negative EP_HOST_* code; `trace` receives a short log
 // ("claimed=1 prepacked=1,2,3 ...").
+//
+// With `add` the graph has a second node, Add(product, operand) in either input order.  The plugin is then expected
+// to claim both nodes as one group (EpGraphSupportInfo_AddNodesToFuse); the host calls OrtEp::Compile on that group
+// and runs the OrtNodeComputeInfo it returns, feeding only the non-constant inputs as ONNX Runtime does when the
+// group was fused with drop_constant_initializers.  A pair the plugin leaves un-fused ends with EP_HOST_NOT_FUSED.
 int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTensor* inputs, int constant_mask,
-            EpHostOutput* outs, int repeat, char* trace_buf, size_t trace_len, char* err, size_t err_len) {
+            EpHostOutput* outs, int repeat, char* trace_buf, size_t trace_len, char* err, size_t err_len,
+            const EpHostAddSpec* add = nullptr) {
   const size_t NI = spec.num_inputs;
   FillApis();
   Trace trace{trace_buf, trace_len};
@@ -705,7 +774,23 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
   if (registry == nullptr) return HostFail(EP_HOST_PROTOCOL, "GetKernelRegistry returned NULL", err, err_len);
   trace.add("kernels=%zu ", registry->entries.size());
 
-  // ---- the graph: one node
+  // ---- host views of the caller's tensors (initializers stay host tensors, as in a loaded model)
+  auto host_view = [&](const EpHostTensor& t) {
+    auto v = std::make_unique<OrtValue>();
+    v->dims.assign(t.dims, t.dims + t.rank);
+    v->type = static_cast<ONNXTensorElementDataType>(t.dtype);
+    v->bytes = ByteSize(v->dims, v->type);
+    v->data = const_cast<void*>(t.data);
+    v->mem = &cpu_mem;
+    return v;
+  };
+  std::vector<std::unique_ptr<OrtValue>> host_values(NI), device_values(NI);
+  for (size_t i = 0; i < NI; ++i)
+    if (inputs[i].data != nullptr) host_values[i] = host_view(inputs[i]);
+  std::unique_ptr<OrtValue> add_operand_value;
+  if (add != nullptr && add->operand.data != nullptr) add_operand_value = host_view(add->operand);
+
+  // ---- the graph: the node under test, optionally followed by an Add
   OrtNode node;
   node.op = spec.op_type;
   node.domain = "com.microsoft";
@@ -732,16 +817,66 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
       continue;
     }
     node.inputs.emplace_back(new OrtValueInfo{kInputNames[i]});
+    if (i != 0 && ((constant_mask >> i) & 1)) node.inputs.back()->initializer = host_values[i].get();
     auto t = static_cast<ONNXTensorElementDataType>(inputs[i].dtype);
     auto it = node.types.find(kInputTypes[i]);
     if (it == node.types.end()) node.types[kInputTypes[i]] = t;
   }
+  for (size_t o = 0; o < spec.num_outputs; ++o) {
+    node.outputs.emplace_back(new OrtValueInfo{"out" + std::to_string(o)});
+    node.outputs.back()->is_graph_output = true;
+  }
+  OrtNode add_node, other_consumer;
   OrtGraph graph;
   graph.nodes.push_back(&node);
+  if (add != nullptr) {
+    OrtValueInfo& product = *node.outputs[0];
+    const int pi = add->product_input_index ? 1 : 0;
+    product.is_graph_output = add->product_is_graph_output != 0;
+    product.consumers.emplace_back(&add_node, pi);
+    if (add->extra_consumer) product.consumers.emplace_back(&other_consumer, 0);
+    add_node.op = "Add";
+    add_node.domain = "";
+    add_node.name = "add0";
+    add_node.since_version = 14;
+    add_node.inputs.resize(2);
+    add_node.inputs[pi].reset(new OrtValueInfo{product.name});
+    add_node.inputs[1 - pi].reset(new OrtValueInfo{"add_operand"});
+    if (add->operand_is_constant) add_node.inputs[1 - pi]->initializer = add_operand_value.get();
+    add_node.outputs.emplace_back(new OrtValueInfo{"sum"});
+    add_node.outputs.back()->is_graph_output = true;
+    add_node.types["T"] = static_cast<ONNXTensorElementDataType>(inputs[0].dtype);
+    graph.nodes.push_back(&add_node);
+    if (add->extra_consumer) {
+      other_consumer.op = "Identity";
+      other_consumer.domain = "";
+      other_consumer.name = "identity0";
+      other_consumer.since_version = 14;
+      other_consumer.inputs.emplace_back(new OrtValueInfo{product.name});
+      other_consumer.outputs.emplace_back(new OrtValueInfo{"copy"});
+      other_consumer.outputs.back()->is_graph_output = true;
+      other_consumer.types["T"] = add_node.types["T"];
+      graph.nodes.push_back(&other_consumer);
+    }
+  }
   OrtEpGraphSupportInfo support{registry, ep_name, {}};
   if (OrtStatus* st = ep->GetCapability(ep, &graph, &support)) return Fail(st, "GetCapability", err, err_len);
-  trace.add("claimed=%zu ", support.claimed.size());
-  if (support.claimed.empty()) return HostFail(EP_HOST_NOT_CLAIMED, "node not claimed", err, err_len);
+  trace.add("claimed=%zu fused=%zu ", support.claimed.size(), support.fused.size());
+  if (support.claimed.empty() && support.fused.empty())
+    return HostFail(EP_HOST_NOT_CLAIMED, "node not claimed", err, err_len);
+  // A node may be claimed once: singly or in one fused group.
+  for (const auto& group : support.fused)
+    for (const OrtNode* n : group)
+      for (const OrtNode* c : support.claimed)
+        if (c == n) return HostFail(EP_HOST_PROTOCOL, "a node was claimed both singly and in a fused group", err, err_len);
+  const bool compiled = add != nullptr && support.fused.size() == 1 && support.fused[0].size() == 2 &&
+                        support.fused[0][0] == &node && support.fused[0][1] == &add_node;
+  if (add != nullptr && !compiled) {
+    if (!support.fused.empty()) return HostFail(EP_HOST_PROTOCOL, "unexpected fused group", err, err_len);
+    return HostFail(EP_HOST_NOT_FUSED, "the MatMulNBits + Add pair was not fused", err, err_len);
+  }
+  if (add == nullptr && !support.fused.empty())
+    return HostFail(EP_HOST_PROTOCOL, "a fused group in a graph of one node", err, err_len);
 
   // ---- session resources
   OrtAllocator* allocator = nullptr;
@@ -770,17 +905,6 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
   OrtSyncStream stream{stream_impl};
 
   // ---- values. Host copies wrap the caller's memory; constants go to the device through the data transfer.
-  std::vector<std::unique_ptr<OrtValue>> host_values(NI), device_values(NI);
-  for (size_t i = 0; i < NI; ++i) {
-    if (inputs[i].data == nullptr) continue;
-    auto v = std::make_unique<OrtValue>();
-    v->dims.assign(inputs[i].dims, inputs[i].dims + inputs[i].rank);
-    v->type = static_cast<ONNXTensorElementDataType>(inputs[i].dtype);
-    v->bytes = ByteSize(v->dims, v->type);
-    v->data = const_cast<void*>(inputs[i].data);
-    v->mem = &cpu_mem;
-    host_values[i] = std::move(v);
-  }
   auto to_device = [&](size_t i, bool with_stream) -> OrtStatus* {
     auto d = std::make_unique<OrtValue>();
     d->dims = host_values[i]->dims;
@@ -797,29 +921,73 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     device_values[i] = std::move(d);
     return st;
   };
-  for (size_t i = 1; i < NI; ++i) {
+  for (size_t i = 1; i < NI && !compiled; ++i) {
     if (!host_values[i]) continue;
     // initializers are copied without a stream at session initialisation, run inputs on the run's stream
     if (OrtStatus* st = to_device(i, !((constant_mask >> i) & 1))) return Fail(st, "CopyTensors", err, err_len);
   }
 
+  // ---- the compiled route: OrtEp::Compile on the fused group
+  struct ComputeInfoGuard {
+    OrtEp* e;
+    OrtNodeComputeInfo* info = nullptr;
+    void* state = nullptr;
+    bool has_state = false;
+    ~ComputeInfoGuard() {
+      if (info == nullptr) return;
+      if (has_state) info->ReleaseState(info, state);
+      e->ReleaseNodeComputeInfos(e, &info, 1);
+    }
+  } compute_info{ep};
+  if (compiled) {
+    if (!support.fused_drops_constants[0])
+      return HostFail(EP_HOST_PROTOCOL, "this host models fused nodes without their constant initializers only", err, err_len);
+    if (ep->Compile == nullptr || ep->ReleaseNodeComputeInfos == nullptr)
+      return HostFail(EP_HOST_PROTOCOL, "nodes were fused but OrtEp::Compile is not implemented", err, err_len);
+    OrtGraph subgraph;
+    subgraph.nodes = support.fused[0];
+    OrtNode fused_node;
+    fused_node.op = ep_name + "_fused_0";
+    fused_node.name = fused_node.op;
+    fused_node.inputs.emplace_back(new OrtValueInfo{kInputNames[0]});
+    fused_node.outputs.emplace_back(new OrtValueInfo{"sum"});
+    const OrtGraph* graphs[1] = {&subgraph};
+    const OrtNode* fused_nodes[1] = {&fused_node};
+    OrtNodeComputeInfo* infos[1] = {nullptr};
+    OrtNode* ep_context_nodes[1] = {nullptr};
+    if (OrtStatus* st = ep->Compile(ep, graphs, fused_nodes, 1, infos, ep_context_nodes)) return Fail(st, "Compile", err, err_len);
+    if (infos[0] == nullptr) return HostFail(EP_HOST_PROTOCOL, "Compile returned no OrtNodeComputeInfo", err, err_len);
+    compute_info.info = infos[0];
+    OrtNodeComputeContext node_context{fused_node.name};
+    if (OrtStatus* st = infos[0]->CreateState(infos[0], &node_context, &compute_info.state))
+      return Fail(st, "CreateState", err, err_len);
+    compute_info.has_state = true;
+    trace.add("compiled=1 ");
+  }
+
   // ---- kernel creation + PrePack
-  const auto* entry = LookUp(*registry, ep_name, node);
-  if (entry == nullptr) return HostFail(EP_HOST_PROTOCOL, "claimed node without a kernel", err, err_len);
+  struct KernelGuard {
+    OrtKernelImpl* k;
+    ~KernelGuard() {
+      if (k != nullptr) k->Release(k);
+    }
+  };
+  const auto* entry = compiled ? nullptr : LookUp(*registry, ep_name, node);
+  if (!compiled && entry == nullptr) return HostFail(EP_HOST_PROTOCOL, "claimed node without a kernel", err, err_len);
   OrtKernelInfo info{&node, {}};
   for (size_t i = 1; i < NI; ++i)
     if (device_values[i] && ((constant_mask >> i) & 1)) info.constants[i] = device_values[i].get();
   OrtKernelImpl* kernel = nullptr;
-  if (OrtStatus* st = entry->fn(entry->state, &info, &kernel)) return Fail(st, "kernel creation", err, err_len);
-  if (kernel == nullptr) return HostFail(EP_HOST_PROTOCOL, "kernel creation returned NULL", err, err_len);
-  struct KernelGuard {
-    OrtKernelImpl* k;
-    ~KernelGuard() { k->Release(k); }
-  } kernel_guard{kernel};
-  if (kernel->flags != 0) return HostFail(EP_HOST_PROTOCOL, "OrtKernelImpl::flags must start as 0", err, err_len);
+  if (!compiled) {
+    if (OrtStatus* st = entry->fn(entry->state, &info, &kernel)) return Fail(st, "kernel creation", err, err_len);
+    if (kernel == nullptr) return HostFail(EP_HOST_PROTOCOL, "kernel creation returned NULL", err, err_len);
+  }
+  KernelGuard kernel_guard{kernel};
+  if (kernel != nullptr && kernel->flags != 0)
+    return HostFail(EP_HOST_PROTOCOL, "OrtKernelImpl::flags must start as 0", err, err_len);
   trace.add("prepacked=");
   std::vector<bool> packed(NI, false);
-  if (kernel->PrePackWeight != nullptr) {
+  if (kernel != nullptr && kernel->PrePackWeight != nullptr) {
     for (size_t i = 1; i < NI; ++i) {
       if (!info.constants.count(i)) continue;
       bool is_packed = false;
@@ -865,11 +1033,17 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     ctx.output_on_host.assign(spec.num_outputs, false);
     ctx.output_skipped.assign(spec.num_outputs, false);
     for (size_t o = 0; o < spec.num_outputs; ++o) ctx.output_skipped[o] = (spec.skipped_output_mask >> o) & 1;
-    ctx.inputs.assign(node.inputs.size(), nullptr);
-    ctx.inputs[0] = copy_in.outputs[0].get();
-    for (size_t i = 1; i < node.inputs.size(); ++i)
-      if (!packed[i] && device_values[i]) ctx.inputs[i] = device_values[i].get();
-    if (OrtStatus* st = kernel->Compute(kernel, &ctx)) return Fail(st, "Compute", err, err_len);
+    if (compiled) {
+      ctx.inputs.assign(1, copy_in.outputs[0].get());  // the fused node's only non-constant input
+      if (OrtStatus* st = compute_info.info->Compute(compute_info.info, compute_info.state, &ctx))
+        return Fail(st, "compiled Compute", err, err_len);
+    } else {
+      ctx.inputs.assign(node.inputs.size(), nullptr);
+      ctx.inputs[0] = copy_in.outputs[0].get();
+      for (size_t i = 1; i < node.inputs.size(); ++i)
+        if (!packed[i] && device_values[i]) ctx.inputs[i] = device_values[i].get();
+      if (OrtStatus* st = kernel->Compute(kernel, &ctx)) return Fail(st, "Compute", err, err_len);
+    }
     for (size_t o = 0; o < spec.num_outputs; ++o) {
       outs[o].produced = 0;
       if (ctx.output_skipped[o]) continue;
@@ -908,6 +1082,32 @@ __attribute__((visibility("default"))) int EpHostRunNode(const char* plugin_path
                                                         EpHostOutput* outs, int repeat, char* trace_buf,
                                                         size_t trace_len, char* err, size_t err_len) {
   return RunNode(plugin_path, *spec, inputs, constant_mask, outs, repeat, trace_buf, trace_len, err, err_len);
+}
+
+// com.microsoft::MatMulNBits followed by Add(product, operand): the pair the plugin is expected to fuse and compile.
+// `inputs` as for EpHostRunMatMulNBits; the sum is copied to `y`.
+__attribute__((visibility("default"))) int EpHostRunMatMulNBitsAdd(
+    const char* plugin_path, int64_t N, int64_t K, int64_t bits, int64_t block_size, const EpHostTensor* inputs,
+    int constant_mask, const EpHostAddSpec* add, void* y, size_t y_bytes, int64_t* y_dims, size_t* y_rank, int repeat,
+    char* trace_buf, size_t trace_len, char* err, size_t err_len) {
+  const EpHostAttr attrs[4] = {{"K", 0, K, 0.f, nullptr},
+                               {"N", 0, N, 0.f, nullptr},
+                               {"bits", 0, bits, 0.f, nullptr},
+                               {"block_size", 0, block_size, 0.f, nullptr}};
+  static const char* kSchemaAttrs[5] = {"K", "N", "bits", "block_size", "accuracy_level"};
+  static const char* kInputNames[6] = {"A", "B", "scales", "zero_points", "g_idx", "bias"};
+  static const char* kInputTypes[6] = {"T1", "T2", "T1", "T3", "T4", "T1"};
+  const EpHostNodeSpec spec{"MatMulNBits", attrs, 4, kSchemaAttrs, 5, kInputNames, kInputTypes, 6, 1, 0};
+  EpHostOutput out{};
+  out.data = y;
+  out.capacity = y_bytes;
+  const int rc =
+      RunNode(plugin_path, spec, inputs, constant_mask, &out, repeat, trace_buf, trace_len, err, err_len, add);
+  if (rc == 0) {
+    *y_rank = out.rank;
+    for (size_t i = 0; i < out.rank; ++i) y_dims[i] = out.dims[i];
+  }
+  return rc;
 }
 
 // One com.microsoft::MatMulNBits node; `inputs` has six entries (A, B, scales, zero_points, g_idx, bias).  The result
