@@ -47,7 +47,8 @@ typedef enum MnbDataType {
   MNB_DTYPE_FLOAT = 1,
   MNB_DTYPE_UINT8 = 2,
   MNB_DTYPE_INT32 = 6,
-  MNB_DTYPE_FLOAT16 = 10
+  MNB_DTYPE_FLOAT16 = 10,
+  MNB_DTYPE_BFLOAT16 = 16 /* activations of the rare-variant entry points only (MnbVariant*) */
 } MnbDataType;
 
 /* Shape of one operator input for MnbCheckInputs; dims == NULL means the optional input is absent. */
@@ -194,6 +195,69 @@ MNB_API int MnbQkvGemm(size_t M, size_t Nq, size_t Nkv, size_t K, int bits, int 
 /* The prologue alone (what the fused calls run first): a_norm_dev T[M][K], dense. */
 MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* a_dev, size_t lda,
                                    const MnbNormPrologue* norm, void* a_norm_dev, void* stream);
+
+/* ---- rare operand variants -----------------------------------------------------------------------------------------
+ * The inputs the reference kernel serves through its dequantise-everything route and calls "very rare"
+ * (MatMulNBits<T>::ComputeBUnpacked, onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc:1184-1333, fp16
+ * :1336-1510): zero points in the activation type (input zero_points of type T1, shape [N][k_blocks]), a group index
+ * (input g_idx, int32[K] or [k_blocks*block_size]: element k of every column uses scale and zero point of block
+ * g_idx[k]; dequantisation onnxruntime/contrib_ops/cpu/quantization/matmul_nbits_impl.cc:19-75), and bfloat16
+ * activations (type constraint T1 of the schema, contrib_defs.cc:3782-3849; the reference has no CPU kernel for it).
+ *
+ * They run on the same GEMM kernels as MnbGemm after a transformation made once, at pack time:
+ *   g_idx            the k index is permuted so that the elements of one group are adjacent, every group is padded to
+ *                    a multiple of 16 elements, and the matrix is packed with block size 16; the activation columns
+ *                    are gathered into that order (zeros in the padding) in front of every GEMM.  A g_idx equal to
+ *                    k / block_size is recognised and dropped.
+ *   typed zero points, bfloat16:  scales and zero points are widened to fp32 (exactly) and the fp32 kernels run on
+ *                    a widened copy of the activations; the fp32 result plus bias is narrowed once.  This is the
+ *                    reference's own arithmetic for these inputs (fp32 SGEMM on widened operands, :1336-1510).
+ * Zero points are honoured together with g_idx for both zero-point types, as the schema defines; the reference's CPU
+ * dequantiser reads uint8 zero points in that combination but then uses 8 (matmul_nbits_impl.cc:56-66).
+ * Supported: g_idx with bits = 4; typed zero points with bits = 2 or 4 (the reference rejects 8, :1251-1252). */
+typedef enum MnbZeroPointKind {
+  MNB_ZP_NONE = 0,  /* no zero_points input: 2^(bits-1) */
+  MNB_ZP_UINT8 = 1, /* packed uint8, [N][ceil(k_blocks*bits/8)] */
+  MNB_ZP_TYPED = 2  /* activation type, [N][k_blocks] */
+} MnbZeroPointKind;
+
+/* Filled by MnbVariantMakePlan; plain data the caller keeps next to the packed buffer. */
+typedef struct MnbVariantPlan {
+  int64_t N, K;
+  int bits, block_size; /* of the operator */
+  int a_dtype;          /* MNB_DTYPE_FLOAT, MNB_DTYPE_FLOAT16 or MNB_DTYPE_BFLOAT16 */
+  int zp_kind;          /* MnbZeroPointKind */
+  int has_g_idx;        /* a g_idx that is not k / block_size: activations are gathered per call */
+  int compute_dtype;    /* element type the GEMM kernels run in: a_dtype or MNB_DTYPE_FLOAT */
+  int64_t packed_k;     /* k extent of the packed matrix (K without g_idx) */
+  int packed_block_size;
+  int reserved;
+  uint64_t gather_offset; /* byte offset of the int32 gather table inside the packed buffer */
+  uint64_t packed_bytes;  /* size of the packed buffer */
+} MnbVariantPlan;
+
+/* g_idx_host: HOST pointer to g_idx_len int32 values, or NULL.  Fails with MNB_INVALID_ARGUMENT when a value lies
+ * outside [0, k_blocks) and with MNB_NOT_IMPLEMENTED for a combination without kernels. */
+MNB_API int MnbVariantMakePlan(size_t N, size_t K, int bits, int block_size, int a_dtype, int zp_kind,
+                               const int32_t* g_idx_host, size_t g_idx_len, MnbVariantPlan* plan);
+/* Packs the canonical operands (device pointers; scales and typed zero points in a_dtype) into packed_dev
+ * (plan->packed_bytes, 256-byte aligned).  g_idx_host must be the array the plan was made from.  Synchronises the
+ * stream when the plan has a g_idx (the gather table is uploaded from pageable host memory). */
+MNB_API int MnbVariantPack(const MnbVariantPlan* plan, const void* b_dev, const void* scales_dev,
+                           const void* zero_points_dev, const int32_t* g_idx_host, size_t g_idx_len, void* packed_dev,
+                           void* stream);
+MNB_API size_t MnbVariantGemmWorkspaceSize(const MnbVariantPlan* plan, size_t M);
+/* Y[M][ldy] = A[M][lda] x W (+ bias), A, bias and Y in plan->a_dtype. */
+MNB_API int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size_t lda, const void* packed_dev,
+                           const void* bias_dev, void* y_dev, size_t ldy, void* workspace_dev, size_t workspace_bytes,
+                           void* stream);
+/* The reference's dequantiser for these inputs, dst_dev float[N][K] whatever a_dtype is
+ * (Dequantize4BitsKernelReOrder, matmul_nbits_impl.cc:19-75; 2 bits: MlasDequantizeBlockwiseFpZeroPoint,
+ * onnxruntime/core/mlas/lib/q4_dq.cpp:2187-2241): scales and zero points widened to fp32,
+ * w = float(q) * scale + (-scale * zp), each operation rounded on its own.  g_idx_dev: device pointer or NULL. */
+MNB_API int MnbVariantDequantize(float* dst_dev, const void* b_dev, const void* scales_dev,
+                                 const void* zero_points_dev, int zp_kind, const int32_t* g_idx_dev, size_t N,
+                                 size_t K, int bits, int block_size, int a_dtype, void* stream);
 
 /* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
 MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);

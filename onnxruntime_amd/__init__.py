@@ -3,7 +3,8 @@ from ._lib import MnbError, LIB_PATH  # noqa: F401
 
 
 def __getattr__(name):
-    if name in ("MatMulNBits", "check_inputs", "dequantize_blockwise", "quantize_blockwise", "MatMulNBitsMlp",
+    if name in ("MatMulNBits", "check_inputs", "dequantize_blockwise", "dequantize_blockwise_variant", "quantize_blockwise",
+                "MatMulNBitsMlp",
                 "MatMulNBitsQkv", "simplified_layer_norm"):
         from . import matmul_nbits
         return getattr(matmul_nbits, name)

@@ -17,6 +17,7 @@ DTYPE_FLOAT = 1
 DTYPE_UINT8 = 2
 DTYPE_INT32 = 6
 DTYPE_FLOAT16 = 10
+DTYPE_BFLOAT16 = 16
 
 OK, FAIL, INVALID_ARGUMENT, NOT_IMPLEMENTED, EP_FAIL = 0, 1, 2, 9, 11
 
@@ -37,6 +38,19 @@ class MnbNormPrologue(ctypes.Structure):
 
 
 _NORM_P = ctypes.POINTER(MnbNormPrologue)
+
+ZP_NONE, ZP_UINT8, ZP_TYPED = 0, 1, 2
+
+
+class MnbVariantPlan(ctypes.Structure):
+    _fields_ = [("N", c_int64), ("K", c_int64), ("bits", c_int), ("block_size", c_int), ("a_dtype", c_int),
+                ("zp_kind", c_int), ("has_g_idx", c_int), ("compute_dtype", c_int), ("packed_k", c_int64),
+                ("packed_block_size", c_int), ("reserved", c_int), ("gather_offset", ctypes.c_uint64),
+                ("packed_bytes", ctypes.c_uint64)]
+
+
+_PLAN_P = ctypes.POINTER(MnbVariantPlan)
+_I32_P = ctypes.POINTER(ctypes.c_int32)
 
 # name -> (restype, argtypes); every symbol include/mnb_mi355x.h declares
 SIGNATURES = {
@@ -71,6 +85,13 @@ SIGNATURES = {
                            c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t,
                            c_void_p]),
     "MnbSimplifiedLayerNorm": (c_int, [c_size_t, c_size_t, c_int, c_void_p, c_size_t, _NORM_P, c_void_p, c_void_p]),
+    "MnbVariantMakePlan": (c_int, [c_size_t, c_size_t, c_int, c_int, c_int, c_int, _I32_P, c_size_t, _PLAN_P]),
+    "MnbVariantPack": (c_int, [_PLAN_P, c_void_p, c_void_p, c_void_p, _I32_P, c_size_t, c_void_p, c_void_p]),
+    "MnbVariantGemmWorkspaceSize": (c_size_t, [_PLAN_P, c_size_t]),
+    "MnbVariantGemm": (c_int, [_PLAN_P, c_size_t, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p,
+                               c_size_t, c_void_p]),
+    "MnbVariantDequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_size_t,
+                                     c_int, c_int, c_int, c_void_p]),
     "MnbMeasureReadBandwidth": (c_int, [c_size_t, c_int, ctypes.POINTER(ctypes.c_double)]),
     "MnbMeasureMfmaRate": (c_int, [c_int, ctypes.POINTER(ctypes.c_double)]),
     "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),

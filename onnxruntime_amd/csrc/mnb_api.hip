@@ -81,6 +81,11 @@ bool present(const MnbTensorInfo* t) { return t != nullptr && t->dims != nullptr
 
 }  // namespace
 
+int mnb_report_error(int code, const char* message) {
+  g_last_error = message;
+  return code;
+}
+
 extern "C" {
 
 const char* MnbGetLastErrorMessage(void) { return g_last_error.c_str(); }

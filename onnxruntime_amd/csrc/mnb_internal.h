@@ -39,6 +39,11 @@ enum MnbKernelKind {
 MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a);
 const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout& L);
 
+// records `message` as the calling thread's last error (MnbGetLastErrorMessage) and returns `code`
+int mnb_report_error(int code, const char* message);
+
+// weights only, one source matrix (the meta part of the packed buffer is written by the caller)
+hipError_t mnb_launch_pack_weights(const MnbLayout& L, const void* B, void* packed, hipStream_t s);
 hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
                            hipStream_t s);
 hipError_t mnb_launch_pack_fused(const MnbFusedLayout& F, const void* const* B, const void* const* scales,

@@ -215,6 +215,25 @@ static hipError_t pack_t(const MnbLayout& L, const MnbPackSrc& S, const void* zp
   return hipGetLastError();
 }
 
+hipError_t mnb_launch_pack_weights(const MnbLayout& L, const void* B, void* packed, hipStream_t s) {
+  MnbPackSrc S{};
+  S.B[0] = reinterpret_cast<const uint8_t*>(B);
+  S.map.kind = kMnbFusedNone;
+  S.map.nsrc = 1;
+  S.map.n[0] = L.N;
+  S.map.Np = L.N;
+  uint4* W = reinterpret_cast<uint4*>(packed);
+  const int64_t wn = L.Npad * L.KG;
+  const dim3 grid((unsigned)((wn + 255) / 256)), blk(256);
+  if (L.src_bits == 2)
+    mnb_pack_weights_kernel<2><<<grid, blk, 0, s>>>(S, W, L);
+  else if (L.bits == 4)
+    mnb_pack_weights_kernel<4><<<grid, blk, 0, s>>>(S, W, L);
+  else
+    mnb_pack_weights_kernel<8><<<grid, blk, 0, s>>>(S, W, L);
+  return hipGetLastError();
+}
+
 hipError_t mnb_launch_pack(const MnbLayout& L, const void* B, const void* scales, const void* zp, void* packed,
                            hipStream_t s) {
   MnbPackSrc S{};

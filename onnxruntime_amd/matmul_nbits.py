@@ -5,6 +5,8 @@ The class follows contrib::MatMulNBits<T1> (onnxruntime/contrib_ops/cpu/quantiza
   PrePack       shape guards + repack of B / scales / zero points  :252-724 (fp16: :729-859)
   Compute       CheckInputs, output shape, empty-output return,    :1513-1570
                 packed or unpacked route
+The inputs the reference serves through its dequantise-everything route (:1248-1295: zero points in the activation
+type, a group index) and bfloat16 activations go through the library's variant entry points.
 Tensors are torch tensors on a HIP device; torch only provides memory and streams here.
 """
 from __future__ import annotations
@@ -20,7 +22,7 @@ from ._lib import MnbError, MnbTensorInfo
 A, B, SCALES, ZERO_POINTS, G_IDX, BIAS = range(6)  # operator input indices (contrib_defs.cc:3794-3828)
 
 _DTYPES = {torch.float32: _lib.DTYPE_FLOAT, torch.float16: _lib.DTYPE_FLOAT16, torch.uint8: _lib.DTYPE_UINT8,
-           torch.int32: _lib.DTYPE_INT32}
+           torch.int32: _lib.DTYPE_INT32, torch.bfloat16: _lib.DTYPE_BFLOAT16}
 
 
 def _info(shape: Optional[Sequence[int]], dtype) -> MnbTensorInfo:
@@ -70,12 +72,26 @@ class MatMulNBits:
         self.blob_size = self.block_size * self.bits // 8
         self.zp_row = (self.k_blocks * self.bits + 7) // 8
         self.lib = _lib.load()
+        # typed zero points, a group index, bfloat16: the variant entry points
+        self.variant = has_g_idx or zero_points_dtype != torch.uint8 or dtype == torch.bfloat16
         # what this device path takes; everything else stays with the CPU provider
-        self.supported = (dtype in (torch.float16, torch.float32) and bits in (2, 4, 8) and not has_g_idx
-                          and zero_points_dtype == torch.uint8
-                          and bool(self.lib.MnbIsAvailable(bits, block_size, _DTYPES[dtype])))
+        if self.variant:
+            self.supported = (dtype in (torch.float16, torch.float32, torch.bfloat16)
+                              and zero_points_dtype in (torch.uint8, dtype)
+                              and (zero_points_dtype == torch.uint8 or bits in (2, 4))   # matmul_nbits.cc:1251-1252
+                              and (not has_g_idx or bits == 4))
+        else:
+            self.supported = (dtype in (torch.float16, torch.float32) and bits in (2, 4, 8)
+                              and bool(self.lib.MnbIsAvailable(bits, block_size, _DTYPES[dtype])))
         self.packed: Optional[torch.Tensor] = None
+        self.plan: Optional[_lib.MnbVariantPlan] = None
         self._workspace = {}
+
+    @property
+    def zp_kind(self) -> int:
+        if not self.has_zero_points:
+            return _lib.ZP_NONE
+        return _lib.ZP_UINT8 if self.zero_points_dtype == torch.uint8 else _lib.ZP_TYPED
 
     # -- PrePack ------------------------------------------------------------------------------------------------
     def _validate_initializer(self, idx: int, t: torch.Tensor) -> None:
@@ -103,7 +119,27 @@ class MatMulNBits:
                                f"MatMulNBits PrePack: zero_points initializer shape {s} does not match "
                                f"attribute-derived shape [{n * kb}] or [{n},{kb}]")
 
-    def PrePack(self, b: torch.Tensor, scales: torch.Tensor, zero_points: Optional[torch.Tensor] = None) -> bool:
+    def _pack_variant(self, b, scales, zero_points, g_idx):
+        """(plan, packed buffer) for the variant route; g_idx is copied to the host, where the k order is planned."""
+        if (g_idx is not None) != self.has_g_idx:
+            raise MnbError(_lib.INVALID_ARGUMENT, "MatMulNBits PrePack: g_idx presence differs from the node")
+        if scales.dtype != self.dtype or (zero_points is not None and zero_points.dtype != self.zero_points_dtype):
+            raise MnbError(_lib.INVALID_ARGUMENT, "MatMulNBits PrePack: scales / zero_points types differ from the node")
+        g_host, g_ptr, g_len = None, None, 0
+        if g_idx is not None:
+            g_host = g_idx.to(device="cpu", dtype=torch.int32).contiguous().numpy()
+            g_ptr, g_len = g_host.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), g_host.size
+        plan = _lib.MnbVariantPlan()
+        _lib.check(self.lib.MnbVariantMakePlan(self.N, self.K, self.bits, self.block_size, _DTYPES[self.dtype],
+                                               self.zp_kind, g_ptr, g_len, ctypes.byref(plan)))
+        packed = torch.empty(plan.packed_bytes, dtype=torch.uint8, device=b.device)
+        _lib.check(self.lib.MnbVariantPack(ctypes.byref(plan), _ptr(b.contiguous()), _ptr(scales.contiguous()),
+                                           _ptr(None if zero_points is None else zero_points.contiguous()), g_ptr,
+                                           g_len, _ptr(packed), _stream_ptr(b.device)))
+        return plan, packed
+
+    def PrePack(self, b: torch.Tensor, scales: torch.Tensor, zero_points: Optional[torch.Tensor] = None,
+                g_idx: Optional[torch.Tensor] = None) -> bool:
         """Repacks constant B / scales / zero_points (device tensors, canonical layout) into the tiled layout.
 
         Returns True when the weights were packed (the caller may then drop the originals), False when this
@@ -116,6 +152,9 @@ class MatMulNBits:
             return False
         if (zero_points is not None) != self.has_zero_points:
             raise MnbError(_lib.INVALID_ARGUMENT, "MatMulNBits PrePack: zero_points presence differs from the node")
+        if self.variant:
+            self.plan, self.packed = self._pack_variant(b, scales, zero_points, g_idx)
+            return True
         dt = _DTYPES[self.dtype]
         size = self.lib.MnbPackQuantBDataSize(self.N, self.K, self.bits, self.block_size,
                                               int(self.has_zero_points), dt)
@@ -140,14 +179,15 @@ class MatMulNBits:
 
     def Compute(self, a: torch.Tensor, b: Optional[torch.Tensor] = None, scales: Optional[torch.Tensor] = None,
                 zero_points: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """Y = A x dequant(B)^T (+ bias). b/scales/zero_points are only needed when PrePack did not run."""
+                out: Optional[torch.Tensor] = None, g_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Y = A x dequant(B)^T (+ bias). b/scales/zero_points/g_idx are only needed when PrePack did not run."""
         if not self.supported:
             raise MnbError(_lib.NOT_IMPLEMENTED, "this MatMulNBits configuration has no MI355X kernel")
         check_inputs(None if b is None else tuple(b.shape), None if scales is None else tuple(scales.shape),
-                     None if zero_points is None else tuple(zero_points.shape), None,
+                     None if zero_points is None else tuple(zero_points.shape),
+                     None if g_idx is None else tuple(g_idx.shape),
                      None if bias is None else tuple(bias.shape), self.N, self.K, self.block_size, self.bits,
-                     scales_dtype=self.dtype)
+                     scales_dtype=self.dtype, zp_dtype=self.zero_points_dtype)
         if a.dtype != self.dtype:
             raise MnbError(_lib.INVALID_ARGUMENT, f"A has dtype {a.dtype}, the node was built for {self.dtype}")
         if a.shape[-1] != self.K:
@@ -165,6 +205,18 @@ class MatMulNBits:
         dt = _DTYPES[self.dtype]
         lda = a2.stride(0) if M > 1 else self.K
         stream = _stream_ptr(a.device)
+        if self.variant:
+            plan, packed = self.plan, self.packed
+            if packed is None:  # operands fed per run: plan and pack per call, like the reference's unpacked route
+                if b is None or scales is None:
+                    raise MnbError(_lib.INVALID_ARGUMENT,
+                                   "MatMulNBits: B and scales are required when B was not prepacked")
+                plan, packed = self._pack_variant(b, scales, zero_points, g_idx)
+            wsz = self.lib.MnbVariantGemmWorkspaceSize(ctypes.byref(plan), M)
+            ws = self._get_workspace(a.device, wsz)
+            _lib.check(self.lib.MnbVariantGemm(ctypes.byref(plan), M, _ptr(a2), lda, _ptr(packed), _ptr(bias),
+                                               _ptr(y2), self.N, _ptr(ws), wsz, stream))
+            return y
         if self.packed is not None:
             wsz = self.lib.MnbGemmWorkspaceSize(M, self.N, self.K, self.bits, self.block_size,
                                                 int(self.has_zero_points), dt)
@@ -417,3 +469,22 @@ def quantize_blockwise(w: torch.Tensor, bits: int, block_size: int, symmetric: b
     _lib.check(lib.MnbQuantizeBlockwise(_ptr(b), _ptr(scales), _ptr(zp), _ptr(w), block_size, bits, K, N,
                                         w.stride(0) if K > 1 else N, _DTYPES[w.dtype], _stream_ptr(w.device)))
     return b, scales, zp
+
+
+def dequantize_blockwise_variant(b: torch.Tensor, scales: torch.Tensor, zero_points: Optional[torch.Tensor],
+                                 g_idx: Optional[torch.Tensor], N: int, K: int, bits: int,
+                                 block_size: int) -> torch.Tensor:
+    """The reference's dequantiser for typed zero points and / or a group index on the device
+    (matmul_nbits_impl.cc:19-75): W float32 [N, K] = float(q) * scale + (-scale * zp), whatever the scales' type."""
+    lib = _lib.load()
+    w = torch.empty(N, K, dtype=torch.float32, device=b.device)
+    if zero_points is None:
+        kind = _lib.ZP_NONE
+    else:
+        kind = _lib.ZP_UINT8 if zero_points.dtype == torch.uint8 else _lib.ZP_TYPED
+    g = None if g_idx is None else g_idx.to(torch.int32).contiguous()
+    _lib.check(lib.MnbVariantDequantize(_ptr(w), _ptr(b.contiguous()), _ptr(scales.contiguous()),
+                                        _ptr(None if zero_points is None else zero_points.contiguous()), kind,
+                                        _ptr(g), N, K, bits, block_size, _DTYPES[scales.dtype],
+                                        _stream_ptr(b.device)))
+    return w

@@ -27,6 +27,15 @@
  *   mnbo_matmul_{f32,f16,f64}           pinned: the 23 vectors (exact), integer special cases against
  *                                       numpy int64 matmul, linearity, fp64 agreement
  *   mnbo_quantize_*                     see the header comment of that section
+ *   mnbo_variant_dequantize_f32         typed zero points / g_idx (the reference's "very rare" route,
+ *                                       onnxruntime/contrib_ops/cpu/quantization/matmul_nbits_impl.cc:19-75 and
+ *                                       onnxruntime/core/mlas/lib/q4_dq.cpp:2187-2241).  Pinned by mathematics only
+ *                                       (the reference's tests recompute their expectations and its dequantiser for
+ *                                       this route does not build without the whole runtime): exact cases where no
+ *                                       operation rounds, equality with mnbo_dequantize_f32 on the inputs where both
+ *                                       routes are defined and exact, group selection read back through power-of-two
+ *                                       scales, closeness to the fp64 value.  The last-ulp behaviour of the two-step
+ *                                       formula is PARITY UNPINNED.
  */
 #include <math.h>
 #include <pthread.h>
@@ -148,6 +157,34 @@ void mnbo_dequantize_f16(uint16_t* dst, const uint8_t* B, const uint16_t* scales
       int d = q_at(B, n, k, kbc, bs, bits) - zp_at(zp, n, kb, kbc, bits);
       volatile float v = (float)d * mnbo_f16_to_f32(scales[n * kbc + kb]);
       dst[n * K + k] = mnbo_f32_to_f16(v);
+    }
+}
+
+/* Typed zero points and/or a group index: dst[n*K + k] = float(q) * scale + (-scale * zp), every operation rounded to
+ * fp32 by itself (matmul_nbits_impl.cc:66-73 for T = float; 2 bits: q4_dq.cpp:2227-2238 hands scale and -scale*zp to
+ * a kernel that computes q*scale + that).  Scales and typed zero points arrive widened to fp32 (the fp16 operator
+ * widens them first, matmul_nbits.cc:1352-1366).  block index = g_idx[k] when a group index is given, else k / bs.
+ * zp_kind: 0 none (2^(bits-1)), 1 packed uint8, 2 float [N][k_blocks].
+ * honour_u8_zp_with_g_idx = 0 restates the reference's CPU code literally: with a group index, packed uint8 zero
+ * points are read and then ignored in favour of 8 (matmul_nbits_impl.cc:56-66); 1 applies them, as the operator's
+ * schema defines and as the reference does without a group index. */
+void mnbo_variant_dequantize_f32(float* dst, const uint8_t* B, const float* scales, int zp_kind, const void* zp,
+                                 const int32_t* g_idx, int64_t N, int64_t K, int bits, int64_t bs,
+                                 int honour_u8_zp_with_g_idx) {
+  int64_t kbc = k_blocks_of(K, bs);
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t k = 0; k < K; ++k) {
+      int64_t b = g_idx ? g_idx[k] : k / bs;
+      float s = scales[n * kbc + b];
+      float z = (float)(1 << (bits - 1));
+      if (zp_kind == 2)
+        z = ((const float*)zp)[n * kbc + b];
+      else if (zp_kind == 1 && (!g_idx || honour_u8_zp_with_g_idx))
+        z = (float)zp_at((const uint8_t*)zp, n, b, kbc, bits);
+      volatile float adjust = -s * z;
+      volatile float prod = (float)q_at(B, n, k, kbc, bs, bits) * s;
+      volatile float v = prod + adjust;
+      dst[n * K + k] = v;
     }
 }
 

@@ -77,6 +77,9 @@ class _C:
             lib.mnbo_quantize_f32.argtypes = [_u8p, _f32p, _u8p, _f32p, _i64, _i64, _int, _i64, _int]
             lib.mnbo_quantize_f16.argtypes = [_u8p, _u16p, _u8p, _u16p, _i64, _i64, _int, _i64, _int]
             lib.mnbo_quantize_f16.restype = None
+            lib.mnbo_variant_dequantize_f32.argtypes = [_f32p, _u8p, _f32p, _int, ctypes.c_void_p,
+                                                        ctypes.POINTER(ctypes.c_int32), _i64, _i64, _int, _i64, _int]
+            lib.mnbo_variant_dequantize_f32.restype = None
             lib.mnbo_skip_simplified_layer_norm_f32.argtypes = [_f32p, _f32p, _f32p, _f32p, _i64, _f32p, _f32p,
                                                                 ctypes.c_float, _i64, _i64]
             lib.mnbo_skip_simplified_layer_norm_f32.restype = None
@@ -117,6 +120,27 @@ class _C:
         s = np.ascontiguousarray(scales, np.float32)
         out = np.empty((N, K), np.float32)
         self.lib.mnbo_dequantize_f32(_ptr(out, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), N, K, bits, bs)
+        return out
+
+    def variant_dequantize(self, B, scales, zp, g_idx, N, K, bits, bs, honour_u8_zp_with_g_idx=True) -> np.ndarray:
+        """The reference's dequantiser for typed zero points and / or a group index: W as float32 [N, K].
+
+        ``scales`` float32, float16 or bfloat16-as-uint16 (see ``widen``); ``zp`` None, uint8 (packed) or an array of
+        the scales' type (typed, [N, k_blocks])."""
+        B = np.ascontiguousarray(B, np.uint8)
+        s = np.ascontiguousarray(widen(scales), np.float32)
+        if zp is None:
+            kind, z = 0, None
+        elif zp.dtype == np.uint8 and scales.dtype != np.uint8:
+            kind, z = 1, np.ascontiguousarray(zp)
+        else:
+            kind, z = 2, np.ascontiguousarray(widen(zp), np.float32)
+        g = None if g_idx is None else np.ascontiguousarray(g_idx, np.int32)
+        out = np.empty((N, K), np.float32)
+        self.lib.mnbo_variant_dequantize_f32(_ptr(out, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), kind,
+                                             None if z is None else z.ctypes.data,
+                                             _ptr(g, ctypes.POINTER(ctypes.c_int32)), N, K, bits, bs,
+                                             int(bool(honour_u8_zp_with_g_idx)))
         return out
 
     # -- matmul ---------------------------------------------------------------
@@ -255,6 +279,35 @@ C = _C()
 
 
 # ----------------------------------------------------------------------------- numpy restatement
+
+def widen(x: np.ndarray) -> np.ndarray:
+    """float32 view of a float32 / float16 array, or of bfloat16 values held in a uint16 array (exact)."""
+    x = np.asarray(x)
+    if x.dtype == np.uint16:
+        return (x.astype(np.uint32) << 16).view(np.float32)
+    return x.astype(np.float32)
+
+
+def narrow_bf16(x: np.ndarray) -> np.ndarray:
+    """float32 -> bfloat16 (as uint16), round to nearest even; finite inputs only."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def dense_matmul_f64(A, W, bias=None):
+    """Y = A x W^T (+ bias) in float64 over float32 operands, and the row bound sum_k |a*w| (+ |bias|).
+    W is [N, K] as the dequantisers return it."""
+    a = widen(A).astype(np.float64)
+    a = a.reshape(-1, a.shape[-1])
+    w = np.asarray(W, np.float32).astype(np.float64)
+    y = a @ w.T
+    bound = np.abs(a) @ np.abs(w).T
+    if bias is not None:
+        b = widen(bias).astype(np.float64)
+        y = y + b
+        bound = bound + np.abs(b)
+    return y, bound
+
 
 def np_unpack_q(B: np.ndarray, N: int, K: int, bits: int, bs: int) -> np.ndarray:
     """Quantised integers as int32 [N, k_blocks*bs] from canonical B [N, k_blocks, bs*bits/8]."""

@@ -92,9 +92,52 @@ def test_constructor_and_prepack_guards():
         op.PrePack(b, s, torch.zeros(8, 2, dtype=torch.uint8))
     # configurations the device path declines (they stay on the CPU provider)
     assert MatMulNBits(32, 8, bits=2, block_size=16).supported
-    assert not MatMulNBits(32, 8, has_g_idx=True).supported
-    assert not MatMulNBits(32, 8, has_zero_points=True, zero_points_dtype=torch.float16).supported
-    assert not MatMulNBits(32, 8, dtype=torch.bfloat16).supported
+    # the reference's "very rare" inputs run through the variant entry points, within the reference's own limits
+    assert MatMulNBits(32, 8, has_g_idx=True).supported and MatMulNBits(32, 8, has_g_idx=True).variant
+    assert MatMulNBits(32, 8, has_zero_points=True, zero_points_dtype=torch.float16).supported
+    assert MatMulNBits(32, 8, dtype=torch.bfloat16).supported
+    assert not MatMulNBits(32, 8, bits=8, has_g_idx=True).supported
+    assert not MatMulNBits(32, 8, bits=8, has_zero_points=True, zero_points_dtype=torch.float16).supported
+    assert not MatMulNBits(32, 8, has_zero_points=True, zero_points_dtype=torch.float32).supported  # T3 must be T1
+
+
+def test_variant_plans_without_a_gpu():
+    """Planning is host work: block size 16 in group order, padding, trivial group indices, the reference's limits."""
+    import ctypes
+    import numpy as np
+    lib = _lib.load()
+
+    def plan(N, K, bits, bs, dtype, zp_kind, g=None):
+        p = _lib.MnbVariantPlan()
+        gp, gl = (None, 0) if g is None else (np.ascontiguousarray(g, np.int32), len(g))
+        rc = lib.MnbVariantMakePlan(N, K, bits, bs, dtype, zp_kind,
+                                    None if gp is None else gp.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), gl,
+                                    ctypes.byref(p))
+        return rc, p
+
+    K, bs = 200, 32
+    kb = (K + bs - 1) // bs
+    rc, p = plan(8, K, 4, bs, _lib.DTYPE_FLOAT16, _lib.ZP_NONE, np.arange(K) // bs)
+    assert rc == 0 and not p.has_g_idx and p.packed_k == K and p.packed_block_size == bs   # trivial: dropped
+    assert p.compute_dtype == _lib.DTYPE_FLOAT16
+    g = np.arange(K) % kb                                                                  # groups interleaved
+    rc, p = plan(8, K, 4, bs, _lib.DTYPE_FLOAT16, _lib.ZP_UINT8, g)
+    counts = np.bincount(g, minlength=kb)
+    assert rc == 0 and p.has_g_idx and p.packed_block_size == 16
+    assert p.packed_k == int(((counts + 15) // 16 * 16).sum())
+    assert p.gather_offset < p.packed_bytes
+    rc, p = plan(8, K, 4, bs, _lib.DTYPE_FLOAT16, _lib.ZP_TYPED)
+    assert rc == 0 and p.compute_dtype == _lib.DTYPE_FLOAT and not p.has_g_idx
+    rc, p = plan(8, K, 4, bs, _lib.DTYPE_BFLOAT16, _lib.ZP_NONE)
+    assert rc == 0 and p.compute_dtype == _lib.DTYPE_FLOAT
+    rc, _ = plan(8, K, 4, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, np.full(K, kb))              # group out of range
+    assert rc == _lib.INVALID_ARGUMENT and "outside [0, 7)" in _lib.last_error()
+    rc, _ = plan(8, K, 4, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, np.zeros(K + 1))             # wrong length
+    assert rc == _lib.INVALID_ARGUMENT and "group_index" in _lib.last_error()
+    rc, _ = plan(8, K, 8, bs, _lib.DTYPE_FLOAT, _lib.ZP_TYPED)
+    assert rc == _lib.NOT_IMPLEMENTED and "Only 2b and 4b quantization is supported for unpacked compute" in _lib.last_error()
+    rc, _ = plan(8, K, 8, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, g)
+    assert rc == _lib.NOT_IMPLEMENTED
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
