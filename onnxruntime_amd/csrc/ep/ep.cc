@@ -40,6 +40,27 @@ OrtStatus* ReadIntAttr(const Apis& a, const OrtNode* node, const char* name, int
 
 namespace {
 
+bool IsConstant(const Apis& a, const OrtValueInfo* v) {
+  bool c = false;
+  if (v == nullptr) return false;
+  if (OrtStatus* st = a.ort->ValueInfo_IsConstantInitializer(v, &c)) {
+    a.ort->ReleaseStatus(st);
+    return false;
+  }
+  return c;
+}
+
+// Element type of a tensor value; UNDEFINED when the value is not a tensor.
+OrtStatus* ElementTypeOf(const Apis& a, const OrtValueInfo* v, ONNXTensorElementDataType* type) {
+  *type = ONNX_TENSOR_ELEMENT_DATA_TYPE_UNDEFINED;
+  const OrtTypeInfo* info = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->GetValueInfoTypeInfo(v, &info));
+  const OrtTensorTypeAndShapeInfo* tensor = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->CastTypeInfoToTensorInfo(info, &tensor));
+  if (tensor == nullptr) return nullptr;
+  return a.ort->GetTensorElementType(tensor, type);
+}
+
 // Static screening of one MatMulNBits node: the conditions under which the reference kernel itself would not run
 // its fast path are kept on the CPU provider instead of failing at run time on the device
 // (onnxruntime/contrib_ops/cpu/quantization/matmul_nbits.cc:112-139 for the attribute checks).
@@ -56,9 +77,30 @@ OrtStatus* MatMulNBitsNodeSupported(const Apis& a, const OrtNode* node, bool* su
   if (num_inputs < 3) return nullptr;
   std::vector<const OrtValueInfo*> inputs(num_inputs, nullptr);
   MI_RETURN_IF_ERROR(a.ort->Node_GetInputs(node, inputs.data(), num_inputs));
-  if (num_inputs > 4 && inputs[4] != nullptr) return nullptr;  // g_idx: no device kernel
-  // The activation type decides the kernel family; both registered types have kernels for every (bits, block).
-  *supported = MnbIsAvailable(static_cast<int>(bits), static_cast<int>(block_size), MNB_DTYPE_FLOAT16) != 0;
+  if (inputs[0] == nullptr || inputs[1] == nullptr || inputs[2] == nullptr) return nullptr;
+  // Both plain activation types have kernels for every (bits, block).
+  if (!MnbIsAvailable(static_cast<int>(bits), static_cast<int>(block_size), MNB_DTYPE_FLOAT16)) return nullptr;
+
+  // A group index, zero points in the activation type and bfloat16 activations - the inputs the reference serves
+  // through its dequantise-everything route (matmul_nbits.cc:1248-1295) - are transformed once, when the weights are
+  // packed, so everything the packed buffer depends on has to be a constant initializer; the limits on bits are the
+  // reference's own (:1251-1252, :1258-1259).
+  const OrtValueInfo* zp = num_inputs > 3 ? inputs[3] : nullptr;
+  const OrtValueInfo* g_idx = num_inputs > 4 ? inputs[4] : nullptr;
+  ONNXTensorElementDataType t1 = ONNX_TENSOR_ELEMENT_DATA_TYPE_UNDEFINED;
+  ONNXTensorElementDataType t3 = ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8;
+  MI_RETURN_IF_ERROR(ElementTypeOf(a, inputs[0], &t1));
+  if (zp != nullptr) MI_RETURN_IF_ERROR(ElementTypeOf(a, zp, &t3));
+  const bool typed_zp = t3 != ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8;
+  const bool bf16 = t1 == ONNX_TENSOR_ELEMENT_DATA_TYPE_BFLOAT16;
+  if (g_idx != nullptr || typed_zp || bf16) {
+    if (typed_zp && (t3 != t1 || (bits != 2 && bits != 4))) return nullptr;
+    if (g_idx != nullptr && bits != 4) return nullptr;
+    if (!IsConstant(a, inputs[1]) || !IsConstant(a, inputs[2])) return nullptr;
+    if (zp != nullptr && !IsConstant(a, zp)) return nullptr;
+    if (g_idx != nullptr && !IsConstant(a, g_idx)) return nullptr;
+  }
+  *supported = true;
   return nullptr;
 }
 
@@ -91,16 +133,6 @@ OrtStatus* FusedProjectionNodeSupported(const Apis& a, const OrtNode* node, bool
   return nullptr;
 }
 
-bool IsConstant(const Apis& a, const OrtValueInfo* v) {
-  bool c = false;
-  if (v == nullptr) return false;
-  if (OrtStatus* st = a.ort->ValueInfo_IsConstantInitializer(v, &c)) {
-    a.ort->ReleaseStatus(st);
-    return false;
-  }
-  return c;
-}
-
 // MatMulNBits -> Add(constant [N]) is the pair ONNX Runtime's MatMulNBitsFusion folds into the operator's bias input,
 // but only for its own CPU and CUDA providers (onnxruntime/core/optimizer/graph_transformer_utils.cc:343-344,459;
 // matmul_nbits_fusion.cc).  For this provider the Add would stay behind as a CPU node with a device-to-host copy in
@@ -119,6 +151,7 @@ OrtStatus* FindBiasAdd(const Apis& a, const OrtNode* mm, const OrtNode** add_out
   std::vector<const OrtValueInfo*> in(num_inputs, nullptr);
   MI_RETURN_IF_ERROR(a.ort->Node_GetInputs(mm, in.data(), num_inputs));
   if (num_inputs > 5 && in[5] != nullptr) return nullptr;               // already has a bias
+  if (num_inputs > 4 && in[4] != nullptr) return nullptr;               // group index: the kernel's variant route
   if (num_inputs < 3 || !IsConstant(a, in[1]) || !IsConstant(a, in[2])) return nullptr;
   if (num_inputs > 3 && in[3] != nullptr && !IsConstant(a, in[3])) return nullptr;
   MI_RETURN_IF_ERROR(a.ort->Node_GetNumOutputs(mm, &num_outputs));

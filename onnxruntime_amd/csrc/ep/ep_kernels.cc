@@ -22,8 +22,14 @@ struct MatMulNBitsKernel : OrtKernelImpl {
   // constant initializers seen at kernel creation (owned by the session; valid until they are reported packed)
   const OrtValue* const_scales = nullptr;
   const OrtValue* const_zero_points = nullptr;
+  const OrtValue* const_g_idx = nullptr;  // host memory (the kernel definition asks for input 4 on the CPU)
   bool has_zp_arg = false;    // the node has a zero_points input, constant or not
   bool has_g_idx = false;
+  // Inputs the reference serves through its dequantise-everything route (matmul_nbits.cc:1248-1295): a group index,
+  // zero points in the activation type, and bfloat16 activations.  They run through the library's variant entry
+  // points; the plan describes the transformed problem.
+  bool variant = false;
+  MnbVariantPlan plan{};
   // packed weights (weights + scales + zero points in the device layout)
   void* packed = nullptr;
   OrtAllocator* packed_allocator = nullptr;
@@ -44,6 +50,198 @@ void ORT_API_CALL MatMulNBitsRelease(OrtKernelImpl* this_ptr) noexcept {
   delete k;
 }
 
+// ---- variant route -------------------------------------------------------------------------------------------
+int ZpKind(const TensorDesc* zp) {
+  if (zp == nullptr) return MNB_ZP_NONE;
+  return zp->type == ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8 ? MNB_ZP_UINT8 : MNB_ZP_TYPED;
+}
+
+// g_idx values in host memory: the tensor's own storage, or a copy when it lives on the device after all.
+OrtStatus* HostGroupIndex(const Apis& a, const OrtValue* g_idx, std::vector<int32_t>* copy, const int32_t** out,
+                          size_t* len) {
+  *out = nullptr;
+  *len = 0;
+  if (g_idx == nullptr) return nullptr;
+  TensorDesc d;
+  MI_RETURN_IF_ERROR(Describe(a, g_idx, &d));
+  if (d.type != ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: g_idx must be an int32 tensor");
+  }
+  const void* p = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->GetTensorData(g_idx, &p));
+  *len = static_cast<size_t>(d.count());
+  if (OnHost(a, g_idx)) {
+    *out = static_cast<const int32_t*>(p);
+    return nullptr;
+  }
+  copy->resize(*len);
+  MI_RETURN_IF_HIP(a, hipMemcpy(copy->data(), p, *len * sizeof(int32_t), hipMemcpyDeviceToHost));
+  *out = copy->data();
+  return nullptr;
+}
+
+// Validates the operands, plans the transformed problem and packs it into `*packed` (allocated by `alloc`).
+template <typename Alloc>
+OrtStatus* VariantPack(MatMulNBitsKernel& k, const OrtValue* b, const OrtValue* scales, const OrtValue* zp,
+                       const OrtValue* g_idx, hipStream_t stream, Alloc alloc, MnbVariantPlan* plan, void** packed) {
+  const Apis& a = k.apis;
+  *packed = nullptr;
+  TensorDesc b_desc, s_desc, z_desc, g_desc;
+  MI_RETURN_IF_ERROR(Describe(a, b, &b_desc));
+  MI_RETURN_IF_ERROR(Describe(a, scales, &s_desc));
+  if (zp != nullptr) MI_RETURN_IF_ERROR(Describe(a, zp, &z_desc));
+  if (g_idx != nullptr) MI_RETURN_IF_ERROR(Describe(a, g_idx, &g_desc));
+  MnbTensorInfo bi = ToMnb(&b_desc), si = ToMnb(&s_desc), zi = ToMnb(zp ? &z_desc : nullptr),
+                gi = ToMnb(g_idx ? &g_desc : nullptr), none = ToMnb(nullptr);
+  MI_RETURN_IF_ERROR(StatusFromMnb(a, MnbCheckInputs(&bi, &si, &zi, &gi, &none, k.N, k.K, k.block_size, k.bits)));
+  std::vector<int32_t> g_copy;
+  const int32_t* g_host = nullptr;
+  size_t g_len = 0;
+  MI_RETURN_IF_ERROR(HostGroupIndex(a, g_idx, &g_copy, &g_host, &g_len));
+  MI_RETURN_IF_ERROR(StatusFromMnb(
+      a, MnbVariantMakePlan(static_cast<size_t>(k.N), static_cast<size_t>(k.K), static_cast<int>(k.bits),
+                            static_cast<int>(k.block_size), static_cast<int>(s_desc.type),
+                            ZpKind(zp ? &z_desc : nullptr), g_host, g_len, plan)));
+  DeviceView b_dev, s_dev, z_dev;
+  MI_RETURN_IF_ERROR(b_dev.Init(a, b));
+  MI_RETURN_IF_ERROR(s_dev.Init(a, scales));
+  if (zp != nullptr) MI_RETURN_IF_ERROR(z_dev.Init(a, zp));
+  void* buffer = nullptr;
+  MI_RETURN_IF_ERROR(alloc(static_cast<size_t>(plan->packed_bytes), &buffer));
+  *packed = buffer;  // the caller frees it, also on failure below
+  MI_RETURN_IF_ERROR(StatusFromMnb(a, MnbVariantPack(plan, b_dev.get(), s_dev.get(), z_dev.get(), g_host, g_len, buffer,
+                                                     stream)));
+  MI_RETURN_IF_HIP(a, hipStreamSynchronize(stream));  // the temporary device copies go away with this scope
+  return nullptr;
+}
+
+void FreePacked(MatMulNBitsKernel& k) {
+  if (k.packed == nullptr) return;
+  if (k.packed_allocator != nullptr)
+    k.packed_allocator->Free(k.packed_allocator, k.packed);
+  else
+    (void)hipFree(k.packed);
+  k.packed = nullptr;
+}
+
+OrtStatus* VariantPrePack(MatMulNBitsKernel& k, const OrtValue* tensor, int input_index, OrtAllocator* allocator,
+                          bool* is_packed) {
+  const Apis& a = k.apis;
+  if (input_index == static_cast<int>(kScales) || input_index == static_cast<int>(kZeroPoints) ||
+      input_index == static_cast<int>(kGIdx)) {
+    *is_packed = k.packed != nullptr;  // consumed by the B call
+    return nullptr;
+  }
+  if (input_index != static_cast<int>(kB)) return nullptr;
+  // everything the packed buffer depends on must be a constant initializer; otherwise Compute packs per call
+  if (k.const_scales == nullptr) return nullptr;
+  if (k.has_zp_arg && k.const_zero_points == nullptr) return nullptr;
+  if (k.has_g_idx && k.const_g_idx == nullptr) return nullptr;
+  OrtAllocator* owner = allocator;
+  auto alloc = [&](size_t bytes, void** out) -> OrtStatus* {
+    *out = allocator != nullptr ? allocator->Alloc(allocator, bytes) : nullptr;
+    if (*out == nullptr) {
+      owner = nullptr;
+      MI_RETURN_IF_HIP(a, hipMalloc(out, bytes));
+    }
+    return nullptr;
+  };
+  void* buffer = nullptr;
+  OrtStatus* st = VariantPack(k, tensor, k.const_scales, k.const_zero_points, k.const_g_idx, nullptr, alloc, &k.plan,
+                              &buffer);
+  k.packed = buffer;
+  k.packed_allocator = owner;
+  if (st != nullptr) {
+    FreePacked(k);
+    return st;
+  }
+  *is_packed = true;
+  return nullptr;
+}
+
+OrtStatus* VariantCompute(MatMulNBitsKernel& k, OrtKernelContext* ctx) {
+  const Apis& a = k.apis;
+  size_t num_inputs = 0;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetInputCount(ctx, &num_inputs));
+  const OrtValue* in[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  for (size_t i = 0; i < 6 && i < num_inputs; ++i) {
+    if (k.packed != nullptr && (i == kB || i == kScales || i == kZeroPoints || i == kGIdx)) continue;
+    MI_RETURN_IF_ERROR(a.ort->KernelContext_GetInput(ctx, i, &in[i]));
+  }
+  if (in[kA] == nullptr) return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: input A is missing");
+  TensorDesc ad, bias_desc;
+  MI_RETURN_IF_ERROR(Describe(a, in[kA], &ad));
+  if (in[kBias] != nullptr) {
+    MI_RETURN_IF_ERROR(Describe(a, in[kBias], &bias_desc));
+    if (bias_desc.dims.size() != 1 || bias_desc.dims[0] != k.N) {
+      return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "bias must be a 1D tensor with shape [N]");
+    }
+  }
+  if (ad.dims.empty() || ad.dims.back() != k.K) {
+    return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMul dimension mismatch");
+  }
+  std::vector<int64_t> y_dims(ad.dims.begin(), ad.dims.end() - 1);
+  y_dims.push_back(k.N);
+  int64_t M = 1;
+  for (size_t i = 0; i + 1 < ad.dims.size(); ++i) M *= ad.dims[i];
+  OrtValue* y = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetOutput(ctx, 0, y_dims.data(), y_dims.size(), &y));
+  if (M == 0 || k.N == 0) return nullptr;
+
+  void* stream = nullptr;
+  MI_RETURN_IF_ERROR(a.ort->KernelContext_GetGPUComputeStream(ctx, &stream));
+  hipStream_t hs = static_cast<hipStream_t>(stream);
+
+  // operands fed per run (or prepacking disabled): plan and pack per call into stream-ordered memory
+  MnbVariantPlan call_plan{};
+  const MnbVariantPlan* plan = &k.plan;
+  void* call_packed = nullptr;
+  const void* packed = k.packed;
+  if (packed == nullptr) {
+    if (in[kB] == nullptr || in[kScales] == nullptr) {
+      return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: B and scales are required when B was not prepacked");
+    }
+    auto alloc = [&](size_t bytes, void** out) -> OrtStatus* {
+      MI_RETURN_IF_HIP(a, hipMallocAsync(out, bytes, hs));
+      return nullptr;
+    };
+    OrtStatus* st = VariantPack(k, in[kB], in[kScales], in[kZeroPoints], in[kGIdx], hs, alloc, &call_plan, &call_packed);
+    if (st != nullptr) {
+      if (call_packed != nullptr) (void)hipFreeAsync(call_packed, hs);
+      return st;
+    }
+    plan = &call_plan;
+    packed = call_packed;
+  }
+  OrtStatus* result = nullptr;
+  if (static_cast<int>(ad.type) != plan->a_dtype) {
+    result = a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A and scales must have the same element type");
+  } else {
+    const void* a_ptr = nullptr;
+    const void* bias_ptr = nullptr;
+    void* y_ptr = nullptr;
+    result = a.ort->GetTensorData(in[kA], &a_ptr);
+    if (result == nullptr && in[kBias] != nullptr) result = a.ort->GetTensorData(in[kBias], &bias_ptr);
+    if (result == nullptr) result = a.ort->GetTensorMutableData(y, &y_ptr);
+    if (result == nullptr) {
+      const size_t Mz = static_cast<size_t>(M);
+      const size_t ws_bytes = MnbVariantGemmWorkspaceSize(plan, Mz);
+      void* ws = nullptr;
+      hipError_t e = ws_bytes > 0 ? hipMallocAsync(&ws, ws_bytes, hs) : hipSuccess;
+      if (e != hipSuccess) {
+        result = a.ort->CreateStatus(ORT_EP_FAIL, hipGetErrorString(e));
+      } else {
+        const int rc = MnbVariantGemm(plan, Mz, a_ptr, static_cast<size_t>(k.K), packed, bias_ptr, y_ptr,
+                                      static_cast<size_t>(k.N), ws, ws_bytes, stream);
+        if (ws != nullptr) (void)hipFreeAsync(ws, hs);
+        result = StatusFromMnb(a, rc);
+      }
+    }
+  }
+  if (call_packed != nullptr) (void)hipFreeAsync(call_packed, hs);
+  return result;
+}
+
 // PrePack(B) folds the constant scales and zero points into one device buffer in the gfx950 layout, the way the
 // reference folds them into its packed buffer on the B call (matmul_nbits.cc:252-330).  The later calls for scales
 // and zero points then only report those inputs as consumed.
@@ -53,7 +251,7 @@ OrtStatus* ORT_API_CALL MatMulNBitsPrePack(OrtKernelImpl* this_ptr, const OrtVal
   MatMulNBitsKernel& k = *Self(this_ptr);
   const Apis& a = k.apis;
   *is_packed = false;
-  if (k.has_g_idx) return nullptr;  // no packed kernel with a group index (matmul_nbits.cc:258-262)
+  if (k.variant) return VariantPrePack(k, tensor, input_index, allocator, is_packed);
 
   if (input_index == static_cast<int>(kScales) || input_index == static_cast<int>(kZeroPoints)) {
     // consumed by the B call: ONNX Runtime may drop the initializer
@@ -115,6 +313,7 @@ OrtStatus* ORT_API_CALL MatMulNBitsPrePack(OrtKernelImpl* this_ptr, const OrtVal
 OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelContext* ctx) noexcept {
   MatMulNBitsKernel& k = *Self(this_ptr);
   const Apis& a = k.apis;
+  if (k.variant) return VariantCompute(k, ctx);
   size_t num_inputs = 0;
   MI_RETURN_IF_ERROR(a.ort->KernelContext_GetInputCount(ctx, &num_inputs));
   const OrtValue* in[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -272,6 +471,27 @@ OrtStatus* ORT_API_CALL CreateMatMulNBits(void* state, const OrtKernelInfo* info
     MI_RETURN_IF_ERROR(a.ort->KernelInfoGetConstantInput_tensor(info, kZeroPoints, &is_constant, &value));
     if (is_constant) k->const_zero_points = value;
   }
+  if (k->has_g_idx) {
+    is_constant = 0;
+    value = nullptr;
+    MI_RETURN_IF_ERROR(a.ort->KernelInfoGetConstantInput_tensor(info, kGIdx, &is_constant, &value));
+    if (is_constant) k->const_g_idx = value;
+  }
+  // The element types are read from the constant initializers: GetCapability claims a node with typed zero points
+  // or bfloat16 activations only when scales and zero points are constant.
+  bool typed_zp = false;
+  if (k->const_zero_points != nullptr) {
+    TensorDesc z;
+    MI_RETURN_IF_ERROR(Describe(a, k->const_zero_points, &z));
+    typed_zp = z.type != ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8;
+  }
+  bool bf16 = false;
+  if (k->const_scales != nullptr) {
+    TensorDesc sd;
+    MI_RETURN_IF_ERROR(Describe(a, k->const_scales, &sd));
+    bf16 = sd.type == ONNX_TENSOR_ELEMENT_DATA_TYPE_BFLOAT16;
+  }
+  k->variant = k->has_g_idx || typed_zp || bf16;
   *kernel_out = k.release();
   return nullptr;
 }
@@ -341,8 +561,11 @@ OrtStatus* AddMatMulNBits(const Apis& a, const Apis* state, const char* ep_name,
   MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T1", types.data(), types.size()));
   MI_RETURN_IF_ERROR(TypeList(a, {ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8}, &types));
   MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T2", types.data(), types.size()));
-  // Zero points in the activation type (the reference's "unquantized zero point" route) stay on the CPU provider.
+  // zero points: packed uint8, or the activation type (the reference's "unquantized zero point" route)
+  MI_RETURN_IF_ERROR(TypeList(a, {ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8, t1}, &types));
   MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T3", types.data(), types.size()));
+  // the group index is analysed on the host when the weights are packed
+  MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_SetInputMemType(db.b, kGIdx, OrtMemTypeCPUInput));
   MI_RETURN_IF_ERROR(TypeList(a, {ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32}, &types));
   MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T4", types.data(), types.size()));
   OrtKernelDef* def = nullptr;
@@ -368,7 +591,8 @@ OrtStatus* AddMemcpy(const Apis& a, const Apis* state, const char* ep_name, OrtK
   std::vector<const OrtDataType*> types;
   MI_RETURN_IF_ERROR(TypeList(a,
                               {ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16,
-                               ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8, ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32},
+                               ONNX_TENSOR_ELEMENT_DATA_TYPE_BFLOAT16, ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8,
+                               ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32},
                               &types));
   MI_RETURN_IF_ERROR(a.ep->KernelDefBuilder_AddTypeConstraint(db.b, "T", types.data(), types.size()));
   OrtKernelDef* def = nullptr;
@@ -388,6 +612,7 @@ OrtStatus* CreateKernelRegistry(const Apis& apis, const char* ep_name, OrtKernel
   MI_RETURN_IF_ERROR(apis.ep->CreateKernelRegistry(&registry));
   OrtStatus* st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT);
   if (st == nullptr) st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16);
+  if (st == nullptr) st = AddMatMulNBits(apis, state, ep_name, registry, ONNX_TENSOR_ELEMENT_DATA_TYPE_BFLOAT16);
   if (st == nullptr) st = AddFusedProjectionKernels(apis, state, ep_name, registry);
   if (st == nullptr) st = AddMemcpy(apis, state, ep_name, registry, /*from_host*/ true);
   if (st == nullptr) st = AddMemcpy(apis, state, ep_name, registry, /*from_host*/ false);

@@ -11,7 +11,9 @@ SHIM = HERE / "libort_host_shim.so"
 PLUGIN = HERE.parent.parent / "onnxruntime_amd" / "libonnxruntime_mi355x_ep.so"
 
 NOT_CLAIMED, LOAD_FAILED, NO_DEVICE, PROTOCOL, NOT_FUSED = -1, -2, -3, -4, -5
-_ONNX_TYPE = {np.dtype(np.float32): 1, np.dtype(np.uint8): 2, np.dtype(np.int32): 6, np.dtype(np.float16): 10}
+# bfloat16 tensors travel as uint16 arrays of their bit patterns
+_ONNX_TYPE = {np.dtype(np.float32): 1, np.dtype(np.uint8): 2, np.dtype(np.int32): 6, np.dtype(np.float16): 10,
+              np.dtype(np.uint16): 16}
 
 
 class EpHostTensor(ctypes.Structure):

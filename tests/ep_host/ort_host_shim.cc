@@ -97,8 +97,12 @@ struct OrtOpAttr {
   float f = 0.f;
   std::string s;
 };
+struct OrtTypeInfo {
+  OrtTensorTypeAndShapeInfo tensor;
+};
 struct OrtValueInfo {
   std::string name;
+  OrtTypeInfo type_info = {{{}, ONNX_TENSOR_ELEMENT_DATA_TYPE_UNDEFINED}};
   const OrtValue* initializer = nullptr;  // host tensor of a constant initializer
   bool is_graph_output = false;
   std::vector<std::pair<const OrtNode*, int64_t>> consumers = {};  // (node, input index)
@@ -150,6 +154,7 @@ size_t ElemSize(ONNXTensorElementDataType t) {
     case ONNX_TENSOR_ELEMENT_DATA_TYPE_INT32:
       return 4;
     case ONNX_TENSOR_ELEMENT_DATA_TYPE_FLOAT16:
+    case ONNX_TENSOR_ELEMENT_DATA_TYPE_BFLOAT16:
       return 2;
     case ONNX_TENSOR_ELEMENT_DATA_TYPE_UINT8:
       return 1;
@@ -387,6 +392,15 @@ void FillApisOnce() {
   };
   g_ort.GetValueInfoName = [](const OrtValueInfo* v, const char** out) noexcept -> OrtStatus* {
     *out = v->name.c_str();
+    return nullptr;
+  };
+  g_ort.GetValueInfoTypeInfo = [](const OrtValueInfo* v, const OrtTypeInfo** out) noexcept -> OrtStatus* {
+    *out = &v->type_info;
+    return nullptr;
+  };
+  g_ort.CastTypeInfoToTensorInfo = [](const OrtTypeInfo* t, const OrtTensorTypeAndShapeInfo** out) noexcept
+      -> OrtStatus* {
+    *out = &t->tensor;
     return nullptr;
   };
   g_ort.ValueInfo_IsConstantInitializer = [](const OrtValueInfo* v, bool* out) noexcept -> OrtStatus* {
@@ -819,6 +833,7 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     node.inputs.emplace_back(new OrtValueInfo{kInputNames[i]});
     if (i != 0 && ((constant_mask >> i) & 1)) node.inputs.back()->initializer = host_values[i].get();
     auto t = static_cast<ONNXTensorElementDataType>(inputs[i].dtype);
+    node.inputs.back()->type_info.tensor = {host_values[i]->dims, t};
     auto it = node.types.find(kInputTypes[i]);
     if (it == node.types.end()) node.types[kInputTypes[i]] = t;
   }
@@ -974,9 +989,20 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
   };
   const auto* entry = compiled ? nullptr : LookUp(*registry, ep_name, node);
   if (!compiled && entry == nullptr) return HostFail(EP_HOST_PROTOCOL, "claimed node without a kernel", err, err_len);
+  // inputs the kernel definition wants in host memory (OrtMemTypeCPUInput) are never copied to the device
+  auto wants_host = [&](size_t i) {
+    if (entry == nullptr) return false;
+    auto it = entry->def.input_mem.find(i);
+    return it != entry->def.input_mem.end() && it->second == OrtMemTypeCPUInput;
+  };
+  for (size_t i = 1; i < NI; ++i)
+    if (device_values[i] && wants_host(i)) device_values[i].reset();
+  auto fed_value = [&](size_t i) -> const OrtValue* {
+    return wants_host(i) ? host_values[i].get() : device_values[i].get();
+  };
   OrtKernelInfo info{&node, {}};
   for (size_t i = 1; i < NI; ++i)
-    if (device_values[i] && ((constant_mask >> i) & 1)) info.constants[i] = device_values[i].get();
+    if (fed_value(i) && ((constant_mask >> i) & 1)) info.constants[i] = fed_value(i);
   OrtKernelImpl* kernel = nullptr;
   if (!compiled) {
     if (OrtStatus* st = entry->fn(entry->state, &info, &kernel)) return Fail(st, "kernel creation", err, err_len);
@@ -991,8 +1017,8 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     for (size_t i = 1; i < NI; ++i) {
       if (!info.constants.count(i)) continue;
       bool is_packed = false;
-      if (OrtStatus* st = kernel->PrePackWeight(kernel, device_values[i].get(), static_cast<int>(i), allocator,
-                                                nullptr, &is_packed))
+      if (OrtStatus* st = kernel->PrePackWeight(kernel, fed_value(i), static_cast<int>(i), allocator, nullptr,
+                                                &is_packed))
         return Fail(st, "PrePackWeight", err, err_len);
       packed[i] = is_packed;
       if (is_packed) trace.add("%zu,", i);
@@ -1001,6 +1027,7 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     for (size_t i = 1; i < NI; ++i)
       if (packed[i]) device_values[i].reset();
   }
+  std::vector<bool> dropped = packed;  // initializers the kernel took over are gone, host-side ones included
   trace.add(" ");
 
   // ---- Memcpy kernels around the node
@@ -1041,7 +1068,7 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
       ctx.inputs.assign(node.inputs.size(), nullptr);
       ctx.inputs[0] = copy_in.outputs[0].get();
       for (size_t i = 1; i < node.inputs.size(); ++i)
-        if (!packed[i] && device_values[i]) ctx.inputs[i] = device_values[i].get();
+        if (!dropped[i] && fed_value(i)) ctx.inputs[i] = fed_value(i);
       if (OrtStatus* st = kernel->Compute(kernel, &ctx)) return Fail(st, "Compute", err, err_len);
     }
     for (size_t o = 0; o < spec.num_outputs; ++o) {

@@ -64,14 +64,26 @@ def test_batched_activations_and_empty_output(oracle):
 
 def test_nodes_left_to_the_cpu_provider():
     c = make_case(2, 64, 128, 4, 32, np.float32, has_zp=True, seed=5)
-    # g_idx present: not claimed
-    with pytest.raises(host.EpHostError) as e:
-        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A, c.B, c.scales, c.zero_points, np.zeros(c.K, np.int32), None)
-    assert e.value.code == host.NOT_CLAIMED
-    # zero points in the activation type: no kernel registered for T3 = float
-    with pytest.raises(host.EpHostError) as e:
-        host.run_matmul_nbits(c.N, c.K, 4, 32, c.A, c.B, c.scales, c.scales.copy(), None, None)
-    assert e.value.code == host.NOT_CLAIMED
+    g = (np.arange(c.K) // 32).astype(np.int32)
+
+    def not_claimed(**kw):
+        args = dict(zero_points=c.zero_points, g_idx=None, bits=4, B=c.B, scales=c.scales)
+        args.update(kw)
+        with pytest.raises(host.EpHostError) as e:
+            host.run_matmul_nbits(c.N, c.K, args["bits"], 32, c.A, args["B"], args["scales"], args["zero_points"],
+                                  args["g_idx"], None, constant=args.get("constant", ("B", "scales", "zero_points",
+                                                                                      "g_idx")))
+        assert e.value.code == host.NOT_CLAIMED
+
+    # a group index, typed zero points: transformed when the weights are packed, so every operand must be constant
+    not_claimed(g_idx=g, constant=("B", "scales", "zero_points"))
+    not_claimed(g_idx=g, constant=("B", "zero_points", "g_idx"))
+    not_claimed(zero_points=np.full((c.N, 4), 7.5, np.float32), constant=("B", "scales"))
+    # the reference's own limits: 8-bit weights with either, zero points of another float type
+    c8 = make_case(2, 64, 128, 8, 32, np.float32, seed=5)
+    not_claimed(bits=8, B=c8.B, scales=c8.scales, zero_points=None, g_idx=g)
+    not_claimed(bits=8, B=c8.B, scales=c8.scales, zero_points=np.full((c.N, 4), 100.5, np.float32))
+    not_claimed(zero_points=np.full((c.N, 4), 7.5, np.float16))
 
 
 def test_shape_errors_carry_the_reference_messages():
