@@ -66,7 +66,7 @@ def build(force: bool = True, jobs: int = 4) -> Path:
 
 
 EP_LIB = PKG / "libonnxruntime_mi355x_ep.so"
-EP_SOURCES = ["ep_lib_entry.cc", "ep_factory.cc", "ep.cc", "ep_kernels.cc", "ep_fused_kernels.cc", "ep_compile.cc",
+EP_SOURCES = ["ep_lib_entry.cc", "ep_factory.cc", "ep.cc", "ep_kernels.cc", "ep_fused_kernels.cc", "ep_compile.cc", "ep_profiler.cc",
               "ep_device_runtime.cc"]
 
 

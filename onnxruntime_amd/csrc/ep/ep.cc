@@ -289,6 +289,10 @@ void ORT_API_CALL ReleaseNodeComputeInfosImpl(OrtEp*, OrtNodeComputeInfo** infos
   for (size_t i = 0; i < count; ++i) ReleaseFusedNode(infos[i]);
 }
 
+OrtStatus* ORT_API_CALL CreateProfilerImpl(OrtEp* this_ptr, OrtEpProfilerImpl** profiler) noexcept {
+  return CreateEpProfiler(Self(this_ptr)->apis, profiler);
+}
+
 OrtStatus* ORT_API_CALL SyncImpl(OrtEp* this_ptr) noexcept {
   Ep& ep = *Self(this_ptr);
   MI_RETURN_IF_HIP(ep.apis, hipSetDevice(ep.device));
@@ -310,6 +314,7 @@ OrtEp* CreateEp(Factory& factory, const Apis& apis, int device) {
   ep->IsConcurrentRunSupported = IsConcurrentRunSupportedImpl;
   ep->Sync = SyncImpl;
   // the only subgraph the provider compiles is MatMulNBits + Add(bias); everything else runs registered kernels
+  ep->CreateProfiler = CreateProfilerImpl;
   ep->Compile = CompileImpl;
   ep->ReleaseNodeComputeInfos = ReleaseNodeComputeInfosImpl;
   return ep;

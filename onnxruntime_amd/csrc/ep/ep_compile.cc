@@ -85,6 +85,7 @@ OrtStatus* ORT_API_CALL ComputeImpl(OrtNodeComputeInfo* this_ptr, void* /*comput
   const size_t ws_bytes = MnbGemmWorkspaceSize(Mz, Nz, Kz, bits, bs, k.has_zp, k.dtype);
   void* ws = nullptr;
   if (ws_bytes > 0) MI_RETURN_IF_HIP(a, hipMallocAsync(&ws, ws_bytes, hs));  // per call: concurrent runs never share it
+  KernelTimer timer(hs, "MatMulNBits+Add", MnbGemmKernelName(Mz, Nz, Kz, bits, bs, k.dtype), M, k.N, k.K);
   const int rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.has_zp, k.dtype, a_ptr, Kz, k.packed, k.bias, y_ptr, Nz, ws, ws_bytes,
                          stream);
   const hipError_t free_err = ws != nullptr ? hipFreeAsync(ws, hs) : hipSuccess;

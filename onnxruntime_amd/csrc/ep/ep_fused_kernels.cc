@@ -250,6 +250,8 @@ OrtStatus* ORT_API_CALL FusedCompute(OrtKernelImpl* this_ptr, OrtKernelContext* 
   }
   void* ws = ws_bytes > 0 ? scratch + pack_bytes : nullptr;
   if (rc == MNB_OK) {
+    KernelTimer timer(hs, k.op(), has_norm ? "norm + fused projections" : "fused projections", static_cast<int64_t>(Mz),
+                      static_cast<int64_t>(k.is_qkv ? n0 + 2 * n1 : 2 * n0), static_cast<int64_t>(Kz));
     if (k.is_qkv)
       rc = MnbQkvGemm(Mz, n0, n1, Kz, bits, bs, dtype, a_ptr, Kz, has_norm ? &norm : nullptr, packed, out_ptr[0], n0,
                       out_ptr[1], n1, out_ptr[2], n1, ws, ws_bytes, stream);

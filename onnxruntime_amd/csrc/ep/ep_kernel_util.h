@@ -107,6 +107,24 @@ inline OrtStatus* TypeList(const Apis& a, const std::vector<ONNXTensorElementDat
   return nullptr;
 }
 
+// ---- profiling (ep_profiler.cc)
+OrtStatus* CreateEpProfiler(const Apis& a, OrtEpProfilerImpl** out);
+
+// Times what the enclosing scope enqueues on `stream` when the calling thread is inside an ONNX Runtime event that
+// a profiler of this provider is following; does nothing otherwise.
+class KernelTimer {
+ public:
+  KernelTimer(hipStream_t stream, const char* op, const char* kernel_name, int64_t M, int64_t N, int64_t K);
+  ~KernelTimer();
+  KernelTimer(const KernelTimer&) = delete;
+  KernelTimer& operator=(const KernelTimer&) = delete;
+
+ private:
+  hipStream_t stream_;
+  void* pending_ = nullptr;   // the launch record, until the stop event is in the stream
+  void* profiler_ = nullptr;
+};
+
 // ---- compiled subgraphs (ep_compile.cc): MatMulNBits + Add(bias) as one node
 OrtStatus* ReadIntAttr(const Apis& a, const OrtNode* node, const char* name, int64_t* value, bool* found);  // ep.cc
 OrtStatus* CompileFusedNodes(const Apis& a, const OrtGraph** graphs, const OrtNode** fused_nodes, size_t count,

@@ -231,6 +231,8 @@ OrtStatus* VariantCompute(MatMulNBitsKernel& k, OrtKernelContext* ctx) {
       if (e != hipSuccess) {
         result = a.ort->CreateStatus(ORT_EP_FAIL, hipGetErrorString(e));
       } else {
+        KernelTimer timer(hs, "MatMulNBits", plan->has_g_idx ? "gather + MatMulNBits" : "MatMulNBits (widened)", M,
+                          k.N, k.K);
         const int rc = MnbVariantGemm(plan, Mz, a_ptr, static_cast<size_t>(k.K), packed, bias_ptr, y_ptr,
                                       static_cast<size_t>(k.N), ws, ws_bytes, stream);
         if (ws != nullptr) (void)hipFreeAsync(ws, hs);
@@ -385,6 +387,7 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
     void* gemm_scratch = nullptr;
     hipStream_t gs = static_cast<hipStream_t>(stream);
     if (gemm_ws > 0) MI_RETURN_IF_HIP(a, hipMallocAsync(&gemm_scratch, gemm_ws, gs));
+    KernelTimer timer(gs, "MatMulNBits", MnbGemmKernelName(Mz, Nz, Kz, bits, bs, dtype), M, k.N, k.K);
     const int gemm_rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr, Nz,
                                 gemm_scratch, gemm_ws, stream);
     const hipError_t gemm_free = gemm_scratch != nullptr ? hipFreeAsync(gemm_scratch, gs) : hipSuccess;
@@ -413,6 +416,7 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
   void* ws = nullptr;
   hipStream_t hs = static_cast<hipStream_t>(stream);
   MI_RETURN_IF_HIP(a, hipMallocAsync(&ws, ws_bytes, hs));
+  KernelTimer timer(hs, "MatMulNBits", "pack + MatMulNBits", M, k.N, k.K);
   int rc = MnbGemmUnpacked(Mz, Nz, Kz, bits, bs, dtype, a_ptr, Kz, b_ptr, s_ptr, z_ptr, bias_ptr, y_ptr, Nz, ws,
                            ws_bytes, stream);
   hipError_t free_err = hipFreeAsync(ws, hs);

@@ -51,6 +51,28 @@ class EpHostError(RuntimeError):
         self.code, self.message, self.trace = code, message, trace
 
 
+class profiled:
+    """Context manager: the next run_* call inside it is followed by the plugin's profiler; ``events`` then holds
+    dicts with category, name, timestamp_us, duration_us and the event's arguments."""
+
+    def __enter__(self):
+        self._buf = ctypes.create_string_buffer(8192)
+        lib = _load()
+        lib.EpHostProfileNextRun.restype = None
+        lib.EpHostProfileNextRun.argtypes = [ctypes.c_char_p, ctypes.c_size_t]
+        lib.EpHostProfileNextRun(self._buf, len(self._buf))
+        self.events = []
+        return self
+
+    def __exit__(self, *exc):
+        for line in self._buf.value.decode().splitlines():
+            cat, name, ts, dur, *args = line.split("|")
+            self.events.append(dict(category=int(cat), name=name, timestamp_us=int(ts), duration_us=int(dur),
+                                    **dict(a.split("=", 1) for a in args)))
+        _load().EpHostProfileNextRun(None, 0)
+        return False
+
+
 def available() -> bool:
     return SHIM.exists() and PLUGIN.exists()
 

@@ -129,6 +129,16 @@ struct OrtEpGraphSupportInfo {
 struct OrtNodeComputeContext {
   std::string node_name;
 };
+struct OrtProfilingEvent {
+  OrtProfilingEventCategory category;
+  int32_t pid, tid;
+  std::string name;
+  int64_t timestamp_us, duration_us;
+  std::vector<std::pair<std::string, std::string>> args;
+};
+struct OrtProfilingEventsContainer {
+  std::vector<OrtProfilingEvent> events;
+};
 struct OrtKernelInfo {
   const OrtNode* node;
   std::map<size_t, const OrtValue*> constants;
@@ -483,6 +493,23 @@ void FillApisOnce() {
     g->fused_drops_constants.push_back(options != nullptr && options->drop_constant_initializers);
     return nullptr;
   };
+  g_ep.CreateProfilingEvent = [](OrtProfilingEventCategory category, int32_t pid, int32_t tid, const char* name,
+                                 int64_t timestamp_us, int64_t duration_us, const char* const* keys,
+                                 const char* const* values, size_t num_args, OrtProfilingEvent** out) noexcept
+      -> OrtStatus* {
+    if (name == nullptr) return MakeStatus(ORT_INVALID_ARGUMENT, "event_name must not be NULL");
+    auto* e = new OrtProfilingEvent{category, pid, tid, name, timestamp_us, duration_us, {}};
+    for (size_t i = 0; i < num_args; ++i) e->args.emplace_back(keys[i], values[i]);
+    *out = e;
+    return nullptr;
+  };
+  g_ep.ReleaseProfilingEvent = [](OrtProfilingEvent* e) noexcept { delete e; };
+  g_ep.ProfilingEventsContainer_AddEvents = [](OrtProfilingEventsContainer* c, const OrtProfilingEvent* const* events,
+                                               size_t n) noexcept -> OrtStatus* {
+    if (n == 0) return MakeStatus(ORT_INVALID_ARGUMENT, "num_events must be greater than 0");
+    for (size_t i = 0; i < n; ++i) c->events.push_back(*events[i]);  // ORT copies the event data
+    return nullptr;
+  };
   g_ep.EpGraphSupportInfo_LookUpKernel = [](OrtEpGraphSupportInfo* g, const OrtNode* n,
                                             const OrtKernelDef** out) noexcept -> OrtStatus* {
     const auto* e = LookUp(*g->registry, g->ep_name, *n);
@@ -615,6 +642,12 @@ Plugin* LoadPlugin(const char* path, std::string* error) {
   }
   return &(loaded[path] = p);
 }
+
+// Set by EpHostProfileNextRun: the next RunNode on this thread drives the plugin's profiler the way ONNX Runtime's
+// session profiling does and writes one line per reported event into the buffer.
+thread_local char* tl_profile_buf = nullptr;
+thread_local size_t tl_profile_len = 0;
+constexpr int64_t kProfilingStartOffsetNs = 5000000;  // pretend ORT's profiling began 5 ms before the EP's
 
 int Fail(OrtStatus* st, const char* where, char* err, size_t err_len) {
   int code = st->code == ORT_OK ? ORT_FAIL : static_cast<int>(st->code);
@@ -782,6 +815,29 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     ~EpGuard() { f->ReleaseEp(f, e); }
   } ep_guard{factory, ep};
   const std::string ep_name = ep->GetName(ep);
+
+  // ---- optional: follow the run with the plugin's profiler (OrtEp::CreateProfiler)
+  char* profile_buf = tl_profile_buf;
+  const size_t profile_len = tl_profile_len;
+  tl_profile_buf = nullptr;
+  OrtEpProfilerImpl* profiler = nullptr;
+  struct ProfilerGuard {
+    OrtEpProfilerImpl*& p;
+    ~ProfilerGuard() {
+      if (p != nullptr) p->Release(p);
+    }
+  } profiler_guard{profiler};
+  if (profile_buf != nullptr) {
+    profile_buf[0] = 0;
+    if (ep->CreateProfiler == nullptr) return HostFail(EP_HOST_PROTOCOL, "the plugin has no CreateProfiler", err, err_len);
+    if (OrtStatus* st = ep->CreateProfiler(ep, &profiler)) return Fail(st, "CreateProfiler", err, err_len);
+    if (profiler == nullptr) return HostFail(EP_HOST_PROTOCOL, "CreateProfiler returned NULL", err, err_len);
+    if (profiler->ort_version_supported < 25 || profiler->Release == nullptr || profiler->StartProfiling == nullptr ||
+        profiler->EndProfiling == nullptr)
+      return HostFail(EP_HOST_PROTOCOL, "OrtEpProfilerImpl lacks a required member", err, err_len);
+    if (OrtStatus* st = profiler->StartProfiling(profiler, kProfilingStartOffsetNs))
+      return Fail(st, "StartProfiling", err, err_len);
+  }
 
   const OrtKernelRegistry* registry = nullptr;
   if (OrtStatus* st = ep->GetKernelRegistry(ep, &registry)) return Fail(st, "GetKernelRegistry", err, err_len);
@@ -1060,6 +1116,18 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     ctx.output_on_host.assign(spec.num_outputs, false);
     ctx.output_skipped.assign(spec.num_outputs, false);
     for (size_t o = 0; o < spec.num_outputs; ++o) ctx.output_skipped[o] = (spec.skipped_output_mask >> o) & 1;
+    const uint64_t correlation = 1700000000000000ull + static_cast<uint64_t>(r);  // epoch-based, like ORT's
+    if (profiler != nullptr && profiler->StartEvent != nullptr)
+      if (OrtStatus* st = profiler->StartEvent(profiler, correlation)) return Fail(st, "StartEvent", err, err_len);
+    struct EventGuard {
+      OrtEpProfilerImpl* p;
+      uint64_t id;
+      ~EventGuard() {
+        if (p == nullptr || p->StopEvent == nullptr) return;
+        OrtProfilingEvent node_event{OrtProfilingEventCategory_NODE, -1, -1, "node0_kernel_time", 0, 0, {}};
+        if (OrtStatus* st = p->StopEvent(p, id, &node_event)) delete st;
+      }
+    } event_guard{profiler, correlation};
     if (compiled) {
       ctx.inputs.assign(1, copy_in.outputs[0].get());  // the fused node's only non-constant input
       if (OrtStatus* st = compute_info.info->Compute(compute_info.info, compute_info.state, &ctx))
@@ -1092,6 +1160,20 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
       outs[o].produced = 1;
     }
   }
+  if (profiler != nullptr) {
+    OrtProfilingEventsContainer container;
+    if (OrtStatus* st = profiler->EndProfiling(profiler, &container)) return Fail(st, "EndProfiling", err, err_len);
+    size_t used = 0;
+    for (const auto& e : container.events) {
+      std::string line = std::to_string(static_cast<int>(e.category)) + "|" + e.name + "|" +
+                         std::to_string(e.timestamp_us) + "|" + std::to_string(e.duration_us);
+      for (const auto& kv : e.args) line += "|" + kv.first + "=" + kv.second;
+      line += "\n";
+      if (used + line.size() + 1 > profile_len) break;
+      std::memcpy(profile_buf + used, line.c_str(), line.size() + 1);
+      used += line.size();
+    }
+  }
   if (OrtStatus* st = ep->Sync(ep)) return Fail(st, "OrtEp::Sync", err, err_len);
   bool concurrent = false;
   if (OrtStatus* st = ep->IsConcurrentRunSupported(ep, &concurrent)) return Fail(st, "IsConcurrentRunSupported", err, err_len);
@@ -1102,6 +1184,13 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
 }  // namespace
 
 extern "C" {
+
+// The next EpHostRun* call on the calling thread is profiled: CreateProfiler, StartProfiling, StartEvent / StopEvent
+// around every Compute, EndProfiling; `buf` receives "category|name|timestamp_us|duration_us|key=value..." lines.
+__attribute__((visibility("default"))) void EpHostProfileNextRun(char* buf, size_t len) {
+  tl_profile_buf = len > 0 ? buf : nullptr;
+  tl_profile_len = len;
+}
 
 // Any operator of the com.microsoft domain the plugin registers (MatMulNBitsMlp, MatMulNBitsQkv, ...).
 __attribute__((visibility("default"))) int EpHostRunNode(const char* plugin_path, const EpHostNodeSpec* spec,
