@@ -183,10 +183,8 @@ static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
   }();
   if (mid_max_m >= 0) return M > mid_max_m;
   const double t_mid = 2.0 * (double)M * (double)L.N * (double)L.K / 550e12;
-  const int64_t tiles = ((M + 255) / 256) * ((L.N + 255) / 256);
-  // 8-bit weights with 16-wide blocks run a register-spilling variant of the tile kernel
-  const double step = L.bits == 4 ? 1.45e-6 : (L.bs >= 32 ? 1.65e-6 : 2.95e-6);
-  const double t_256 = (double)((tiles + 255) / 256) * (double)(L.K / 64) * step;
+  double t_256 = 0.0;
+  (void)mnb_gemm256_tile_rows(L, M, &t_256);
   return t_256 < t_mid;
 }
 

@@ -19,6 +19,8 @@
 //     the price here is that the two wavefront rows dequantise the same columns.
 //   * one barrier per step; the dequantisation of slab s+1 and the A staging run in the shadow of slab s's MFMAs.
 // Bias add and the single fp32 -> fp16 narrowing happen in the epilogue.
+#include <cstdlib>
+
 #include "mnb_device.cuh"
 #include "mnb_internal.h"
 
@@ -27,10 +29,15 @@ namespace {
 typedef uint32_t u4_t __attribute__((ext_vector_type(4)));  // plain register quad (HIP's uint4 struct resists SROA)
 typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int BN = 256, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // halves per staged A row
 constexpr int THREADS = 512;
-constexpr int STAGE_HALVES = BM * LDS_STRIDE;  // one A buffer
+// Rows of the tile: 64 * TM, TM = 32-row matrix-core tiles per wavefront (4: 256 x 256, 2: 128 x 256 for grids that
+// leave most of the chip idle with the large tile).  The dynamic LDS allocation is that of TM = 4 for both: the
+// epilogue stages 64 x 64 outputs per wavefront in it.
+constexpr int SMEM_HALVES = 2 * 256 * LDS_STRIDE;
+// cost of a k-step of the 128-row tile relative to the 256-row one (measured)
+constexpr double kMnbGemm128StepRatio = 0.88;
 
 struct Gemm256Params {
   const _Float16* A;
@@ -42,6 +49,7 @@ struct Gemm256Params {
   int M, N, K, bs_shift;
   int ksteps;
   int tiles_m, tiles_n;
+  int tile_rows;  // 256 or 128
   int c_vec_ok;  // C allows 16-byte stores of 8 columns: aligned base and pitch, N a multiple of 8
   uint32_t uc[4];  // unpack constants (see UnpackConsts)
   // several matrices packed as one (mnb_layout.h); these kinds always take the 16-byte store path
@@ -93,13 +101,13 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
   return __builtin_bit_cast(h8_t, o);
 }
 
-// Scheduling pipeline of one slab section (8 MFMAs): after every MFMA a few of the other instructions of the
+// Scheduling pipeline of one slab section (NM MFMAs): after every MFMA a few of the other instructions of the
 // section, so they run in the MFMA's shadow.  The closing sched_barrier keeps the scheduler from mixing the MFMAs
 // of different slabs (they reuse the same accumulators).
-template <int LDS_READS, int VMEM, int VALU, int LDS_WRITE_EVERY>
+template <int NM, int LDS_READS, int VMEM, int VALU, int LDS_WRITE_EVERY>
 __device__ __forceinline__ void slab_pipeline() {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < NM; ++i) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                             // 1 MFMA
     if (i < LDS_READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);          // 1 LDS read
     if (i < VMEM) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);               // 2 VMEM reads
@@ -114,16 +122,17 @@ __device__ __forceinline__ void slab_pipeline() {
 // Slab 0 of a k-step when the activations share one register set: the four LDS writes of the next A tile go first,
 // the four global loads that refill their registers follow (the loads must not overtake the writes that still read
 // those registers).
+template <int TM>
 __device__ __forceinline__ void slab0_shared_a_pipeline() {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // 1 MFMA
-    if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
-    __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);             // VALU
-    if (i < 4)
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);           // 1 LDS write
-    else if (i < 6)
-      __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);           // 2 VMEM reads
+  for (int i = 0; i < 2 * TM; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // 1 MFMA
+    if (i < TM) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 LDS read
+    __builtin_amdgcn_sched_group_barrier(0x002, 32 / (2 * TM), 0);  // VALU
+    if (i < TM)
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);            // 1 LDS write
+    else if (i < TM + TM / 2)
+      __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);            // 2 VMEM reads
   }
   __builtin_amdgcn_sched_barrier(0);
 }
@@ -131,9 +140,13 @@ __device__ __forceinline__ void slab0_shared_a_pipeline() {
 // MPS: meta entries (scale, zero point) a lane keeps per k-step and column tile.  A k-step of 64 spans 64 / block_size
 // blocks; 4-bit vectors cover 32 k, so two entries serve every block size (16-wide blocks through the lane's half
 // kq); 8-bit vectors cover 16 k: 4 entries for blocks of 16, 2 for blocks of 32 and more.
-template <int BITS, bool HAS_ZP, int MPS>
+template <int BITS, bool HAS_ZP, int MPS, int TM>
 __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
-  constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 16-byte activation loads per thread per k-step: 4
+  constexpr int BM = 64 * TM;                       // rows of the tile
+  constexpr int STAGE_HALVES = BM * LDS_STRIDE;     // one A buffer
+  constexpr int NM = 2 * TM;                        // MFMAs per slab
+  constexpr int VALU_PER_MFMA = 32 / NM;            // the slab's dequantisation spread over its MFMAs
+  constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 16-byte activation loads per thread per k-step: TM
   // 4-bit: a 16-byte vector spans two slabs (one word each per lane); 8-bit: one slab (two words per lane)
   constexpr int VEC_PER_STEP = (BITS == 4) ? 2 : 4;  // 8-byte weight loads per lane, column tile and k-step
   constexpr int GK = 128 / BITS;
@@ -142,15 +155,15 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts: rows wm*128, columns wn*64
+  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts: rows wm*32*TM, columns wn*64
   // column-fastest tile order: the workgroups resident at one time share a few 256-row slabs of A
   const int m0 = (blockIdx.x / p.tiles_n) * BM;
   const int n0 = (blockIdx.x % p.tiles_n) * BN;
   const int li = lane & 31, kq = lane >> 5;
 
-  f16_t acc[4][2];
+  f16_t acc[TM][2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -168,7 +181,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   };
   Stage R0, R1;
   u4_t RA[A_LOADS];
-  h8_t FA0[4], FA1[4];  // A operands, double buffered over slabs
+  h8_t FA0[TM], FA1[TM];  // A operands, double buffered over slabs
   h8_t FB0[2], FB1[2];  // B operands, double buffered over slabs
 
   const UnpackConsts uc = make_unpack_consts(p.uc);
@@ -274,14 +287,14 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // A operands of slab kk: lane (row li, half kq).  The k permutation matches the weights' (see the file header).
   auto read_a = [&](int buf, int kk, h8_t* FA) {
     const int koff = (BITS == 4) ? 32 * (kk >> 1) + 16 * kq + 8 * (kk & 1) : 16 * kk + 8 * kq;
-    const _Float16* As = lds + buf * STAGE_HALVES + (wm * 128 + li) * LDS_STRIDE + koff;
+    const _Float16* As = lds + buf * STAGE_HALVES + (wm * 32 * TM + li) * LDS_STRIDE + koff;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) FA[t] = *reinterpret_cast<const h8_t*>(As + t * 32 * LDS_STRIDE);
+    for (int t = 0; t < TM; ++t) FA[t] = *reinterpret_cast<const h8_t*>(As + t * 32 * LDS_STRIDE);
   };
 
   auto mfma_slab = [&](const h8_t* FA, const h8_t* FB) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(FA[i], FB[j], acc[i][j], 0, 0, 0);
@@ -301,27 +314,27 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     for (int i = 0; i < A_LOADS; ++i) store_a(nxt, i, Rn);
     if constexpr (SHARED_A) {
       load_a(ks + 2, Rc);
-      slab0_shared_a_pipeline();
+      slab0_shared_a_pipeline<TM>();
     } else {
-      slab_pipeline<4, 2, 4, 2>();
+      slab_pipeline<NM, TM, TM / 2, VALU_PER_MFMA, 2>();
     }
     // slab 1: operands of slab 2
     read_a(cur, 2, FA0);
     make_b(2, Rc, FB0);
     mfma_slab(FA1, FB1);
-    slab_pipeline<4, 0, 4, 0>();
+    slab_pipeline<NM, TM, 0, VALU_PER_MFMA, 0>();
     // slab 2: operands of slab 3; after that the weight registers of Rc are free: weights of step ks+2
     read_a(cur, 3, FA1);
     make_b(3, Rc, FB1);
     mfma_slab(FA0, FB0);
     load_b(ks + 2, Rc);
-    slab_pipeline<4, 4, 4, 0>();
+    slab_pipeline<NM, TM, 4, VALU_PER_MFMA, 0>();
     __syncthreads();
     // slab 3, behind the barrier: operands of slab 0 of step ks+1
     read_a(nxt, 0, FA0);
     make_b(0, Rn, FB0);
     mfma_slab(FA1, FB1);
-    slab_pipeline<4, 0, 4, 0>();
+    slab_pipeline<NM, TM, 0, VALU_PER_MFMA, 0>();
   };
 
   // ---- prologue: steps 0 and 1 in flight, A of step 0 staged, operands of slab 0 ready
@@ -358,7 +371,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     const int erow = lane >> 3, ecol = (lane & 7) * 8;
     const int n_out = n0 + wn * 64 + ecol;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < TM / 2; ++h) {
 #pragma unroll
       for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
@@ -385,7 +398,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
             const float gf = (float)g[e];
             y[e] = (_Float16)(gf / (1.0f + __expf(-gf)) * (float)u[e]);
           }
-          const int m = m0 + wm * 128 + h * 64 + row;
+          const int m = m0 + wm * 32 * TM + h * 64 + row;
           if (m < p.M && n_glu < p.n_out0) *reinterpret_cast<h8_t*>(p.C + (int64_t)m * p.ldc + n_glu) = y;
         }
       } else {
@@ -405,7 +418,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
         for (int ps = 0; ps < 8; ++ps) {
           const int row = ps * 8 + erow;
           const u4_t v = *reinterpret_cast<const u4_t*>(ep + row * EP_STRIDE + ecol);
-          const int m = m0 + wm * 128 + h * 64 + row;
+          const int m = m0 + wm * 32 * TM + h * 64 + row;
           if (m < p.M && n_loc < n_lim) *reinterpret_cast<u4_t*>(dst + (int64_t)m * ld + n_loc) = v;
         }
       }
@@ -416,10 +429,10 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       const int n = n0 + wn * 64 + j * 32 + li;
       if (n >= p.N) continue;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * 128 + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
+          const int m = m0 + wm * 32 * TM + i * 32 + (r >> 2) * 8 + kq * 4 + (r & 3);
           if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + bcol[j]);
         }
       }
@@ -433,11 +446,11 @@ int log2i(int v) {
   return s;
 }
 
-template <int BITS, bool HAS_ZP, int MPS>
-hipError_t launch(const Gemm256Params& p, hipStream_t s) {
-  const size_t smem = (size_t)2 * STAGE_HALVES * sizeof(_Float16);  // 73728 bytes
+template <int BITS, bool HAS_ZP, int MPS, int TM>
+hipError_t launch_tm(const Gemm256Params& p, hipStream_t s) {
+  const size_t smem = (size_t)SMEM_HALVES * sizeof(_Float16);  // 73728 bytes
   static bool configured = false;  // per instantiation; the attribute is sticky for the function
-  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS>;
+  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM>;
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -449,7 +462,30 @@ hipError_t launch(const Gemm256Params& p, hipStream_t s) {
   return hipGetLastError();
 }
 
+template <int BITS, bool HAS_ZP, int MPS>
+hipError_t launch(const Gemm256Params& p, hipStream_t s) {
+  return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2>(p, s) : launch_tm<BITS, HAS_ZP, MPS, 4>(p, s);
+}
+
 }  // namespace
+
+// Rows of the tile for a problem: the 128-row tile when its grid fills the 256 compute units in fewer, or at the
+// measured step costs cheaper, rounds than the 256-row one.
+int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds) {
+  const int64_t tiles_n = (L.N + BN - 1) / BN;
+  const double ksteps = (double)(L.K / BK);
+  const double step256 = L.bits == 4 ? 1.45e-6 : (L.bs >= 32 ? 1.65e-6 : 2.95e-6);
+  const double step128 = step256 * kMnbGemm128StepRatio;
+  const double t256 = (double)((((M + 255) / 256) * tiles_n + 255) / 256) * ksteps * step256;
+  const double t128 = (double)((((M + 127) / 128) * tiles_n + 255) / 256) * ksteps * step128;
+  static const int forced = [] {
+    const char* e = getenv("MNB_GEMM256_TILE_ROWS");  // tuning override: 128 or 256
+    return e ? atoi(e) : 0;
+  }();
+  const bool small = forced ? forced == 128 : t128 < t256;
+  if (seconds) *seconds = small ? t128 : t256;
+  return small ? 128 : 256;
+}
 
 // The fused outputs are written with 16-byte stores of 8 columns: every output 16-byte aligned, with a pitch and a
 // width that are multiples of 8 elements.
@@ -475,7 +511,8 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.K = (int)a.L.K;
   p.bs_shift = log2i(a.L.bs);
   p.ksteps = (int)(a.L.K / BK);  // K is a multiple of 2 * BK
-  p.tiles_m = (int)((a.M + BM - 1) / BM);
+  p.tile_rows = mnb_gemm256_tile_rows(a.L, a.M, nullptr);
+  p.tiles_m = (int)((a.M + p.tile_rows - 1) / p.tile_rows);
   p.tiles_n = (int)((a.L.N + BN - 1) / BN);
   p.uc[0] = 0x000F000Fu;
   p.uc[1] = 0x00F000F0u;

@@ -62,6 +62,8 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M);  // staged copy o
 bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
+// rows of the tile the tile GEMM would use (256 or 128) and, optionally, its estimated run time
+int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds);
 bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
 

@@ -76,10 +76,11 @@ def test_config4_prefill(oracle):
 @pytest.mark.parametrize("shape", list(synthetic.C5_SHAPES))
 def test_config5_layer_sweep(oracle, bits, bs, shape):
     K, N = synthetic.C5_SHAPES[shape]
-    for M in (1, 64, 256):
+    # M = 256 and 1024 reach the tile GEMM with 128-row tiles on the wide shapes and the streaming kernel on the others
+    for M in (1, 64, 256, 1024):
         c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, seed=0)
         y = run_case(c)
-        rows = np.unique(np.linspace(0, M - 1, 6).astype(int))
+        rows = np.unique(np.concatenate([np.linspace(0, M - 1, 6).astype(int), [min(127, M - 1), min(128, M - 1)]]))
         sub = make_case(len(rows), N, K, bits, bs, np.float16, has_zp=True, seed=0)
         sub.B, sub.scales, sub.zero_points = c.B, c.scales, c.zero_points
         sub.A = c.A[rows]
