@@ -10,6 +10,14 @@ Two independent restatements of the reference's arithmetic contract live here:
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this module.
 The product (``onnxruntime_amd``) never does.
 
+Parity status of what is defined here on top of the C functions (whose own status is in the header of mnb_oracle.c):
+  ``mlp`` / ``qkv``           compositions of pinned parts (matmul, layer normalisation) with silu(g) * u in float64;
+                              the reference ships only WebGPU shaders for these operators and no stored outputs, so
+                              beyond that composition their parity is PARITY UNPINNED
+  ``variant_dequantize``      wrapper of mnbo_variant_dequantize_f32: pinned by mathematics only, last ulp on inexact
+                              inputs PARITY UNPINNED; bfloat16 operands have no CPU kernel in the reference at all
+  ``dense_matmul_f64``        numpy float64 product over a dequantised W, the checker of the variant route
+
 Reference definitions followed (onnxruntime 1.30.0):
   canonical layout + ``(q - zp) * scale``      onnxruntime/core/mlas/lib/q4_dq.cpp:587-641
   operator contract (shapes, optional inputs)   onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3782-3849
