@@ -129,6 +129,30 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
   for (int t = 0; t < T; ++t) R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + col0 + t * 16];
 }
 
+// The same loads for slabs that do not start at a multiple of 64 columns (the meta entries of a lane's tiles are then
+// not adjacent): colw[t] is the lane's packed column in tile t, mcol[t] the position of its meta entry.
+template <int BITS, bool HAS_ZP, int MODE, int T>
+__device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, int kq, const int32_t* colw,
+                                                const int32_t* mcol, ChunkRegs<BITS, T>& R) {
+  constexpr int GK = 128 / BITS;
+  constexpr int CK = 4 * GK;
+  if constexpr (MODE == 0) {
+    const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
+#pragma unroll
+    for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t]);
+  } else {
+    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      load_meta_vec<HAS_ZP, 1>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol[t], &R.m0[t]);
+      if constexpr (BITS == 4)
+        load_meta_vec<HAS_ZP, 1>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol[t], &R.m1[t]);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < T; ++t) R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + colw[t]];
+}
+
 template <int BITS, bool HAS_ZP>
 __device__ __forceinline__ void decode_meta(uint32_t raw, _Float16& s, _Float16& neg_1024_plus_zp) {
   if constexpr (HAS_ZP) {

@@ -207,6 +207,86 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams
   skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
 }
 
+// ---- direct variant for slabs of three tiles ----------------------------------------------------------------------
+// A workgroup's run time is a fixed part plus a part proportional to its tiles, and hardly depends on how many of the
+// 256 compute units are busy, so 513..768 column tiles are best cut into slabs of three (at most 256 workgroups, one
+// round) rather than two (up to 384): N = 12288 runs 12 % faster.  Slabs of 48 columns are not aligned to the 64-column
+// groups in which the meta entries of a lane's tiles are adjacent, so the tiles are addressed one by one.
+// (Slabs with half a tile at the end - 56 columns for N = 14336, which would put exactly one workgroup on every
+// compute unit - were measured too: the half tile costs the instructions of a whole one, and the run time did not
+// improve.)
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW>
+__global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(SkinnyParams p) {
+  constexpr int GK = 128 / BITS;
+  constexpr int NI = GK / 8;
+  constexpr int CW = 16 * T;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int j = lane & 15, kq = lane >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * CW;
+  const int arow = j < p.M ? j : p.M - 1;
+  const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
+
+  int32_t colw[T], mcol[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    int64_t col = n0 + 16 * t + j;
+    col = col < p.Npad ? col : p.Npad - 1;  // beyond the matrix: padding, never stored
+    colw[t] = (int32_t)col;
+    mcol[t] = (int32_t)mnb_meta_col(col);
+  }
+
+  f4_t y[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const BConst bconst = make_bconst<BITS, HAS_ZP>();
+  const UnpackConsts uc = make_unpack_consts(p.uc);
+
+  auto load_a = [&](int c, h8_t* af) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i) af[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
+  };
+
+  if constexpr (CPW > 0) {
+    ChunkRegs<BITS, T> R[CPW];
+    h8_t a[CPW][NI];
+#pragma unroll
+    for (int q = 0; q < CPW; ++q) load_a(wave + q * NW, a[q]);
+#pragma unroll
+    for (int q = 0; q < CPW; ++q) load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, wave + q * NW, kq, colw, mcol, R[q]);
+#pragma unroll
+    for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, y);
+  } else {
+    ChunkRegs<BITS, T> R0, R1;
+    h8_t a0[NI], a1[NI];
+    int c = wave;
+    if (c < p.chunks) {
+      load_a(c, a0);
+      load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c, kq, colw, mcol, R0);
+    }
+    if (c + NW < p.chunks) {
+      load_a(c + NW, a1);
+      load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, colw, mcol, R1);
+    }
+    for (; c < p.chunks; c += 2 * NW) {
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
+      if (c + 2 * NW < p.chunks) {
+        load_a(c + 2 * NW, a0);
+        load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c + 2 * NW, kq, colw, mcol, R0);
+      }
+      if (c + NW < p.chunks) {
+        compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
+        if (c + 3 * NW < p.chunks) {
+          load_a(c + 3 * NW, a1);
+          load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c + 3 * NW, kq, colw, mcol, R1);
+        }
+      }
+    }
+  }
+  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
+}
+
 // ---- staged variant: any alignment of A; rows staged in LDS phase by phase -------------------------------------
 template <int BITS, bool HAS_ZP, int MODE, int T, int NW>
 __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams p) {
@@ -293,6 +373,8 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
     }
   }
   if (pl.t < min_t) pl.t = min_t;  // gate/up pairs live in one workgroup
+  // three tiles per workgroup (slab kernel): one round of at most 256 workgroups where two tiles would need up to 384
+  if (direct && min_t == 1 && tiles > 512 && tiles <= 768 && !getenv("MNB_SKINNY_PLAN")) pl.t = 3;
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
   pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
@@ -301,6 +383,32 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   const size_t red_bytes = (size_t)pl.nw * pl.t * 4 * 64 * 4;
   pl.smem = a_bytes > red_bytes ? a_bytes : red_bytes;
   return pl;
+}
+
+template <int BITS, bool HAS_ZP, int MODE, int T>
+hipError_t launch_slab(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
+  constexpr int CW = 16 * T;
+  dim3 grid((unsigned)((p.N + CW - 1) / CW));
+  const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
+#define MNB_SLAB_LAUNCH(NW_, CPW_) \
+  mnb_skinny_slab_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
+#define MNB_SLAB_CPW(NW_)            \
+  do {                               \
+    if (cpw == 1)                    \
+      MNB_SLAB_LAUNCH(NW_, 1);       \
+    else if (cpw == 2)               \
+      MNB_SLAB_LAUNCH(NW_, 2);       \
+    else                             \
+      MNB_SLAB_LAUNCH(NW_, 0);       \
+  } while (0)
+  switch (pl.nw) {
+    case 16: MNB_SLAB_CPW(16); break;
+    case 8: MNB_SLAB_CPW(8); break;
+    default: MNB_SLAB_CPW(4); break;
+  }
+#undef MNB_SLAB_CPW
+#undef MNB_SLAB_LAUNCH
+  return hipGetLastError();
 }
 
 template <int BITS, bool HAS_ZP, int MODE, int T>
@@ -335,6 +443,7 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
 
 template <int BITS, bool HAS_ZP, int MODE>
 hipError_t launch_mode(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
+  if (pl.t == 3) return launch_slab<BITS, HAS_ZP, MODE, 3>(p, pl, s);  // offered to the direct variant only
   switch (pl.t) {
     case 4: return launch_t<BITS, HAS_ZP, MODE, 4>(p, pl, s);
     case 2: return launch_t<BITS, HAS_ZP, MODE, 2>(p, pl, s);

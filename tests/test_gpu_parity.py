@@ -131,6 +131,25 @@ def test_gemm_parity(oracle, dtype, bits, bs, zp, bias):
         check_against_oracle(oracle, c, y)
 
 
+@pytest.mark.parametrize("bits,bs,zp", [(4, 128, False), (4, 128, True), (4, 32, True), (8, 64, True), (8, 16, False)])
+@pytest.mark.parametrize("N,K,M", [(8200, 512, 1), (9000, 1024, 5), (12288, 2048, 16), (11008, 4096, 1),
+                                   (12281, 640, 3)])
+def test_decode_with_three_tile_slabs(oracle, bits, bs, zp, N, K, M):
+    """513..768 column tiles: the decode kernel cuts N into slabs of 48 columns that do not start at multiples of 64
+    (tiles addressed one by one); every chunk schedule (one, two, many chunks per wavefront), both dequantisation
+    modes, ragged N, and unit vectors that recover W bit for bit across slab boundaries."""
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + bits)
+    y = run_case(c)
+    check_against_oracle(oracle, c, y)
+    if K <= 1024:
+        eye = np.zeros((16, K), np.float16)
+        ks = np.linspace(0, K - 1, 16).astype(int)
+        eye[np.arange(16), ks] = 1
+        c0 = make_case(16, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + bits)
+        w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
+        assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+
+
 def test_unpacked_route_matches_packed():
     for dtype in (np.float16, np.float32):
         for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128)]:
