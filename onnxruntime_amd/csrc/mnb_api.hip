@@ -199,6 +199,7 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
     return kMnbKernelSkinny;
   }
   if (mnb_gemv_applicable(a)) return kMnbKernelGemv;
+  if (mnb_gemm32_applicable(a)) return kMnbKernelGemm32;
   if (a.L.dtype == kMnbDtypeFloat16) {
     // the tile GEMM loads activations 16 bytes at a time: base and row pitch aligned
     const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
@@ -215,6 +216,7 @@ const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout&) {
     case kMnbKernelGemv: return "mnb_gemv_kernel";
     case kMnbKernelMid: return "mnb_mid_kernel";
     case kMnbKernelGemm256: return "mnb_gemm256_kernel";
+    case kMnbKernelGemm32: return "mnb_gemm32_kernel";
     case kMnbKernelGemmGeneric: return "mnb_gemm_generic_kernel";
     default: return "none";
   }
@@ -270,6 +272,7 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
       break;
     }
     case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
+    case kMnbKernelGemm32: e = mnb_launch_gemm32(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }
   return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbGemm");
@@ -412,6 +415,7 @@ int fused_gemm(const char* fn, const MnbFusedLayout& F, size_t M, const void* a_
     case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
     case kMnbKernelMid: e = mnb_launch_mid(a, s); break;
     case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
+    case kMnbKernelGemm32: e = mnb_launch_gemm32(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }
   if (e != hipSuccess) return hip_fail(e, fn);

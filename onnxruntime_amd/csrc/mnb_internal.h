@@ -33,7 +33,8 @@ enum MnbKernelKind {
   kMnbKernelGemv,       // fp32, M <= 16: dequantising GEMV (VALU dot products, activations in SGPRs)
   kMnbKernelMid,        // fp16, M > 16: weights from registers to the matrix cores, K split over waves (any shape)
   kMnbKernelGemm256,    // fp16, MFMA GEMM with 256 x 256 tiles: large M, enough tiles to fill the chip
-  kMnbKernelGemmGeneric // any shape / fp32 large M: simple tile kernel
+  kMnbKernelGemm32,     // fp32, M > 16: tile GEMM on the fp32 matrix cores
+  kMnbKernelGemmGeneric // any shape: simple tile kernel (fallback)
 };
 
 MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a);
@@ -66,6 +67,8 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
 int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds);
 bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
+bool mnb_gemm32_applicable(const MnbGemmArgs& a);
+hipError_t mnb_launch_gemm32(const MnbGemmArgs& a, hipStream_t s);
 
 // kernels around the fused operators (mnb_fused.hip)
 // A (+ skip) -> A_norm = x / sqrt(mean(x^2) + eps) * scale per row; sum_out (optional) = A + skip
