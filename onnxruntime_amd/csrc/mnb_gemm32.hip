@@ -7,7 +7,7 @@
 // bfloat16 activations run on after widening (mnb_variant.hip).
 //
 // 128 x 128 output tile per workgroup of four wavefronts (2 x 2), each owning 64 x 64 as 2 x 2
-// v_mfma_f32_32x32x2_f32 accumulators.  Per k-step of 32:
+// v_mfma_f32_32x32x2_f32 accumulators (64 x 128 with 32 x 64 per wavefront while such tiles fit the chip in one round).  Per k-step of 32:
 //   * every thread fetches 4 x 16 B of A and 8 bytes (4-bit) or 16 bytes (8-bit) of packed weights for the NEXT step
 //     into registers while the matrix cores work on the current one;
 //   * the weights are dequantised to fp32 in registers - float(q) - zp, one multiply by the scale: the bits of
@@ -29,7 +29,7 @@ namespace {
 typedef float f16v_t __attribute__((ext_vector_type(16)));
 typedef float f4v_t __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int BN = 128, BK = 32;  // rows of the tile: 64 TM, TM = 32-row matrix-core tiles per wavefront (2, or 1 for M <= 64)
 constexpr int THREADS = 256;
 constexpr int STRIDE = BK + 4;  // floats per staged row
 
@@ -46,8 +46,10 @@ struct Gemm32Params {
   int a_vec_ok;  // A allows 16-byte loads: aligned base, row pitch and K multiples of 4 floats
 };
 
-template <int BITS, bool HAS_ZP>
+template <int BITS, bool HAS_ZP, int TM>
 __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
+  constexpr int BM = 64 * TM;
+  constexpr int A_LOADS = 2 * TM;  // 16-byte activation loads per thread and step
   __shared__ __align__(16) float As[BM * STRIDE];
   __shared__ __align__(16) float Bs[BN * STRIDE];
 
@@ -59,20 +61,21 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
   const int m0 = (blockIdx.x / p.tiles_n) * BM;
   const int n0 = (blockIdx.x % p.tiles_n) * BN;
 
-  f16v_t acc[2][2];
+  f16v_t acc[TM][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
 
   // ---- this thread's share of the tiles
-  // A: rows a_row + 32 i (i < 4), floats [a_kc, a_kc + 4) of the step; rows beyond M repeat row M - 1 (never stored)
+  // A: rows a_row + 32 i (i < A_LOADS), floats [a_kc, a_kc + 4) of the step; rows beyond M repeat row M - 1 (never
+  // stored)
   const int a_row = tid >> 3, a_kc = (tid & 7) * 4;
-  const float* a_ptr[4];
+  const float* a_ptr[A_LOADS];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < A_LOADS; ++i) {
     int m = m0 + a_row + 32 * i;
     m = m < p.M ? m : p.M - 1;
     a_ptr[i] = p.A + (int64_t)m * p.lda + a_kc;
@@ -83,14 +86,14 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
   const int64_t col = n0 + b_col;  // < Npad: the padding columns hold zero weights and zero scales
   const int64_t mcol = mnb_meta_col(col);
 
-  f4v_t ra[4];
+  f4v_t ra[A_LOADS];
   uint32_t rw[4];
   float rs = 0.f, rz = 0.f;
 
   auto load_step = [&](int ks) {
     const int k0 = ks * BK;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < A_LOADS; ++i) {
       const float* src = a_ptr[i] + k0;
       if (p.a_vec_ok) {  // K is a multiple of 4: a chunk lies wholly below K or wholly beyond it
         ra[i] = (k0 + a_kc < p.K) ? *reinterpret_cast<const f4v_t*>(src) : f4v_t{0.f, 0.f, 0.f, 0.f};
@@ -116,7 +119,7 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
 
   auto store_step = [&]() {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < A_LOADS; ++i)
       *reinterpret_cast<f4v_t*>(&As[(a_row + 32 * i) * STRIDE + a_kc]) = ra[i];
     float wv[16];
     if constexpr (BITS == 4) {
@@ -148,20 +151,19 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
     store_step();
     __syncthreads();
     if (ks + 1 < p.ksteps) load_step(ks + 1);
-    const float* a_base = &As[(wm * 64 + r) * STRIDE + 16 * h];
+    const float* a_base = &As[(wm * 32 * TM + r) * STRIDE + 16 * h];
     const float* b_base = &Bs[(wn * 64 + r) * STRIDE + 16 * h];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      f4v_t a4[2], b4[2];
+      f4v_t a4[TM], b4[2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        a4[t] = *reinterpret_cast<const f4v_t*>(a_base + t * 32 * STRIDE + 4 * c);
-        b4[t] = *reinterpret_cast<const f4v_t*>(b_base + t * 32 * STRIDE + 4 * c);
-      }
+      for (int t = 0; t < TM; ++t) a4[t] = *reinterpret_cast<const f4v_t*>(a_base + t * 32 * STRIDE + 4 * c);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) b4[t] = *reinterpret_cast<const f4v_t*>(b_base + t * 32 * STRIDE + 4 * c);
 #pragma unroll
       for (int e = 0; e < 4; ++e)
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < 2; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[i][e], b4[j][e], acc[i][j], 0, 0, 0);
@@ -175,10 +177,10 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
     if (n >= p.N) continue;
     const float b = p.bias ? p.bias[n] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        const int m = m0 + wm * 64 + i * 32 + (q >> 2) * 8 + h * 4 + (q & 3);
+        const int m = m0 + wm * 32 * TM + i * 32 + (q >> 2) * 8 + h * 4 + (q & 3);
         if (m < p.M) p.C[(int64_t)m * p.ldc + n] = acc[i][j][q] + b;
       }
     }
@@ -192,8 +194,12 @@ int log2i(int v) {
 }
 
 template <int BITS, bool HAS_ZP>
-hipError_t launch(const Gemm32Params& p, int64_t tiles, hipStream_t s) {
-  mnb_gemm32_kernel<BITS, HAS_ZP><<<dim3((unsigned)tiles), dim3(THREADS), 0, s>>>(p);
+hipError_t launch(const Gemm32Params& p, int64_t row_tiles, int tm, hipStream_t s) {
+  const dim3 grid((unsigned)(row_tiles * p.tiles_n)), blk(THREADS);
+  if (tm == 1)
+    mnb_gemm32_kernel<BITS, HAS_ZP, 1><<<grid, blk, 0, s>>>(p);
+  else
+    mnb_gemm32_kernel<BITS, HAS_ZP, 2><<<grid, blk, 0, s>>>(p);
   return hipGetLastError();
 }
 
@@ -225,7 +231,10 @@ hipError_t mnb_launch_gemm32(const MnbGemmArgs& a, hipStream_t s) {
   p.ksteps = (int)((L.K + BK - 1) / BK);  // <= Kpad / 32: steps past K read zero weights
   p.tiles_n = (int)((L.N + BN - 1) / BN);
   p.a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 4 == 0) && (L.K % 4 == 0);
-  const int64_t tiles = (int64_t)p.tiles_n * ((a.M + BM - 1) / BM);
-  if (L.bits == 4) return L.has_zp ? launch<4, true>(p, tiles, s) : launch<4, false>(p, tiles, s);
-  return L.has_zp ? launch<8, true>(p, tiles, s) : launch<8, false>(p, tiles, s);
+  // 64-row tiles while they still fit the 256 compute units in one round: half the latency of a round
+  const int64_t rows64 = (a.M + 63) / 64;
+  const int tm = rows64 * p.tiles_n <= 256 ? 1 : 2;
+  const int64_t row_tiles = (a.M + 64 * tm - 1) / (64 * tm);
+  if (L.bits == 4) return L.has_zp ? launch<4, true>(p, row_tiles, tm, s) : launch<4, false>(p, row_tiles, tm, s);
+  return L.has_zp ? launch<8, true>(p, row_tiles, tm, s) : launch<8, false>(p, row_tiles, tm, s);
 }
