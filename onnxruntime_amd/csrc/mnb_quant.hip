@@ -118,20 +118,29 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
         const float v = (float)tile[r * kCols + c];
         float t = v * rscale;  // separate statements: the product is rounded before the addition
         t = t + zf32;
-        t = roundf(t);
-        t = t < 0.f ? 0.f : t;
-        t = t > (float)MAXQ ? (float)MAXQ : t;
+        // roundf (halves away from zero) followed by the clamp to [0, MAXQ]: round to nearest even, then push the
+        // upward ties up.  Negative ties need no care, everything below 0.5 ends at 0 either way.
+        const float rn = __builtin_rintf(t);
+        const float up = (t - rn == 0.5f) ? 1.0f : 0.0f;  // the difference is exact
+        t = __builtin_amdgcn_fmed3f(rn + up, 0.f, (float)MAXQ);
         return (uint32_t)(int)t;
       };
       uint8_t* out = B + (n * kbc + kb) * blob + (int64_t)r0 / PER_BYTE;
       const int qbytes = qrows / PER_BYTE;  // 1 (2-bit, block 16), 2 (4-bit block 16, 2-bit block 32) or a multiple of 4
-      if (qbytes >= 4) {
-        for (int w = 0; w < qbytes / 4; ++w) {
-          uint32_t word = 0;
+      auto quant_word = [&](int w) -> uint32_t {
+        uint32_t word = 0;
 #pragma unroll
-          for (int e = 0; e < 4 * PER_BYTE; ++e) word |= quant(r0 + w * 4 * PER_BYTE + e) << (e * BITS);
-          *reinterpret_cast<uint32_t*>(out + 4 * w) = word;
+        for (int e = 0; e < 4 * PER_BYTE; ++e) word |= quant(r0 + w * 4 * PER_BYTE + e) << (e * BITS);
+        return word;
+      };
+      if (qbytes >= 16 && (blob % 16) == 0) {
+        // 16-byte stores (the quarter starts at a multiple of 16 bytes of a 16-byte aligned blob)
+        for (int w = 0; w < qbytes / 16; ++w) {
+          const uint4 v = make_uint4(quant_word(4 * w), quant_word(4 * w + 1), quant_word(4 * w + 2), quant_word(4 * w + 3));
+          *reinterpret_cast<uint4*>(out + 16 * w) = v;
         }
+      } else if (qbytes >= 4) {
+        for (int w = 0; w < qbytes / 4; ++w) *reinterpret_cast<uint32_t*>(out + 4 * w) = quant_word(w);
       } else {
         uint32_t word = 0;
         for (int e = 0; e < qrows; ++e) word |= quant(r0 + e) << (e * BITS);
