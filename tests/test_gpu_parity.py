@@ -131,6 +131,27 @@ def test_gemm_parity(oracle, dtype, bits, bs, zp, bias):
         check_against_oracle(oracle, c, y)
 
 
+@pytest.mark.parametrize("bits,bs,zp", [(4, 32, True), (4, 16, False), (8, 64, True), (2, 32, True)])
+@pytest.mark.parametrize("M,N,K,offset", [(1100, 2100, 160, 0), (1100, 2100, 100, 0), (700, 4100, 93, 1)])
+def test_fp32_matrix_core_gemm_with_128_row_tiles(oracle, bits, bs, zp, M, N, K, offset):
+    """fp32 problems whose 64-row tiles no longer fit the chip in one round run 128 x 128 tiles; K that is not a
+    multiple of the 32-deep step (tail guarded), A that is not 16-byte aligned (element-wise loads), and unit-vector
+    rows that must come back as the fp32 dequantisation, bit for bit, through the fp32 matrix instruction."""
+    c = make_case(M, N, K, bits, bs, np.float32, has_zp=zp, has_bias=True, seed=M + K + bits)
+    ks = np.arange(K)
+    c.A[:K] = 0
+    c.A[ks, ks] = 1                                   # rows 0..K-1: unit vectors
+    op = make_op(c)
+    a = torch.zeros(M * K + 4, dtype=torch.float32, device="cuda:0")
+    a_view = a[offset:offset + M * K].view(M, K)
+    a_view.copy_(dev(c.A))
+    y = op.Compute(a_view, bias=dev(c.bias)).cpu().numpy()
+    check_against_oracle(oracle, c, y)
+    w = oracle.C.dequantize(c.B, c.scales, c.zero_points, N, K, bits, bs)          # [N, K] fp32
+    want = (w.T.astype(np.float32) + c.bias[None, :]).astype(np.float32)            # one fp32 addition per element
+    assert np.array_equal(_bits_view(y[:K]), _bits_view(want))
+
+
 @pytest.mark.parametrize("bits,bs,zp", [(4, 128, False), (4, 128, True), (4, 32, True), (8, 64, True), (8, 16, False)])
 @pytest.mark.parametrize("N,K,M", [(8200, 512, 1), (9000, 1024, 5), (12288, 2048, 16), (11008, 4096, 1),
                                    (12281, 640, 3)])
