@@ -28,8 +28,8 @@ sys.path.insert(0, str(ROOT))
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
 # for a plain copy of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs are summarised in
 # profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md.  They are properties of the kernels, not of one run.
-MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14847.3 * 2.0 + 28.0) * 1024), "c4_prefill": int((109683.5 * 2.0 + 57344.0) * 1024),
-                          "quantize": int((57409.6 * 2.0 + 41462.0) * 1024)}
+MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14853.8 * 2.0 + 28.0) * 1024), "c4_prefill": int((109699.9 * 2.0 + 57344.0) * 1024),
+                          "quantize": int((57404.1 * 2.0 + 33747.9) * 1024), "mlp_decode": int((29669.4 * 2.0 + 28.0) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
 LAYERS = 32
@@ -328,7 +328,7 @@ def main() -> int:
             "ms_per_launch_with_skip_layer_norm_prologue": round(legs["skip_norm"], 5),
             "kernel": "mnb_skinny_kernel",
             "roofline": {"bound": "hbm", "achieved": round(gbs_f, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs_f / HBM_PEAK_GBS, 4), "traffic": None},
+                         "frac": round(gbs_f / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["mlp_decode"]},
         }
         del ops
         torch.cuda.empty_cache()
