@@ -440,12 +440,6 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   }
 }
 
-int log2i(int v) {
-  int s = 0;
-  while ((1 << s) < v) ++s;
-  return s;
-}
-
 template <int BITS, bool HAS_ZP, int MPS, int TM>
 hipError_t launch_tm(const Gemm256Params& p, hipStream_t s) {
   const size_t smem = (size_t)SMEM_HALVES * sizeof(_Float16);  // 73728 bytes
@@ -509,7 +503,7 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.M = (int)a.M;
   p.N = (int)a.L.N;
   p.K = (int)a.L.K;
-  p.bs_shift = log2i(a.L.bs);
+  p.bs_shift = mnb_log2i(a.L.bs);
   p.ksteps = (int)(a.L.K / BK);  // K is a multiple of 2 * BK
   p.tile_rows = mnb_gemm256_tile_rows(a.L, a.M, nullptr);
   p.tiles_m = (int)((a.M + p.tile_rows - 1) / p.tile_rows);

@@ -187,12 +187,6 @@ __global__ void __launch_bounds__(THREADS) mnb_gemm32_kernel(Gemm32Params p) {
   }
 }
 
-int log2i(int v) {
-  int s = 0;
-  while ((1 << s) < v) ++s;
-  return s;
-}
-
 template <int BITS, bool HAS_ZP>
 hipError_t launch(const Gemm32Params& p, int64_t row_tiles, int tm, hipStream_t s) {
   const dim3 grid((unsigned)(row_tiles * p.tiles_n)), blk(THREADS);
@@ -227,7 +221,7 @@ hipError_t mnb_launch_gemm32(const MnbGemmArgs& a, hipStream_t s) {
   p.M = (int)a.M;
   p.N = (int)L.N;
   p.K = (int)L.K;
-  p.bs_shift = log2i(L.bs);
+  p.bs_shift = mnb_log2i(L.bs);
   p.ksteps = (int)((L.K + BK - 1) / BK);  // <= Kpad / 32: steps past K read zero weights
   p.tiles_n = (int)((L.N + BN - 1) / BN);
   p.a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 4 == 0) && (L.K % 4 == 0);

@@ -455,12 +455,6 @@ hipError_t launch_gemv16(const GemvParams& p, hipStream_t s) {
 #undef MNB_G16
 }
 
-int log2i(int v) {
-  int s = 0;
-  while ((1 << s) < v) ++s;
-  return s;
-}
-
 GemvParams make_params(const MnbGemmArgs& a) {
   GemvParams p{};
   p.A = a.A;
@@ -475,7 +469,7 @@ GemvParams make_params(const MnbGemmArgs& a) {
   p.K = (int)a.L.K;
   p.Npad = a.L.Npad;
   p.bs = a.L.bs;
-  p.bs_shift = log2i(a.L.bs);
+  p.bs_shift = mnb_log2i(a.L.bs);
   p.KG = (int)((a.L.K + a.L.group_k - 1) / a.L.group_k);
   return p;
 }

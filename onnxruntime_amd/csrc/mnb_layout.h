@@ -47,6 +47,13 @@ struct MnbLayout {
 
 MNB_HD int64_t mnb_round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+// log2 of a power of two (block sizes)
+MNB_HD int mnb_log2i(int v) {
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+
 // position of column n inside a meta row
 MNB_HD int64_t mnb_meta_col(int64_t n) { return (n & ~(int64_t)63) | ((n & 15) << 2) | ((n >> 4) & 3); }
 

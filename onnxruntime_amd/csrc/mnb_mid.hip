@@ -193,7 +193,8 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   const int64_t row_blocks = (M + 16 * pl.mt - 1) / (16 * pl.mt);
   pl.t = (tiles / 4) * row_blocks >= 192 ? 4 : (tiles / 2) * row_blocks >= 96 ? 2 : 1;
   pl.nw = chunks >= 16 ? 8 : 4;
-  if (const char* e = getenv("MNB_MID_PLAN")) {  // tuning override "<T>,<MT>,<NW>"
+  static const char* const plan_override = getenv("MNB_MID_PLAN");  // tuning override "<T>,<MT>,<NW>", read once
+  if (const char* e = plan_override) {
     int t = 0, mt = 0, nw = 0;
     if (sscanf(e, "%d,%d,%d", &t, &mt, &nw) == 3 && (t == 1 || t == 2 || t == 4) && (mt == 2 || mt == 4) &&
         (nw == 4 || nw == 8)) {
@@ -232,12 +233,6 @@ hipError_t launch_t(const MidParams& p, const MidPlan& pl, hipStream_t s) {
   }
 }
 
-int log2i(int v) {
-  int s = 0;
-  while ((1 << s) < v) ++s;
-  return s;
-}
-
 int mid_row_tiles(int64_t M, int mt) { return (int)((M + 16 * mt - 1) / (16 * mt)) * mt; }
 
 }  // namespace
@@ -269,7 +264,7 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   p.M = (int)a.M;
   p.N = (int)L.N;
   p.K = (int)L.K;
-  p.bs_shift = log2i(L.bs);
+  p.bs_shift = mnb_log2i(L.bs);
   p.chunks = (int)((L.K + CK - 1) / CK);
   p.epi.kind = a.epi.kind;
   if (a.epi.kind != kMnbFusedNone) {

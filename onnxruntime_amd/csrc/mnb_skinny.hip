@@ -365,7 +365,8 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   pl.t = tiles >= 800 ? 4 : tiles >= 320 ? 2 : 1;  // measured: N = 6144 prefers 2 (192 workgroups), N = 4096 prefers 1
   // wavefronts per workgroup: aim for >= 2 chunks per wavefront
   pl.nw = chunks >= 32 ? 16 : chunks >= 16 ? 8 : 4;
-  if (const char* e = getenv("MNB_SKINNY_PLAN")) {  // tuning override "<T>,<NW>"
+  static const char* const plan_override = getenv("MNB_SKINNY_PLAN");  // tuning override "<T>,<NW>", read once
+  if (const char* e = plan_override) {
     int t = 0, nw = 0;
     if (sscanf(e, "%d,%d", &t, &nw) == 2 && (t == 1 || t == 2 || t == 4) && (nw == 4 || nw == 8 || nw == 16)) {
       pl.t = t;
@@ -374,7 +375,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   }
   if (pl.t < min_t) pl.t = min_t;  // gate/up pairs live in one workgroup
   // three tiles per workgroup (slab kernel): one round of at most 256 workgroups where two tiles would need up to 384
-  if (direct && min_t == 1 && tiles > 512 && tiles <= 768 && !getenv("MNB_SKINNY_PLAN")) pl.t = 3;
+  if (direct && min_t == 1 && tiles > 512 && tiles <= 768 && plan_override == nullptr) pl.t = 3;
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
   pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
@@ -456,12 +457,6 @@ hipError_t launch_zp(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s)
   return pl.mode == 0 ? launch_mode<BITS, HAS_ZP, 0>(p, pl, s) : launch_mode<BITS, HAS_ZP, 1>(p, pl, s);
 }
 
-int log2i(int v) {
-  int s = 0;
-  while ((1 << s) < v) ++s;
-  return s;
-}
-
 }  // namespace
 
 bool mnb_skinny_applicable(const MnbGemmArgs& a) {
@@ -485,7 +480,7 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   p.M = (int)a.M;
   p.N = (int)L.N;
   p.K = (int)L.K;
-  p.bs_shift = log2i(L.bs);
+  p.bs_shift = mnb_log2i(L.bs);
   const int CK = 4 * L.group_k;
   p.chunks = (int)((L.K + CK - 1) / CK);
   p.phase_chunks = pl.phase_chunks;
