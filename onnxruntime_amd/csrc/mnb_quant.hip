@@ -13,7 +13,9 @@
 // A workgroup owns 64 neighbouring columns and the 8/bits consecutive blocks that share one zero-point byte.  Each
 // block is first copied to LDS with 16-byte loads (rows of the source are contiguous across the 64 columns), so the
 // source is read from HBM exactly once; the range scan and the quantisation then work from LDS, four threads per
-// column (one quarter of the block each).  The job is bound by that single read of the source.
+// column (one quarter of the block each).  (Reading a thread's elements straight from global memory into registers -
+// no LDS tile, one barrier per block - was measured at less than half the speed: 2-byte loads per lane put too few
+// bytes in flight.)
 #include <hip/hip_runtime.h>
 
 #include "mnb_internal.h"
