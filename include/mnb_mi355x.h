@@ -205,9 +205,11 @@ MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* 
  * activations (type constraint T1 of the schema, contrib_defs.cc:3782-3849; the reference has no CPU kernel for it).
  *
  * They run on the same GEMM kernels as MnbGemm after a transformation made once, at pack time:
- *   g_idx            the k index is permuted so that the elements of one group are adjacent, every group is padded to
- *                    a multiple of 16 elements, and the matrix is packed with block size 16; the activation columns
- *                    are gathered into that order (zeros in the padding) in front of every GEMM.  A g_idx equal to
+ *   g_idx            the k index is permuted so that the elements of one group are adjacent and the matrix is packed
+ *                    in that order: with the operator's block size when every group has a multiple of it (act-order
+ *                    permutations), else with the largest power of two >= 16 that divides every group, else with
+ *                    block size 16 and every group padded to a multiple of 16.  The activation columns are gathered
+ *                    into that order (zeros in the padding) in front of every GEMM.  A g_idx equal to
  *                    k / block_size is recognised and dropped.
  *   typed zero points, bfloat16:  scales and zero points are widened to fp32 (exactly) and the fp32 kernels run on
  *                    a widened copy of the activations; the fp32 result plus bias is narrowed once.  This is the

@@ -5,9 +5,11 @@
 // Nothing here computes a product.  The variants are turned into problems the ordinary kernels run:
 //   * g_idx[k] names the block whose scale and zero point element k uses (Dequantize4BitsKernelReOrder,
 //     onnxruntime/contrib_ops/cpu/quantization/matmul_nbits_impl.cc:19-75).  Sorting k by group makes the members of
-//     a group adjacent; padding every group to a multiple of 16 turns it into whole blocks of 16, the smallest block
-//     size the kernels know.  The weights are packed in that order once; per call the activation columns are
-//     gathered into the same order, with zeros in the padding (so the padded weights never count).
+//     a group adjacent: whole blocks of the operator's block size when every group has a multiple of it (act-order
+//     permutations), otherwise of the largest power of two that divides every group, otherwise - after padding every
+//     group to a multiple of 16 - of 16, the smallest block size the kernels know.  The weights are packed in that
+//     order once; per call the activation columns are gathered into the same order, with zeros in the padding (so
+//     the padded weights never count).
 //   * zero points in the activation type are not integers (HQQ-style quantisers produce them), so they cannot ride
 //     in the fp16 kernels' integer offset.  The fp32 kernels subtract a float zero point anyway: scales and zero
 //     points are widened to fp32, exactly, at pack time, activations are widened per call, and the fp32 result plus
@@ -26,7 +28,7 @@
 namespace {
 
 constexpr int kSrcF32 = 0, kSrcF16 = 1, kSrcBf16 = 2;
-constexpr int kPackedBlock = 16;  // block size of a matrix packed in g_idx order
+constexpr int kMinPackedBlock = 16;  // smallest block size of a matrix packed in g_idx order
 
 int fail(int code, const char* fmt, ...) {
   char buf[1024];
@@ -198,12 +200,15 @@ __global__ void __launch_bounds__(256) mnb_variant_dequant_kernel(float* __restr
 // ---------------------------------------------------------------------------------------------------- planning
 struct GroupOrder {
   bool trivial = true;
+  int packed_block = 0;  // block size of the packed matrix
   int64_t packed_k = 0;
   std::vector<int32_t> gather;       // packed k -> canonical k, -1 in the padding
   std::vector<int32_t> block_group;  // packed block of 16 -> source block
 };
 
-// Sorts k by group (stable), pads every group to whole blocks of 16.
+// Sorts k by group (stable) and pads every group to whole blocks.  The packed block size is the operator's when every
+// group has a multiple of it (GPTQ act-order: a permutation, every group keeps block_size members), else the largest
+// power of two >= 16 that divides every group, else 16 with padding.
 int order_by_group(const int32_t* g_idx, size_t len, int64_t K, int bs, bool tables, GroupOrder* out) {
   const int64_t k_blocks = (K + bs - 1) / bs;
   if ((int64_t)len != K && (int64_t)len != k_blocks * bs)
@@ -221,21 +226,26 @@ int order_by_group(const int32_t* g_idx, size_t len, int64_t K, int bs, bool tab
   }
   if (out->trivial) {
     out->packed_k = K;
+    out->packed_block = bs;
     return MNB_OK;
   }
+  int pb = bs;
+  for (int64_t g = 0; g < k_blocks && pb > kMinPackedBlock; ++g)
+    while (pb > kMinPackedBlock && count[(size_t)g] % pb != 0) pb >>= 1;
+  out->packed_block = pb;
   std::vector<int64_t> start((size_t)k_blocks, 0);
   int64_t total = 0;
   for (int64_t g = 0; g < k_blocks; ++g) {
     start[(size_t)g] = total;
-    total += (count[(size_t)g] + kPackedBlock - 1) / kPackedBlock * kPackedBlock;
+    total += (count[(size_t)g] + pb - 1) / pb * pb;
   }
   out->packed_k = total;
   if (!tables) return MNB_OK;
   out->gather.assign((size_t)total, -1);
-  out->block_group.assign((size_t)(total / kPackedBlock), 0);
+  out->block_group.assign((size_t)(total / pb), 0);
   for (int64_t g = 0; g < k_blocks; ++g) {
-    const int64_t blocks = (count[(size_t)g] + kPackedBlock - 1) / kPackedBlock;
-    for (int64_t b = 0; b < blocks; ++b) out->block_group[(size_t)(start[(size_t)g] / kPackedBlock + b)] = (int32_t)g;
+    const int64_t blocks = (count[(size_t)g] + pb - 1) / pb;
+    for (int64_t b = 0; b < blocks; ++b) out->block_group[(size_t)(start[(size_t)g] / pb + b)] = (int32_t)g;
   }
   std::vector<int64_t> next(start);
   for (int64_t k = 0; k < K; ++k) out->gather[(size_t)next[(size_t)g_idx[k]]++] = (int32_t)k;
@@ -287,6 +297,7 @@ int MnbVariantMakePlan(size_t N, size_t K, int bits, int block_size, int a_dtype
 
   GroupOrder order;
   order.packed_k = (int64_t)K;
+  order.packed_block = block_size;
   if (g_idx_host != nullptr)
     if (int rc = order_by_group(g_idx_host, g_idx_len, (int64_t)K, block_size, false, &order)) return rc;
 
@@ -299,7 +310,7 @@ int MnbVariantMakePlan(size_t N, size_t K, int bits, int block_size, int a_dtype
   plan->has_g_idx = order.trivial ? 0 : 1;
   plan->compute_dtype = (a_dtype == MNB_DTYPE_FLOAT16 && zp_kind != MNB_ZP_TYPED) ? MNB_DTYPE_FLOAT16 : MNB_DTYPE_FLOAT;
   plan->packed_k = order.packed_k;
-  plan->packed_block_size = plan->has_g_idx ? kPackedBlock : block_size;
+  plan->packed_block_size = plan->has_g_idx ? order.packed_block : block_size;
   const MnbLayout L = packed_layout(*plan);
   plan->gather_offset = (uint64_t)L.total_bytes;
   plan->packed_bytes = (uint64_t)L.total_bytes;
@@ -347,7 +358,7 @@ int MnbVariantPack(const MnbVariantPlan* plan, const void* b_dev, const void* sc
   if (g_idx_host == nullptr) return fail(MNB_INVALID_ARGUMENT, "MnbVariantPack: the plan was made with a g_idx");
   GroupOrder order;
   if (int rc = order_by_group(g_idx_host, g_idx_len, plan->K, plan->block_size, true, &order)) return rc;
-  if (order.trivial || order.packed_k != plan->packed_k)
+  if (order.trivial || order.packed_k != plan->packed_k || order.packed_block != plan->packed_block_size)
     return fail(MNB_INVALID_ARGUMENT, "MnbVariantPack: g_idx is not the one the plan was made from");
   const int64_t ld = staged_ld(*plan);
   order.gather.resize((size_t)ld, -1);

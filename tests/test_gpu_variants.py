@@ -137,6 +137,8 @@ def test_gemm_against_float64(kind, zp_kind, g_kind, M):
     assert y.dtype == TORCH[kind] and tuple(y.shape) == (M, N)
     if g_kind in ("none", "trivial"):
         assert not op.plan.has_g_idx
+    elif g_kind == "act_order":   # every group keeps block_size members: the packed matrix keeps the block size
+        assert op.plan.has_g_idx and op.plan.packed_block_size == bs and op.plan.packed_k == K
     else:
         assert op.plan.has_g_idx and op.plan.packed_block_size == 16
     check(kind, c, y, N, K, 4, bs)
