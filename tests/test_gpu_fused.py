@@ -171,6 +171,7 @@ QKV_CASES = [
     (1, 64, 16, 128, 4, 32), (1, 4096, 1024, 4096, 4, 32), (5, 100, 24, 96, 4, 16), (16, 48, 40, 256, 8, 64),
     (33, 128, 32, 512, 4, 128), (100, 72, 8, 200, 4, 32), (300, 512, 128, 256, 4, 32), (600, 768, 256, 512, 8, 32),
     (1024, 4000, 2040, 1024, 4, 32),   # tile GEMM; outputs begin inside a wavefront's 64-column block
+    (2, 6100, 2040, 512, 4, 128),      # decode with 48-column slabs: slabs straddle the borders between Q, K and V
 ]
 
 
