@@ -84,12 +84,14 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
 }
 
 // One chunk: word step i of every column tile against the MT row tiles, then -- the A operands of step i being dead --
-// their reload for the wavefront's next chunk (a_next, when has_next).  The activations are thus prefetched
-// three quarters of a chunk ahead without a second register set.
-template <int BITS, bool HAS_ZP, int T, int MT>
+// their reload for the wavefront's next chunk (a_next, when NEXT_A).  The activations are thus prefetched
+// three quarters of a chunk ahead without a second register set.  NEXT_A is a compile-time flag on purpose: a load
+// under a run-time condition makes the number of outstanding loads unknown to the compiler at the join, and every
+// later wait then degenerates to "wait for all loads", the weight prefetch issued just before included.
+template <int BITS, bool HAS_ZP, int T, int MT, bool NEXT_A>
 __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h8_t (*af)[(128 / BITS) / 8],
-                                                  const uint4* a_next, bool has_next, int64_t a_step,
-                                                  const UnpackConsts& uc, f4_t (*y)[T]) {
+                                                  const uint4* a_next, int64_t a_step, const UnpackConsts& uc,
+                                                  f4_t (*y)[T]) {
   constexpr int NI = (128 / BITS) / 8;
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
@@ -107,9 +109,13 @@ __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) y[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][i], b, y[mt][t], 0, 0, 0);
     }
-    if (has_next) {  // wave-uniform: no divergent branch inside the chunk
+    // Nothing moves across the end of a word step: loads hoisted above the matrix instructions that still read
+    // af[.][i] would need a second register set, and so would dequantised operands prepared steps ahead.
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NEXT_A) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) af[mt][i] = __builtin_bit_cast(h8_t, a_next[i * a_step + mt * 64]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
@@ -147,23 +153,27 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
         af[mt][i] = __builtin_bit_cast(h8_t, a_lane[((int64_t)c * NI + i) * a_step + mt * 64]);
   };
 
-  // weights two chunks ahead (double buffer); activations reloaded word step by word step inside the chunk
+  // Weights two chunks ahead (double buffer), activations reloaded word step by word step inside the chunk.  No load
+  // of the loop sits under a condition, so every wait counts exactly the loads it needs and leaves the younger
+  // prefetches in flight; a prefetch beyond the wavefront's last chunk is clamped to the last chunk of the matrix
+  // instead of skipped (valid memory that another wavefront of the workgroup is reading anyway, never used here).
   auto a_of = [&](int c) -> const uint4* { return a_lane + (int64_t)c * NI * a_step; };
   ChunkRegs<BITS, T> R0, R1;
+  const int last = p.chunks - 1;
   int c = wave;
-  if (c < p.chunks) {
-    load_chunk<BITS, HAS_ZP, 1, T>(p, c, kq, col0, R0);
-    load_a(c);
+  load_chunk<BITS, HAS_ZP, 1, T>(p, min(c, last), kq, col0, R0);
+  load_a(min(c, last));
+  load_chunk<BITS, HAS_ZP, 1, T>(p, min(c + NW, last), kq, col0, R1);
+  __builtin_amdgcn_sched_barrier(0);
+  for (; c + NW < p.chunks; c += 2 * NW) {
+    mid_compute_chunk<BITS, HAS_ZP, T, MT, true>(R0, af, a_of(c + NW), a_step, uc, y);
+    load_chunk<BITS, HAS_ZP, 1, T>(p, min(c + 2 * NW, last), kq, col0, R0);
+    __builtin_amdgcn_sched_barrier(0);
+    mid_compute_chunk<BITS, HAS_ZP, T, MT, true>(R1, af, a_of(min(c + 2 * NW, last)), a_step, uc, y);
+    load_chunk<BITS, HAS_ZP, 1, T>(p, min(c + 3 * NW, last), kq, col0, R1);
+    __builtin_amdgcn_sched_barrier(0);
   }
-  if (c + NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + NW, kq, col0, R1);
-  for (; c < p.chunks; c += 2 * NW) {
-    mid_compute_chunk<BITS, HAS_ZP, T, MT>(R0, af, a_of(c + NW), c + NW < p.chunks, a_step, uc, y);
-    if (c + 2 * NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + 2 * NW, kq, col0, R0);
-    if (c + NW < p.chunks) {
-      mid_compute_chunk<BITS, HAS_ZP, T, MT>(R1, af, a_of(c + 2 * NW), c + 2 * NW < p.chunks, a_step, uc, y);
-      if (c + 3 * NW < p.chunks) load_chunk<BITS, HAS_ZP, 1, T>(p, c + 3 * NW, kq, col0, R1);
-    }
-  }
+  if (c < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false>(R0, af, nullptr, a_step, uc, y);
 
   // reduce over the wavefronts, one row tile at a time: lane (j, kq), register r of y[mt][t] holds
   // row m0 + 16 mt + 4 kq + r, column n0 + 16 t + j
@@ -188,11 +198,32 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   const int CK = 4 * L.group_k;
   const int chunks = (int)((L.K + CK - 1) / CK);
   const int64_t tiles = (L.N + 15) / 16;
-  pl.mt = M <= 32 ? 2 : 4;
-  // the widest column slab (best reuse of the activations) that still leaves the chip enough workgroups
-  const int64_t row_blocks = (M + 16 * pl.mt - 1) / (16 * pl.mt);
-  pl.t = (tiles / 4) * row_blocks >= 192 ? 4 : (tiles / 2) * row_blocks >= 96 ? 2 : 1;
-  pl.nw = chunks >= 16 ? 8 : 4;
+  // A workgroup's tile of 16 T columns x 16 MT rows decides how often a dequantised weight (MT) and a loaded
+  // activation operand (T) are reused; the grid has to give every CU a workgroup first.  Among the shapes that
+  // reach 192 workgroups the largest tile wins, at equal area the wider one (measured: the activations are the
+  // larger stream); if none does, the shape with the most workgroups.
+  int64_t best_wgs = -1;
+  int best_area = 0;
+  pl.t = min_t;
+  pl.mt = 2;
+  for (int t = 4; t >= min_t; t >>= 1) {
+    for (int mt = M <= 32 ? 2 : 4; mt >= 2; mt >>= 1) {
+      const int64_t wgs = ((tiles + t - 1) / t) * ((M + 16 * mt - 1) / (16 * mt));
+      const int area = t * mt;
+      const bool full = wgs >= 192, best_full = best_wgs >= 192;
+      const bool better = best_wgs < 0 || (full && !best_full) || (full && best_full && area > best_area) ||
+                          (!full && !best_full && (wgs > best_wgs || (wgs == best_wgs && area > best_area)));
+      if (better) {
+        best_wgs = wgs;
+        best_area = area;
+        pl.t = t;
+        pl.mt = mt;
+      }
+    }
+  }
+  // eight wavefronts split K further and hide more latency in a single round of workgroups; with several rounds of
+  // the largest tile, two workgroups of four wavefronts share a CU instead
+  pl.nw = chunks < 16 || (best_area == 16 && best_wgs >= 384) ? 4 : 8;
   static const char* const plan_override = getenv("MNB_MID_PLAN");  // tuning override "<T>,<MT>,<NW>", read once
   if (const char* e = plan_override) {
     int t = 0, mt = 0, nw = 0;
@@ -241,10 +272,9 @@ bool mnb_mid_applicable(const MnbGemmArgs& a) { return a.L.dtype == kMnbDtypeFlo
 
 // bytes of the staged copy of A
 size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
-  const MidPlan pl = mid_plan(L, M);
   const int CK = 4 * L.group_k;
   const int64_t chunks = (L.K + CK - 1) / CK;
-  return (size_t)chunks * (L.group_k / 8) * mid_row_tiles(M, pl.mt) * 64 * 16;
+  return (size_t)chunks * (L.group_k / 8) * mid_row_tiles(M, 4) * 64 * 16;  // the larger of the two row blockings
 }
 
 hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
