@@ -35,14 +35,6 @@ template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t* af, const BConst& bc,
                                               const UnpackConsts& uc, f4_t* y) {
   constexpr int NI = (128 / BITS) / 8;
-#if defined(MNB_EXPERIMENT) && MNB_EXPERIMENT == 1
-  // loads only: fold every loaded register into y so nothing is optimised away
-  for (int t = 0; t < T; ++t) {
-    y[t][0] += __builtin_bit_cast(float, R.w[t].x ^ R.w[t].y ^ R.w[t].z ^ R.w[t].w ^ R.m0[t]);
-    y[t][1] += (float)af[t % NI][0];
-  }
-  return;
-#endif
   if constexpr (MODE == 0) {
     // init[m] = -sum_k (off_k + zp) a[m][k] (no zero points) or -sum_k off_k a[m][k]; nc2[m] = -sum_k a[m][k].
     // The constant operands are the same in every lane, so every lane receives the value of its own rows.
@@ -139,112 +131,181 @@ __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* re
   reduce_and_store_tiles<T, NW>(p, red, 0, n0);
 }
 
-// ---- direct variant: A operands straight from global memory (16-byte aligned rows), no barrier before the end ----
+// ---- activations through LDS for 4 < M <= 16 -----------------------------------------------------------------------
+// Lane (j, kq) needs 16 bytes of row j at a 64-byte stride between the kq: read straight from A, one load
+// instruction of a wavefront touches two cache lines per row -- 8 lines for up to four rows, 32 for sixteen -- and the
+// vector cache looks lines up one after the other.  For more than four rows a wavefront therefore reads its chunk of
+// A row-contiguously (64 lanes x 16 bytes = 4 rows x 256 bytes: 8 lines per instruction whatever M is), passes it
+// through a private 4 KiB of LDS and picks its operands up from there.  No barrier is involved: the region belongs
+// to one wavefront and LDS executes a wavefront's accesses in order.  16-byte pieces are XOR-swizzled with the row
+// so that both the row-contiguous writes and the operand reads are free of bank conflicts.
+template <int BITS>
+struct AStage {
+  static constexpr int GK = 128 / BITS, NI = GK / 8;
+  static constexpr int PIECES = 4 * NI;     // 16-byte pieces per row of a chunk
+  static constexpr int RPI = 64 / PIECES;   // rows per load instruction; 16 / RPI == NI instructions
+  static __device__ __forceinline__ int swz(int row) { return PIECES == 16 ? row : (row >> 1); }
+
+  // global -> registers: g[I] = piece (lane % PIECES) of row I * RPI + lane / PIECES (rows >= M re-read row M - 1)
+  static __device__ __forceinline__ void fetch(const SkinnyParams& p, int c, int lane, h8_t* g) {
+    const int piece = lane % PIECES, r0 = lane / PIECES;
+#pragma unroll
+    for (int I = 0; I < NI; ++I) {
+      int row = I * RPI + r0;
+      row = row < p.M ? row : p.M - 1;
+      g[I] = *reinterpret_cast<const h8_t*>(p.A + (int64_t)row * p.lda + (int64_t)c * 4 * GK + piece * 8);
+    }
+  }
+  // registers -> LDS -> operands of lane (j, kq)
+  static __device__ __forceinline__ void pass(h8_t* mine, const h8_t* g, int lane, h8_t* af) {
+    const int piece = lane % PIECES, r0 = lane / PIECES;
+    const int j = lane & 15, kq = lane >> 4;
+#pragma unroll
+    for (int I = 0; I < NI; ++I) {
+      const int row = I * RPI + r0;
+      mine[row * PIECES + (piece ^ swz(row))] = g[I];
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) af[i] = mine[j * PIECES + ((kq * NI + i) ^ swz(j))];
+  }
+};
+
+// ---- direct variants: A operands from global memory (16-byte aligned rows), no barrier before the end -----------
+// The chunk pipeline of a wavefront; `load_w(c, R)` issues the weight and meta loads of chunk c.
 // CPW = chunks per wavefront when that is 1 or 2 for every wavefront (chunks == CPW * NW): everything is loaded up
 // front in straight-line code, so the compiler's s_waitcnt counts are exact and each tile is processed as soon as
 // its own vector has landed.  CPW = 0: general loop with two chunks in flight.
-template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW>
-__global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams p) {
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS, class LoadW>
+__device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned char* smem, int wave, int lane,
+                                              const LoadW& load_w, f4_t* y) {
   constexpr int GK = 128 / BITS;
   constexpr int NI = GK / 8;
-  extern __shared__ __align__(16) unsigned char smem[];
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int j = lane & 15, kq = lane >> 4;
-  const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
-  const int64_t col0 = n0 + j;
-  const int arow = j < p.M ? j : p.M - 1;
+  const int arow = j < p.M ? j : p.M - 1;  // rows >= M of the MFMA A operand re-read row M-1: they are never stored
   const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
-
-  f4_t y[T];
-#pragma unroll
-  for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  h8_t* mine = reinterpret_cast<h8_t*>(smem) + wave * (16 * AStage<BITS>::PIECES);  // A_LDS only
   const BConst bconst = make_bconst<BITS, HAS_ZP>();
   const UnpackConsts uc = make_unpack_consts(p.uc);
 
-  // rows >= M of the MFMA A operand re-read row M-1: they are never stored
-  auto load_a = [&](int c, h8_t* af) {
+  // the activation loads of chunk c: the operands themselves, or the row-contiguous pieces that pass through LDS
+  auto fetch_a = [&](int c, h8_t* a) {
+    if constexpr (A_LDS) {
+      AStage<BITS>::fetch(p, c, lane, a);
+    } else {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) af[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
+      for (int i = 0; i < NI; ++i) a[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
+    }
+  };
+  auto run = [&](const ChunkRegs<BITS, T>& R, const h8_t* a) {
+    if constexpr (A_LDS) {
+      h8_t af[NI];
+      AStage<BITS>::pass(mine, a, lane, af);
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R, af, bconst, uc, y);
+    } else {
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R, a, bconst, uc, y);
+    }
   };
 
   if constexpr (CPW > 0) {
     ChunkRegs<BITS, T> R[CPW];
     h8_t a[CPW][NI];
 #pragma unroll
-    for (int q = 0; q < CPW; ++q) load_a(wave + q * NW, a[q]);
+    for (int q = 0; q < CPW; ++q) fetch_a(wave + q * NW, a[q]);
 #pragma unroll
-    for (int q = 0; q < CPW; ++q) load_chunk<BITS, HAS_ZP, MODE, T>(p, wave + q * NW, kq, col0, R[q]);
+    for (int q = 0; q < CPW; ++q) load_w(wave + q * NW, R[q]);
+    if constexpr (A_LDS) {
+      h8_t af[CPW][NI];
 #pragma unroll
-    for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, y);
-  } else {
-    if constexpr (T <= 2) {
-      // Two chunks in flight.  Loads under a run-time condition would leave the compiler unable to count the
-      // outstanding loads at the join, and every wait of the loop would then be for all of them, the prefetch issued
-      // a moment earlier included.  So the steady state and each possible tail are straight-line code, and the two
-      // loads in front of the loop are clamped to the last chunk instead of skipped (valid memory, not used).
-      ChunkRegs<BITS, T> R0, R1;
-      h8_t a0[NI], a1[NI];
-      auto load = [&](int c, h8_t* a, ChunkRegs<BITS, T>& R) {
-        __builtin_amdgcn_sched_barrier(0);  // the loads stay between the two chunks they are written between
-        load_a(c, a);
-        load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R);
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      const int last = p.chunks - 1;
-      const int mine = wave < p.chunks ? (p.chunks - wave + NW - 1) / NW : 0;  // chunks of this wavefront
-      int c = wave;
-      load(min(c, last), a0, R0);
-      load(min(c + NW, last), a1, R1);
-      int q = 0;
-      for (; q + 3 < mine; q += 2, c += 2 * NW) {
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-        load(c + 2 * NW, a0, R0);
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
-        load(c + 3 * NW, a1, R1);
-      }
-      const int left = mine - q;  // 0 .. 3
-      if (left == 3) {
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-        load(c + 2 * NW, a0, R0);
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-      } else if (left == 2) {
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
-      } else if (left == 1) {
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-      }
+      for (int q = 0; q < CPW; ++q) AStage<BITS>::pass(mine, a[q], lane, af[q]);
+#pragma unroll
+      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], af[q], bconst, uc, y);
     } else {
-      // Wide slabs keep the loop with conditional prefetches: the straight-line form needs 30-50 registers more
-      // there, which 16 wavefronts do not have (measured 11 % slower for T = 4; 2-9 % faster for T = 1, 2).
-      ChunkRegs<BITS, T> R0, R1;
-      h8_t a0[NI], a1[NI];
-      int c = wave;
-      if (c < p.chunks) {
-        load_a(c, a0);
-        load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R0);
+#pragma unroll
+      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, y);
+    }
+  } else if constexpr (T <= 2) {
+    // Two chunks in flight.  Loads under a run-time condition would leave the compiler unable to count the
+    // outstanding loads at the join, and every wait of the loop would then be for all of them, the prefetch issued
+    // a moment earlier included.  So the steady state and each possible tail are straight-line code, and the two
+    // loads in front of the loop are clamped to the last chunk instead of skipped (valid memory, not used).
+    ChunkRegs<BITS, T> R0, R1;
+    h8_t a0[NI], a1[NI];
+    auto load = [&](int c, h8_t* a, ChunkRegs<BITS, T>& R) {
+      __builtin_amdgcn_sched_barrier(0);  // the loads stay between the two chunks they are written between
+      fetch_a(c, a);
+      load_w(c, R);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    const int last = p.chunks - 1;
+    const int own = wave < p.chunks ? (p.chunks - wave + NW - 1) / NW : 0;  // chunks of this wavefront
+    int c = wave;
+    load(min(c, last), a0, R0);
+    load(min(c + NW, last), a1, R1);
+    int q = 0;
+    for (; q + 3 < own; q += 2, c += 2 * NW) {
+      run(R0, a0);
+      load(c + 2 * NW, a0, R0);
+      run(R1, a1);
+      load(c + 3 * NW, a1, R1);
+    }
+    const int left = own - q;  // 0 .. 3
+    if (left == 3) {
+      run(R0, a0);
+      load(c + 2 * NW, a0, R0);
+      run(R1, a1);
+      run(R0, a0);
+    } else if (left == 2) {
+      run(R0, a0);
+      run(R1, a1);
+    } else if (left == 1) {
+      run(R0, a0);
+    }
+  } else {
+    // Wide slabs keep the loop with conditional prefetches: the straight-line form needs 30-50 registers more
+    // there, which 16 wavefronts do not have (measured 11 % slower for T = 4; 2-9 % faster for T = 1, 2).
+    ChunkRegs<BITS, T> R0, R1;
+    h8_t a0[NI], a1[NI];
+    int c = wave;
+    if (c < p.chunks) {
+      fetch_a(c, a0);
+      load_w(c, R0);
+    }
+    if (c + NW < p.chunks) {
+      fetch_a(c + NW, a1);
+      load_w(c + NW, R1);
+    }
+    for (; c < p.chunks; c += 2 * NW) {
+      run(R0, a0);
+      if (c + 2 * NW < p.chunks) {
+        fetch_a(c + 2 * NW, a0);
+        load_w(c + 2 * NW, R0);
       }
       if (c + NW < p.chunks) {
-        load_a(c + NW, a1);
-        load_chunk<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, col0, R1);
-      }
-      for (; c < p.chunks; c += 2 * NW) {
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-        if (c + 2 * NW < p.chunks) {
-          load_a(c + 2 * NW, a0);
-          load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 2 * NW, kq, col0, R0);
-        }
-        if (c + NW < p.chunks) {
-          compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
-          if (c + 3 * NW < p.chunks) {
-            load_a(c + 3 * NW, a1);
-            load_chunk<BITS, HAS_ZP, MODE, T>(p, c + 3 * NW, kq, col0, R1);
-          }
+        run(R1, a1);
+        if (c + 3 * NW < p.chunks) {
+          fetch_a(c + 3 * NW, a1);
+          load_w(c + 3 * NW, R1);
         }
       }
     }
   }
+  if constexpr (A_LDS) __syncthreads();  // the reduction buffer overlays the staging regions of all wavefronts
+}
+
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS>
+__global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kq = lane >> 4;
+  const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
+  const int64_t col0 = n0 + (lane & 15);
+  f4_t y[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  skinny_chunks<BITS, HAS_ZP, MODE, T, NW, CPW, A_LDS>(
+      p, smem, wave, lane,
+      [&](int c, ChunkRegs<BITS, T>& R) { load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R); }, y);
   skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
 }
 
@@ -256,19 +317,13 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams
 // (Slabs with half a tile at the end - 56 columns for N = 14336, which would put exactly one workgroup on every
 // compute unit - were measured too: the half tile costs the instructions of a whole one, and the run time did not
 // improve.)
-template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW>
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS>
 __global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(SkinnyParams p) {
-  constexpr int GK = 128 / BITS;
-  constexpr int NI = GK / 8;
-  constexpr int CW = 16 * T;
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int j = lane & 15, kq = lane >> 4;
-  const int64_t n0 = (int64_t)blockIdx.x * CW;
-  const int arow = j < p.M ? j : p.M - 1;
-  const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
-
+  const int64_t n0 = (int64_t)blockIdx.x * (16 * T);
   int32_t colw[T], mcol[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) {
@@ -277,54 +332,12 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(SkinnyParams p
     colw[t] = (int32_t)col;
     mcol[t] = (int32_t)mnb_meta_col(col);
   }
-
   f4_t y[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-  const BConst bconst = make_bconst<BITS, HAS_ZP>();
-  const UnpackConsts uc = make_unpack_consts(p.uc);
-
-  auto load_a = [&](int c, h8_t* af) {
-#pragma unroll
-    for (int i = 0; i < NI; ++i) af[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
-  };
-
-  if constexpr (CPW > 0) {
-    ChunkRegs<BITS, T> R[CPW];
-    h8_t a[CPW][NI];
-#pragma unroll
-    for (int q = 0; q < CPW; ++q) load_a(wave + q * NW, a[q]);
-#pragma unroll
-    for (int q = 0; q < CPW; ++q) load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, wave + q * NW, kq, colw, mcol, R[q]);
-#pragma unroll
-    for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, y);
-  } else {
-    ChunkRegs<BITS, T> R0, R1;
-    h8_t a0[NI], a1[NI];
-    int c = wave;
-    if (c < p.chunks) {
-      load_a(c, a0);
-      load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c, kq, colw, mcol, R0);
-    }
-    if (c + NW < p.chunks) {
-      load_a(c + NW, a1);
-      load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c + NW, kq, colw, mcol, R1);
-    }
-    for (; c < p.chunks; c += 2 * NW) {
-      compute_chunk<BITS, HAS_ZP, MODE, T>(R0, a0, bconst, uc, y);
-      if (c + 2 * NW < p.chunks) {
-        load_a(c + 2 * NW, a0);
-        load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c + 2 * NW, kq, colw, mcol, R0);
-      }
-      if (c + NW < p.chunks) {
-        compute_chunk<BITS, HAS_ZP, MODE, T>(R1, a1, bconst, uc, y);
-        if (c + 3 * NW < p.chunks) {
-          load_a(c + 3 * NW, a1);
-          load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c + 3 * NW, kq, colw, mcol, R1);
-        }
-      }
-    }
-  }
+  skinny_chunks<BITS, HAS_ZP, MODE, T, NW, CPW, A_LDS>(
+      p, smem, wave, lane,
+      [&](int c, ChunkRegs<BITS, T>& R) { load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c, kq, colw, mcol, R); }, y);
   skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
 }
 
@@ -386,6 +399,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
 
 struct SkinnyPlan {
   int mode, t, nw, phase_chunks, mtr;
+  bool a_lds;  // activations row-contiguously through LDS (more than four rows, one or two chunks per wavefront)
   size_t smem;
 };
 
@@ -417,6 +431,14 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   if (pl.t < min_t) pl.t = min_t;  // gate/up pairs live in one workgroup
   // three tiles per workgroup (slab kernel): one round of at most 256 workgroups where two tiles would need up to 384
   if (direct && min_t == 1 && tiles > 512 && tiles <= 768 && plan_override == nullptr) pl.t = 3;
+  // Activations through LDS (see AStage) pay from nine rows on, for single-tile slabs from five (measured: at
+  // M = 8 the wider slabs gain or lose a few per cent either way; at M = 16 everything gains 10-35 % except the
+  // general loop of four-tile slabs).  The general loop needs one more operand set for it, which sixteen wavefronts
+  // of 4-bit weights cannot hold in their 128 registers: those run with eight (K = 14336, M = 16: 20 -> 13 us).
+  static const int a_lds_from = getenv("MNB_SKINNY_ALDS_FROM") ? atoi(getenv("MNB_SKINNY_ALDS_FROM")) : 5;
+  const bool up_front = chunks == pl.nw || chunks == 2 * pl.nw;  // everything loaded before the first wait
+  pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4);
+  if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
   pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
@@ -424,6 +446,10 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   const size_t a_bytes = direct ? 0 : (size_t)pl.mtr * (pl.phase_chunks * CK + kLdsPad) * 2;
   const size_t red_bytes = (size_t)pl.nw * pl.t * 4 * 64 * 4;
   pl.smem = a_bytes > red_bytes ? a_bytes : red_bytes;
+  if (pl.a_lds) {
+    const size_t stage_bytes = (size_t)pl.nw * GK * 128;  // 16 rows x one chunk of halves per wavefront
+    if (stage_bytes > pl.smem) pl.smem = stage_bytes;
+  }
   return pl;
 }
 
@@ -432,16 +458,27 @@ hipError_t launch_slab(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
   constexpr int CW = 16 * T;
   dim3 grid((unsigned)((p.N + CW - 1) / CW));
   const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
-#define MNB_SLAB_LAUNCH(NW_, CPW_) \
-  mnb_skinny_slab_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
-#define MNB_SLAB_CPW(NW_)            \
-  do {                               \
-    if (cpw == 1)                    \
-      MNB_SLAB_LAUNCH(NW_, 1);       \
-    else if (cpw == 2)               \
-      MNB_SLAB_LAUNCH(NW_, 2);       \
-    else                             \
-      MNB_SLAB_LAUNCH(NW_, 0);       \
+  // the plan never asks for the LDS route in the general loop of sixteen wavefronts on 4-bit weights: not instantiated
+  if (pl.a_lds && cpw == 0 && BITS == 4 && pl.nw == 16) return hipErrorInvalidConfiguration;
+#define MNB_SLAB_LAUNCH(NW_, CPW_, LDS_) \
+  mnb_skinny_slab_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
+#define MNB_SLAB_CPW(NW_)                                           \
+  do {                                                              \
+    if (pl.a_lds) {                                                 \
+      if (cpw == 1)                                                 \
+        MNB_SLAB_LAUNCH(NW_, 1, true);                              \
+      else if (cpw == 2)                                            \
+        MNB_SLAB_LAUNCH(NW_, 2, true);                              \
+      else if constexpr (!(BITS == 4 && NW_ == 16))                 \
+        MNB_SLAB_LAUNCH(NW_, 0, true);                              \
+    } else {                                                        \
+      if (cpw == 1)                                                 \
+        MNB_SLAB_LAUNCH(NW_, 1, false);                             \
+      else if (cpw == 2)                                            \
+        MNB_SLAB_LAUNCH(NW_, 2, false);                             \
+      else                                                          \
+        MNB_SLAB_LAUNCH(NW_, 0, false);                             \
+    }                                                               \
   } while (0)
   switch (pl.nw) {
     case 16: MNB_SLAB_CPW(16); break;
@@ -458,16 +495,27 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
   dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)));
   if (p.a_vec_ok) {
     const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
-#define MNB_SKINNY_LAUNCH(NW_, CPW_) \
-  mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
-#define MNB_SKINNY_CPW(NW_)               \
-  do {                                    \
-    if (cpw == 1)                         \
-      MNB_SKINNY_LAUNCH(NW_, 1);          \
-    else if (cpw == 2)                    \
-      MNB_SKINNY_LAUNCH(NW_, 2);          \
-    else                                  \
-      MNB_SKINNY_LAUNCH(NW_, 0);          \
+    // not instantiated, never planned: LDS route in the general loop of four-tile slabs or of sixteen 4-bit wavefronts
+    if (pl.a_lds && cpw == 0 && (T == 4 || (BITS == 4 && pl.nw == 16))) return hipErrorInvalidConfiguration;
+#define MNB_SKINNY_LAUNCH(NW_, CPW_, LDS_) \
+  mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
+#define MNB_SKINNY_CPW(NW_)                                         \
+  do {                                                              \
+    if (pl.a_lds) {                                                 \
+      if (cpw == 1)                                                 \
+        MNB_SKINNY_LAUNCH(NW_, 1, true);                            \
+      else if (cpw == 2)                                            \
+        MNB_SKINNY_LAUNCH(NW_, 2, true);                            \
+      else if constexpr (!(BITS == 4 && NW_ == 16) && T < 4)        \
+        MNB_SKINNY_LAUNCH(NW_, 0, true);                            \
+    } else {                                                        \
+      if (cpw == 1)                                                 \
+        MNB_SKINNY_LAUNCH(NW_, 1, false);                           \
+      else if (cpw == 2)                                            \
+        MNB_SKINNY_LAUNCH(NW_, 2, false);                           \
+      else                                                          \
+        MNB_SKINNY_LAUNCH(NW_, 0, false);                           \
+    }                                                               \
   } while (0)
     switch (pl.nw) {
       case 16: MNB_SKINNY_CPW(16); break;

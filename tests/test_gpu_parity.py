@@ -171,6 +171,27 @@ def test_decode_with_three_tile_slabs(oracle, bits, bs, zp, N, K, M):
         assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
 
 
+@pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (8, 64, True), (8, 128, False)])
+@pytest.mark.parametrize("N,K", [(100, 4096), (6144, 2048), (9000, 1024), (14400, 512), (200, 14336), (5200, 8320),
+                                 (300, 4160)])
+@pytest.mark.parametrize("M", [5, 9, 16])
+def test_decode_with_activations_through_lds(oracle, bits, bs, zp, N, K, M):
+    """More than four rows (single-tile slabs) or eight: the decode kernel reads its chunk of A row-contiguously and
+    passes it through LDS in a swizzled layout.  Shapes cover one, two and many chunks per wavefront (also unevenly
+    many), slabs of one to four tiles, and long K on 4-bit weights (eight wavefronts); with unit-vector rows the
+    product must return columns of W bit for bit, so a wrong piece, row or swizzle cannot hide in a tolerance."""
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + M)
+    check_against_oracle(oracle, c, run_case(c))
+    if N <= 300:
+        rng = np.random.default_rng(M + K)
+        ks = rng.choice(K, size=M, replace=False)
+        eye = np.zeros((M, K), np.float16)
+        eye[np.arange(M), ks] = 1
+        c0 = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + M)
+        w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
+        assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+
+
 def test_unpacked_route_matches_packed():
     for dtype in (np.float16, np.float32):
         for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128)]:
