@@ -85,11 +85,21 @@ class Problem:
             self.launch(i)
 
 
-def time_steps(torch, run_step, steps: int, warmup: int) -> float:
-    """Milliseconds per step, HIP events on the launch stream, barrier + synchronize on both sides."""
+def time_steps(torch, run_step, steps: int, warmup: int, warm_ms: float = 0.0) -> float:
+    """Milliseconds per step, HIP events on the launch stream, barrier + synchronize on both sides.
+
+    warm_ms > 0 keeps the warm-up going until that much wall time has passed: from idle the matrix-core clock needs
+    about 15 ms of load to settle (measured on the M=2048 GEMM: 305, 241, 230, 225, 225 ... us per launch over
+    consecutive groups of 20 launches), so a compute-bound leg that is timed after a handful of launches reports the
+    ramp, not the kernel.  The decode GEMV shows no such ramp (8.34-8.42 us per launch from the first replay on)."""
     for _ in range(warmup):
         run_step()
     torch.cuda.synchronize()
+    if warm_ms > 0:
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < warm_ms:
+            run_step()
+            torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
     start.record()
@@ -237,8 +247,8 @@ def main() -> int:
     if not args.no_prefill:
         c4 = synthetic.config_c4(seed=0)
         p4 = Problem(c4, 2, torch, _lib)
-        k4 = max(4, args.steps // 5)
-        ms4 = time_steps(torch, p4.step, k4, max(1, args.warmup // 2)) / 2
+        k4 = max(50, args.steps)  # 100+ launches, about 25 ms
+        ms4 = time_steps(torch, p4.step, k4, max(1, args.warmup // 2), warm_ms=30.0) / 2
         tflops = c4.flops() / (ms4 * 1e-3) / 1e12
         out["prefill"] = {
             "workload": "BASELINE configs[3]: M=2048 K=4096 N=14336 bits=4 block_size=32 zero_points bias fp16",
@@ -277,7 +287,7 @@ def main() -> int:
             for w in ws:  # 4 x 117 MB of distinct sources: beyond the Infinity Cache
                 quantize_blockwise(w, c2.bits, c2.block_size, symmetric=True)
 
-        msq = time_steps(torch, qstep, max(4, args.steps // 5), 2) / copies
+        msq = time_steps(torch, qstep, max(4, args.steps // 5), 2, warm_ms=20.0) / copies
         kbq = Kq // c2.block_size
         qbytes = Kq * Nq * 2 + Nq * kbq * (c2.block_size * c2.bits // 8) + Nq * kbq * 2
         out["quantize"] = {
@@ -364,7 +374,7 @@ def sweep(torch, _lib, synthetic):
             g = graph_of(torch, p.step)
             ms = time_steps(torch, g.replay, 20, 3) / copies
         else:
-            ms = time_steps(torch, p.step, 5, 1) / copies
+            ms = time_steps(torch, p.step, 20, 1, warm_ms=30.0) / copies
         gb = case.algorithmic_bytes() / (ms * 1e-3) / 1e9
         tf = case.flops() / (ms * 1e-3) / 1e12
         rows.append((name, p.kernel, ms * 1e3, gb, tf))

@@ -125,7 +125,8 @@ hipError_t mnb_probe_mfma(int random_operands, double* tflops) {
   err = hipMalloc(&out, (size_t)cus * 512 * sizeof(float));
   if (err != hipSuccess) return err;
   hipEvent_t e0 = nullptr, e1 = nullptr;
-  const int iters = 20000;  // a few milliseconds: long enough for the clocks to settle
+  // From idle the matrix-core clock needs about 15 ms of load to settle: one untimed launch of 25 ms, then the timed one.
+  const int iters = 100000;
   auto launch = [&](int n) {
     if (random_operands)
       mnb_probe_mfma_kernel<1><<<cus, 512, 0, nullptr>>>(out, n);
@@ -133,7 +134,7 @@ hipError_t mnb_probe_mfma(int random_operands, double* tflops) {
       mnb_probe_mfma_kernel<0><<<cus, 512, 0, nullptr>>>(out, n);
   };
   if ((err = hipEventCreate(&e0)) == hipSuccess && (err = hipEventCreate(&e1)) == hipSuccess) {
-    launch(200);
+    launch(iters);
     if ((err = hipDeviceSynchronize()) == hipSuccess) {
       (void)hipEventRecord(e0, nullptr);
       launch(iters);
