@@ -29,7 +29,7 @@ sys.path.insert(0, str(ROOT))
 # for a plain copy of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs are summarised in
 # profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md.  They are properties of the kernels, not of one run.
 MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14853.8 * 2.0 + 28.0) * 1024), "c4_prefill": int((109699.9 * 2.0 + 57344.0) * 1024),
-                          "quantize": int((57404.1 * 2.0 + 33747.9) * 1024), "mlp_decode": int((29669.4 * 2.0 + 28.0) * 1024)}
+                          "quantize": int((57399.0 * 2.0 + 30478.3) * 1024), "mlp_decode": int((29669.4 * 2.0 + 28.0) * 1024)}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
 LAYERS = 32

@@ -42,7 +42,6 @@ template <typename T, int BITS, bool HAS_ZP, bool SMALL_BS, int MT>
 __device__ __forceinline__ void mnb_gemv_group(const uint4& wv, const uint8_t* __restrict__ meta, int64_t midx,
                                                int64_t Npad, const T* __restrict__ a_grp, int64_t lda, int M,
                                                float* acc) {
-  constexpr int GK = 128 / BITS;
   constexpr int NBLK = SMALL_BS ? 2 : 1;   // quantisation blocks inside one group
   constexpr int WORDS = 4 / NBLK;          // 32-bit words per block
   const uint32_t wd[4] = {wv.x, wv.y, wv.z, wv.w};

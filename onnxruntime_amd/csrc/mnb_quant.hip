@@ -12,10 +12,11 @@
 //
 // A workgroup owns 64 neighbouring columns and the 8/bits consecutive blocks that share one zero-point byte.  Each
 // block is first copied to LDS with 16-byte loads (rows of the source are contiguous across the 64 columns), so the
-// source is read from HBM exactly once; the range scan and the quantisation then work from LDS, four threads per
-// column (one quarter of the block each).  (Reading a thread's elements straight from global memory into registers -
-// no LDS tile, one barrier per block - was measured at less than half the speed: 2-byte loads per lane put too few
-// bytes in flight.)
+// source is read from HBM exactly once.  Four threads per column take one quarter of the block each: a thread reads
+// its quarter from LDS once, keeps it widened to fp32 in registers across the range scan, and quantises from there
+// (the block size is a template parameter for that reason).  (Reading a thread's elements straight from global
+// memory into registers - no LDS tile, one barrier per block - was measured at less than half the speed: 2-byte
+// loads per lane put too few bytes in flight.)
 #include <hip/hip_runtime.h>
 
 #include "mnb_internal.h"
@@ -25,15 +26,21 @@ namespace {
 constexpr int kCols = 64;      // columns per workgroup
 constexpr int kQuarters = 4;   // threads per column (each takes one quarter of the block)
 
-template <typename T, int BITS>
+// QROWS = block size / 4: the elements of a thread's quarter.  A compile-time constant so that the quarter, widened
+// to fp32, stays in registers between the range scan and the quantisation (each element leaves LDS once).
+template <typename T, int BITS, int QROWS>
 __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t* __restrict__ B, T* __restrict__ scales,
                                                                          uint8_t* __restrict__ zp,
                                                                          const T* __restrict__ src, int64_t K, int64_t N,
-                                                                         int64_t ld, int bs, int vec_ok) {
+                                                                         int64_t ld, int vec_ok, int nsub) {
   constexpr int PER_BYTE = 8 / BITS;  // blocks per zero-point byte, elements per weight byte
   constexpr int MAXQ = (1 << BITS) - 1;
   constexpr int MID = 1 << (BITS - 1);
   constexpr int VEC = 16 / (int)sizeof(T);  // elements per 16-byte load
+  constexpr int bs = QROWS * kQuarters;
+  constexpr int blob = bs * BITS / 8;
+  constexpr int QBITS = QROWS * BITS;       // bits a thread produces per block: 8 (2-bit, block 16), 16, or words
+  constexpr int QWORDS = (QBITS + 31) / 32;
   extern __shared__ __align__(16) unsigned char smem[];
   T* tile = reinterpret_cast<T*>(smem);                                    // [bs][kCols]
   float* red = reinterpret_cast<float*>(smem + (size_t)bs * kCols * sizeof(T));  // [2][kQuarters][kCols]
@@ -43,28 +50,46 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
   const int64_t n0 = (int64_t)blockIdx.x * kCols;
   const int64_t n = n0 + c;
   const int64_t kbc = (K + bs - 1) / bs;
-  const int64_t blob = (int64_t)bs * BITS / 8;
   const int64_t zrow = (kbc * BITS + 7) / 8;
-  const int64_t kb0 = (int64_t)blockIdx.y * PER_BYTE;
+  const int64_t kb0 = (int64_t)blockIdx.y * nsub;
+  const int nb = (int)(kbc - kb0 < nsub ? kbc - kb0 : nsub);  // blocks of this workgroup, consecutive along K
   const bool full_cols = n0 + kCols <= N;
+  const bool fast = vec_ok && full_cols;
+  const int q0 = qr * QROWS;
   uint32_t zbyte = 0;
 
-  for (int sub = 0; sub < PER_BYTE; ++sub) {
-    const int64_t kb = kb0 + sub;
-    if (kb >= kbc) {
-      // the unused part of the last zero-point byte keeps the reference's filler, the default zero point
-      zbyte |= (uint32_t)MID << (sub * BITS);
-      continue;
-    }
+  // The next block travels from global memory into registers while the current one is worked on from LDS.
+  constexpr int CH = kCols / VEC;                                // 16-byte chunks per row
+  constexpr int PRE = (bs * CH + kCols * kQuarters - 1) / (kCols * kQuarters);  // chunks per thread and block
+  // chunk u of a thread: row (tid + 256 u) / CH of the block (rows beyond the block's last re-read that row and are
+  // never used, so that no load sits under a condition), 16-byte piece (tid + 256 u) % CH of the strip
+  auto chunk_ptr = [&](int64_t kb, int u) -> const uint4* {
+    const int64_t k0 = kb * bs;
+    const int rows = (int)(k0 + bs < K ? bs : K - k0);
+    const int i = tid + u * kCols * kQuarters;
+    const int r = i / CH < rows ? i / CH : rows - 1;
+    return reinterpret_cast<const uint4*>(src + (k0 + r) * ld + n0 + (i % CH) * VEC);
+  };
+  uint4 pre[PRE];
+#pragma unroll
+  for (int u = 0; u < PRE; ++u) pre[u] = fast ? *chunk_ptr(kb0, u) : make_uint4(0u, 0u, 0u, 0u);
+
+  for (int sb = 0; sb < nb; ++sb) {
+    const int sub = sb % PER_BYTE;
+    const int64_t kb = kb0 + sb;
     const int64_t k0 = kb * bs;
     const int rows = (int)(k0 + bs < K ? bs : K - k0);
     __syncthreads();  // the previous block's tile is no longer read
-    if (vec_ok && full_cols) {
-      constexpr int CH = kCols / VEC;  // 16-byte chunks per row
-      for (int i = tid; i < rows * CH; i += kCols * kQuarters) {
-        const int r = i / CH, ch = i % CH;
-        *reinterpret_cast<uint4*>(tile + r * kCols + ch * VEC) =
-            *reinterpret_cast<const uint4*>(src + (k0 + r) * ld + n0 + ch * VEC);
+    if (fast) {
+#pragma unroll
+      for (int u = 0; u < PRE; ++u) {
+        const int i = tid + u * kCols * kQuarters;
+        if (bs * CH % (kCols * kQuarters) == 0 || i < bs * CH)
+          *reinterpret_cast<uint4*>(tile + (i / CH) * kCols + (i % CH) * VEC) = pre[u];
+      }
+      if (sb + 1 < nb) {
+#pragma unroll
+        for (int u = 0; u < PRE; ++u) pre[u] = *chunk_ptr(kb + 1, u);
       }
     } else {
       for (int i = tid; i < rows * kCols; i += kCols * kQuarters) {
@@ -74,14 +99,18 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
     }
     __syncthreads();
     // range of this thread's quarter, then of the whole block
-    const int qrows = bs / kQuarters;
-    const int r0 = qr * qrows;
-    const int r1 = r0 + qrows < rows ? r0 + qrows : rows;
+    const int mine = rows - q0 < QROWS ? rows - q0 : QROWS;  // rows of the quarter that exist (may be <= 0)
+    float held[QROWS];
     float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
-    for (int r = r0; r < r1; ++r) {
-      const float v = (float)tile[r * kCols + c];
-      mn = v < mn ? v : mn;
-      mx = v > mx ? v : mx;
+#pragma unroll
+    for (int e = 0; e < QROWS; ++e) {
+      float v = 0.f;
+      if (e < mine) {
+        v = (float)tile[(q0 + e) * kCols + c];
+        mn = v < mn ? v : mn;
+        mx = v > mx ? v : mx;
+      }
+      held[e] = v;
     }
     red[qr * kCols + c] = mn;
     red[(kQuarters + qr) * kCols + c] = mx;
@@ -109,73 +138,96 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
       z = MID;
     }
     zbyte |= (uint32_t)z << (sub * BITS);
+    if (zp && (sub == PER_BYTE - 1 || kb == kbc - 1)) {
+      // the unused part of the last zero-point byte keeps the reference's filler, the default zero point
+      for (int f = sub + 1; f < PER_BYTE; ++f) zbyte |= (uint32_t)MID << (f * BITS);
+      if (n < N && qr == 0) zp[n * zrow + kb / PER_BYTE] = (uint8_t)zbyte;
+      zbyte = 0;
+    }
     const T stored = (T)scale;
     const float sf = (float)stored;
     const float rscale = sf != 0.f ? 1.0f / sf : 0.f;
     const float zf32 = (float)z;
     if (n < N) {
       if (qr == 0) scales[n * kbc + kb] = stored;
-      auto quant = [&](int r) -> uint32_t {
-        if (r >= rows) return (uint32_t)z;
-        const float v = (float)tile[r * kCols + c];
-        float t = v * rscale;  // separate statements: the product is rounded before the addition
-        t = t + zf32;
-        // roundf (halves away from zero) followed by the clamp to [0, MAXQ]: round to nearest even, then push the
-        // upward ties up.  Negative ties need no care, everything below 0.5 ends at 0 either way.
-        const float rn = __builtin_rintf(t);
-        const float up = (t - rn == 0.5f) ? 1.0f : 0.0f;  // the difference is exact
-        t = __builtin_amdgcn_fmed3f(rn + up, 0.f, (float)MAXQ);
-        return (uint32_t)(int)t;
-      };
-      uint8_t* out = B + (n * kbc + kb) * blob + (int64_t)r0 / PER_BYTE;
-      const int qbytes = qrows / PER_BYTE;  // 1 (2-bit, block 16), 2 (4-bit block 16, 2-bit block 32) or a multiple of 4
-      auto quant_word = [&](int w) -> uint32_t {
-        uint32_t word = 0;
+      uint32_t word[QWORDS];
 #pragma unroll
-        for (int e = 0; e < 4 * PER_BYTE; ++e) word |= quant(r0 + w * 4 * PER_BYTE + e) << (e * BITS);
-        return word;
-      };
-      if (qbytes >= 16 && (blob % 16) == 0) {
-        // 16-byte stores (the quarter starts at a multiple of 16 bytes of a 16-byte aligned blob)
-        for (int w = 0; w < qbytes / 16; ++w) {
-          const uint4 v = make_uint4(quant_word(4 * w), quant_word(4 * w + 1), quant_word(4 * w + 2), quant_word(4 * w + 3));
-          *reinterpret_cast<uint4*>(out + 16 * w) = v;
+      for (int w = 0; w < QWORDS; ++w) word[w] = 0;
+#pragma unroll
+      for (int e = 0; e < QROWS; ++e) {
+        uint32_t q = (uint32_t)z;
+        if (e < mine) {
+          float t = held[e] * rscale;  // separate statements: the product is rounded before the addition
+          t = t + zf32;
+          // clamp(roundf(t), 0, MAXQ), roundf rounding halves away from zero: for t >= 0 that is
+          // trunc(t + 0.49999997f) (the largest float below one half: a sum that lands exactly between two floats
+          // rounds to the even one, which is the integer, only when t itself is a tie), everything below 0.5 ends
+          // at 0 either way, and the clamp commutes with the truncation because its bounds are integers.
+          t = t + 0.49999997f;
+          t = __builtin_amdgcn_fmed3f(t, 0.f, (float)MAXQ);
+          q = (uint32_t)t;
         }
-      } else if (qbytes >= 4) {
-        for (int w = 0; w < qbytes / 4; ++w) *reinterpret_cast<uint32_t*>(out + 4 * w) = quant_word(w);
+        word[(e * BITS) / 32] |= q << ((e * BITS) % 32);
+      }
+      uint8_t* out = B + (n * kbc + kb) * blob + qr * (QBITS / 8);
+      if constexpr (QBITS == 8) {
+        *out = (uint8_t)word[0];
+      } else if constexpr (QBITS == 16) {
+        *reinterpret_cast<uint16_t*>(out) = (uint16_t)word[0];
+      } else if constexpr (QWORDS % 4 == 0) {
+        // 16-byte stores (the quarter starts at a multiple of 16 bytes of a 16-byte aligned blob)
+#pragma unroll
+        for (int w = 0; w < QWORDS; w += 4)
+          *reinterpret_cast<uint4*>(out + 4 * w) = make_uint4(word[w], word[w + 1], word[w + 2], word[w + 3]);
       } else {
-        uint32_t word = 0;
-        for (int e = 0; e < qrows; ++e) word |= quant(r0 + e) << (e * BITS);
-        if (qbytes == 1)
-          *out = (uint8_t)word;  // 2-bit, block 16: four elements per thread
-        else
-          *reinterpret_cast<uint16_t*>(out) = (uint16_t)word;
+#pragma unroll
+        for (int w = 0; w < QWORDS; ++w) *reinterpret_cast<uint32_t*>(out + 4 * w) = word[w];
       }
     }
   }
-  if (zp && n < N && qr == 0) zp[n * zrow + blockIdx.y] = (uint8_t)zbyte;
+}
+
+template <typename T, int BITS, int QROWS>
+hipError_t launch_k(void* B, void* scales, void* zp, const void* src, int64_t K, int64_t N, int64_t ld, hipStream_t s) {
+  constexpr int bs = QROWS * kQuarters;
+  const auto kernel = mnb_quantize_kernel<T, BITS, QROWS>;
+  const size_t smem = (size_t)bs * kCols * sizeof(T) + 2 * kQuarters * kCols * sizeof(float);
+  // fp32 sources with 256-deep blocks need 66 KiB of LDS: above the default limit, within the CU's 160 KiB
+  if (smem > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)smem);
+    if (e != hipSuccess) return e;
+  }
+  const int64_t kbc = (K + bs - 1) / bs;
+  // Blocks per workgroup: the 8/bits blocks of one zero-point byte when zero points are written, else one.  Many
+  // small workgroups beat few long ones here: [4096, 14336] fp16 to 4 bits, blocks of 128, takes 36 us with one
+  // block per workgroup (7168 workgroups), 41 us with two and 44-46 us with four to eight.
+  const int nsub = zp ? 8 / BITS : 1;
+  const int64_t strips = (N + kCols - 1) / kCols;
+  dim3 grid((unsigned)strips, (unsigned)((kbc + nsub - 1) / nsub)), blk(kCols * kQuarters);
+  const int vec_ok = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (ld % (16 / sizeof(T)) == 0);
+  kernel<<<grid, blk, smem, s>>>((uint8_t*)B, (T*)scales, (uint8_t*)zp, (const T*)src, K, N, ld, vec_ok, nsub);
+  return hipGetLastError();
+}
+
+template <typename T, int BITS>
+hipError_t launch_b(void* B, void* scales, void* zp, const void* src, int64_t K, int64_t N, int64_t ld, int bs,
+                    hipStream_t s) {
+  switch (bs) {
+    case 16: return launch_k<T, BITS, 4>(B, scales, zp, src, K, N, ld, s);
+    case 32: return launch_k<T, BITS, 8>(B, scales, zp, src, K, N, ld, s);
+    case 64: return launch_k<T, BITS, 16>(B, scales, zp, src, K, N, ld, s);
+    case 128: return launch_k<T, BITS, 32>(B, scales, zp, src, K, N, ld, s);
+    case 256: return launch_k<T, BITS, 64>(B, scales, zp, src, K, N, ld, s);
+    default: return hipErrorInvalidValue;
+  }
 }
 
 template <typename T>
 hipError_t launch_t(void* B, void* scales, void* zp, const void* src, int64_t K, int64_t N, int64_t ld, int bits,
                     int bs, hipStream_t s) {
-  const int64_t kbc = (K + bs - 1) / bs;
-  const int per_byte = 8 / bits;
-  dim3 grid((unsigned)((N + kCols - 1) / kCols), (unsigned)((kbc + per_byte - 1) / per_byte)), blk(kCols * kQuarters);
-  const size_t smem = (size_t)bs * kCols * sizeof(T) + 2 * kQuarters * kCols * sizeof(float);
-  const int vec_ok = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (ld % (16 / sizeof(T)) == 0);
-  auto launch = [&](auto kernel) -> hipError_t {
-    // fp32 sources with 256-deep blocks need 66 KiB of LDS: above the default limit, within the CU's 160 KiB
-    if (smem > 64 * 1024) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-      if (e != hipSuccess) return e;
-    }
-    kernel<<<grid, blk, smem, s>>>((uint8_t*)B, (T*)scales, (uint8_t*)zp, (const T*)src, K, N, ld, bs, vec_ok);
-    return hipGetLastError();
-  };
-  if (bits == 2) return launch(mnb_quantize_kernel<T, 2>);
-  return bits == 4 ? launch(mnb_quantize_kernel<T, 4>) : launch(mnb_quantize_kernel<T, 8>);
+  if (bits == 2) return launch_b<T, 2>(B, scales, zp, src, K, N, ld, bs, s);
+  return bits == 4 ? launch_b<T, 4>(B, scales, zp, src, K, N, ld, bs, s) : launch_b<T, 8>(B, scales, zp, src, K, N, ld, bs, s);
 }
 
 }  // namespace

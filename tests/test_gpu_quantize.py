@@ -19,7 +19,7 @@ def _bits(a):
 @pytest.mark.parametrize("bs", [16, 32, 64, 128, 256])
 @pytest.mark.parametrize("symmetric", [False, True])
 def test_identical_to_oracle(oracle, dtype, bits, bs, symmetric):
-    for (K, N) in [(64, 8), (93, 33), (260, 300), (1234, 5), (512, 257)]:
+    for (K, N) in [(64, 8), (93, 33), (260, 300), (1234, 5), (512, 257), (200, 128), (1000, 192)]:
         rng = np.random.default_rng(K * 7 + N + bits + bs)
         W = (rng.standard_normal((K, N)) * rng.uniform(0.01, 2.0, size=(1, N))).astype(dtype)
         W[:, 0] = 0                                   # an all-zero column: scale 0
@@ -35,6 +35,29 @@ def test_identical_to_oracle(oracle, dtype, bits, bs, symmetric):
         else:
             assert np.array_equal(zp.cpu().numpy(), z), (K, N, "zero points")
         assert np.array_equal(b.cpu().numpy(), Bq), (K, N, "weights")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_exact_ties_round_away_from_zero(oracle, dtype, bits):
+    """Elements that land exactly half way between two integers (power-of-two scale) round like roundf in the oracle."""
+    bs, N, kb = 32, 128, 6
+    mid, maxq = 1 << (bits - 1), (1 << bits) - 1
+    rng = np.random.default_rng(bits)
+    scale = np.ldexp(1.0, -rng.integers(1, 6, size=(kb, 1, N)))
+    steps = rng.integers(-2 * mid - 2, 2 * mid + 2, size=(kb, bs, N)) * 0.5       # multiples of one half, some clamp
+    steps[:, 0, :] = -mid                                                         # pins the symmetric scale to `scale`
+    steps = np.clip(steps, -mid, mid)
+    W = (steps * scale).reshape(kb * bs, N).astype(dtype)                         # exact in fp16
+    for symmetric in (True, False):
+        Bq, s, z = oracle.C.quantize(W, bits, bs, symmetric)
+        b, sc, zp = quantize_blockwise(dev(W), bits, bs, symmetric)
+        torch.cuda.synchronize()
+        assert np.array_equal(_bits(sc.cpu().numpy()), _bits(s))
+        assert np.array_equal(b.cpu().numpy(), Bq)
+        if not symmetric:
+            assert np.array_equal(zp.cpu().numpy(), z)
+    assert maxq == 2 * mid - 1
 
 
 def test_strided_source_and_grid_round_trip():
