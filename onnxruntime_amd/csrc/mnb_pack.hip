@@ -72,6 +72,81 @@ __global__ void __launch_bounds__(256) mnb_pack_weights_kernel(MnbPackSrc S, uin
   W[g * L.Npad + n] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The same transformation as a tiled transpose, for 4- and 8-bit sources whose columns are whole 16-byte groups at
+// 16-byte aligned addresses (every block size but 16 with an odd block count).  In the kernel above a wavefront reads
+// 64 x 16 single bytes and writes 64 vectors to 64 different cache lines; here a workgroup moves a tile of 32 columns
+// x 32 groups through LDS: 16-byte loads with the lanes along a column (512-byte runs of the canonical matrix),
+// 16-byte stores with the lanes along the columns (512-byte runs of the packed one).  LDS rows are padded by one
+// vector, so the transposed reads are free of bank conflicts.
+constexpr int kPackTile = 32;
+
+// canonical nibble i of a word holds element e_i; the packed word holds e0 e2 e4 e6 e1 e3 e5 e7
+__device__ __forceinline__ uint32_t mnb_pack_nibble_order(uint32_t v) {
+  uint32_t lo = v & 0x0F0F0F0Fu, hi = (v >> 4) & 0x0F0F0F0Fu;  // even / odd elements, one per byte
+  lo = (lo | (lo >> 4)) & 0x00FF00FFu;
+  hi = (hi | (hi >> 4)) & 0x00FF00FFu;
+  lo = (lo | (lo >> 8)) & 0x0000FFFFu;
+  hi = (hi | (hi >> 8)) & 0x0000FFFFu;
+  return lo | (hi << 16);
+}
+
+template <int BITS>
+__global__ void __launch_bounds__(256) mnb_pack_weights_tiled_kernel(MnbPackSrc S, uint4* __restrict__ W, MnbLayout L) {
+  static_assert(BITS == 4 || BITS == 8, "2-bit sources take the element-wise kernel");
+  __shared__ uint4 tile[kPackTile][kPackTile + 1];
+  const int64_t n0 = (int64_t)blockIdx.x * kPackTile, g0 = (int64_t)blockIdx.y * kPackTile;
+  const int64_t col_groups = L.k_blocks * L.bs * BITS / 128;  // whole 16-byte groups of one canonical column
+#pragma unroll
+  for (int r = 0; r < kPackTile * kPackTile / 256; ++r) {
+    const int i = threadIdx.x + 256 * r;
+    const int gl = i % kPackTile, nl = i / kPackTile;
+    const int64_t g = g0 + gl;
+    int m;
+    int64_t col;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (g < col_groups && mnb_map_col(S.map, n0 + nl, &m, &col))
+      v = reinterpret_cast<const uint4*>(S.B[m])[col * col_groups + g];
+    if constexpr (BITS == 4) {
+      v.x = mnb_pack_nibble_order(v.x);
+      v.y = mnb_pack_nibble_order(v.y);
+      v.z = mnb_pack_nibble_order(v.z);
+      v.w = mnb_pack_nibble_order(v.w);
+    }
+    tile[nl][gl] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kPackTile * kPackTile / 256; ++r) {
+    const int i = threadIdx.x + 256 * r;
+    const int nl = i % kPackTile, gl = i / kPackTile;
+    if (g0 + gl < L.KG) W[(g0 + gl) * L.Npad + n0 + nl] = tile[nl][gl];  // Npad is a multiple of the tile
+  }
+}
+
+// Launches the weight repacking: the tiled kernel where its alignment conditions hold, else the element-wise one.
+static void mnb_pack_weights_dispatch(const MnbPackSrc& S, uint4* W, const MnbLayout& L, hipStream_t s) {
+  const int64_t wn = L.Npad * L.KG;
+  const dim3 grid((unsigned)((wn + 255) / 256)), blk(256);
+  if (L.src_bits == 2) {
+    mnb_pack_weights_kernel<2><<<grid, blk, 0, s>>>(S, W, L);
+    return;
+  }
+  bool tiled = (L.k_blocks * L.bs * L.bits) % 128 == 0 && L.Npad % kPackTile == 0;
+  for (int m = 0; m < 3; ++m) tiled = tiled && reinterpret_cast<uintptr_t>(S.B[m]) % 16 == 0;
+  const dim3 tgrid((unsigned)(L.Npad / kPackTile), (unsigned)((L.KG + kPackTile - 1) / kPackTile));
+  if (L.bits == 4) {
+    if (tiled)
+      mnb_pack_weights_tiled_kernel<4><<<tgrid, blk, 0, s>>>(S, W, L);
+    else
+      mnb_pack_weights_kernel<4><<<grid, blk, 0, s>>>(S, W, L);
+  } else {
+    if (tiled)
+      mnb_pack_weights_tiled_kernel<8><<<tgrid, blk, 0, s>>>(S, W, L);
+    else
+      mnb_pack_weights_kernel<8><<<grid, blk, 0, s>>>(S, W, L);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ pack meta
 // One thread per (block kb, column n).
 template <typename T, int BITS, bool HAS_ZP>
@@ -191,22 +266,19 @@ template <typename T>
 static hipError_t pack_t(const MnbLayout& L, const MnbPackSrc& S, const void* zp, void* packed, hipStream_t s) {
   uint4* W = reinterpret_cast<uint4*>(packed);
   uint8_t* meta = reinterpret_cast<uint8_t*>(packed) + L.meta_off;
-  const int64_t wn = L.Npad * L.KG;
   const int64_t mn = L.KBp * L.Npad;
   dim3 blk(256);
-  const dim3 wgrid((unsigned)((wn + 255) / 256)), mgrid((unsigned)((mn + 255) / 256));
+  const dim3 mgrid((unsigned)((mn + 255) / 256));
   const uint8_t* z = (const uint8_t*)zp;
+  mnb_pack_weights_dispatch(S, W, L, s);
   if (L.src_bits == 2) {
-    mnb_pack_weights_kernel<2><<<wgrid, blk, 0, s>>>(S, W, L);
     mnb_pack_meta_kernel<T, 2, true><<<mgrid, blk, 0, s>>>(S, z, meta, L);  // z may be NULL: default stored
   } else if (L.bits == 4) {
-    mnb_pack_weights_kernel<4><<<wgrid, blk, 0, s>>>(S, W, L);
     if (zp)
       mnb_pack_meta_kernel<T, 4, true><<<mgrid, blk, 0, s>>>(S, z, meta, L);
     else
       mnb_pack_meta_kernel<T, 4, false><<<mgrid, blk, 0, s>>>(S, nullptr, meta, L);
   } else {
-    mnb_pack_weights_kernel<8><<<wgrid, blk, 0, s>>>(S, W, L);
     if (zp)
       mnb_pack_meta_kernel<T, 8, true><<<mgrid, blk, 0, s>>>(S, z, meta, L);
     else
@@ -222,15 +294,7 @@ hipError_t mnb_launch_pack_weights(const MnbLayout& L, const void* B, void* pack
   S.map.nsrc = 1;
   S.map.n[0] = L.N;
   S.map.Np = L.N;
-  uint4* W = reinterpret_cast<uint4*>(packed);
-  const int64_t wn = L.Npad * L.KG;
-  const dim3 grid((unsigned)((wn + 255) / 256)), blk(256);
-  if (L.src_bits == 2)
-    mnb_pack_weights_kernel<2><<<grid, blk, 0, s>>>(S, W, L);
-  else if (L.bits == 4)
-    mnb_pack_weights_kernel<4><<<grid, blk, 0, s>>>(S, W, L);
-  else
-    mnb_pack_weights_kernel<8><<<grid, blk, 0, s>>>(S, W, L);
+  mnb_pack_weights_dispatch(S, reinterpret_cast<uint4*>(packed), L, s);
   return hipGetLastError();
 }
 
