@@ -300,7 +300,27 @@ def main() -> int:
                          "unit": "GB/s", "frac": round(qbytes / (msq * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                          "traffic": MEASURED_TRAFFIC_BYTES["quantize"]},
         }
+        # ---- and back: MlasDequantizeBlockwise semantics on the quantiser's output (4 distinct operand sets) --------
+        from onnxruntime_amd.matmul_nbits import dequantize_blockwise
+        qs = [quantize_blockwise(w, c2.bits, c2.block_size, symmetric=True) for w in ws]
         del ws
+        torch.cuda.empty_cache()
+
+        def dstep():
+            for (b, sc, z) in qs:  # the allocator hands every call the 117 MB block the previous result just freed
+                dequantize_blockwise(b, sc, z, Nq, Kq, c2.bits, c2.block_size)
+
+        msd = time_steps(torch, dstep, max(4, args.steps // 5), 2, warm_ms=20.0) / copies
+        out["dequantize"] = {
+            "workload": "MlasDequantizeBlockwise semantics: int4 block_size=128 symmetric [14336, 32, 64] -> fp16 [14336, 4096]",
+            "value": round(qbytes / (msd * 1e-3) / 1e9, 1),
+            "unit": "GB/s",
+            "ms_per_launch": round(msd, 4),
+            "kernel": "mnb_dequant_canonical_vec_kernel",
+            "roofline": {"bound": "hbm", "achieved": round(qbytes / (msd * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(qbytes / (msd * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None},
+        }
+        del qs
         torch.cuda.empty_cache()
 
     # ---- MatMulNBitsMlp: the gate and up projections of configs[1]'s shape in one launch ------------------------

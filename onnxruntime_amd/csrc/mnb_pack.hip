@@ -238,10 +238,61 @@ __global__ void __launch_bounds__(256) mnb_dequant_canonical_kernel(T* __restric
   }
 }
 
+// The same for K % 8 == 0 and aligned operands: one thread per 8 consecutive k of one column (they share a block,
+// block sizes being multiples of 16): one 2-, 4- or 8-byte load of weights, 16- or 32-byte stores, consecutive
+// threads on consecutive addresses of both.  Arithmetic per element as above.
+template <typename T, int BITS>
+__global__ void __launch_bounds__(256) mnb_dequant_canonical_vec_kernel(T* __restrict__ dst,
+                                                                        const uint8_t* __restrict__ B,
+                                                                        const T* __restrict__ scales,
+                                                                        const uint8_t* __restrict__ zp, int64_t N,
+                                                                        int64_t K, int bs) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // 8-element unit
+  const int64_t upr = K / 8;                                            // units per row of dst
+  if (idx >= N * upr) return;
+  const int64_t n = idx / upr, k = (idx % upr) * 8;
+  const int64_t kbc = (K + bs - 1) / bs;
+  const int64_t kb = k / bs, r = k % bs;
+  const uint8_t* src = B + (n * kbc + kb) * (bs * BITS / 8) + r * BITS / 8;
+  int q[8], z = 1 << (BITS - 1);
+  if constexpr (BITS == 8) {
+    const uint2 w = *reinterpret_cast<const uint2*>(src);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      q[e] = (w.x >> (8 * e)) & 0xFF;
+      q[4 + e] = (w.y >> (8 * e)) & 0xFF;
+    }
+    if (zp) z = zp[n * kbc + kb];
+  } else if constexpr (BITS == 4) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(src);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q[e] = (w >> (4 * e)) & 0xF;
+    if (zp) z = (zp[n * ((kbc + 1) / 2) + (kb >> 1)] >> ((kb & 1) * 4)) & 0xF;
+  } else {
+    const uint32_t w = *reinterpret_cast<const uint16_t*>(src);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) q[e] = (w >> (2 * e)) & 0x3;
+    if (zp) z = (zp[n * ((kbc + 3) / 4) + (kb >> 2)] >> ((kb & 3) * 2)) & 0x3;
+  }
+  const T s = scales[n * kbc + kb];
+  __align__(16) T out[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    if constexpr (sizeof(T) == 2)
+      out[e] = (_Float16)(q[e] - z) * s;  // exact integer half times half: one RNE rounding
+    else
+      out[e] = (float)(q[e] - z) * s;
+  }
+  uint4* d = reinterpret_cast<uint4*>(dst + n * K + k);
+  const uint4* o = reinterpret_cast<const uint4*>(out);
+#pragma unroll
+  for (int v = 0; v < (int)(8 * sizeof(T) / 16); ++v) d[v] = o[v];
+}
+
 // Packed buffer -> dst[n*K + k], through the same unpack code the GEMV/GEMM kernels use.
 template <typename T, int BITS, bool HAS_ZP>
 __global__ void __launch_bounds__(256) mnb_dequant_packed_kernel(T* __restrict__ dst, const uint8_t* __restrict__ packed,
-                                                                 MnbLayout L) {
+                                                                 MnbLayout L, int vec_ok) {
   constexpr int GK = 128 / BITS;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t g = idx / L.Npad;
@@ -249,11 +300,19 @@ __global__ void __launch_bounds__(256) mnb_dequant_packed_kernel(T* __restrict__
   if (g >= L.KG || n >= L.N) return;
   const uint4 v = reinterpret_cast<const uint4*>(packed)[g * L.Npad + n];
   const uint8_t* meta = packed + L.meta_off;
-  T out[GK];
+  __align__(16) T out[GK];
   if constexpr (sizeof(T) == 2) {
     mnb_dequant_group_h<BITS, HAS_ZP>(v, meta, g, n, L.Npad, L.bs, out);
   } else {
     mnb_dequant_group_f<BITS, HAS_ZP>(v, meta, g, n, L.Npad, L.bs, out);
+  }
+  if (vec_ok && (g + 1) * GK <= L.K) {
+    // whole group inside the row, 16-byte aligned (K % 8 == 0, aligned dst): 16-byte stores
+    uint4* d = reinterpret_cast<uint4*>(dst + n * L.K + g * GK);
+    const uint4* o = reinterpret_cast<const uint4*>(out);
+#pragma unroll
+    for (int i = 0; i < (int)(GK * sizeof(T) / 16); ++i) d[i] = o[i];
+    return;
   }
   for (int i = 0; i < GK; ++i) {
     const int64_t k = g * GK + i;
@@ -331,39 +390,35 @@ hipError_t mnb_launch_pack_fused(const MnbFusedLayout& F, const void* const* B, 
   return hipGetLastError();
 }
 
-hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,
-                                        int64_t K, int bits, int bs, int dtype, hipStream_t s) {
-  const int64_t total = N * K;
-  if (total == 0) return hipSuccess;
-  dim3 grid((unsigned)((total + 255) / 256)), blk(256);
-  if (bits == 2) {
-    if (dtype == kMnbDtypeFloat16)
-      mnb_dequant_canonical_kernel<_Float16, 2><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,
-                                                                     (const _Float16*)scales, (const uint8_t*)zp, N, K,
-                                                                     bs);
-    else
-      mnb_dequant_canonical_kernel<float, 2><<<grid, blk, 0, s>>>((float*)dst, (const uint8_t*)B, (const float*)scales,
-                                                                  (const uint8_t*)zp, N, K, bs);
-    return hipGetLastError();
-  }
-  if (dtype == kMnbDtypeFloat16) {
-    if (bits == 4)
-      mnb_dequant_canonical_kernel<_Float16, 4><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,
-                                                                     (const _Float16*)scales, (const uint8_t*)zp, N, K,
-                                                                     bs);
-    else
-      mnb_dequant_canonical_kernel<_Float16, 8><<<grid, blk, 0, s>>>((_Float16*)dst, (const uint8_t*)B,
-                                                                     (const _Float16*)scales, (const uint8_t*)zp, N, K,
-                                                                     bs);
+template <typename T, int BITS>
+static hipError_t dequant_canonical_t(void* dst, const void* B, const void* scales, const void* zp, int64_t N, int64_t K,
+                                      int bs, hipStream_t s) {
+  const dim3 blk(256);
+  // vector kernel: 8 k per thread; needs whole units per row and naturally aligned loads and stores
+  const bool vec = K % 8 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && reinterpret_cast<uintptr_t>(B) % BITS == 0;
+  if (vec) {
+    const int64_t units = N * (K / 8);
+    mnb_dequant_canonical_vec_kernel<T, BITS><<<dim3((unsigned)((units + 255) / 256)), blk, 0, s>>>(
+        (T*)dst, (const uint8_t*)B, (const T*)scales, (const uint8_t*)zp, N, K, bs);
   } else {
-    if (bits == 4)
-      mnb_dequant_canonical_kernel<float, 4><<<grid, blk, 0, s>>>((float*)dst, (const uint8_t*)B, (const float*)scales,
-                                                                  (const uint8_t*)zp, N, K, bs);
-    else
-      mnb_dequant_canonical_kernel<float, 8><<<grid, blk, 0, s>>>((float*)dst, (const uint8_t*)B, (const float*)scales,
-                                                                  (const uint8_t*)zp, N, K, bs);
+    const int64_t total = N * K;
+    mnb_dequant_canonical_kernel<T, BITS><<<dim3((unsigned)((total + 255) / 256)), blk, 0, s>>>(
+        (T*)dst, (const uint8_t*)B, (const T*)scales, (const uint8_t*)zp, N, K, bs);
   }
   return hipGetLastError();
+}
+
+hipError_t mnb_launch_dequant_canonical(void* dst, const void* B, const void* scales, const void* zp, int64_t N,
+                                        int64_t K, int bits, int bs, int dtype, hipStream_t s) {
+  if (N * K == 0) return hipSuccess;
+  if (dtype == kMnbDtypeFloat16) {
+    if (bits == 2) return dequant_canonical_t<_Float16, 2>(dst, B, scales, zp, N, K, bs, s);
+    if (bits == 4) return dequant_canonical_t<_Float16, 4>(dst, B, scales, zp, N, K, bs, s);
+    return dequant_canonical_t<_Float16, 8>(dst, B, scales, zp, N, K, bs, s);
+  }
+  if (bits == 2) return dequant_canonical_t<float, 2>(dst, B, scales, zp, N, K, bs, s);
+  if (bits == 4) return dequant_canonical_t<float, 4>(dst, B, scales, zp, N, K, bs, s);
+  return dequant_canonical_t<float, 8>(dst, B, scales, zp, N, K, bs, s);
 }
 
 template <typename T>
@@ -371,16 +426,17 @@ static hipError_t dequant_packed_t(void* dst, const void* packed, const MnbLayou
   const int64_t total = L.KG * L.Npad;
   dim3 grid((unsigned)((total + 255) / 256)), blk(256);
   const uint8_t* p = (const uint8_t*)packed;
+  const int vec_ok = L.K % 8 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0;
   if (L.bits == 4) {
     if (L.has_zp)
-      mnb_dequant_packed_kernel<T, 4, true><<<grid, blk, 0, s>>>((T*)dst, p, L);
+      mnb_dequant_packed_kernel<T, 4, true><<<grid, blk, 0, s>>>((T*)dst, p, L, vec_ok);
     else
-      mnb_dequant_packed_kernel<T, 4, false><<<grid, blk, 0, s>>>((T*)dst, p, L);
+      mnb_dequant_packed_kernel<T, 4, false><<<grid, blk, 0, s>>>((T*)dst, p, L, vec_ok);
   } else {
     if (L.has_zp)
-      mnb_dequant_packed_kernel<T, 8, true><<<grid, blk, 0, s>>>((T*)dst, p, L);
+      mnb_dequant_packed_kernel<T, 8, true><<<grid, blk, 0, s>>>((T*)dst, p, L, vec_ok);
     else
-      mnb_dequant_packed_kernel<T, 8, false><<<grid, blk, 0, s>>>((T*)dst, p, L);
+      mnb_dequant_packed_kernel<T, 8, false><<<grid, blk, 0, s>>>((T*)dst, p, L, vec_ok);
   }
   return hipGetLastError();
 }
