@@ -62,7 +62,21 @@ class Problem:
             assert op.PrePack(bi, s, z)
             self.packed.append(op.packed)
         torch.cuda.synchronize()
-        self.prepack_ms = (time.perf_counter() - t0) * 1e3 / copies
+        self.prepack_ms = (time.perf_counter() - t0) * 1e3 / copies   # host view: allocation, roll and launch included
+
+        from onnxruntime_amd.matmul_nbits import _stream_ptr
+        stream = _stream_ptr(b.device)
+
+        def repack():  # device view: the pack kernels alone, into the buffers that exist by now
+            for pk in self.packed:
+                lib_mod.check(self.lib.MnbPackQuantBData(case.N, case.K, case.bits, case.block_size, self.dt, _ptr(b),
+                                                         _ptr(s), _ptr(z), _ptr(pk), stream))
+        self.prepack_device_us = time_steps(torch, repack, 3, 1) / copies * 1e3
+        for i, pk in enumerate(self.packed):  # restore the distinct contents
+            bi = torch.roll(b, shifts=i, dims=0) if i else b
+            lib_mod.check(self.lib.MnbPackQuantBData(case.N, case.K, case.bits, case.block_size, self.dt, _ptr(bi),
+                                                     _ptr(s), _ptr(z), _ptr(pk), stream))
+        torch.cuda.synchronize()
         self.a = dev(case.A.reshape(-1, case.K))
         self.bias = dev(case.bias)
         self.M = self.a.shape[0]
@@ -212,6 +226,7 @@ def main() -> int:
             "algorithmic_bytes_per_launch": bytes_per_launch,
             "kernel": p2.kernel,
             "prepack_ms_per_matrix": round(p2.prepack_ms, 3),
+            "prepack_device_us_per_matrix": round(p2.prepack_device_us, 1),
             "us_per_launch_weights_in_infinity_cache": round(ms_hot * 1e3 / LAYERS, 3),
         },
         "roofline": {
