@@ -25,11 +25,18 @@ import numpy as np
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the same counters read
-# for a plain copy of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the runs are summarised in
-# profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md.  They are properties of the kernels, not of one run.
-MEASURED_TRAFFIC_BYTES = {"c2_decode": int((14853.8 * 2.0 + 28.0) * 1024), "c4_prefill": int((109699.9 * 2.0 + 57344.0) * 1024),
-                          "quantize": int((57399.0 * 2.0 + 30478.3) * 1024), "mlp_decode": int((29669.4 * 2.0 + 28.0) * 1024)}
+# HBM bytes per launch are NOT measured by this program: they come from separate rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of this same command, scaled by what the same counters read for a plain copy of known size
+# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000), and are copied here from the summary named in TRAFFIC_SOURCE (KiB per
+# dispatch as printed there).  Every `traffic` value in the output carries `traffic_source` beside it.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md (rocprofv3 --pmc; a constant, not this run)"
+PROFILED_TRAFFIC_BYTES = {"c2_decode": int((14851.8 * 2.0 + 28.0) * 1024), "c4_prefill": int((109697.9 * 2.0 + 57344.0) * 1024),
+                          "quantize": int((57399.0 * 2.0 + 30478.3) * 1024), "mlp_decode": int((29667.4 * 2.0 + 28.0) * 1024)}
+# The reference's own MLAS kernel on the headline shape, timed by the survey on an 8-vCPU Sapphire-Rapids-class host
+# (standalone MLAS build, SQNBIT_CompFp32, N sliced over 8 threads): quoted beside the port so that the port's
+# figure is not read as the reference's.
+REFERENCE_MLAS_US_SURVEY = {"us_per_call": 1353.0, "threads": 8, "algorithmic_GBs": 23.1,
+                            "source": "BASELINE.md section 2 (survey container, not this host)"}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
 LAYERS = 32
@@ -124,6 +131,22 @@ def time_steps(torch, run_step, steps: int, warmup: int, warm_ms: float = 0.0) -
     return start.elapsed_time(stop) / steps
 
 
+def load_probe():
+    """libmnb_probe.so: the read-bandwidth and matrix-core-rate probes (onnxruntime_amd/csrc/mnb_probe.h)."""
+    path = ROOT / "onnxruntime_amd" / "libmnb_probe.so"
+    if not path.exists():
+        raise RuntimeError(f"{path} is missing: build it with `python -m onnxruntime_amd.build`")
+    lib = ctypes.CDLL(str(path))
+    lib.MnbProbeReadBandwidth.restype = ctypes.c_int
+    lib.MnbProbeReadBandwidth.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                          ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeMfmaRate.restype = ctypes.c_int
+    lib.MnbProbeMfmaRate.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeRelease.restype = None
+    lib.MnbProbeRelease.argtypes = []
+    return lib
+
+
 def graph_of(torch, run_step):
     """Captures one step into a HIP graph (the launches are ~5 us each: Python cannot issue them that fast)."""
     side = torch.cuda.Stream()
@@ -167,6 +190,7 @@ def main() -> int:
                     help="skip the read-only / MFMA-only probe kernels that report what the machine sustains")
     ap.add_argument("--no-quantize", action="store_true", help="skip the blockwise quantiser (producer of the format)")
     ap.add_argument("--no-fused", action="store_true", help="skip the fused gate/up projection (MatMulNBitsMlp)")
+    ap.add_argument("--no-sizes", action="store_true", help="skip the decode kernel on the larger gate+up matrices")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -235,7 +259,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES["c2_decode"],
+            "traffic": PROFILED_TRAFFIC_BYTES["c2_decode"], "traffic_source": TRAFFIC_SOURCE,
             "kernel": p2.kernel,
             "us_per_launch": round(us_per_launch, 3),
         },
@@ -245,18 +269,34 @@ def main() -> int:
 
     # ---- what this GPU sustains with the plainest kernels (context for the fractions above and below) ----------
     if not args.no_ceilings:
-        import ctypes
-        lib = _lib.load()
+        probe = load_probe()
         v = ctypes.c_double(0.0)
-        _lib.check(lib.MnbMeasureReadBandwidth(bytes_per_launch, LAYERS, ctypes.byref(v)))
-        read_same = v.value
-        _lib.check(lib.MnbMeasureReadBandwidth(1 << 30, 2, ctypes.byref(v)))
+        sweep_rows = []
+        for threads in (256, 512, 1024):
+            for inflight in (4, 8, 16, 32):
+                for batches in (1, 2, 4):
+                    rc = probe.MnbProbeReadBandwidth(bytes_per_launch, LAYERS, threads, inflight, batches,
+                                                     ctypes.byref(v))
+                    assert rc == 0, f"read probe failed ({rc})"
+                    sweep_rows.append((v.value, threads, inflight, batches))
+        best = max(sweep_rows)
+        probe.MnbProbeRelease()
+        assert probe.MnbProbeReadBandwidth(1 << 30, 2, 256, 8, 1, ctypes.byref(v)) == 0
         read_big = v.value
+        probe.MnbProbeRelease()
         out["roofline"]["measured_ceiling"] = {
-            "read_only_kernel_same_bytes_per_launch_GBs": round(read_same, 1),
+            "read_only_kernel_same_bytes_per_launch_GBs": round(best[0], 1),
+            "read_only_kernel_best_config": {"threads": best[1], "loads_in_flight": best[2], "batches": best[3]},
+            "read_only_kernel_sweep_GBs_min_median_max": [round(x, 1) for x in (
+                min(sweep_rows)[0], sorted(sweep_rows)[len(sweep_rows) // 2][0], best[0])],
+            "read_only_kernel_configs_swept": len(sweep_rows),
             "read_only_kernel_1GiB_per_launch_GBs": round(read_big, 1),
-            "frac_of_read_only_kernel": round(gbs / read_same, 4) if read_same > 0 else None,
+            "frac_of_read_only_kernel": round(gbs / best[0], 4) if best[0] > 0 else None,
         }
+        if args.sweep:
+            for r in sorted(sweep_rows, reverse=True):
+                print(f"read probe: {r[0]:8.1f} GB/s threads={r[1]} loads_in_flight={r[2]} batches={r[3]}",
+                      file=sys.stderr)
 
     # ---- prefill GEMM ----------------------------------------------------------------------------------------
     if not args.no_prefill:
@@ -273,15 +313,14 @@ def main() -> int:
             "kernel": p4.kernel,
             "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_FP16_PEAK_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(tflops / MFMA_FP16_PEAK_TFLOPS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES["c4_prefill"]},
+                         "traffic": PROFILED_TRAFFIC_BYTES["c4_prefill"], "traffic_source": TRAFFIC_SOURCE},
         }
         if not args.no_ceilings:
-            import ctypes
-            lib = _lib.load()
+            probe = load_probe()
             v = ctypes.c_double(0.0)
-            _lib.check(lib.MnbMeasureMfmaRate(0, ctypes.byref(v)))
+            assert probe.MnbProbeMfmaRate(0, ctypes.byref(v)) == 0
             mfma_const = v.value
-            _lib.check(lib.MnbMeasureMfmaRate(1, ctypes.byref(v)))
+            assert probe.MnbProbeMfmaRate(1, ctypes.byref(v)) == 0
             mfma_rand = v.value
             out["prefill"]["roofline"]["measured_ceiling"] = {
                 "mfma_only_loop_constant_operands_TFLOPs": round(mfma_const, 1),
@@ -313,7 +352,7 @@ def main() -> int:
             "kernel": "mnb_quantize_kernel",
             "roofline": {"bound": "hbm", "achieved": round(qbytes / (msq * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(qbytes / (msq * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES["quantize"]},
+                         "traffic": PROFILED_TRAFFIC_BYTES["quantize"], "traffic_source": TRAFFIC_SOURCE},
         }
         # ---- and back: MlasDequantizeBlockwise semantics on the quantiser's output (4 distinct operand sets) --------
         from onnxruntime_amd.matmul_nbits import dequantize_blockwise
@@ -373,10 +412,28 @@ def main() -> int:
             "ms_per_launch_with_skip_layer_norm_prologue": round(legs["skip_norm"], 5),
             "kernel": "mnb_skinny_kernel",
             "roofline": {"bound": "hbm", "achieved": round(gbs_f, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs_f / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["mlp_decode"]},
+                         "frac": round(gbs_f / HBM_PEAK_GBS, 4), "traffic": PROFILED_TRAFFIC_BYTES["mlp_decode"], "traffic_source": TRAFFIC_SOURCE},
         }
         del ops
         torch.cuda.empty_cache()
+
+    # ---- the same decode kernel on larger matrices: how the fixed part of a launch weighs against its size ----------
+    if not args.no_sizes:
+        rows = []
+        for label, bits, bs in (("gate+up int4 bs128 zp", 4, 128), ("gate+up int8 bs64 zp", 8, 64)):
+            K5, N5 = synthetic.C5_SHAPES["gate_up"]
+            case = synthetic.make_case(1, N5, K5, bits, bs, np.float16, has_zp=True, seed=0)
+            copies = 8  # 8 x 60 / 123 MB of distinct weights: beyond the Infinity Cache
+            p5 = Problem(case, copies, torch, _lib)
+            g5 = graph_of(torch, p5.step)
+            us5 = time_steps(torch, g5.replay, max(4, args.steps // 2), 2) / copies * 1e3
+            gb5 = case.algorithmic_bytes() / (us5 * 1e-6) / 1e9
+            rows.append({"workload": f"BASELINE configs[4] M=1 K={K5} N={N5} {label} fp16", "kernel": p5.kernel,
+                         "algorithmic_bytes_per_launch": case.algorithmic_bytes(), "us_per_launch": round(us5, 3),
+                         "value": round(gb5, 1), "unit": "GB/s", "frac_of_hbm_peak": round(gb5 / HBM_PEAK_GBS, 4)})
+            del g5, p5
+            torch.cuda.empty_cache()
+        out["decode_sizes"] = rows
 
     # ---- the other configurations (not part of the JSON contract) ---------------------------------------------
     if args.sweep:
@@ -393,6 +450,7 @@ def main() -> int:
             "kind": "port",
             "sample": f"{n} calls of the same M=1 K=4096 N=14336 problem on the C oracle, N sliced over {threads} "
                       f"threads, {sec * 1e3:.2f} ms per call",
+            "reference_mlas_us_survey": REFERENCE_MLAS_US_SURVEY,
         }
     print(json.dumps(out))
     return 0

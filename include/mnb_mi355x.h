@@ -263,16 +263,11 @@ MNB_API int MnbVariantDequantize(float* dst_dev, const void* b_dev, const void* 
 
 /* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
 MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);
-
-/* Diagnostics without a counterpart in the reference: ceilings of the machine the library runs on, measured with
- * the plainest kernels, so that the throughput of the real kernels can be read against what the device sustains.
- * Both calls allocate their own buffers, run for a few milliseconds and synchronise the device.
- * MnbMeasureReadBandwidth: GB/s of `launches` back-to-back kernels (one HIP graph) that each only read their own
- * `bytes_per_launch` bytes of device memory once.
- * MnbMeasureMfmaRate: TFLOP/s of a loop of nothing but v_mfma_f32_32x32x16_f16 on every CU, with constant operands
- * (random_operands = 0) or random fp16 operands (1): the sustained matrix-core clock depends on operand toggling. */
-MNB_API int MnbMeasureReadBandwidth(size_t bytes_per_launch, int launches, double* gb_per_s);
-MNB_API int MnbMeasureMfmaRate(int random_operands, double* tflops);
+/* The same for activations with a row pitch of lda elements (MnbGemmKernelName assumes K rounded up to 8).  The tile
+ * GEMM addresses a tile's activations with 32-bit byte offsets from the tile's first row, 255 * lda + 63 elements at
+ * most; pitches beyond that range select the streaming kernel, whose addressing is 64-bit. */
+MNB_API const char* MnbGemmKernelNameStrided(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype,
+                                             size_t lda);
 
 #ifdef __cplusplus
 }

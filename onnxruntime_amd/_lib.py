@@ -8,10 +8,7 @@ import ctypes
 from ctypes import c_int, c_int64, c_size_t, c_void_p, c_char_p
 from pathlib import Path
 
-import os
-
-# MNB_LIB_PATH points at an alternative build of the same library (kernel experiments); default: the in-tree one.
-LIB_PATH = Path(os.environ.get("MNB_LIB_PATH") or Path(__file__).resolve().parent / "libmnb_mi355x.so")
+LIB_PATH = Path(__file__).resolve().parent / "libmnb_mi355x.so"
 
 DTYPE_FLOAT = 1
 DTYPE_UINT8 = 2
@@ -92,9 +89,8 @@ SIGNATURES = {
                                c_size_t, c_void_p]),
     "MnbVariantDequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_size_t,
                                      c_int, c_int, c_int, c_void_p]),
-    "MnbMeasureReadBandwidth": (c_int, [c_size_t, c_int, ctypes.POINTER(ctypes.c_double)]),
-    "MnbMeasureMfmaRate": (c_int, [c_int, ctypes.POINTER(ctypes.c_double)]),
     "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
+    "MnbGemmKernelNameStrided": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_size_t]),
 }
 
 _lib = None

@@ -1,5 +1,6 @@
 """Builds, in-tree and with hipcc:
   libmnb_mi355x.so            HIP kernels + C ABI for gfx950
+  libmnb_probe.so             read-bandwidth and matrix-core-rate probes that only bench.py loads (csrc/mnb_probe.h)
   libonnxruntime_mi355x_ep.so the ONNX Runtime plugin execution provider above that C ABI (needs the ONNX Runtime
                               C API headers: directory given by ORT_INCLUDE_DIR, or an onnxruntime checkout at
                               ORT_SOURCE_DIR / /root/reference)
@@ -20,8 +21,9 @@ CSRC = PKG / "csrc"
 LIB = PKG / "libmnb_mi355x.so"
 OBJ_DIR = PKG / "build"
 
-SOURCES = ["mnb_api.hip", "mnb_pack.hip", "mnb_quant.hip", "mnb_gemv.hip", "mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_gemm32.hip", "mnb_fused.hip", "mnb_variant.hip",
-           "mnb_probe.hip"]
+SOURCES = ["mnb_api.hip", "mnb_pack.hip", "mnb_quant.hip", "mnb_gemv.hip", "mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_gemm32.hip", "mnb_fused.hip", "mnb_variant.hip"]
+PROBE_LIB = PKG / "libmnb_probe.so"
+PROBE_SOURCES = ["mnb_probe.hip"]
 
 # -packed-fp32-ops is switched off on purpose: scalar fp32 code must not be fused into v_pk_*_f32.
 HIPCC_FLAGS = [
@@ -53,15 +55,17 @@ def _compile(src: str, extra=()) -> Path:
 def build(force: bool = True, jobs: int = 4) -> Path:
     """Compiles every HIP source and links the shared library. Always recompiles when force is set."""
     srcs = [CSRC / s for s in SOURCES]
-    hdrs = list(CSRC.glob("*.h")) + list(CSRC.glob("*.cuh")) + [PKG.parent / "include" / "mnb_mi355x.h"]
+    hdrs = list(CSRC.glob("*.h")) + [PKG.parent / "include" / "mnb_mi355x.h"]
     if not force and LIB.exists():
         newest = max(p.stat().st_mtime for p in srcs + hdrs)
         if LIB.stat().st_mtime >= newest:
             return LIB
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(_compile, SOURCES))
-    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)]
-    subprocess.check_call(cmd)
+        objs = list(ex.map(_compile, SOURCES + PROBE_SOURCES))
+    n = len(SOURCES)
+    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs[:n])])
+    subprocess.check_call([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(PROBE_LIB),
+                           *map(str, objs[n:])])
     return LIB
 
 

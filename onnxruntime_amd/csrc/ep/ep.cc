@@ -72,6 +72,12 @@ OrtStatus* MatMulNBitsNodeSupported(const Apis& a, const OrtNode* node, bool* su
   if (!found) bits = 4;
   MI_RETURN_IF_ERROR(ReadIntAttr(a, node, "block_size", &block_size, &found));
   if (!found) return nullptr;
+  // weight_prepacked != 0 says that B already is in a CUDA-specific layout (1: SM80, 2: SM90 fpA_intB,
+  // onnxruntime/core/graph/contrib_ops/contrib_defs.cc:3800-3805), not in the canonical one this provider repacks:
+  // such a node is left to a provider that knows that layout.
+  int64_t weight_prepacked = 0;
+  MI_RETURN_IF_ERROR(ReadIntAttr(a, node, "weight_prepacked", &weight_prepacked, &found));
+  if (found && weight_prepacked != 0) return nullptr;
   size_t num_inputs = 0;
   MI_RETURN_IF_ERROR(a.ort->Node_GetNumInputs(node, &num_inputs));
   if (num_inputs < 3) return nullptr;

@@ -5,6 +5,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 
 #include "../../include/mnb_mi355x.h"
@@ -171,10 +172,39 @@ int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int a_dtype,
 
 }  // extern "C"
 
+// ------------------------------------------------------------------------------------------------ device facts
+// Compute units and engine clock of the current device, asked once per device and process.  The kernel-choice
+// estimates below are stated in cycles and per compute unit and scaled by these, so they follow the part the library
+// runs on.  Without a usable device (a host that only asks for kernel names) the MI355X figures stand in.
+const MnbDeviceInfo& mnb_device_info() {
+  constexpr int kMaxDevices = 64;
+  static MnbDeviceInfo info[kMaxDevices];
+  static std::once_flag once[kMaxDevices];
+  static const MnbDeviceInfo fallback{256, 2.4e9};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return fallback;
+  }
+  std::call_once(once[dev], [dev] {
+    int cus = 0, khz = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    if (hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, dev) != hipSuccess || khz <= 0) khz = 2400000;
+    (void)hipGetLastError();
+    info[dev] = MnbDeviceInfo{cus, (double)khz * 1e3};
+  });
+  return info[dev];
+}
+
 // ------------------------------------------------------------------------------------------------ kernel choice
 // fp16, M > 16: the weight-streaming kernel (mnb_mid.hip) takes any shape; the 256 x 256 tile GEMM wins once its tiles
-// fill the chip.  The estimate compares 2MNK at the streaming kernel's measured rate with whole rounds of 256 tiles
-// at the tile kernel's measured time per 64-deep k-step.
+// fill the chip.  The estimate compares 2MNK at the streaming kernel's rate with whole rounds of tiles at the tile
+// kernel's cycles per 64-deep k-step.
+// What the streaming kernel sustains per compute unit and cycle in the range where the two compete (M = 128 ... 1024
+// on the Llama-3-8B projections: 0.9 flop in 4 of the matrix cores' 4096 per cycle, the rest is weight dequantisation,
+// activation operand traffic and the reduction epilogue).
+constexpr double kMnbMidFlopsPerCuCycle = 895.0;
+
 static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
   if (M <= 128 || L.K % 128 != 0) return false;
   static const int64_t mid_max_m = [] {
@@ -182,7 +212,8 @@ static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
     return e ? (int64_t)atoll(e) : (int64_t)-1;
   }();
   if (mid_max_m >= 0) return M > mid_max_m;
-  const double t_mid = 2.0 * (double)M * (double)L.N * (double)L.K / 550e12;
+  const MnbDeviceInfo& dev = mnb_device_info();
+  const double t_mid = 2.0 * (double)M * (double)L.N * (double)L.K / (kMnbMidFlopsPerCuCycle * dev.cus * dev.clock_hz);
   double t_256 = 0.0;
   (void)mnb_gemm256_tile_rows(L, M, &t_256);
   return t_256 < t_mid;
@@ -202,7 +233,9 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
   if (mnb_gemm32_applicable(a)) return kMnbKernelGemm32;
   if (a.L.dtype == kMnbDtypeFloat16) {
     // the tile GEMM loads activations 16 bytes at a time: base and row pitch aligned
-    const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
+    // and addresses them with 32-bit offsets from a per-tile base
+    const bool aligned = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) &&
+                         mnb_gemm256_addressable(a.lda, a.L.Npad);
     if (aligned && mnb_prefer_gemm256(a.L, a.M)) return kMnbKernelGemm256;
     // the workspace is sized for the streaming kernel only when the shape alone selects it
     if (!mnb_prefer_gemm256(a.L, a.M) || a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;
@@ -237,16 +270,18 @@ size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_si
   return 0;
 }
 
-int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
-            const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev, size_t ldc,
-            void* workspace_dev, size_t workspace_bytes, void* stream) {
-  if (int rc = check_config("MnbGemm", bits, block_size, a_dtype)) return rc;
+// Validation and dispatch shared by MnbGemm and MnbGemmStaticScratch.
+static int gemm_checked(const char* fn, size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                        int a_dtype, const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev,
+                        void* c_dev, size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream) {
+  if (int rc = check_config(fn, bits, block_size, a_dtype)) return rc;
   if (M == 0 || N == 0) return MNB_OK;  // empty output: nothing to compute (matmul_nbits.cc:1533-1536)
-  if (K == 0) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: K must be positive");
-  if (!a_dev || !packed_dev || !c_dev) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: A, packed B and C must not be NULL");
-  if (lda < K || ldc < N) return fail(MNB_INVALID_ARGUMENT, "MnbGemm: lda (%zu) < K (%zu) or ldc (%zu) < N (%zu)", lda, K, ldc, N);
+  if (K == 0) return fail(MNB_INVALID_ARGUMENT, "%s: K must be positive", fn);
+  if (!a_dev || !packed_dev || !c_dev) return fail(MNB_INVALID_ARGUMENT, "%s: A, packed B and C must not be NULL", fn);
+  if (lda < K || ldc < N)
+    return fail(MNB_INVALID_ARGUMENT, "%s: lda (%zu) < K (%zu) or ldc (%zu) < N (%zu)", fn, lda, K, ldc, N);
   if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff)
-    return fail(MNB_INVALID_ARGUMENT, "MnbGemm: M, N and K must fit in 31 bits");
+    return fail(MNB_INVALID_ARGUMENT, "%s: M, N and K must fit in 31 bits", fn);
   MnbGemmArgs a{};  // epi: plain output
   a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
   a.M = (int64_t)M;
@@ -266,7 +301,7 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
     case kMnbKernelMid: {
       const size_t need = mnb_mid_workspace_bytes(a.L, a.M);
       if (a.workspace_bytes < need)
-        return fail(MNB_INVALID_ARGUMENT, "MnbGemm: workspace of %zu bytes needed (MnbGemmWorkspaceSize), %zu given", need,
+        return fail(MNB_INVALID_ARGUMENT, "%s: workspace of %zu bytes needed (MnbGemmWorkspaceSize), %zu given", fn, need,
                     a.workspace_bytes);
       e = mnb_launch_mid(a, s);
       break;
@@ -275,7 +310,14 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
     case kMnbKernelGemm32: e = mnb_launch_gemm32(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }
-  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbGemm");
+  return e == hipSuccess ? MNB_OK : hip_fail(e, fn);
+}
+
+int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+            const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev, size_t ldc,
+            void* workspace_dev, size_t workspace_bytes, void* stream) {
+  return gemm_checked("MnbGemm", M, N, K, bits, block_size, has_zero_points, a_dtype, a_dev, lda, packed_dev, bias_dev,
+                      c_dev, ldc, workspace_dev, workspace_bytes, stream);
 }
 
 size_t MnbGemmUnpackedWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
@@ -563,19 +605,6 @@ int MnbQuantizeBlockwise(void* b_dev, void* scales_dev, void* zero_points_dev, c
   return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbQuantizeBlockwise");
 }
 
-int MnbMeasureReadBandwidth(size_t bytes_per_launch, int launches, double* gb_per_s) {
-  if (!gb_per_s || bytes_per_launch < 16 || launches < 1 || (double)bytes_per_launch * launches > 8e9)
-    return fail(MNB_INVALID_ARGUMENT, "MnbMeasureReadBandwidth: need gb_per_s, >= 16 bytes, >= 1 launch, <= 8 GB in total");
-  hipError_t e = mnb_probe_read(bytes_per_launch, launches, gb_per_s);
-  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbMeasureReadBandwidth");
-}
-
-int MnbMeasureMfmaRate(int random_operands, double* tflops) {
-  if (!tflops) return fail(MNB_INVALID_ARGUMENT, "MnbMeasureMfmaRate: tflops must not be NULL");
-  hipError_t e = mnb_probe_mfma(random_operands, tflops);
-  return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbMeasureMfmaRate");
-}
-
 int MnbDequantizeBlockwise(void* dst_dev, const void* b_dev, const void* scales_dev, const void* zero_points_dev,
                            int block_size, int bits, size_t K, size_t N, int a_dtype, void* stream) {
   if (int rc = check_config("MnbDequantizeBlockwise", bits, block_size, a_dtype)) return rc;
@@ -597,15 +626,19 @@ int MnbDequantizePacked(void* dst_dev, const void* packed_dev, size_t N, size_t 
   return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbDequantizePacked");
 }
 
-const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype) {
-  if (!supported(bits, block_size, a_dtype)) return "none";
+const char* MnbGemmKernelNameStrided(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype, size_t lda) {
+  if (!supported(bits, block_size, a_dtype) || lda < K) return "none";
   MnbGemmArgs a{};
   a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, 0);
   a.M = (int64_t)M;
-  a.lda = (int64_t)((K + 7) / 8 * 8);  // assume the usual aligned activations
-  a.A = nullptr;
+  a.lda = (int64_t)lda;
+  a.A = nullptr;  // an aligned base
   a.workspace_bytes = ~(size_t)0;  // a caller that follows MnbGemmWorkspaceSize
   return mnb_kernel_name(mnb_select_kernel(a), a.L);
+}
+
+const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype) {
+  return MnbGemmKernelNameStrided(M, N, K, bits, block_size, a_dtype, (K + 7) / 8 * 8);  // the usual aligned rows
 }
 
 }  // extern "C"

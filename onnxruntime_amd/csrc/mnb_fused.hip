@@ -8,7 +8,7 @@
 //     fp32 arithmetic, one narrowing of each output);
 //   * the finishing pass for the GEMM kernels that cannot write the operator's outputs themselves: they produce the
 //     plain product over the packed columns, and this pass applies silu(gate) * up or splits Q, K and V.
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 namespace {

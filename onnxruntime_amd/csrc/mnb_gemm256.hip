@@ -21,7 +21,7 @@
 // Bias add and the single fp32 -> fp16 narrowing happen in the epilogue.
 #include <cstdlib>
 
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 namespace {
@@ -188,14 +188,17 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 
   // Addressing: every global access is  uniform base (SGPRs, advanced per k-step)  +  32-bit per-lane offset (a VGPR
   // computed once), so the loads cost no VALU work inside the loop.
+  // The tile's first row is part of the uniform base, so a lane's offset spans at most 255 rows: it fits 32 bits
+  // for every M as long as 512 * lda does (mnb_gemm256_addressable; larger pitches take the streaming kernel).
   const int a_row = tid >> 3, a_kc = tid & 7;  // thread's first A chunk: row a_row (+64 per load), k chunk a_kc
-  uint32_t a_off[A_LOADS];                     // byte offsets from p.A + k0
+  const _Float16* a_tile = p.A + (int64_t)m0 * p.lda;
+  uint32_t a_off[A_LOADS];                     // byte offsets from a_tile + k0
 #pragma unroll
   for (int i = 0; i < A_LOADS; ++i) {
     // rows beyond M re-read row M-1 and are never stored (a predicated load would serialise the loop)
-    int m = m0 + a_row + i * 64;
-    m = m < p.M ? m : p.M - 1;
-    a_off[i] = (uint32_t)(((int64_t)m * p.lda + a_kc * 8) * 2);
+    int r = a_row + i * 64;
+    r = m0 + r < p.M ? r : p.M - 1 - m0;
+    a_off[i] = (uint32_t)(((int64_t)r * p.lda + a_kc * 8) * 2);
   }
   // this lane's weight columns (one per column tile): its 8 bytes inside each 16-byte vector, and its meta entries.
   // The block of a lane's half vector is (k-group base >> bs_shift), plus kq when 4-bit blocks are 16 wide.
@@ -215,7 +218,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // k-steps past the end are clamped to the last one: the loop body stays branch free, the data is never used
   auto load_a = [&](int ks_raw, Stage& R) {
     const int ks = ks_raw < last_step ? ks_raw : last_step;
-    const uint8_t* base = reinterpret_cast<const uint8_t*>(p.A + (int64_t)ks * BK);
+    const uint8_t* base = reinterpret_cast<const uint8_t*>(a_tile + (int64_t)ks * BK);
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       const u4_t v = *reinterpret_cast<const u4_t*>(base + a_off[i]);
@@ -443,14 +446,13 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 template <int BITS, bool HAS_ZP, int MPS, int TM>
 hipError_t launch_tm(const Gemm256Params& p, hipStream_t s) {
   const size_t smem = (size_t)SMEM_HALVES * sizeof(_Float16);  // 73728 bytes
-  static bool configured = false;  // per instantiation; the attribute is sticky for the function
   auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM>;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  // The attribute belongs to the function on the current device, so it is set on every launch (a host-side table
+  // update, no device work): callers on several threads or devices need no shared flag.
+  if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      e != hipSuccess)
+    return e;
   dim3 grid((unsigned)(p.tiles_n * p.tiles_m)), blk(THREADS);
   kernel<<<grid, blk, smem, s>>>(p);
   return hipGetLastError();
@@ -466,12 +468,17 @@ hipError_t launch(const Gemm256Params& p, hipStream_t s) {
 // Rows of the tile for a problem: the 128-row tile when its grid fills the 256 compute units in fewer, or at the
 // measured step costs cheaper, rounds than the 256-row one.
 int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds) {
+  const MnbDeviceInfo& dev = mnb_device_info();
   const int64_t tiles_n = (L.N + BN - 1) / BN;
   const double ksteps = (double)(L.K / BK);
-  const double step256 = L.bits == 4 ? 1.45e-6 : (L.bs >= 32 ? 1.65e-6 : 2.95e-6);
+  // cycles of one 64-deep k-step of a 256-row tile with the whole chip busy (4-bit; 8-bit; 8-bit with 16-wide blocks,
+  // whose four meta entries per step spill): properties of the kernel's instruction schedule
+  const double cycles256 = L.bits == 4 ? 3480.0 : (L.bs >= 32 ? 3960.0 : 7080.0);
+  const double step256 = cycles256 / dev.clock_hz;
   const double step128 = step256 * kMnbGemm128StepRatio;
-  const double t256 = (double)((((M + 255) / 256) * tiles_n + 255) / 256) * ksteps * step256;
-  const double t128 = (double)((((M + 127) / 128) * tiles_n + 255) / 256) * ksteps * step128;
+  const int64_t cus = dev.cus;
+  const double t256 = (double)((((M + 255) / 256) * tiles_n + cus - 1) / cus) * ksteps * step256;
+  const double t128 = (double)((((M + 127) / 128) * tiles_n + cus - 1) / cus) * ksteps * step128;
   static const int forced = [] {
     const char* e = getenv("MNB_GEMM256_TILE_ROWS");  // tuning override: 128 or 256
     return e ? atoi(e) : 0;
@@ -479,6 +486,16 @@ int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds) {
   const bool small = forced ? forced == 128 : t128 < t256;
   if (seconds) *seconds = small ? t128 : t256;
   return small ? 128 : 256;
+}
+
+// Per-lane offsets of the tile GEMM are 32-bit byte counts from a base that moves with the tile: activations span
+// 255 rows of lda halves plus one k-step (mnb_gemm256_max_lane_offset), weights one k-group row of Npad columns x 16
+// bytes, meta entries two block rows of Npad x 4 bytes.  Problems beyond that take the streaming kernel, whose
+// addressing is 64-bit throughout.
+uint64_t mnb_gemm256_max_lane_offset(int64_t lda) { return ((uint64_t)255 * (uint64_t)lda + 7 * 8 + 7) * 2 + 1; }
+
+bool mnb_gemm256_addressable(int64_t lda, int64_t Npad) {
+  return mnb_gemm256_max_lane_offset(lda) < ((uint64_t)1 << 32) && (uint64_t)Npad * 16 + 16 <= ((uint64_t)1 << 32);
 }
 
 // The fused outputs are written with 16-byte stores of 8 columns: every output 16-byte aligned, with a pitch and a
@@ -491,6 +508,7 @@ bool mnb_gemm256_fused_ok(const MnbEpilogue& e) {
 }
 
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
+  if (!mnb_gemm256_addressable(a.lda, a.L.Npad)) return hipErrorInvalidValue;  // the dispatcher never sends these
   Gemm256Params p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
   p.W = reinterpret_cast<const uint8_t*>(a.packed);

@@ -21,7 +21,7 @@
 // kernel it replaces for these shapes.
 #include <cstdlib>
 
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 namespace {

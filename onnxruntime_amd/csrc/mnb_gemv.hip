@@ -15,7 +15,7 @@
 #include <cstdio>
 #include <cstdlib>
 
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 struct GemvParams {

@@ -63,9 +63,18 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M);  // staged copy o
 bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
+// compute units and engine clock (Hz) of the current device; asked once per device (mnb_api.hip)
+struct MnbDeviceInfo {
+  int cus;
+  double clock_hz;
+};
+const MnbDeviceInfo& mnb_device_info();
 // rows of the tile the tile GEMM would use (256 or 128) and, optionally, its estimated run time
 int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds);
 bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
+// the tile GEMM's 32-bit per-lane offsets reach every element of this problem
+uint64_t mnb_gemm256_max_lane_offset(int64_t lda);
+bool mnb_gemm256_addressable(int64_t lda, int64_t Npad);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
 bool mnb_gemm32_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemm32(const MnbGemmArgs& a, hipStream_t s);
@@ -79,6 +88,3 @@ hipError_t mnb_launch_rmsnorm(void* a_norm, void* sum_out, int64_t ld_sum, const
 hipError_t mnb_launch_fused_finish(const MnbEpilogue& epi, const void* tmp, int64_t ld_tmp, int64_t M, int dtype,
                                    hipStream_t s);
 
-// machine ceilings (mnb_probe.hip); diagnostics, synchronous
-hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s);
-hipError_t mnb_probe_mfma(int random_operands, double* tflops);

@@ -2,7 +2,7 @@
 // registers (mnb_skinny.hip for M <= 16, mnb_mid.hip for 16 < M): kernel parameters, the nibble/byte to "magic half"
 // conversion, the per-chunk register block with its loads, and the constant operands of the correction MFMAs.
 #pragma once
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 namespace {

@@ -14,7 +14,7 @@
 // into operand order in the caller's workspace, [chunk][word i][row tile][kq][j] in 16-byte units (zero-filled beyond
 // M and K, any alignment of the source), so that every operand load of a wavefront is 1 KiB contiguous.  The staged
 // copy is M x K halves (at most a few MB) and is re-read from L2 by every workgroup.
-#include "mnb_mfma16_common.cuh"
+#include "mnb_mfma16_common.hip.h"
 
 namespace {
 

@@ -4,7 +4,7 @@
 // (onnxruntime/core/mlas/lib/sqnbitgemm_kernel_avx_common.h:39-115) with the gfx950 k-group-major layout described
 // in mnb_layout.h.  The dequantise kernels restate BlockwiseQuantizer::dequantize
 // (onnxruntime/core/mlas/lib/q4_dq.cpp:587-641) on the device.
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 // ------------------------------------------------------------------------------------------------ pack weights

@@ -1,0 +1,34 @@
+/*
+ * mnb_probe.h -- C entry points of libmnb_probe.so: diagnostics for the benchmark, NOT part of the operator's C ABI
+ * (that is include/mnb_mi355x.h).  They have no counterpart in the reference: they measure what the device sustains
+ * with the plainest kernels, so that the throughput of the real kernels can be read against it.  Every call
+ * allocates device memory, runs for a few milliseconds and synchronises the device.  Return 0 on success, 1 on a HIP
+ * error, 2 on an invalid argument.
+ */
+#ifndef MNB_PROBE_H_
+#define MNB_PROBE_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MNB_PROBE_API __attribute__((visibility("default")))
+
+/* GB/s of `launches` back-to-back kernels (one HIP graph) that each only read their own `bytes_per_launch` bytes of
+ * device memory once: workgroups of `threads` threads (multiple of 64, at most 1024), every thread issuing
+ * `loads_in_flight` (2, 4, 8, 16 or 32) independent 16-byte loads `batches` times; the grid covers the buffer.
+ * The buffers are kept between calls with the same sizes (a sweep allocates once); MnbProbeRelease frees them. */
+MNB_PROBE_API int MnbProbeReadBandwidth(size_t bytes_per_launch, int launches, int threads, int loads_in_flight,
+                                        int batches, double* gb_per_s);
+MNB_PROBE_API void MnbProbeRelease(void);
+
+/* TFLOP/s of a loop of nothing but v_mfma_f32_32x32x16_f16 on every CU, with constant operands
+ * (random_operands = 0) or random fp16 operands (1): the sustained matrix-core clock depends on operand toggling. */
+MNB_PROBE_API int MnbProbeMfmaRate(int random_operands, double* tflops);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MNB_PROBE_H_ */

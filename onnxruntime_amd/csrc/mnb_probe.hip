@@ -1,30 +1,36 @@
 // Machine ceilings measured with the plainest possible kernels, for reading the roofline fractions of the real ones:
-//   * what a kernel that only reads N bytes per launch achieves (launch ramp and tail included), and
+//   * what a kernel that only reads N bytes per launch achieves (launch ramp and tail included), swept over workgroup
+//     size, 16-byte loads in flight per thread and batches per thread, and
 //   * what a loop of nothing but v_mfma_f32_32x32x16_f16 achieves with constant and with random fp16 operands
 //     (matrix-core power draw, hence the sustained clock, depends on how many operand bits toggle).
-// Diagnostics only: nothing on the operator's path calls them.
+// Built as a library of its own (libmnb_probe.so) that only the benchmark loads: diagnostics, not part of the
+// operator's C ABI, and nothing on the operator's path calls them.
+#include "mnb_probe.h"
+
 #include <hip/hip_runtime.h>
 
 #include <vector>
 
-#include "mnb_device.cuh"
-#include "mnb_internal.h"
+#include "mnb_device.hip.h"
 
 namespace {
 
+// Each thread issues U independent 16-byte loads (a wavefront reads 1 KiB contiguous per load), `batches` times.
 template <int U>
-__global__ void __launch_bounds__(256) mnb_probe_read_kernel(const uint4* __restrict__ p, float* out, size_t n_vec) {
+__global__ void mnb_probe_read_kernel(const uint4* __restrict__ p, float* out, size_t n_vec, int batches) {
   const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
-  uint4 v[U];
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const size_t i = tid + u * stride;
-    v[u] = i < n_vec ? p[i] : make_uint4(0, 0, 0, 0);
-  }
   uint32_t s = 0;
+  for (int b = 0; b < batches; ++b) {
+    uint4 v[U];
 #pragma unroll
-  for (int u = 0; u < U; ++u) s += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    for (int u = 0; u < U; ++u) {
+      const size_t i = tid + ((size_t)b * U + u) * stride;
+      v[u] = i < n_vec ? p[i] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) s += v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
   if (s == 0x12345678u) out[0] = 1.f;  // keeps the loads alive; practically never taken
 }
 
@@ -62,15 +68,43 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_mfma_kernel(float* out, int 
   out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
-}  // namespace
+// Buffers of the read probe, kept between calls so that a sweep allocates once.
+std::vector<uint4*> g_bufs;
+size_t g_buf_vecs = 0;
+float* g_out = nullptr;
+
+void release_buffers() {
+  for (uint4* b : g_bufs)
+    if (b) (void)hipFree(b);
+  g_bufs.clear();
+  g_buf_vecs = 0;
+  if (g_out) (void)hipFree(g_out);
+  g_out = nullptr;
+}
+
+hipError_t ensure_buffers(size_t n_vec, int launches) {
+  if (g_buf_vecs == n_vec && (int)g_bufs.size() == launches && g_out) return hipSuccess;
+  release_buffers();
+  hipError_t e = hipMalloc(&g_out, 256);
+  if (e != hipSuccess) return e;
+  g_bufs.assign((size_t)launches, nullptr);
+  for (int i = 0; i < launches; ++i) {
+    if ((e = hipMalloc(&g_bufs[i], n_vec * 16)) != hipSuccess) return e;
+    if ((e = hipMemset(g_bufs[i], i + 1, n_vec * 16)) != hipSuccess) return e;
+  }
+  g_buf_vecs = n_vec;
+  return hipSuccess;
+}
+
+template <int U>
+void launch_read(unsigned blocks, int threads, hipStream_t s, const uint4* p, size_t n_vec, int batches) {
+  mnb_probe_read_kernel<U><<<blocks, threads, 0, s>>>(p, g_out, n_vec, batches);
+}
 
 // `launches` back-to-back kernels (one HIP graph), each reading its own `bytes` of device memory once.
-hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s) {
+hipError_t probe_read(size_t bytes, int launches, int threads, int loads_in_flight, int batches, double* gb_per_s) {
   *gb_per_s = 0.0;
   const size_t n_vec = bytes / 16;
-  if (n_vec == 0 || launches < 1) return hipErrorInvalidValue;
-  std::vector<uint4*> bufs((size_t)launches, nullptr);
-  float* out = nullptr;
   hipStream_t s = nullptr;
   hipEvent_t e0 = nullptr, e1 = nullptr;
   hipGraph_t g = nullptr;
@@ -80,15 +114,21 @@ hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s) {
     if (err == hipSuccess && e != hipSuccess) err = e;
     return err == hipSuccess;
   };
-  constexpr int U = 8;
-  const unsigned blocks = (unsigned)((n_vec + 256 * U - 1) / (256 * U));
-  if (ok(hipMalloc(&out, 256))) {
-    for (int i = 0; i < launches && err == hipSuccess; ++i)
-      if (ok(hipMalloc(&bufs[i], n_vec * 16))) ok(hipMemset(bufs[i], i + 1, n_vec * 16));
-  }
-  if (ok(hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) && ok(hipEventCreate(&e0)) && ok(hipEventCreate(&e1)) &&
-      ok(hipDeviceSynchronize()) && ok(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal))) {
-    for (int i = 0; i < launches; ++i) mnb_probe_read_kernel<U><<<blocks, 256, 0, s>>>(bufs[i], out, n_vec);
+  const size_t per_block = (size_t)threads * loads_in_flight * batches;
+  const unsigned blocks = (unsigned)((n_vec + per_block - 1) / per_block);
+  ok(ensure_buffers(n_vec, launches));
+  if (ok(err) && ok(hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) && ok(hipEventCreate(&e0)) &&
+      ok(hipEventCreate(&e1)) && ok(hipDeviceSynchronize()) &&
+      ok(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal))) {
+    for (int i = 0; i < launches; ++i) {
+      switch (loads_in_flight) {
+        case 2: launch_read<2>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
+        case 4: launch_read<4>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
+        case 8: launch_read<8>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
+        case 16: launch_read<16>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
+        default: launch_read<32>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
+      }
+    }
     ok(hipStreamEndCapture(s, &g));
     if (ok(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0))) {
       for (int w = 0; w < 3; ++w) ok(hipGraphLaunch(ge, s));
@@ -108,13 +148,10 @@ hipError_t mnb_probe_read(size_t bytes, int launches, double* gb_per_s) {
   if (e0) (void)hipEventDestroy(e0);
   if (e1) (void)hipEventDestroy(e1);
   if (s) (void)hipStreamDestroy(s);
-  for (uint4* b : bufs)
-    if (b) (void)hipFree(b);
-  if (out) (void)hipFree(out);
   return err;
 }
 
-hipError_t mnb_probe_mfma(int random_operands, double* tflops) {
+hipError_t probe_mfma(int random_operands, double* tflops) {
   *tflops = 0.0;
   int dev = 0, cus = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -150,3 +187,26 @@ hipError_t mnb_probe_mfma(int random_operands, double* tflops) {
   (void)hipFree(out);
   return err;
 }
+
+}  // namespace
+
+extern "C" {
+
+int MnbProbeReadBandwidth(size_t bytes_per_launch, int launches, int threads, int loads_in_flight, int batches,
+                          double* gb_per_s) {
+  const bool u_ok = loads_in_flight == 2 || loads_in_flight == 4 || loads_in_flight == 8 || loads_in_flight == 16 ||
+                    loads_in_flight == 32;
+  if (!gb_per_s || bytes_per_launch < 16 || launches < 1 || (double)bytes_per_launch * launches > 8e9 || !u_ok ||
+      threads < 64 || threads > 1024 || threads % 64 != 0 || batches < 1 || batches > 64)
+    return 2;
+  return probe_read(bytes_per_launch, launches, threads, loads_in_flight, batches, gb_per_s) == hipSuccess ? 0 : 1;
+}
+
+void MnbProbeRelease(void) { release_buffers(); }
+
+int MnbProbeMfmaRate(int random_operands, double* tflops) {
+  if (!tflops) return 2;
+  return probe_mfma(random_operands, tflops) == hipSuccess ? 0 : 1;
+}
+
+}  // extern "C"

@@ -26,7 +26,7 @@
 #include <cstdio>
 #include <cstdlib>
 
-#include "mnb_mfma16_common.cuh"
+#include "mnb_mfma16_common.hip.h"
 
 namespace {
 

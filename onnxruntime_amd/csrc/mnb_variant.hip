@@ -22,7 +22,7 @@
 #include <vector>
 
 #include "../../include/mnb_mi355x.h"
-#include "mnb_device.cuh"
+#include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
 namespace {
@@ -184,7 +184,13 @@ __global__ void __launch_bounds__(256) mnb_variant_dequant_kernel(float* __restr
   const int64_t kbc = (K + bs - 1) / bs;
   const uint8_t* col = B + n * (kbc * bs * bits / 8);
   const float q = bits == 4 ? (float)((col[k >> 1] >> ((k & 1) * 4)) & 0xF) : (float)((col[k >> 2] >> ((k & 3) * 2)) & 0x3);
-  const int64_t b = g_idx ? g_idx[k] : k / bs;
+  int64_t b = g_idx ? g_idx[k] : k / bs;
+  if (b < 0 || b >= kbc) {
+    // a group index outside [0, k_blocks) lives on the device, where the host cannot vet it: nothing is read through
+    // it and the element becomes NaN, which no valid input produces
+    dst[idx] = __builtin_nanf("");
+    return;
+  }
   const float s = widen(scales, n * kbc + b, kind);
   float z = (float)(1 << (bits - 1));
   if (zp_kind == MNB_ZP_TYPED) {
@@ -216,11 +222,14 @@ int order_by_group(const int32_t* g_idx, size_t len, int64_t K, int bs, bool tab
                 (long long)K, (long long)(k_blocks * bs), len);
   std::vector<int64_t> count((size_t)k_blocks, 0);
   out->trivial = true;
-  for (int64_t k = 0; k < K; ++k) {
+  // every entry is checked, the padded tail beyond K included, with the reference's message
+  // (matmul_nbits_helper.h:92-103)
+  for (int64_t k = 0; k < (int64_t)len; ++k) {
     const int64_t g = g_idx[k];
     if (g < 0 || g >= k_blocks)
-      return fail(MNB_INVALID_ARGUMENT, "g_idx[%lld] = %lld is outside [0, %lld)", (long long)k, (long long)g,
-                  (long long)k_blocks);
+      return fail(MNB_INVALID_ARGUMENT, "group_index value at index %lld is %lld, which is out of valid range [0, %lld)",
+                  (long long)k, (long long)g, (long long)k_blocks);
+    if (k >= K) continue;  // padding: validated, not used
     if (g != k / bs) out->trivial = false;
     ++count[(size_t)g];
   }

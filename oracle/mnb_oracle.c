@@ -34,8 +34,10 @@
  *                                       this route does not build without the whole runtime): exact cases where no
  *                                       operation rounds, equality with mnbo_dequantize_f32 on the inputs where both
  *                                       routes are defined and exact, group selection read back through power-of-two
- *                                       scales, closeness to the fp64 value.  The last-ulp behaviour of the two-step
- *                                       formula is PARITY UNPINNED.
+ *                                       scales, closeness to the fp64 value, and the last place of the three-rounding
+ *                                       formula against exact rational arithmetic rounded to fp32 after each
+ *                                       operation (tests/test_oracle_variants.py), on inputs where a contracted
+ *                                       multiply-add and the one-rounding form both differ from it.
  */
 #include <math.h>
 #include <pthread.h>
@@ -324,8 +326,10 @@ void mnbo_matmul_f16(const uint16_t* A, const uint8_t* B, const uint16_t* scales
  * are widened to fp32, the scale is computed in fp32 and stored as fp16 (RNE); the zero point comes from the
  * unrounded scale, the reciprocal from the stored one.  Positions k >= K of the last block, which the reference
  * leaves unwritten, hold the zero point here (they dequantise to 0).
- * Parity: pinned only by round-trip and closed-form properties (tests/test_oracle_quantize.py); tie-breaking
- * on exact .5 values is "parity unpinned" because the compiled reference is not available in this build.
+ * Parity: pinned by round-trip and closed-form properties and an independent numpy restatement
+ * (tests/test_oracle_quantize.py); rounding of exact .5 values, of elements and of the zero point, is pinned by
+ * grids on which scale, zero point and every expected integer are a closed form of roundf (x + 0.5 -> x + 1 for even
+ * and odd x: tests/tie_cases.py), which a round-half-to-even quantiser fails.
  */
 static void quantize_core(uint8_t* B, float* scales, uint8_t* zp, const float* src, int64_t K, int64_t N, int bits,
                           int64_t bs, int symmetric, int scale_is_f16) {

@@ -14,8 +14,9 @@ Parity status of what is defined here on top of the C functions (whose own statu
   ``mlp`` / ``qkv``           compositions of pinned parts (matmul, layer normalisation) with silu(g) * u in float64;
                               the reference ships only WebGPU shaders for these operators and no stored outputs, so
                               beyond that composition their parity is PARITY UNPINNED
-  ``variant_dequantize``      wrapper of mnbo_variant_dequantize_f32: pinned by mathematics only, last ulp on inexact
-                              inputs PARITY UNPINNED; bfloat16 operands have no CPU kernel in the reference at all
+  ``variant_dequantize``      wrapper of mnbo_variant_dequantize_f32: pinned by mathematics, the last place of its
+                              three roundings included (exact rational arithmetic, tests/test_oracle_variants.py);
+                              bfloat16 operands have no CPU kernel in the reference at all: PARITY UNPINNED
   ``dense_matmul_f64``        numpy float64 product over a dequantised W, the checker of the variant route
 
 Reference definitions followed (onnxruntime 1.30.0):

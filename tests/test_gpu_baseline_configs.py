@@ -76,12 +76,19 @@ def test_config4_prefill(oracle):
 @pytest.mark.parametrize("shape", list(synthetic.C5_SHAPES))
 def test_config5_layer_sweep(oracle, bits, bs, shape):
     K, N = synthetic.C5_SHAPES[shape]
-    # M = 256 and 1024 reach the tile GEMM with 128-row tiles on the wide shapes and the streaming kernel on the others
-    for M in (1, 64, 256, 1024):
+    # M = 256 and 1024 reach the tile GEMM with 128-row tiles on the wide shapes and the streaming kernel on the others;
+    # M = 4096 runs the tile GEMM over several rounds of the chip (up to seven on the gate+up shape)
+    for M in (1, 64, 256, 1024, 4096):
         c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, seed=0)
         y = run_case(c)
-        rows = np.unique(np.concatenate([np.linspace(0, M - 1, 6).astype(int), [min(127, M - 1), min(128, M - 1)]]))
+        rows = np.unique(np.concatenate([np.linspace(0, M - 1, 6).astype(int), [min(127, M - 1), min(128, M - 1)],
+                                         [min(r, M - 1) for r in (255, 256, 2047, 2048, 3839, 3840)]]))
         sub = make_case(len(rows), N, K, bits, bs, np.float16, has_zp=True, seed=0)
         sub.B, sub.scales, sub.zero_points = c.B, c.scales, c.zero_points
         sub.A = c.A[rows]
         check_against_oracle(oracle, sub, y[rows], A=sub.A)
+        if M == 4096:
+            # every 256 x 256 tile of the output was written: finite, and not the zeros the buffer could start with
+            yt = torch.from_numpy(y).float()
+            assert torch.isfinite(yt).all()
+            assert (yt.view(M // 256, 256, N // 256, 256).abs().amax(dim=(1, 3)) > 0).all()

@@ -104,8 +104,6 @@ def test_mlp_cases_cover_every_kernel():
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("M,N,K,bits,bs", MLP_CASES)
 def test_mlp_parity(oracle, dtype, bias, M, N, K, bits, bs):
-    if dtype == np.float32 and M > 100:
-        pytest.skip("fp32 large M runs the same any-shape kernel as M = 100")
     g, gm = _mats(M, N, K, bits, bs, dtype, bias, 11)
     u, um = _mats(M, N, K, bits, bs, dtype, bias and N % 2 == 0, 12)  # sometimes only one of the two biases
     op = MatMulNBitsMlp(K, N, bits, bs, dtype=tdtype(dtype))
@@ -179,8 +177,6 @@ QKV_CASES = [
 @pytest.mark.parametrize("norm", [None, "simplified", "skip"])
 @pytest.mark.parametrize("M,Nq,Nkv,K,bits,bs", QKV_CASES)
 def test_qkv_parity(oracle, dtype, norm, M, Nq, Nkv, K, bits, bs):
-    if dtype == np.float32 and (M > 100 or K > 1024):
-        pytest.skip("fp32 large shapes run the same any-shape kernel")
     q, qm = _mats(M, Nq, K, bits, bs, dtype, True, 41)
     k, km = _mats(M, Nkv, K, bits, bs, dtype, False, 42)
     v, vm = _mats(M, Nkv, K, bits, bs, dtype, True, 43)

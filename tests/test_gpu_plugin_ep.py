@@ -86,6 +86,32 @@ def test_nodes_left_to_the_cpu_provider():
     not_claimed(zero_points=np.full((c.N, 4), 7.5, np.float16))
 
 
+def test_weights_prepacked_for_another_provider_are_not_claimed(oracle):
+    """weight_prepacked = 1 / 2 marks B as being in a CUDA fpA_intB layout (contrib_defs.cc:3800-3805): this provider
+    would repack it as if it were canonical, so it leaves the node alone; 0 (or the attribute absent) is claimed."""
+    c = make_case(2, 64, 128, 4, 32, np.float16, has_zp=True, seed=8)
+    names = ["A", "B", "scales", "zero_points", "g_idx", "bias"]
+    types = ["T1", "T2", "T1", "T3", "T4", "T1"]
+    schema = ["K", "N", "bits", "block_size", "accuracy_level", "weight_prepacked"]
+
+    def run(prepacked):
+        attrs = {"K": c.K, "N": c.N, "bits": 4, "block_size": 32, "accuracy_level": 0}
+        if prepacked is not None:
+            attrs["weight_prepacked"] = prepacked
+        return host.run_node("MatMulNBits", attrs, schema, names, types,
+                             [c.A, c.B, c.scales, c.zero_points, None, None], ("B", "scales", "zero_points"),
+                             [(c.M, c.N)])
+
+    for prepacked in (1, 2):
+        with pytest.raises(host.EpHostError) as e:
+            run(prepacked)
+        assert e.value.code == host.NOT_CLAIMED
+    for prepacked in (None, 0):
+        (y,), trace = run(prepacked)
+        assert "claimed=1" in trace
+        check_against_oracle(oracle, c, y)
+
+
 def test_shape_errors_carry_the_reference_messages():
     c = make_case(2, 64, 128, 4, 32, np.float32, has_zp=True, seed=6)
     INVALID_ARGUMENT = 2

@@ -55,7 +55,7 @@ def test_errors_surface_at_prepack():
     c["g"][5] = 2
     with pytest.raises(host.EpHostError) as e:
         _run(c, N, K, 4, bs)
-    assert e.value.code == 2 and "g_idx[5] = 2 is outside [0, 2)" in e.value.message
+    assert e.value.code == 2 and "group_index value at index 5 is 2, which is out of valid range [0, 2)" in e.value.message
     c = make("f16", N, K, 4, bs, "typed", "none", 2, seed=1)
     c["zp"] = c["zp"][:, :1]
     with pytest.raises(host.EpHostError) as e:

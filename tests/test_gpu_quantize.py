@@ -4,7 +4,9 @@ import numpy as np
 import pytest
 import torch
 
+import tie_cases
 from gpu_util import dev
+from oracle.oracle import np_unpack_q, np_unpack_zp
 from onnxruntime_amd.matmul_nbits import MatMulNBits, dequantize_blockwise, quantize_blockwise
 
 pytestmark = pytest.mark.gpu
@@ -39,25 +41,32 @@ def test_identical_to_oracle(oracle, dtype, bits, bs, symmetric):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("bits", [2, 4, 8])
-def test_exact_ties_round_away_from_zero(oracle, dtype, bits):
-    """Elements that land exactly half way between two integers (power-of-two scale) round like roundf in the oracle."""
-    bs, N, kb = 32, 128, 6
-    mid, maxq = 1 << (bits - 1), (1 << bits) - 1
-    rng = np.random.default_rng(bits)
-    scale = np.ldexp(1.0, -rng.integers(1, 6, size=(kb, 1, N)))
-    steps = rng.integers(-2 * mid - 2, 2 * mid + 2, size=(kb, bs, N)) * 0.5       # multiples of one half, some clamp
-    steps[:, 0, :] = -mid                                                         # pins the symmetric scale to `scale`
-    steps = np.clip(steps, -mid, mid)
-    W = (steps * scale).reshape(kb * bs, N).astype(dtype)                         # exact in fp16
-    for symmetric in (True, False):
-        Bq, s, z = oracle.C.quantize(W, bits, bs, symmetric)
-        b, sc, zp = quantize_blockwise(dev(W), bits, bs, symmetric)
-        torch.cuda.synchronize()
-        assert np.array_equal(_bits(sc.cpu().numpy()), _bits(s))
-        assert np.array_equal(b.cpu().numpy(), Bq)
-        if not symmetric:
-            assert np.array_equal(zp.cpu().numpy(), z)
-    assert maxq == 2 * mid - 1
+@pytest.mark.parametrize("bs", [16, 64])
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_exact_ties_round_away_from_zero(dtype, bits, bs, symmetric):
+    """Elements exactly half way between two integers: the device returns the closed-form integers of the reference's
+    roundf (x + 0.5 -> x + 1, q4_dq.cpp:558), the same ones tests/test_oracle_quantize.py demands of the oracle."""
+    W, scale, zp_want, want = tie_cases.element_ties(bits, bs, dtype, symmetric)
+    K, N = W.shape
+    b, sc, zp = quantize_blockwise(dev(W), bits, bs, symmetric)
+    torch.cuda.synchronize()
+    assert np.array_equal(sc.cpu().numpy(), scale)
+    if not symmetric:
+        assert np.array_equal(np_unpack_zp(zp.cpu().numpy(), N, K, bits, bs), zp_want)
+    assert np.array_equal(np_unpack_q(b.cpu().numpy(), N, K, bits, bs), want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_zero_point_ties_round_away_from_zero(dtype, bits):
+    """-min / scale = z + 0.5 -> zero point z + 1 (roundf, q4_dq.cpp:367), and the elements that become ties with it."""
+    W, scale, zp_want, want = tie_cases.zero_point_ties(bits, 32, dtype)
+    K, N = W.shape
+    b, sc, zp = quantize_blockwise(dev(W), bits, 32, symmetric=False)
+    torch.cuda.synchronize()
+    assert np.array_equal(sc.cpu().numpy(), scale)
+    assert np.array_equal(np_unpack_zp(zp.cpu().numpy(), N, K, bits, 32), zp_want)
+    assert np.array_equal(np_unpack_q(b.cpu().numpy(), N, K, bits, 32), want)
 
 
 def test_strided_source_and_grid_round_trip():

@@ -114,6 +114,21 @@ def test_device_dequantiser_is_bit_exact(kind, zp_kind, g_kind):
     assert np.array_equal(w.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+def test_device_dequantiser_never_reads_through_a_bad_group_index():
+    """The group index of this entry point lives on the device: values outside [0, k_blocks) yield NaN, read nothing."""
+    N, K, bs = 9, 200, 32
+    c = make("f32", N, K, 4, bs, "typed", "ragged", 1, seed=3)
+    want = C.variant_dequantize(c["B"], c["scales"], c["zp"], c["g"], N, K, 4, bs)
+    g = c["g"].copy()
+    g[[7, 150]] = [1 << 30, -5]
+    w = ort_amd.dequantize_blockwise_variant(to_dev(c["B"]), to_dev(c["scales"]), to_dev(c["zp"]), to_dev(g), N, K, 4,
+                                             bs).cpu().numpy()
+    bad = np.zeros(K, bool)
+    bad[[7, 150]] = True
+    assert np.isnan(w[:, bad]).all()
+    assert np.array_equal(w[:, ~bad].view(np.uint32), want[:, ~bad].view(np.uint32))
+
+
 @pytest.mark.parametrize("kind", ["f32", "f16"])
 def test_device_dequantiser_two_bits_typed(kind):
     N, K, bs = 5, 100, 16
@@ -196,7 +211,7 @@ def test_errors():
     N, K, bs = 16, 64, 32
     c = make("f32", N, K, 4, bs, "none", "ragged", 2, seed=1)
     c["g"][5] = 2                                            # k_blocks = 2: valid indices are 0 and 1
-    with pytest.raises(MnbError, match=r"g_idx\[5\] = 2 is outside \[0, 2\)") as e:
+    with pytest.raises(MnbError, match=r"group_index value at index 5 is 2, which is out of valid range \[0, 2\)") as e:
         run_op("f32", c, N, K, 4, bs)
     assert e.value.code == _lib.INVALID_ARGUMENT
     op = MatMulNBits(K, N, bits=8, block_size=bs, dtype=torch.float16, has_zero_points=True,

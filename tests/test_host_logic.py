@@ -131,7 +131,15 @@ def test_variant_plans_without_a_gpu():
     rc, p = plan(8, K, 4, bs, _lib.DTYPE_BFLOAT16, _lib.ZP_NONE)
     assert rc == 0 and p.compute_dtype == _lib.DTYPE_FLOAT
     rc, _ = plan(8, K, 4, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, np.full(K, kb))              # group out of range
-    assert rc == _lib.INVALID_ARGUMENT and "outside [0, 7)" in _lib.last_error()
+    assert rc == _lib.INVALID_ARGUMENT and "which is out of valid range [0, 7)" in _lib.last_error()
+    # the padded form [k_blocks * block_size] is checked to its end, as the reference does (matmul_nbits_helper.h:92-103)
+    padded = np.concatenate([np.arange(K) // bs, np.full(kb * bs - K, kb - 1)])
+    rc, p = plan(8, K, 4, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, padded)
+    assert rc == 0 and not p.has_g_idx
+    padded[K + 3] = -1
+    rc, _ = plan(8, K, 4, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, padded)
+    assert rc == _lib.INVALID_ARGUMENT
+    assert f"group_index value at index {K + 3} is -1, which is out of valid range [0, 7)" in _lib.last_error()
     rc, _ = plan(8, K, 4, bs, _lib.DTYPE_FLOAT, _lib.ZP_NONE, np.zeros(K + 1))             # wrong length
     assert rc == _lib.INVALID_ARGUMENT and "group_index" in _lib.last_error()
     rc, _ = plan(8, K, 8, bs, _lib.DTYPE_FLOAT, _lib.ZP_TYPED)
@@ -153,3 +161,25 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert lib.MnbGemm(0, 8, 32, 4, 16, 0, _lib.DTYPE_FLOAT16, None, 32, None, None, None, 8, None, 0, None) == 0
     rc = lib.MnbPackQuantBData(8, 32, 4, 16, _lib.DTYPE_FLOAT16, None, None, None, None, None)
     assert rc == _lib.INVALID_ARGUMENT
+
+
+def test_tile_gemm_offsets_stay_below_four_gib():
+    """The tile GEMM adds a 32-bit per-lane byte offset to a base that holds the tile's first row and the k-step: the
+    largest offset is that of row 255 of the tile, k chunk 7, last byte = (255 * lda + 63) * 2 + 1, whatever M is.
+    Rows beyond 4 GiB from the start of A (M * lda * 2 >= 2^32) therefore stay reachable; a pitch that alone
+    overflows 32 bits must select another kernel."""
+    lib = _lib.load()
+    N, K, bits, bs = 14336, 14336, 4, 32
+    name = lambda M, lda: lib.MnbGemmKernelNameStrided(M, N, K, bits, bs, _lib.DTYPE_FLOAT16, lda).decode()
+    largest = lambda lda: (255 * lda + 7 * 8 + 7) * 2 + 1          # exact integer arithmetic
+    # M beyond the old limit (M * lda * 2 >= 2^32 at M >= 149797 for lda = 14336): offsets do not depend on M
+    for M in (2048, 149796, 149797, 262144, 1 << 21):
+        assert M * K * 2 < (1 << 32) or M >= 149797
+        assert name(M, K) == "mnb_gemm256_kernel" and largest(K) < (1 << 32)
+    # pitches around the limit: 255 * lda * 2 crosses 2^32 between lda = 8421496 and 8421504 (multiples of 8)
+    limit = max(l for l in range(8421000, 8422000, 8) if largest(l) < (1 << 32))
+    assert largest(limit) < (1 << 32) <= largest(limit + 8)
+    assert name(2048, limit) == "mnb_gemm256_kernel"
+    for lda in (limit + 8, limit + 4096, 1 << 24, 1 << 30):
+        assert largest(lda) >= (1 << 32)
+        assert name(2048, lda) != "mnb_gemm256_kernel"

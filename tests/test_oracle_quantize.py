@@ -5,12 +5,13 @@ The compiled reference is not available, so the pins are what the mathematics fi
   * the error bound |w - dequant(quant(w))| <= scale / 2 inside the representable range,
   * an independent vectorised numpy statement of the published algorithm
     (onnxruntime/core/mlas/lib/q4_dq.cpp:347-386, 468-574; numpy spec in
-    onnxruntime/test/python/quantization/test_quantizeblockwise_4bits.py:25-86), compared away from rounding ties.
-Rounding of exact .5 ties is parity unpinned (documented in the oracle's header).
+    onnxruntime/test/python/quantization/test_quantizeblockwise_4bits.py:25-86), compared away from rounding ties,
+  * exact .5 ties, whose expected integers are a closed form of the reference's roundf (tests/tie_cases.py).
 """
 import numpy as np
 import pytest
 
+import tie_cases
 from oracle.oracle import np_unpack_q, np_unpack_zp
 
 
@@ -116,3 +117,34 @@ def test_all_zero_block_and_padding(oracle):
     assert s[0, 0] == 0 and np_unpack_zp(z, 3, 40, 4, 32)[0, 0] == 0
     deq = oracle.C.dequantize(Bq, s, z, 3, 40, 4, 32)
     assert np.array_equal(deq, W.T)                                           # 0 and 1 are both on the grid
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("bs", [16, 64])
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_element_ties_round_half_away_from_zero(oracle, dtype, bits, bs, symmetric):
+    """x + 0.5 -> x + 1 for every x, even ones included (roundf, q4_dq.cpp:558); rint would give x for even x."""
+    W, scale, zp, want = tie_cases.element_ties(bits, bs, dtype, symmetric)
+    K, N = W.shape
+    Bq, s, z = oracle.C.quantize(W, bits, bs, symmetric)
+    assert np.array_equal(s, scale)
+    if not symmetric:
+        assert np.array_equal(np_unpack_zp(z, N, K, bits, bs), zp)
+    q = np_unpack_q(Bq, N, K, bits, bs)
+    assert np.array_equal(q, want)
+    even_ties = (want % 2 == 1) & (want < (1 << bits) - 1)
+    assert even_ties.sum() > 50                       # cases where half-to-even would have returned want - 1
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_zero_point_ties_round_half_away_from_zero(oracle, dtype, bits):
+    """-min / scale = z + 0.5 -> zero point z + 1 (roundf, q4_dq.cpp:367), for even and odd z."""
+    W, scale, zp, want = tie_cases.zero_point_ties(bits, 32, dtype)
+    K, N = W.shape
+    Bq, s, z = oracle.C.quantize(W, bits, 32, symmetric=False)
+    assert np.array_equal(s, scale)
+    assert np.array_equal(np_unpack_zp(z, N, K, bits, 32), zp)
+    assert ((zp - 1) % 2 == 0).sum() > 4              # even z among them
+    assert np.array_equal(np_unpack_q(Bq, N, K, bits, 32), want)

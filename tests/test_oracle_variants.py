@@ -5,8 +5,10 @@ The reference's own tests recompute their expectations for these inputs (matmul_
 expected output from its own dequantiser) and its code for this route does not build without the whole runtime, so
 what pins the restatement is mathematics: inputs on which no operation rounds (the result must equal the exact
 (q - zp) * scale), agreement with the canonical dequantiser where both are defined, group selection read back through
-power-of-two scales, and closeness to the float64 value everywhere.  The last ulp of the two-step formula
-float(q)*s + (-s*zp) on inexact inputs is not pinned by anything the reference holds."""
+power-of-two scales, closeness to the float64 value everywhere, and - for the last ulp of the three-rounding formula
+fl(fl(float(q)*s) + fl(-s*zp)) on inexact inputs - exact rational arithmetic rounded to fp32 after every operation."""
+from fractions import Fraction
+
 import numpy as np
 import pytest
 
@@ -115,3 +117,58 @@ def test_bfloat16_helpers():
     assert back[0] == 1.0 and back[3] == -2.5
     assert oracle.widen(oracle.narrow_bf16(np.float32([1.00390625])))[0] == 1.0          # tie -> even
     assert oracle.widen(oracle.narrow_bf16(np.float32([1.01171875])))[0] == 1.015625     # tie -> even (up)
+
+
+def _round_to_f32(x: Fraction) -> np.float32:
+    """Round-to-nearest-even of an exact rational to IEEE binary32 (normal and subnormal range; no overflow here)."""
+    if x == 0:
+        return np.float32(0.0)
+    sign, a = (-1 if x < 0 else 1), abs(x)
+    e = a.numerator.bit_length() - a.denominator.bit_length()      # 2^(e-1) < a < 2^(e+1)
+    if Fraction(2) ** e > a:
+        e -= 1                                                     # now 2^e <= a < 2^(e+1)
+    q = max(e - 23, -149)                                          # exponent of the last kept bit
+    scaled = a / Fraction(2) ** q
+    n = scaled.numerator // scaled.denominator
+    rem = scaled - n
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+        n += 1
+    return np.float32(sign * float(n) * 2.0 ** q)                  # n < 2^25 and a power of two: exact in double
+
+
+def test_round_to_f32_helper_against_numpy():
+    rng = np.random.default_rng(0)
+    d = np.concatenate([rng.standard_normal(2000) * 10.0 ** rng.integers(-30, 30, 2000),
+                        [1 + 2.0 ** -24, 1 + 3 * 2.0 ** -24, 1 - 2.0 ** -25, 2.0 ** -140 * 1.3, 2.0 ** -149 * 0.5]])
+    for v in d:                                                    # doubles are exact rationals; numpy rounds them RNE
+        assert _round_to_f32(Fraction(float(v))) == np.float32(v)
+
+
+@pytest.mark.parametrize("bits,zp_kind", [(4, "typed"), (2, "typed"), (4, "uint8+g_idx"), (4, "none+g_idx")])
+def test_three_roundings_against_exact_rational_arithmetic(bits, zp_kind):
+    """w = fl(fl(float(q) * s) + fl(-s * zp)), every operation rounded to fp32 by itself
+    (matmul_nbits_impl.cc:66-73 with T = float).  A contracted multiply-add, a (q - zp) * s evaluation or a float64
+    intermediate each differ from this in the last place on part of these inputs (counted below)."""
+    N, K, bs = 5, 96, 16
+    B, scales, zt, zu, kb, rng = _case(N, K, bits, bs, seed=31 + bits)
+    g = rng.integers(0, kb, size=K).astype(np.int32) if "g_idx" in zp_kind else None
+    if zp_kind == "typed":
+        zp_arg, zf = zt, zt
+    elif zp_kind.startswith("uint8"):
+        zp_arg, zf = zu, np_unpack_zp(zu, N, K, bits, bs).astype(np.float32)
+    else:
+        zp_arg, zf = None, np.full((N, kb), 2 ** (bits - 1), np.float32)
+    w = C.variant_dequantize(B, scales, zp_arg, g, N, K, bits, bs)
+    q = np_unpack_q(B, N, K, bits, bs)
+    blk = g if g is not None else np.arange(K) // bs
+    fused_differs = single_differs = 0
+    for n in range(N):
+        for k in range(K):
+            s, z = Fraction(float(scales[n, blk[k]])), Fraction(float(zf[n, blk[k]]))
+            adjust = Fraction(float(_round_to_f32(-s * z)))
+            prod = Fraction(float(_round_to_f32(int(q[n, k]) * s)))
+            want = _round_to_f32(prod + adjust)
+            assert w[n, k] == want, (n, k, float(w[n, k]), float(want))
+            fused_differs += _round_to_f32(int(q[n, k]) * s + adjust) != want
+            single_differs += _round_to_f32((int(q[n, k]) - z) * s) != want
+    assert fused_differs > 0 and single_differs > 0      # the inputs do tell the formulas apart
