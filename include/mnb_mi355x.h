@@ -111,6 +111,18 @@ MNB_API int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int 
                     const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev,
                     size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* MnbGemm for callers that cannot allocate or carry device memory of their own: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results
+ * as MnbGemm (bit for bit) minus the workspace: the scratch MnbGemm would ask for lives in a device array inside the
+ * library (MnbGemmStaticScratchCapacity bytes, 32 MiB, held on every device the library runs on until the process
+ * ends).  The call allocates and frees nothing.  A problem whose MnbGemmWorkspaceSize exceeds the capacity is rejected
+ * with MNB_INVALID_ARGUMENT.  Every call on a device shares that device's array: calls that may overlap on one device
+ * (different streams, several threads) race on it and must be serialised by the caller. */
+MNB_API size_t MnbGemmStaticScratchCapacity(void);
+MNB_API int MnbGemmStaticScratch(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                                 int a_dtype, const void* a_dev, size_t lda, const void* packed_dev,
+                                 const void* bias_dev, void* c_dev, size_t ldc, void* stream);
+
 /* Workspace bytes MnbGemmUnpacked needs (packed copy + MnbGemmWorkspaceSize). */
 MNB_API size_t MnbGemmUnpackedWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size,
                                             int has_zero_points, int a_dtype);

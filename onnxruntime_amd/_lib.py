@@ -62,6 +62,9 @@ SIGNATURES = {
     "MnbGemmWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
     "MnbGemm": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
                         c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "MnbGemmStaticScratchCapacity": (c_size_t, []),
+    "MnbGemmStaticScratch": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
+                                     c_void_p, c_void_p, c_size_t, c_void_p]),
     "MnbGemmUnpackedWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
     "MnbGemmUnpacked": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
                                 c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),

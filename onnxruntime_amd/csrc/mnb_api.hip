@@ -320,6 +320,65 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
                       c_dev, ldc, workspace_dev, workspace_bytes, stream);
 }
 
+}  // extern "C"
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------------------------
+// The per-call scratch of MnbGemm (the streaming kernel's copy of A in matrix-core operand order) as a file-scope
+// device array: every device the library runs on holds its own copy, at its own address, until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+constexpr size_t kMnbStaticScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kMnbStaticScratchBytes];
+
+namespace {
+
+// Device address of `scratch` on the current device; asked once per device, with that device current.
+int static_scratch_address(void** out) {
+  constexpr int kMaxDevices = 64;
+  static void* address[kMaxDevices];
+  static hipError_t status[kMaxDevices];
+  static std::once_flag once[kMaxDevices];
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return hip_fail(e, "MnbGemmStaticScratch: hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(MNB_NOT_IMPLEMENTED, "MnbGemmStaticScratch: device ordinal %d is beyond the %d this entry point tracks", dev,
+                kMaxDevices);
+  std::call_once(once[dev], [dev] {
+    void* p = nullptr;
+    status[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    address[dev] = status[dev] == hipSuccess ? p : nullptr;
+  });
+  if (status[dev] != hipSuccess) return hip_fail(status[dev], "MnbGemmStaticScratch: hipGetSymbolAddress");
+  if (address[dev] == nullptr) return fail(MNB_EP_FAIL, "MnbGemmStaticScratch: the scratch array has no device address");
+  *out = address[dev];
+  return MNB_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t MnbGemmStaticScratchCapacity(void) { return kMnbStaticScratchBytes; }
+
+int MnbGemmStaticScratch(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                         const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev,
+                         size_t ldc, void* stream) {
+  if (int rc = check_config("MnbGemmStaticScratch", bits, block_size, a_dtype)) return rc;
+  if (M == 0 || N == 0) return MNB_OK;
+  const size_t need = MnbGemmWorkspaceSize(M, N, K, bits, block_size, has_zero_points, a_dtype);
+  if (need > kMnbStaticScratchBytes)
+    return fail(MNB_INVALID_ARGUMENT,
+                "MnbGemmStaticScratch: this problem needs %zu bytes of scratch, the static array holds %zu; use MnbGemm "
+                "with a workspace of MnbGemmWorkspaceSize bytes",
+                need, kMnbStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0)
+    if (int rc = static_scratch_address(&ws)) return rc;
+  // The kernels that use the scratch write every byte they later read (the staging pass covers the whole operand
+  // copy, padding included), so nothing of an earlier call's contents has to be cleared.
+  return gemm_checked("MnbGemmStaticScratch", M, N, K, bits, block_size, has_zero_points, a_dtype, a_dev, lda,
+                      packed_dev, bias_dev, c_dev, ldc, ws, need, stream);
+}
+
 size_t MnbGemmUnpackedWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                     int a_dtype) {
   const size_t pack = MnbPackQuantBDataSize(N, K, bits, block_size, has_zero_points, a_dtype);

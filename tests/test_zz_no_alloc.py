@@ -1,0 +1,98 @@
+"""MnbGemmStaticScratch, the entry point that allocates nothing, against MnbGemm on the same inputs: bit-identical
+outputs, on two calls in a row of which the second is smaller (the scratch array keeps the first call's contents),
+for shapes that use the scratch (the streaming kernel's staged activations) and shapes that do not."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import dev
+from onnxruntime_amd import _lib
+from onnxruntime_amd.matmul_nbits import MatMulNBits
+from onnxruntime_amd.synthetic import make_case
+
+pytestmark = pytest.mark.gpu
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _both(case):
+    """Runs one case through MnbGemm (own workspace) and through MnbGemmStaticScratch; returns the two outputs."""
+    lib = _lib.load()
+    dt = _lib.DTYPE_FLOAT16 if case.dtype == np.float16 else _lib.DTYPE_FLOAT
+    tdt = torch.float16 if case.dtype == np.float16 else torch.float32
+    has_zp = int(case.zero_points is not None)
+    op = MatMulNBits(case.K, case.N, case.bits, case.block_size, dtype=tdt, has_zero_points=bool(has_zp),
+                     has_bias=case.bias is not None)
+    assert op.PrePack(dev(case.B), dev(case.scales), dev(case.zero_points))
+    a, bias = dev(case.A), dev(case.bias)
+    M = a.shape[0]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    need = lib.MnbGemmWorkspaceSize(M, case.N, case.K, case.bits, case.block_size, has_zp, dt)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+    y_ref = torch.full((M, case.N), float("nan"), dtype=tdt, device="cuda")
+    y_new = torch.full((M, case.N), float("nan"), dtype=tdt, device="cuda")
+    _lib.check(lib.MnbGemm(M, case.N, case.K, case.bits, case.block_size, has_zp, dt, _ptr(a), case.K, _ptr(op.packed),
+                           _ptr(bias), _ptr(y_ref), case.N, _ptr(ws), need, stream))
+    _lib.check(lib.MnbGemmStaticScratch(M, case.N, case.K, case.bits, case.block_size, has_zp, dt, _ptr(a), case.K,
+                                        _ptr(op.packed), _ptr(bias), _ptr(y_new), case.N, stream))
+    torch.cuda.synchronize()
+    return y_ref, y_new, need
+
+
+def _bits(t):
+    return t.view(torch.int16 if t.dtype == torch.float16 else torch.int32)
+
+
+# (first call, second and smaller call); M, N, K, bits, block size
+PAIRS = [
+    ((300, 520, 1024, 4, 32), (40, 200, 256, 4, 32)),      # streaming kernel twice: the scratch is used by both
+    ((128, 4096, 4096, 4, 128), (17, 333, 200, 8, 64)),    # a large staged copy, then a ragged small one
+    ((64, 512, 512, 4, 128), (1, 512, 1024, 4, 128)),      # scratch, then the decode kernel (no scratch)
+    ((5, 100, 200, 4, 32), (3, 100, 200, 4, 32)),          # M <= 16 with K that is not whole chunks: staged route
+]
+
+
+@pytest.mark.parametrize("first,second", PAIRS)
+def test_same_bits_as_the_entry_point_with_a_workspace(oracle, first, second):
+    used_scratch = False
+    for (M, N, K, bits, bs) in (first, second):
+        c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, has_bias=True, seed=M + N)
+        y_ref, y_new, need = _both(c)
+        used_scratch |= need > 0
+        assert not torch.isnan(y_new).any()
+        assert torch.equal(_bits(y_ref), _bits(y_new)), (M, N, K, bits, bs)
+        # and MnbGemm itself is right (the oracle's reference-semantics result, fp16 gate)
+        want = oracle.C.matmul(c.A, c.B, c.scales, c.zero_points, c.bias, c.N, c.K, c.bits, c.block_size).astype(np.float64)
+        got = y_new.cpu().numpy().astype(np.float64)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 5e-3
+    assert used_scratch
+
+
+def test_fp32_and_tile_gemm_need_no_scratch():
+    lib = _lib.load()
+    for (M, N, K, bits, bs, dtype, kernel) in [(2048, 8192, 1024, 4, 32, np.float16, "mnb_gemm256_kernel"),
+                                               (64, 256, 512, 8, 64, np.float32, "mnb_gemm32_kernel")]:
+        dt = _lib.DTYPE_FLOAT16 if dtype == np.float16 else _lib.DTYPE_FLOAT
+        assert lib.MnbGemmKernelName(M, N, K, bits, bs, dt).decode() == kernel
+        c = make_case(M, N, K, bits, bs, dtype, has_zp=True, seed=1)
+        y_ref, y_new, need = _both(c)
+        assert need == 0
+        assert torch.equal(_bits(y_ref), _bits(y_new))
+
+
+def test_problems_beyond_the_capacity_are_rejected():
+    lib = _lib.load()
+    cap = lib.MnbGemmStaticScratchCapacity()
+    assert cap == 32 << 20
+    M, N, K = 1024, 4096, 32768 + 64                        # K not a multiple of 128: the streaming kernel at any M
+    need = lib.MnbGemmWorkspaceSize(M, N, K, 4, 32, 0, _lib.DTYPE_FLOAT16)
+    assert need > cap
+    one = torch.zeros(256, dtype=torch.uint8, device="cuda")  # never dereferenced: the size check comes first
+    rc = lib.MnbGemmStaticScratch(M, N, K, 4, 32, 0, _lib.DTYPE_FLOAT16, _ptr(one), K, _ptr(one), None, _ptr(one), N,
+                                  None)
+    assert rc == _lib.INVALID_ARGUMENT
+    assert "the static array holds" in _lib.last_error()
