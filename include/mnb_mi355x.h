@@ -94,9 +94,11 @@ MNB_API int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int 
                               const void* scales_dev, const void* zero_points_dev, void* packed_dev, void* stream);
 
 /* Replaces MlasQNBitGemmBatchWorkspaceSize (mlas_qnbit.h:178-189): bytes of per-call device scratch MnbGemm needs for
- * this problem. Non-zero only for fp16 activations whose shape selects the weight-streaming kernel (M > 16 below the
- * tile GEMM's range, or M <= 16 with K not a multiple of 128 (4-bit) / 64 (8-bit)): a copy of A in matrix-core
- * operand order, about M*K*2 bytes; 0 otherwise. */
+ * this problem.  Non-zero only for fp16 activations: (a) shapes that select the weight-streaming kernel (M > 16 below
+ * the tile GEMM's range, or M <= 16 with K not a multiple of 128 (4-bit) / 64 (8-bit)): a copy of A in matrix-core
+ * operand order, about M*K*2 bytes, which that kernel cannot do without; (b) tall problems with few output tiles on
+ * the tile GEMM, which then cuts every tile along K across workgroups: flags plus one fp32 partial tile per workgroup,
+ * up to about 64 MiB.  Without (or with less than) the scratch of (b) the tile GEMM runs uncut. */
 MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                     int a_dtype);
 
@@ -116,7 +118,8 @@ MNB_API int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int 
  * as MnbGemm (bit for bit) minus the workspace: the scratch MnbGemm would ask for lives in a device array inside the
  * library (MnbGemmStaticScratchCapacity bytes, 32 MiB, held on every device the library runs on until the process
  * ends).  The call allocates and frees nothing.  A problem whose MnbGemmWorkspaceSize exceeds the capacity is rejected
- * with MNB_INVALID_ARGUMENT.  Every call on a device shares that device's array: calls that may overlap on one device
+ * with MNB_INVALID_ARGUMENT, unless the scratch would only serve the tile GEMM's optional cut of tiles along K: that
+ * kernel then runs without the cut (the same sums in another fp32 order).  Every call on a device shares that device's array: calls that may overlap on one device
  * (different streams, several threads) race on it and must be serialised by the caller. */
 MNB_API size_t MnbGemmStaticScratchCapacity(void);
 MNB_API int MnbGemmStaticScratch(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,

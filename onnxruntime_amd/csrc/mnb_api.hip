@@ -214,9 +214,8 @@ static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
   if (mid_max_m >= 0) return M > mid_max_m;
   const MnbDeviceInfo& dev = mnb_device_info();
   const double t_mid = 2.0 * (double)M * (double)L.N * (double)L.K / (kMnbMidFlopsPerCuCycle * dev.cus * dev.clock_hz);
-  double t_256 = 0.0;
-  (void)mnb_gemm256_tile_rows(L, M, &t_256);
-  return t_256 < t_mid;
+  // a caller that follows MnbGemmWorkspaceSize hands over the workspace the split needs
+  return mnb_gemm256_plan(L, M, true).seconds < t_mid;
 }
 
 MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
@@ -266,6 +265,8 @@ size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_si
     // M <= 16 needs it only when K is not a whole number of the decode kernel's chunks
     const bool wants = M > 16 ? !mnb_prefer_gemm256(L, (int64_t)M) : (K % (size_t)(4 * L.group_k) != 0);
     if (wants) return mnb_mid_workspace_bytes(L, (int64_t)M);
+    // the tile GEMM: partial tiles and flags when it splits tiles along K across workgroups
+    if (M > 16) return mnb_gemm256_plan(L, (int64_t)M, true).workspace_bytes;
   }
   return 0;
 }
@@ -364,12 +365,22 @@ int MnbGemmStaticScratch(size_t M, size_t N, size_t K, int bits, int block_size,
                          size_t ldc, void* stream) {
   if (int rc = check_config("MnbGemmStaticScratch", bits, block_size, a_dtype)) return rc;
   if (M == 0 || N == 0) return MNB_OK;
-  const size_t need = MnbGemmWorkspaceSize(M, N, K, bits, block_size, has_zero_points, a_dtype);
-  if (need > kMnbStaticScratchBytes)
-    return fail(MNB_INVALID_ARGUMENT,
-                "MnbGemmStaticScratch: this problem needs %zu bytes of scratch, the static array holds %zu; use MnbGemm "
-                "with a workspace of MnbGemmWorkspaceSize bytes",
-                need, kMnbStaticScratchBytes);
+  size_t need = MnbGemmWorkspaceSize(M, N, K, bits, block_size, has_zero_points, a_dtype);
+  if (need > kMnbStaticScratchBytes) {
+    // The tile GEMM uses scratch only to cut tiles along K across workgroups and runs without it otherwise; every
+    // other use of scratch (the streaming kernel's staged activations) is indispensable.
+    MnbGemmArgs probe{};
+    probe.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+    probe.M = (int64_t)M;
+    probe.A = a_dev;
+    probe.lda = (int64_t)lda;
+    if (mnb_select_kernel(probe) != kMnbKernelGemm256)
+      return fail(MNB_INVALID_ARGUMENT,
+                  "MnbGemmStaticScratch: this problem needs %zu bytes of scratch, the static array holds %zu; use "
+                  "MnbGemm with a workspace of MnbGemmWorkspaceSize bytes",
+                  need, kMnbStaticScratchBytes);
+    need = 0;
+  }
   void* ws = nullptr;
   if (need > 0)
     if (int rc = static_scratch_address(&ws)) return rc;

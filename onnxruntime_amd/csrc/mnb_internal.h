@@ -69,8 +69,15 @@ struct MnbDeviceInfo {
   double clock_hz;
 };
 const MnbDeviceInfo& mnb_device_info();
-// rows of the tile the tile GEMM would use (256 or 128) and, optionally, its estimated run time
-int mnb_gemm256_tile_rows(const MnbLayout& L, int64_t M, double* seconds);
+// how the tile GEMM would run a problem (mnb_gemm256.hip)
+struct MnbGemm256Plan {
+  int tile_rows;           // 256 or 128
+  int64_t grid;            // workgroups: the tiles, or one per compute unit when tiles are split along K
+  bool split;              // tiles are computed in parts by several workgroups (needs workspace_bytes of scratch)
+  size_t workspace_bytes;  // flags + one partial tile per workgroup; 0 without a split
+  double seconds;          // estimate, for the choice between kernels
+};
+MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace);
 bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
 // the tile GEMM's 32-bit per-lane offsets reach every element of this problem
 uint64_t mnb_gemm256_max_lane_offset(int64_t lda);
