@@ -39,10 +39,16 @@ def hipcc() -> str:
     return exe
 
 
+# Per-source flags.  The decode kernels take what their first loads need as leading scalar arguments; the compiler is
+# asked to have those preloaded into SGPRs at wavefront start (firmware without the feature runs the compatibility
+# prologue the compiler emits in front of the kernel, which loads them the usual way).
+EXTRA_FLAGS = {"mnb_skinny.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
+
+
 def _compile(src: str, extra=()) -> Path:
     OBJ_DIR.mkdir(exist_ok=True)
     obj = OBJ_DIR / (src + ".o")
-    cmd = [hipcc(), *HIPCC_FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)]
+    cmd = [hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), *extra, "-c", str(CSRC / src), "-o", str(obj)]
     r = subprocess.run(cmd, capture_output=True, text=True)
     msgs = [l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip()]
     if r.returncode != 0:

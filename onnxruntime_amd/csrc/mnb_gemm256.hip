@@ -82,7 +82,6 @@ struct Gemm256Params {
   uint32_t* flags;          // one word per workgroup and wavefront, zero when the kernel starts
   int spin_limit;           // polls of a flag before the wait gives up and the tile is poisoned with NaN
   int c_vec_ok;  // C allows 16-byte stores of 8 columns: aligned base and pitch, N a multiple of 8
-  uint32_t uc[4];  // unpack constants (see UnpackConsts)
   // several matrices packed as one (mnb_layout.h); these kinds always take the 16-byte store path
   int epi_kind;            // kMnbFusedNone / kMnbFusedMlp: C[M][n_out0] = silu(gate) * up / kMnbFusedQkv: three outputs
   int start1, start2;      // qkv: first packed column of the second and third output
@@ -92,18 +91,18 @@ struct Gemm256Params {
   int64_t ld1, ld2;
 };
 
-// The constants of the nibble unpack, passed as kernel arguments: with literals the compiler emits
-// v_and_b32 + v_or_b32 (VOP3 takes no literal on this ISA family); with register operands, one v_and_or_b32.
+// The constants of the nibble unpack.  Written as plain literals the compiler emits v_and_b32 + v_or_b32 (VOP3 takes
+// no literal on this ISA family); held in registers, one v_and_or_b32.  Opaque moves materialise them (the masks in
+// SGPRs, the magic in a VGPR: one SGPR operand per VALU instruction) so that they are not folded back.
 struct UnpackConsts {
   uint32_t mask_lo, mask_hi, magic;  // 0x000F000F, 0x00F000F0, 0x64006400 (two halves of 1024)
 };
 
-__device__ __forceinline__ UnpackConsts make_unpack_consts(const uint32_t* k) {
+__device__ __forceinline__ UnpackConsts make_unpack_consts() {
   UnpackConsts u;
-  u.mask_lo = k[0];
-  u.mask_hi = k[1];
-  // one SGPR operand per VALU instruction: the magic lives in a VGPR (an opaque move, so it is not folded back)
-  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic) : "s"(k[2]));
+  asm("s_mov_b32 %0, 0x000F000F" : "=s"(u.mask_lo));
+  asm("s_mov_b32 %0, 0x00F000F0" : "=s"(u.mask_hi));
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(u.magic));
   return u;
 }
 
@@ -186,7 +185,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   h8_t FA0[TM], FA1[TM];  // A operands, double buffered over slabs
   h8_t FB0[2], FB1[2];  // B operands, double buffered over slabs
 
-  const UnpackConsts uc = make_unpack_consts(p.uc);
+  const UnpackConsts uc = make_unpack_consts();
 
   // Addressing: every global access is  uniform base (SGPRs: the tile's corner, advanced per k-step)  +  32-bit
   // per-lane offset (a VGPR), so the loads cost no VALU work inside the loop.  The tile's first row and column are
@@ -707,10 +706,6 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   }
   const unsigned grid = (unsigned)plan.grid;
-  p.uc[0] = 0x000F000Fu;
-  p.uc[1] = 0x00F000F0u;
-  p.uc[2] = 0x64006400u;
-  p.uc[3] = 0;
   p.c_vec_ok = (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.ldc % 8 == 0) && (a.L.N % 8 == 0);
   p.epi_kind = a.epi.kind;
   if (a.epi.kind != kMnbFusedNone) {

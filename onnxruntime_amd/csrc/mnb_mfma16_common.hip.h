@@ -30,27 +30,25 @@ struct SkinnyParams {
   int phase_chunks; // chunks staged in LDS at a time
   int mtr;          // rows of A staged (power of two >= M, <= 16)
   int a_vec_ok;     // A allows 16-byte loads
-  uint32_t uc[4];   // UnpackConsts
   EpiParams epi;
 };
 
 constexpr int kLdsPad = 8;  // halves of padding per staged row
 
-// The four constants of the nibble unpack.  They are passed as kernel arguments rather than written as literals:
-// VOP3 encodings of this ISA family take no literal, so with literals the compiler emits v_and_b32 + v_or_b32
-// (two instructions); with register operands it selects the single v_and_or_b32.
+// The four constants of the nibble unpack.  Written as plain literals the compiler emits v_and_b32 + v_or_b32 (VOP3
+// encodings of this ISA family take no literal); held in registers it selects the single v_and_or_b32.  They are
+// materialised by opaque moves (an SGPR for each mask, a VGPR for each magic: one SGPR operand per VALU instruction),
+// which the optimiser cannot fold back into literals and which depend on nothing, not even the kernel arguments.
 struct UnpackConsts {
   uint32_t mask_lo, mask_hi, magic_lo, magic_hi;  // 0x000F000F, 0x00F000F0, 0x64006400 (1024), 0x54005400 (64)
 };
 
-// One SGPR operand per VALU instruction: the masks stay scalar, the magics are moved to VGPRs once per kernel.
-// The move is opaque to the optimiser so that it cannot fold the value back into a literal.
-__device__ __forceinline__ UnpackConsts make_unpack_consts(const uint32_t* k) {
+__device__ __forceinline__ UnpackConsts make_unpack_consts() {
   UnpackConsts u;
-  u.mask_lo = k[0];
-  u.mask_hi = k[1];
-  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic_lo) : "s"(k[2]));
-  asm volatile("v_mov_b32 %0, %1" : "=v"(u.magic_hi) : "s"(k[3]));
+  asm("s_mov_b32 %0, 0x000F000F" : "=s"(u.mask_lo));
+  asm("s_mov_b32 %0, 0x00F000F0" : "=s"(u.mask_hi));
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(u.magic_lo));
+  asm("v_mov_b32 %0, 0x54005400" : "=v"(u.magic_hi));
   return u;
 }
 

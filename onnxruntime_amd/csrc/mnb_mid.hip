@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int t = 0; t < T; ++t) y[mt][t] = f4_t{0.f, 0.f, 0.f, 0.f};
-  const UnpackConsts uc = make_unpack_consts(p.uc);
+  const UnpackConsts uc = make_unpack_consts();
 
   h8_t af[MT][NI];
   auto load_a = [&](int c) {
@@ -310,10 +310,6 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
     p.epi.ld1 = a.epi.ld[1];
     p.epi.ld2 = a.epi.ld[2];
   }
-  p.uc[0] = 0x000F000Fu;
-  p.uc[1] = 0x00F000F0u;
-  p.uc[2] = 0x64006400u;
-  p.uc[3] = 0x54005400u;
   mp.As = reinterpret_cast<const uint4*>(a.workspace);
   mp.row_tiles = mid_row_tiles(a.M, pl.mt);
   const int vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);

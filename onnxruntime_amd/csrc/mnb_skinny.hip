@@ -185,7 +185,7 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
   const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
   h8_t* mine = reinterpret_cast<h8_t*>(smem) + wave * (16 * AStage<BITS>::PIECES);  // A_LDS only
   const BConst bconst = make_bconst<BITS, HAS_ZP>();
-  const UnpackConsts uc = make_unpack_consts(p.uc);
+  const UnpackConsts uc = make_unpack_consts();
 
   // the activation loads of chunk c: the operands themselves, or the row-contiguous pieces that pass through LDS
   auto fetch_a = [&](int c, h8_t* a) {
@@ -292,8 +292,30 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
   if constexpr (A_LDS) __syncthreads();  // the reduction buffer overlays the staging regions of all wavefronts
 }
 
+// What a wavefront needs to issue its first loads comes as leading scalar kernel arguments, which the build asks the
+// compiler to have preloaded into SGPRs when the wavefront starts (kernarg preload: no scalar load, about 0.4 us, in
+// front of the first weight load); everything else stays in the parameter block and is fetched where it is used.
+#define MNB_SKINNY_HOT_PARAMS                                                                                 \
+  const uint4 *hot_W, int64_t hot_Npad, const _Float16 *hot_A, int64_t hot_lda, const uint8_t *hot_meta, int hot_M, \
+      int hot_chunks, int hot_bs_shift
+#define MNB_SKINNY_HOT_ARGS(p) (p).W, (p).Npad, (p).A, (p).lda, (p).meta, (p).M, (p).chunks, (p).bs_shift
+
+__device__ __forceinline__ SkinnyParams with_hot_params(SkinnyParams p, MNB_SKINNY_HOT_PARAMS) {
+  p.W = hot_W;
+  p.Npad = hot_Npad;
+  p.A = hot_A;
+  p.lda = hot_lda;
+  p.meta = hot_meta;
+  p.M = hot_M;
+  p.chunks = hot_chunks;
+  p.bs_shift = hot_bs_shift;
+  return p;
+}
+#define MNB_SKINNY_HOT_NAMES hot_W, hot_Npad, hot_A, hot_lda, hot_meta, hot_M, hot_chunks, hot_bs_shift
+
 template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS>
-__global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams p) {
+__global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(MNB_SKINNY_HOT_PARAMS, SkinnyParams rest) {
+  const SkinnyParams p = with_hot_params(rest, MNB_SKINNY_HOT_NAMES);
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -318,7 +340,8 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(SkinnyParams
 // compute unit - were measured too: the half tile costs the instructions of a whole one, and the run time did not
 // improve.)
 template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS>
-__global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(SkinnyParams p) {
+__global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(MNB_SKINNY_HOT_PARAMS, SkinnyParams rest) {
+  const SkinnyParams p = with_hot_params(rest, MNB_SKINNY_HOT_NAMES);
   extern __shared__ __align__(16) unsigned char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -362,7 +385,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
 #pragma unroll
   for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
   const BConst bconst = make_bconst<BITS, HAS_ZP>();
-  const UnpackConsts uc = make_unpack_consts(p.uc);
+  const UnpackConsts uc = make_unpack_consts();
 
   for (int ph0 = 0; ph0 < p.chunks; ph0 += p.phase_chunks) {
     const int ph1 = min(ph0 + p.phase_chunks, p.chunks);
@@ -461,7 +484,8 @@ hipError_t launch_slab(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
   // the plan never asks for the LDS route in the general loop of sixteen wavefronts on 4-bit weights: not instantiated
   if (pl.a_lds && cpw == 0 && BITS == 4 && pl.nw == 16) return hipErrorInvalidConfiguration;
 #define MNB_SLAB_LAUNCH(NW_, CPW_, LDS_) \
-  mnb_skinny_slab_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
+  mnb_skinny_slab_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_>                  \
+      <<<grid, dim3(NW_ * 64), pl.smem, s>>>(MNB_SKINNY_HOT_ARGS(p), p)
 #define MNB_SLAB_CPW(NW_)                                           \
   do {                                                              \
     if (pl.a_lds) {                                                 \
@@ -498,7 +522,8 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
     // not instantiated, never planned: LDS route in the general loop of four-tile slabs or of sixteen 4-bit wavefronts
     if (pl.a_lds && cpw == 0 && (T == 4 || (BITS == 4 && pl.nw == 16))) return hipErrorInvalidConfiguration;
 #define MNB_SKINNY_LAUNCH(NW_, CPW_, LDS_) \
-  mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_><<<grid, dim3(NW_ * 64), pl.smem, s>>>(p)
+  mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_>                \
+      <<<grid, dim3(NW_ * 64), pl.smem, s>>>(MNB_SKINNY_HOT_ARGS(p), p)
 #define MNB_SKINNY_CPW(NW_)                                         \
   do {                                                              \
     if (pl.a_lds) {                                                 \
@@ -589,10 +614,6 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
     p.epi.ld1 = a.epi.ld[1];
     p.epi.ld2 = a.epi.ld[2];
   }
-  p.uc[0] = 0x000F000Fu;
-  p.uc[1] = 0x00F000F0u;
-  p.uc[2] = 0x64006400u;
-  p.uc[3] = 0x54005400u;
   if (L.bits == 4) return L.has_zp ? launch_zp<4, true>(p, pl, s) : launch_zp<4, false>(p, pl, s);
   return L.has_zp ? launch_zp<8, true>(p, pl, s) : launch_zp<8, false>(p, pl, s);
 }
