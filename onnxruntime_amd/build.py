@@ -39,10 +39,11 @@ def hipcc() -> str:
     return exe
 
 
-# Per-source flags.  The decode kernels take what their first loads need as leading scalar arguments; the compiler is
+# Per-source flags.  The decode and streaming kernels take what their first loads need as leading scalar arguments; the compiler is
 # asked to have those preloaded into SGPRs at wavefront start (firmware without the feature runs the compatibility
 # prologue the compiler emits in front of the kernel, which loads them the usual way).
-EXTRA_FLAGS = {"mnb_skinny.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"]}
+_PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=14"]
+EXTRA_FLAGS = {"mnb_skinny.hip": _PRELOAD, "mnb_gemv.hip": _PRELOAD, "mnb_mid.hip": _PRELOAD}
 
 
 def _compile(src: str, extra=()) -> Path:

@@ -197,23 +197,20 @@ const MnbDeviceInfo& mnb_device_info() {
 }
 
 // ------------------------------------------------------------------------------------------------ kernel choice
-// fp16, M > 16: the weight-streaming kernel (mnb_mid.hip) takes any shape; the 256 x 256 tile GEMM wins once its tiles
-// fill the chip.  The estimate compares 2MNK at the streaming kernel's rate with whole rounds of tiles at the tile
-// kernel's cycles per 64-deep k-step.
-// What the streaming kernel sustains per compute unit and cycle in the range where the two compete (M = 128 ... 1024
-// on the Llama-3-8B projections: 0.9 flop in 4 of the matrix cores' 4096 per cycle, the rest is weight dequantisation,
-// activation operand traffic and the reduction epilogue).
-constexpr double kMnbMidFlopsPerCuCycle = 895.0;
+// fp16, M > 16: the weight-streaming kernel (mnb_mid.hip) takes any shape; the tile GEMM wins once its tiles occupy
+// enough of the chip.  The estimate compares the tile GEMM's plan (mnb_gemm256_plan) with the streaming kernel's
+// measured behaviour over the same range of shapes: a fixed 8 us (at 2.4 GHz) plus 2MNK at 1286 flop per compute unit
+// and cycle for 4-bit weights (790 Tflop/s on 256 compute units), 1156 for 8-bit.
+constexpr double kMnbMidStartCycles = 19200.0;
+constexpr double kMnbMidFlopsPerCuCycle[2] = {1286.0, 1156.0};
 
 static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
   if (M <= 128 || L.K % 128 != 0) return false;
-  static const int64_t mid_max_m = [] {
-    const char* e = getenv("MNB_MID_MAX_M");  // tuning override: M up to this value always streams
-    return e ? (int64_t)atoll(e) : (int64_t)-1;
-  }();
-  if (mid_max_m >= 0) return M > mid_max_m;
+  if (const char* e = mnb_tuning_env("MNB_MID_MAX_M")) return M > (int64_t)atoll(e);  // calibration: M up to this streams
   const MnbDeviceInfo& dev = mnb_device_info();
-  const double t_mid = 2.0 * (double)M * (double)L.N * (double)L.K / (kMnbMidFlopsPerCuCycle * dev.cus * dev.clock_hz);
+  const double t_mid = (kMnbMidStartCycles + 2.0 * (double)M * (double)L.N * (double)L.K /
+                                                 (kMnbMidFlopsPerCuCycle[L.bits == 4 ? 0 : 1] * dev.cus)) /
+                       dev.clock_hz;
   // a caller that follows MnbGemmWorkspaceSize hands over the workspace the split needs
   return mnb_gemm256_plan(L, M, true).seconds < t_mid;
 }

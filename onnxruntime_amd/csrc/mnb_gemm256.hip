@@ -5,13 +5,14 @@
 //
 // Eight wavefronts (2 x 4, two per SIMD), each owning a 128 x 64 block of the tile as 4 x 2
 // v_mfma_f32_32x32x16_f16 accumulators.  Per k-step of 64:
-//   * A (activations) goes from global memory straight into LDS (global_load_lds_dwordx4: no registers, no LDS
+//   * A (activations) goes from global memory straight into LDS (buffer_load_dwordx4 ... lds: no registers, no LDS
 //     store instructions), two k-steps ahead, into one of three staged tiles.  Such a load puts the 16 bytes of lane
 //     L at (wave-uniform LDS base) + 16 L, so a wavefront fills 8 rows x 128 bytes with one instruction; the rows are
 //     not padded, instead the lane that fills chunk position p of row r fetches chunk p ^ (r & 7) of that row, and the
 //     readers (ds_read_b128, lane = row) apply the same XOR: conflict free.
 //   * B (weights) never touches LDS.  Lane (column j = lane%32, half kq = lane/32) of a wavefront loads, two steps
-//     ahead, exactly the 8 bytes of packed weights it will feed to the matrix core: the two 32-bit words of its
+//     ahead (each register is reloaded right after its last use, and the loop states its own exact waits: see
+//     LoadPlan), exactly the 8 bytes of packed weights it will feed to the matrix core: the two 32-bit words of its
 //     column's 16-byte vector that belong to its half.  Each word is dequantised in registers to 8 halves -- exact
 //     (q - zp), one rounding by the scale, bit-identical to the reference's fp16 dequantisation -- and IS the MFMA
 //     B operand of one k-slab.  (The contraction index of an MFMA may be permuted freely as long as A uses the same
@@ -57,11 +58,98 @@ constexpr int THREADS = 512;
 constexpr int SMEM_BYTES = 3 * 256 * ROW_BYTES;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// Buffer addressing: a 128-bit resource (uniform base, no range check: every offset is valid by construction) plus a
+// 32-bit per-lane byte offset, so a load costs no 64-bit address arithmetic in the vector unit.  The host pass of the
+// compiler knows these builtins but not the target features they need, and silently drops a whole kernel, launch
+// stub included, that calls one: the calls are for the device pass only.
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t mnb_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, -1, 0x00020000);
+}
+__device__ __forceinline__ u2_t mnb_buffer_load_b64(rsrc_t r, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+}
+__device__ __forceinline__ uint32_t mnb_buffer_load_b32(rsrc_t r, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, (int)off, 0, 0);
+}
+// 16 bytes per lane from the buffer straight into LDS: lane L's bytes land at `lds` (uniform) + 16 L.
+__device__ __forceinline__ void mnb_buffer_load_lds_b128(rsrc_t r, uint32_t off, lds_ptr_t lds) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, lds, 16, (int)off, 0, 0, 0);
+}
+#else
+struct rsrc_t {};
+inline rsrc_t mnb_rsrc(const void*) { return {}; }
+inline u2_t mnb_buffer_load_b64(rsrc_t, uint32_t) { return u2_t{0, 0}; }
+inline uint32_t mnb_buffer_load_b32(rsrc_t, uint32_t) { return 0; }
+inline void mnb_buffer_load_lds_b128(rsrc_t, uint32_t, lds_ptr_t) {}
+#endif
+
 // s_waitcnt immediate that waits until at most VM vector-memory operations are outstanding and every LDS operation
 // of the wavefront has completed (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14).
 constexpr int waitcnt_vm_lds0(int vm) { return (vm & 15) | (7 << 4) | (0 << 8) | ((vm >> 4) << 14); }
-// cost of a k-step of the 128-row tile relative to the 256-row one (measured)
-constexpr double kMnbGemm128StepRatio = 0.88;
+// The same for vector-memory operations only (LDS and scalar-memory counters untouched).
+constexpr int waitcnt_vm(int vm) { return (vm & 15) | (7 << 4) | (15 << 8) | ((vm >> 4) << 14); }
+
+// Order in which a wavefront issues its vector-memory operations in a k-step of the tile GEMM, and what each wait
+// of the step may leave outstanding.  The k-loop states its waits itself (the one in front of the barrier has to: the
+// compiler does not know that other wavefronts read what this one's loads put into LDS; the others pin the weights'
+// two k-steps of latency whatever the scheduler does with the loads).  They are exact as long as the issue order
+// below is the one in the generated code; tests/test_isa_tile_gemm.py checks that, and that the compiler saw no need
+// to add a wait of its own.
+//   slot 0: the A loads into LDS for step s+2 (first thing in slab 0)
+//   slot q = 1, 2, 3: the weight registers last read when the operands of slab q were made (that happens in the
+//           section of slab q-1; the reload follows at once), for step s+2
+//   slot 4: those last read when the operands of slab 0 of step s+1 were made (behind the barrier), for step s+3
+// 4-bit: a vector serves two slabs and has a meta entry of its own; 8-bit: one vector per slab, a meta entry serves
+// 4 / MPS slabs.  A register is reloaded right after its last use, so every datum has about two k-steps to arrive.
+template <int KK>
+struct Slab {
+  static constexpr int value = KK;
+};
+
+template <int BITS, int MPS, int A_LOADS>
+struct LoadPlan {
+  static constexpr int VPS = (BITS == 4) ? 2 : 4;
+  static constexpr int slot_after(int kk) { return kk == 0 ? 4 : kk; }  // slot that follows make_b(kk)
+  static constexpr int vec_of_slab(int kk) { return BITS == 4 ? kk >> 1 : kk; }
+  static constexpr int meta_of_slab(int kk) { return BITS == 4 ? kk >> 1 : kk * MPS / 4; }
+  static constexpr int vec_slot(int v) { return slot_after(BITS == 4 ? 2 * v + 1 : v); }
+  static constexpr int meta_slot(int e) { return slot_after(BITS == 4 ? 2 * e + 1 : (e + 1) * 4 / MPS - 1); }
+  static constexpr int size(int q) {
+    if (q == 0) return A_LOADS;
+    int n = 0;
+    for (int v = 0; v < VPS; ++v) n += vec_slot(v) == q ? 2 : 0;
+    for (int e = 0; e < MPS; ++e) n += meta_slot(e) == q ? 2 : 0;
+    return n;
+  }
+  static constexpr int before(int q) {  // operations of a step in front of slot q
+    int n = 0;
+    for (int i = 0; i < q; ++i) n += size(i);
+    return n;
+  }
+  static constexpr int per_step() { return before(5); }
+  // operations younger than the group of slot q issued `steps` k-steps earlier, seen from in front of slot q_now
+  static constexpr int younger(int q, int steps, int q_now) {
+    return steps * per_step() + before(q_now) - before(q) - size(q);
+  }
+  // what the wait in front of make_b(kk) may leave outstanding.  The data of step u sit in slots 1..3 of step u-2 or
+  // in slot 4 of step u-3; make_b(0) prepares step s+1 during step s, the others step s.
+  static constexpr int wait_of_slab(int kk) {
+    const int ahead = kk == 0 ? 1 : 0, q_now = slot_after(kk);
+    const int qv = vec_slot(vec_of_slab(kk)), qm = meta_slot(meta_of_slab(kk));
+    const int yv = younger(qv, (qv == 4 ? 3 : 2) - ahead, q_now);
+    const int ym = younger(qm, (qm == 4 ? 3 : 2) - ahead, q_now);
+    return yv < ym ? yv : ym;
+  }
+  // the barrier of step s: A of step s+1 (slot 0 of step s-1) has landed, and slab 0's weights of step s+1 are there
+  static constexpr int wait_of_barrier() {
+    const int ya = younger(0, 1, 4), yb = wait_of_slab(0);
+    return ya < yb ? ya : yb;
+  }
+  // a slab whose weights the previous slab's wait has already covered needs none
+  static constexpr bool slab_waits(int kk) { return !(BITS == 4 && (kk & 1)); }
+};
 
 struct Gemm256Params {
   const _Float16* A;
@@ -161,10 +249,8 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 16-byte activation loads per thread per k-step: TM
   // 4-bit: a 16-byte vector spans two slabs (one word each per lane); 8-bit: one slab (two words per lane)
   constexpr int VEC_PER_STEP = (BITS == 4) ? 2 : 4;  // 8-byte weight loads per lane, column tile and k-step
-  constexpr int GK = 128 / BITS;
   constexpr int ACC_PAIRS = TM * 2 * 8;              // 8-byte pairs of accumulators per lane
-  // vector-memory operations a wavefront issues per k-step for the weights (vectors and meta entries)
-  constexpr int B_LOADS = VEC_PER_STEP * 2 + MPS * 2;
+  using Plan = LoadPlan<BITS, MPS, A_LOADS>;
   extern __shared__ __align__(16) unsigned char lds_bytes[];
   _Float16* const lds = reinterpret_cast<_Float16*>(lds_bytes);
 
@@ -179,7 +265,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // Two register sets for the weight prefetch (distance: two k-steps); the activations need none.
   struct Stage {
     u2_t b[VEC_PER_STEP][2];      // [vector of the k-step][column tile]
-    uint32_t m[MPS][2];           // meta entries of the blocks of the k-step
+    uint32_t m[MPS][2];           // meta entries of the blocks of the k-step (see m_off)
   };
   Stage R0, R1;
   h8_t FA0[TM], FA1[TM];  // A operands, double buffered over slabs
@@ -187,8 +273,10 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 
   const UnpackConsts uc = make_unpack_consts();
 
-  // Addressing: every global access is  uniform base (SGPRs: the tile's corner, advanced per k-step)  +  32-bit
-  // per-lane offset (a VGPR), so the loads cost no VALU work inside the loop.  The tile's first row and column are
+  // Addressing: every global access is a buffer access:  uniform base (a resource in SGPRs: the tile's corner,
+  // advanced per k-step)  +  32-bit per-lane offset (a VGPR), so the loads cost no VALU work inside the loop.  (The
+  // flat form of the load into LDS is also what makes the compiler wait for all outstanding loads wherever it needs
+  // one of them; with the buffer form its waits are exact.)  The tile's first row and column are
   // part of the uniform base, so a lane's offsets span at most 255 rows of A and 256 columns of weights: they fit
   // 32 bits for every M and N as long as 512 * lda does (mnb_gemm256_addressable).
   // Load i of a wavefront fills rows i * 64 + wave * 8 + [0, 8) of the staged tile; the lane at chunk position
@@ -199,12 +287,17 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // The block of a lane's half vector is (k-group base >> bs_shift), plus kq when 4-bit blocks are 16 wide.
   constexpr int META_BYTES = HAS_ZP ? 4 : 2;
   const bool small_bs = (BITS == 4) && p.bs_shift == 4;
-  uint32_t w_off[2], m_off[2];
+  // Without zero points an entry is a 16-bit scale.  A 16-bit load would be zero-extended, or packed with its
+  // neighbour, right behind the load, which needs the data at once and defeats the prefetch: the lane loads the
+  // aligned 32-bit word that holds its scale and shifts by m_shift (0 or 16) when it uses it.
+  uint32_t w_off[2], m_off[2], m_shift[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int col = wn * 64 + j * 32 + li;  // within the tile; tiles start at multiples of 256 columns
     w_off[j] = (uint32_t)(col * 16 + kq * 8);
-    m_off[j] = (uint32_t)((mnb_meta_col(col) + (small_bs ? kq * p.Npad : 0)) * META_BYTES);
+    const uint32_t m_byte = (uint32_t)((mnb_meta_col(col) + (small_bs ? kq * p.Npad : 0)) * META_BYTES);
+    m_off[j] = m_byte & ~3u;
+    m_shift[j] = (m_byte & 2u) * 8;
   }
   const int last_step = p.ksteps - 1;
   const int64_t vec_pitch = p.Npad * 16;               // bytes between consecutive k-groups
@@ -219,49 +312,56 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // k-steps past the end are clamped to the last one: the loop body stays branch free, the data is never used
   auto load_a = [&](int ks_raw, int stage_off) {
     const int ks = ks_raw < last_step ? ks_raw : last_step;
-    const uint8_t* base = reinterpret_cast<const uint8_t*>(a_tile + (int64_t)ks * BK);
-    // (The host pass of the compiler knows the builtin but not the target feature it needs, and silently drops the
-    // whole kernel, launch stub included, if it meets the call: the call is for the device pass only.)
+    const rsrc_t r = mnb_rsrc(a_tile + (int64_t)ks * BK);
 #pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-#if defined(__HIP_DEVICE_COMPILE__)
-      __builtin_amdgcn_global_load_lds(base + a_off[i],
-                                       (lds_ptr_t)(lds_bytes + stage_off + (i * 64 + wave * 8) * ROW_BYTES), 16, 0, 0);
-#else
-      (void)base;
-      (void)stage_off;
-#endif
-    }
+    for (int i = 0; i < A_LOADS; ++i)
+      mnb_buffer_load_lds_b128(r, a_off[i], (lds_ptr_t)(lds_bytes + stage_off + (i * 64 + wave * 8) * ROW_BYTES));
   };
-  auto load_b = [&](int ks_raw, Stage& R) {
+  // One issue group of the weight prefetch: the loads of issue slot `slot` (see LoadPlan) for k-step ks_raw.
+  auto load_b_slot = [&](int ks_raw, Stage& R, int slot) {
     const int ks = ks_raw < last_step ? ks_raw : last_step;
 #pragma unroll
     for (int v = 0; v < VEC_PER_STEP; ++v) {
+      if (Plan::vec_slot(v) != slot) continue;
       const int64_t kg = (int64_t)ks * VEC_PER_STEP + v;  // k-group of the vector
-      const int64_t kb = (kg * GK) >> p.bs_shift;         // block of the vector's first element
-      const uint8_t* wbase = w_tile + kg * vec_pitch;
-      const uint8_t* mbase = meta_tile + kb * meta_pitch;
-      constexpr int VEC_PER_META = VEC_PER_STEP / MPS;
+      const rsrc_t r = mnb_rsrc(w_tile + kg * vec_pitch);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        R.b[v][j] = *reinterpret_cast<const u2_t*>(wbase + w_off[j]);
-        if (v % VEC_PER_META == 0) {
-          if constexpr (HAS_ZP)
-            R.m[v / VEC_PER_META][j] = *reinterpret_cast<const uint32_t*>(mbase + m_off[j]);
-          else
-            R.m[v / VEC_PER_META][j] = *reinterpret_cast<const uint16_t*>(mbase + m_off[j]);
-        }
-      }
+      for (int j = 0; j < 2; ++j) R.b[v][j] = mnb_buffer_load_b64(r, w_off[j]);
+    }
+#pragma unroll
+    for (int e = 0; e < MPS; ++e) {
+      if (Plan::meta_slot(e) != slot) continue;
+      const int64_t kb = ((int64_t)ks * BK + e * (BK / MPS)) >> p.bs_shift;  // block of the entry's first element
+      const rsrc_t r = mnb_rsrc(meta_tile + kb * meta_pitch);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) R.m[e][j] = mnb_buffer_load_b32(r, m_off[j]);
+    }
+  };
+  auto load_b = [&](int ks_raw, Stage& R) {
+#pragma unroll
+    for (int slot = 1; slot <= 4; ++slot) load_b_slot(ks_raw, R, slot);
+  };
+  // Waits until the weights that slab kk of a k-step needs have arrived (`vm`: the number of younger vector-memory
+  // operations, from LoadPlan), and ties the registers to the wait: no use of them can be scheduled in front of it.
+  auto await_b = [&](auto slab, Stage& R) {
+    constexpr int kk = decltype(slab)::value;
+    constexpr int vm = kk == 0 ? Plan::wait_of_barrier() : Plan::wait_of_slab(kk);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(vm));
+    constexpr int v = Plan::vec_of_slab(kk), e = Plan::meta_of_slab(kk);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      asm volatile("; b %0" : "+v"(R.b[v][j]));
+      asm volatile("; m %0" : "+v"(R.m[e][j]));
     }
   };
 
-  auto decode = [&](uint32_t raw, h2_t& s2, ZpH& z) {
+  auto decode = [&](uint32_t raw, int j, h2_t& s2, ZpH& z) {
     if constexpr (HAS_ZP) {
       const h2_t m = mnb_as_h2(raw);
       s2 = mnb_h2(m.x);
       z = mnb_zp_h(m.y);
     } else {
-      s2 = mnb_h2(__builtin_bit_cast(_Float16, (uint16_t)raw));
+      s2 = mnb_h2(__builtin_bit_cast(_Float16, (uint16_t)(raw >> m_shift[j])));
       z = mnb_zp_h((_Float16)(-(1024.0f + (float)(1 << (BITS - 1)))));
     }
   };
@@ -274,10 +374,10 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       ZpH z;
       if constexpr (BITS == 4) {
         const int v = kk >> 1;
-        decode(R.m[v][j], s2, z);
+        decode(R.m[v][j], j, s2, z);
         FB[j] = dequant_word<4>(R.b[v][j][kk & 1], 0u, uc, z, s2);
       } else {
-        decode(R.m[kk * MPS / 4][j], s2, z);
+        decode(R.m[kk * MPS / 4][j], j, s2, z);
         FB[j] = dequant_word<8>(R.b[kk][j][0], R.b[kk][j][1], uc, z, s2);
       }
     }
@@ -312,35 +412,43 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     // slab 0: operands of slab 1; A of step ks+2 on its way into the free tile
     load_a(ks + 2, nn);
     read_a(cur, 1, FA1);
+    if constexpr (Plan::slab_waits(1)) await_b(Slab<1>{}, Rc);
     make_b(1, Rc, FB1);
     mfma_slab(FA0, FB0);
-    slab_pipeline<NM, TM, TM / 2, VALU_PER_MFMA, 0>();
+    load_b_slot(ks + 2, Rc, 1);
+    slab_pipeline<NM, TM, (A_LOADS + Plan::size(1) + 1) / 2, VALU_PER_MFMA, 0>();
     // slab 1: operands of slab 2
     read_a(cur, 2, FA0);
+    if constexpr (Plan::slab_waits(2)) await_b(Slab<2>{}, Rc);
     make_b(2, Rc, FB0);
     mfma_slab(FA1, FB1);
-    slab_pipeline<NM, TM, 0, VALU_PER_MFMA, 0>();
-    // slab 2: operands of slab 3; after that the weight registers of Rc are free: weights of step ks+2
+    load_b_slot(ks + 2, Rc, 2);
+    slab_pipeline<NM, TM, (Plan::size(2) + 1) / 2, VALU_PER_MFMA, 0>();
+    // slab 2: operands of slab 3
     read_a(cur, 3, FA1);
+    if constexpr (Plan::slab_waits(3)) await_b(Slab<3>{}, Rc);
     make_b(3, Rc, FB1);
     mfma_slab(FA0, FB0);
-    load_b(ks + 2, Rc);
-    slab_pipeline<NM, TM, 4, VALU_PER_MFMA, 0>();
+    load_b_slot(ks + 2, Rc, 3);
+    slab_pipeline<NM, TM, (Plan::size(3) + 1) / 2, VALU_PER_MFMA, 0>();
     // The barrier of the step.  Before it a wavefront makes sure that its own part of A of step ks+1 has landed in
-    // LDS: those loads are older than the weights fetched in slab 2 of step ks-1, and younger than those are exactly
-    // the A loads of slab 0 and the weight loads of slab 2 above, so "at most A_LOADS + B_LOADS outstanding" covers
-    // them (and nothing issued in this step).  Its LDS reads have completed too, so the tile at `cur` may be
-    // overwritten from the next step on.  No fence: the fence of __syncthreads would wait for every outstanding
-    // load, the weight prefetch included.
+    // LDS (issued in slab 0 of step ks-1) and that the weights of slab 0 of step ks+1 are there; LoadPlan counts the
+    // operations younger than both.  The wavefront's LDS reads have completed too, so the tile at `cur` may be
+    // overwritten from the next step on.  No fence: the fence of __syncthreads would wait for every outstanding load.
+    // Nothing may move across: a dequantisation step of slab 3 hoisted above the wait would need a wait of its own.
+    __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lds0(A_LOADS + B_LOADS));
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lds0(Plan::wait_of_barrier()));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
     // slab 3, behind the barrier: operands of slab 0 of step ks+1
     read_a(nxt, 0, FA0);
+    await_b(Slab<0>{}, Rn);
     make_b(0, Rn, FB0);
     mfma_slab(FA1, FB1);
-    slab_pipeline<NM, TM, 0, VALU_PER_MFMA, 0>();
+    load_b_slot(ks + 3, Rn, 4);
+    slab_pipeline<NM, TM, (Plan::size(4) + 1) / 2, VALU_PER_MFMA, 0>();
   };
 
   // ---- this workgroup's share of the units, walked from the top down
@@ -438,6 +546,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     __syncthreads();
     read_a(st0, 0, FA0);
     make_b(0, R0, FB0);
+    load_b_slot(ks_begin + 2, R0, 4);  // the loop's issue order from here on (LoadPlan)
 
     for (int ks = ks_begin; ks < ks_end; ks += 2) {  // parts begin and end at even k-steps
       k_step(ks, R0, R1, st0, st1, st2);
@@ -603,49 +712,87 @@ size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 // fewer, or at the kernel's step costs cheaper, rounds), the grid, whether tiles are split along K across workgroups
 // (only with a workspace, and only when the tiles leave at least half of the compute units idle), the workspace that
 // takes, and the estimated run time.  The kernel itself takes any division of the units into contiguous shares.
+// ---- the plan: tile height and split, from a cost model calibrated on the device
+// Measured behaviour (all shapes of M = 256 ... 4096, N = 4096 ... 28672, K = 4096 / 8192 / 14336, every tile height
+// and number of parts):
+//   * a workgroup that has its compute unit to itself on a chip at most half busy runs its k-steps at a fixed pace
+//     (kStepCycles), after a fixed start-up (kStartCycles: launch, prologue, epilogue);
+//   * the chip is power-limited: with more than half of the compute units busy every workgroup slows down, by
+//     kLoad[...] at 3/4, 7/8 and all of them (a full chip does 1.3 times the work of half a chip per second, not 2);
+//     kernels that are bound by the vector unit (8-bit weights, 128-row tiles) slow down less;
+//   * more workgroups than compute units run as rounds (128-row tiles share a compute unit in pairs, which costs
+//     what two rounds cost);
+//   * cutting the tiles into `parts` ranges of k costs kFixCycles[0] + parts * kFixCycles[1] for the finishing pass
+//     (the lower parts write their sums, the top part waits for them and adds them one after the other).
+// Times are in cycles of the device's nominal clock.  Variants: 4-bit; 8-bit; 8-bit with 16-wide blocks.
+namespace plan_model {
+struct Variant {
+  double start[2];    // [0]: 256-row tiles, [1]: 128-row tiles
+  double step[2];
+  double load[2][3];  // slow-down at 3/4, 7/8 and all compute units busy (1.0 up to half)
+  double full[2];     // slow-down of a full round when there are several
+};
+constexpr Variant kVariants[3] = {
+    {{16800, 15400}, {2850, 1860}, {{1.31, 1.43, 1.59}, {1.17, 1.28, 1.46}}, {1.59, 1.46}},
+    {{19200, 16800}, {2900, 2360}, {{1.28, 1.41, 1.58}, {1.06, 1.15, 1.24}}, {1.58, 1.35}},
+    {{19200, 16800}, {3820, 3460}, {{1.11, 1.20, 1.35}, {1.05, 1.10, 1.20}}, {1.35, 1.25}},
+};
+constexpr double kFixCycles[2][2] = {{6000, 9400}, {2200, 6700}};  // [tile height][constant, per part]
+
+inline double load_factor(const double (&at)[3], double busy) {  // busy: fraction of the compute units with a workgroup
+  if (busy <= 0.5) return 1.0;
+  if (busy <= 0.75) return 1.0 + (at[0] - 1.0) * (busy - 0.5) / 0.25;
+  if (busy <= 0.875) return at[0] + (at[1] - at[0]) * (busy - 0.75) / 0.125;
+  return at[1] + (at[2] - at[1]) * (busy > 1.0 ? 1.0 : (busy - 0.875) / 0.125);
+}
+
+// cycles for `grid` workgroups of `steps` k-steps each
+inline double cycles(const Variant& v, int h, int64_t grid, int64_t steps, int parts, int64_t cus) {
+  const double part = (double)steps * v.step[h] + (parts > 1 ? kFixCycles[h][0] + parts * kFixCycles[h][1] : 0.0);
+  const int64_t rounds = grid / cus, rest = grid % cus;
+  double t = v.start[h];
+  if (rounds > 0) t += (double)rounds * part * (rounds + (rest ? 1 : 0) > 1 ? v.full[h] : v.load[h][2]);
+  if (rest > 0) t += part * load_factor(v.load[h], (double)rest / (double)cus);
+  return t;
+}
+}  // namespace plan_model
+
 MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace) {
   const MnbDeviceInfo& dev = mnb_device_info();
   const int64_t tiles_n = (L.N + BN - 1) / BN;
   const int64_t ksteps = L.K / BK, upt = ksteps / 2;
-  // cycles of one 64-deep k-step of a 256-row tile with the whole chip busy (4-bit; 8-bit; 8-bit with 16-wide blocks,
-  // whose four meta entries per step spill): properties of the kernel's instruction schedule
-  const double cycles256 = L.bits == 4 ? 3480.0 : (L.bs >= 32 ? 3960.0 : 7080.0);
+  const plan_model::Variant& v = plan_model::kVariants[L.bits == 4 ? 0 : (L.bs >= 32 ? 1 : 2)];
   const int64_t cus = dev.cus;
   MnbGemm256Plan best{};
-  for (int rows = 256; rows >= 128; rows -= 128) {
-    const double step = cycles256 / dev.clock_hz * (rows == 256 ? 1.0 : kMnbGemm128StepRatio);
+  for (int h = 0; h < 2; ++h) {
+    const int rows = h == 0 ? 256 : 128;
     const int64_t tiles = ((M + rows - 1) / rows) * tiles_n;
-    MnbGemm256Plan pl{};
-    pl.tile_rows = rows;
-    pl.grid = tiles;
-    pl.seconds = (double)((tiles + cus - 1) / cus) * (double)ksteps * step;
-    if (with_workspace && tiles * 4 <= cus && M > 768) {
-      // Few tiles of a tall problem: every tile is cut into `parts` equal ranges of k (2 ... 4, each at least 32
-      // k-steps deep), one workgroup per part.  The finishing pass -- every lower part writes its sums, the top part
-      // waits for them and adds them one after the other -- costs about 8 us for two parts plus 8 us for each further
-      // one (256-row tiles), and a part its k-steps at about 1.15 of the steady-state step.  Measured on the
-      // Llama-3-8B projections (M = 1024, N = 4096): K = 4096 in two parts 49 us against 51 us on the streaming kernel
-      // and 59 us unsplit; K = 14336 in four parts 134 us against 141 us and 191 us; 8-bit weights 139 us against
-      // 151 us.  With a quarter of the compute units or more already busy the split loses (96 ... 128 tiles in two
-      // parts: 66 against 63 us, 80 against 76 us), and with whole rounds of tiles equal shares bring nothing either:
-      // the chip is power-limited there, a balanced schedule runs at a lower clock for the same total time
-      // (M = 2048, N = 14336: 223 us of arithmetic in equal shares against 225 us in two unequal rounds, plus the
-      // finishing pass).
-      int64_t parts = cus / tiles < 4 ? cus / tiles : 4;
-      while (parts > 1 && (upt % parts != 0 || ksteps / parts < 32)) --parts;
-      if (parts > 1) {
-        const double pass = rows == 256 ? 8e-6 : 4e-6;
-        const double t = (double)(ksteps / parts) * step * 1.15 + pass * (double)(parts - 1);
-        if (t < pl.seconds) {
-          pl.seconds = t;
-          pl.grid = tiles * parts;
-          pl.split = true;
-          pl.workspace_bytes =
-              round256((size_t)pl.grid * 8 * sizeof(uint32_t)) + (size_t)pl.grid * rows * BN * sizeof(float);
-        }
-      }
+    for (int parts = 1; parts <= 8; ++parts) {
+      // parts are whole units (two k-steps) of at least 16 k-steps, and never more than two rounds of workgroups:
+      // a part waits for the parts below it, which must not sit in a later round than the model assumes
+      if (upt % parts != 0 || (parts > 1 && (!with_workspace || ksteps / parts < 16 || tiles * parts > 2 * cus))) continue;
+      MnbGemm256Plan pl{};
+      pl.tile_rows = rows;
+      pl.grid = tiles * parts;
+      pl.split = parts > 1;
+      pl.seconds = plan_model::cycles(v, h, pl.grid, ksteps / parts, parts, cus) / dev.clock_hz;
+      if (pl.split)
+        pl.workspace_bytes = round256((size_t)pl.grid * 8 * sizeof(uint32_t)) + (size_t)pl.grid * rows * BN * sizeof(float);
+      if (best.grid == 0 || pl.seconds < best.seconds) best = pl;
     }
-    if (rows == 256 || pl.seconds < best.seconds) best = pl;
+  }
+  if (const char* e = mnb_tuning_env("MNB_GEMM256_PLAN")) {  // calibration: "<tile rows>,<parts>"
+    int rows = 0, parts = 0;
+    if (sscanf(e, "%d,%d", &rows, &parts) == 2 && (rows == 128 || rows == 256) && parts >= 1 && parts <= 8 &&
+        upt % parts == 0 && (parts == 1 || with_workspace)) {
+      const int64_t tiles = ((M + rows - 1) / rows) * tiles_n;
+      best = MnbGemm256Plan{};
+      best.tile_rows = rows;
+      best.grid = tiles * parts;
+      best.split = parts > 1;
+      best.workspace_bytes =
+          parts > 1 ? round256((size_t)best.grid * 8 * sizeof(uint32_t)) + (size_t)best.grid * rows * BN * sizeof(float) : 0;
+    }
   }
   return best;
 }
@@ -657,7 +804,7 @@ MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspa
 uint64_t mnb_gemm256_max_lane_offset(int64_t lda) { return ((uint64_t)255 * (uint64_t)lda + 7 * 8 + 7) * 2 + 1; }
 
 bool mnb_gemm256_addressable(int64_t lda, int64_t Npad) {
-  return mnb_gemm256_max_lane_offset(lda) < ((uint64_t)1 << 32) && (uint64_t)Npad * 16 + 16 <= ((uint64_t)1 << 32);
+  return mnb_gemm256_max_lane_offset(lda) < ((uint64_t)1 << 32) - 1 && (uint64_t)Npad * 16 + 16 <= ((uint64_t)1 << 32);
 }
 
 // The fused outputs are written with 16-byte stores of 8 columns: every output 16-byte aligned, with a pitch and a

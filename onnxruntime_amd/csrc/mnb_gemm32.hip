@@ -201,7 +201,7 @@ hipError_t launch(const Gemm32Params& p, int64_t row_tiles, int tm, hipStream_t 
 
 bool mnb_gemm32_applicable(const MnbGemmArgs& a) {
   static const bool disabled = [] {
-    const char* e = getenv("MNB_GEMM32");  // tuning override: "0" sends fp32 problems to the VALU tile kernel
+    const char* e = mnb_tuning_env("MNB_GEMM32");  // tuning override: "0" sends fp32 problems to the VALU tile kernel
     return e != nullptr && e[0] == '0';
   }();
   return !disabled && a.L.dtype == kMnbDtypeFloat && a.M > 16;

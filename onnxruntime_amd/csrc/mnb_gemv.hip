@@ -31,6 +31,27 @@ struct GemvParams {
   int KG;      // k-groups that hold elements below K
 };
 
+// What a wavefront needs to issue its first loads comes as leading scalar kernel arguments, which the build asks the
+// compiler to have preloaded into SGPRs at wavefront start (no scalar load in front of the first weight load); the
+// parameter block carries the rest and is fetched where it is used.
+#define MNB_GEMV_HOT_PARAMS                                                                                    \
+  const uint4 *hot_W, int64_t hot_Npad, const void *hot_A, int64_t hot_lda, const uint8_t *hot_meta, int hot_M, \
+      int hot_KG, int hot_bs_shift
+#define MNB_GEMV_HOT_ARGS(p) (p).W, (p).Npad, (p).A, (p).lda, (p).meta, (p).M, (p).KG, (p).bs_shift
+#define MNB_GEMV_HOT_NAMES hot_W, hot_Npad, hot_A, hot_lda, hot_meta, hot_M, hot_KG, hot_bs_shift
+
+__device__ __forceinline__ GemvParams with_hot_params(GemvParams p, MNB_GEMV_HOT_PARAMS) {
+  p.W = hot_W;
+  p.Npad = hot_Npad;
+  p.A = hot_A;
+  p.lda = hot_lda;
+  p.meta = hot_meta;
+  p.M = hot_M;
+  p.KG = hot_KG;
+  p.bs_shift = hot_bs_shift;
+  return p;
+}
+
 template <typename T>
 __device__ __forceinline__ float mnb_to_float(T v) {
   return (float)v;
@@ -102,7 +123,8 @@ __device__ __forceinline__ void mnb_gemv_group(const uint4& wv, const uint8_t* _
 // Requirements checked by the host: K % GK == 0, A 16-byte aligned with a 16-byte aligned row pitch.
 // Rows [M, MT) of the register tile re-read row M-1 and are never stored.
 template <typename T, int BITS, bool HAS_ZP, bool SMALL_BS, int MT, int NW, int U>
-__global__ void __launch_bounds__(NW * 64) mnb_gemv_kernel(GemvParams p) {
+__global__ void __launch_bounds__(NW * 64) mnb_gemv_kernel(MNB_GEMV_HOT_PARAMS, GemvParams rest) {
+  const GemvParams p = with_hot_params(rest, MNB_GEMV_HOT_NAMES);
   constexpr int GK = 128 / BITS;
   __shared__ float red[NW * MT * 64];
 
@@ -177,7 +199,8 @@ constexpr int kG16Pad = 4;         // floats of padding per staged k-group
 constexpr int kG16PhaseK = 2048;   // k staged at a time (x MT rows x 4 B <= 36 KiB)
 
 template <int BITS, bool HAS_ZP, bool SMALL_BS, int MT, int NW>
-__global__ void __launch_bounds__(NW * 64) mnb_gemv16_kernel(GemvParams p) {
+__global__ void __launch_bounds__(NW * 64) mnb_gemv16_kernel(MNB_GEMV_HOT_PARAMS, GemvParams rest) {
+  const GemvParams p = with_hot_params(rest, MNB_GEMV_HOT_NAMES);
   constexpr int GK = 128 / BITS;                // k per 16-byte vector
   constexpr int GS = GK + kG16Pad;              // staged floats per k-group
   constexpr int PH_GROUPS = kG16PhaseK / GK;    // k-groups per phase
@@ -387,7 +410,7 @@ bool gemv_fast_ok(const MnbGemmArgs& a) {
 template <typename T, int BITS, bool HAS_ZP, bool SMALL_BS, int MT, int NW>
 hipError_t launch_gemv_nw(const GemvParams& p, int64_t col_groups, hipStream_t s) {
   dim3 grid((unsigned)col_groups), blk(NW * 64);
-  mnb_gemv_kernel<T, BITS, HAS_ZP, SMALL_BS, MT, NW, kGemvU><<<grid, blk, 0, s>>>(p);
+  mnb_gemv_kernel<T, BITS, HAS_ZP, SMALL_BS, MT, NW, kGemvU><<<grid, blk, 0, s>>>(MNB_GEMV_HOT_ARGS(p), p);
   return hipGetLastError();
 }
 
@@ -435,9 +458,9 @@ hipError_t launch_gemv16_nw(const GemvParams& p, hipStream_t s) {
   dim3 grid((unsigned)((p.N + 15) / 16));
   const int chunks = (p.KG + 3) / 4;
   if (chunks >= 32) {
-    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 8><<<grid, dim3(512), 0, s>>>(p);
+    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 8><<<grid, dim3(512), 0, s>>>(MNB_GEMV_HOT_ARGS(p), p);
   } else {
-    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 4><<<grid, dim3(256), 0, s>>>(p);
+    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 4><<<grid, dim3(256), 0, s>>>(MNB_GEMV_HOT_ARGS(p), p);
   }
   return hipGetLastError();
 }

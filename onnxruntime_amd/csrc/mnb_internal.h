@@ -1,5 +1,6 @@
 // Launchers implemented in the .hip translation units; called by the C ABI in mnb_api.hip.
 #pragma once
+#include <cstdlib>
 #include <hip/hip_runtime.h>
 
 #include "mnb_layout.h"
@@ -64,6 +65,14 @@ bool mnb_gemv_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_gemv(const MnbGemmArgs& a, hipStream_t s);
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s);
 // compute units and engine clock (Hz) of the current device; asked once per device (mnb_api.hip)
+// Environment overrides of the launch planners exist only in builds made with -DMNB_TUNING_HOOKS (calibration runs);
+// the shipped library reads no environment variable: mnb_tuning_env returns nullptr there.
+#if defined(MNB_TUNING_HOOKS)
+inline const char* mnb_tuning_env(const char* name) { return getenv(name); }
+#else
+inline const char* mnb_tuning_env(const char*) { return nullptr; }
+#endif
+
 struct MnbDeviceInfo {
   int cus;
   double clock_hz;

@@ -120,8 +120,20 @@ __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h
   }
 }
 
+// What a wavefront needs to issue its first loads comes as leading scalar kernel arguments, which the build asks the
+// compiler to have preloaded into SGPRs at wavefront start; the parameter block carries the rest.
 template <int BITS, bool HAS_ZP, int T, int MT, int NW>
-__global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(MidParams mp) {
+__global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, int64_t hot_Npad, const uint4* hot_As,
+                                                          const uint8_t* hot_meta, int hot_row_tiles, int hot_chunks,
+                                                          int hot_bs_shift, MidParams rest) {
+  MidParams mp = rest;
+  mp.s.W = hot_W;
+  mp.s.Npad = hot_Npad;
+  mp.As = hot_As;
+  mp.s.meta = hot_meta;
+  mp.row_tiles = hot_row_tiles;
+  mp.s.chunks = hot_chunks;
+  mp.s.bs_shift = hot_bs_shift;
   const SkinnyParams& p = mp.s;
   constexpr int GK = 128 / BITS;
   constexpr int NI = GK / 8;
@@ -224,7 +236,7 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   // eight wavefronts split K further and hide more latency in a single round of workgroups; with several rounds of
   // the largest tile, two workgroups of four wavefronts share a CU instead
   pl.nw = chunks < 16 || (best_area == 16 && best_wgs >= 384) ? 4 : 8;
-  static const char* const plan_override = getenv("MNB_MID_PLAN");  // tuning override "<T>,<MT>,<NW>", read once
+  static const char* const plan_override = mnb_tuning_env("MNB_MID_PLAN");  // tuning override "<T>,<MT>,<NW>", read once
   if (const char* e = plan_override) {
     int t = 0, mt = 0, nw = 0;
     if (sscanf(e, "%d,%d,%d", &t, &mt, &nw) == 3 && (t == 1 || t == 2 || t == 4) && (mt == 2 || mt == 4) &&
@@ -244,9 +256,11 @@ hipError_t launch_nw(const MidParams& mp, const MidPlan& pl, hipStream_t s) {
   dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)));
   const size_t smem = (size_t)pl.nw * T * 4 * 64 * sizeof(float);
   if (pl.nw == 8)
-    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8><<<grid, dim3(512), smem, s>>>(mp);
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8><<<grid, dim3(512), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
+                                                                        p.chunks, p.bs_shift, mp);
   else
-    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4><<<grid, dim3(256), smem, s>>>(mp);
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4><<<grid, dim3(256), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
+                                                                        p.chunks, p.bs_shift, mp);
   return hipGetLastError();
 }
 

@@ -443,7 +443,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   pl.t = tiles >= 800 ? 4 : tiles >= 320 ? 2 : 1;  // measured: N = 6144 prefers 2 (192 workgroups), N = 4096 prefers 1
   // wavefronts per workgroup: aim for >= 2 chunks per wavefront
   pl.nw = chunks >= 32 ? 16 : chunks >= 16 ? 8 : 4;
-  static const char* const plan_override = getenv("MNB_SKINNY_PLAN");  // tuning override "<T>,<NW>", read once
+  static const char* const plan_override = mnb_tuning_env("MNB_SKINNY_PLAN");  // tuning override "<T>,<NW>", read once
   if (const char* e = plan_override) {
     int t = 0, nw = 0;
     if (sscanf(e, "%d,%d", &t, &nw) == 2 && (t == 1 || t == 2 || t == 4) && (nw == 4 || nw == 8 || nw == 16)) {
@@ -458,7 +458,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   // M = 8 the wider slabs gain or lose a few per cent either way; at M = 16 everything gains 10-35 % except the
   // general loop of four-tile slabs).  The general loop needs one more operand set for it, which sixteen wavefronts
   // of 4-bit weights cannot hold in their 128 registers: those run with eight (K = 14336, M = 16: 20 -> 13 us).
-  static const int a_lds_from = getenv("MNB_SKINNY_ALDS_FROM") ? atoi(getenv("MNB_SKINNY_ALDS_FROM")) : 5;
+  static const int a_lds_from = mnb_tuning_env("MNB_SKINNY_ALDS_FROM") ? atoi(mnb_tuning_env("MNB_SKINNY_ALDS_FROM")) : 5;
   const bool up_front = chunks == pl.nw || chunks == 2 * pl.nw;  // everything loaded before the first wait
   pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4);
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;

@@ -34,9 +34,9 @@ def _gemm(case, op, a, bias, with_workspace):
     return y, need
 
 
-# M, N, K, bits, block size: two parts (K = 4096), four parts (K = 8192, 14336), ragged M / N, 8-bit weights
-SHAPES = [(1024, 4096, 4096, 4, 128), (1000, 4000, 8192, 4, 32), (1024, 2048, 8192, 4, 64), (1024, 4096, 14336, 4, 128),
-          (1024, 4096, 8192, 8, 64), (1000, 4090, 14336, 8, 32)]
+# M, N, K, bits, block size: two and four parts, 128- and 256-row tiles, ragged M / N, 8-bit weights
+SHAPES = [(1024, 4096, 4096, 8, 64), (1000, 4000, 8192, 4, 32), (512, 8192, 8192, 4, 64), (1024, 4096, 14336, 4, 128),
+          (1024, 4096, 8192, 8, 64), (1000, 4090, 14336, 8, 32), (1536, 4096, 8192, 4, 128)]
 
 
 @pytest.mark.parametrize("M,N,K,bits,bs", SHAPES)
@@ -61,7 +61,7 @@ def test_split_matches_unsplit_and_oracle(oracle, M, N, K, bits, bs):
     assert np.linalg.norm(got - y64) / np.linalg.norm(y64) <= FP16_GATE
 
 
-@pytest.mark.parametrize("M,N,K,bits,bs", [(1024, 4096, 4096, 4, 128), (1024, 4096, 8192, 8, 64)])
+@pytest.mark.parametrize("M,N,K,bits,bs", [(1024, 4096, 8192, 4, 128), (1024, 4096, 8192, 8, 64)])
 def test_unit_vectors_come_back_exactly_through_the_split(oracle, M, N, K, bits, bs):
     """Row m of A is the unit vector e_k(m): every partial sum but one is zero, so Y[m] is column k(m) of the
     dequantised weights bit for bit, whichever part of the tile k(m) falls into."""
@@ -83,7 +83,7 @@ def test_unit_vectors_come_back_exactly_through_the_split(oracle, M, N, K, bits,
 def test_fused_gate_up_through_the_split(oracle):
     """MatMulNBitsMlp on a shape whose packed matrix (gate and up interleaved) takes the split: the epilogue that
     applies silu(gate) * up sees complete sums."""
-    M, N, K, bits, bs = 1024, 2048, 4096, 4, 32
+    M, N, K, bits, bs = 1024, 2048, 8192, 4, 32
     g = make_case(M, N, K, bits, bs, np.float16, has_bias=True, seed=5)
     u = make_case(M, N, K, bits, bs, np.float16, has_bias=True, seed=6)
     op = MatMulNBitsMlp(K, N, bits, bs, dtype=torch.float16)
