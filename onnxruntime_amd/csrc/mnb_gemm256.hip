@@ -8,8 +8,10 @@
 //   * A (activations) goes from global memory straight into LDS (buffer_load_dwordx4 ... lds: no registers, no LDS
 //     store instructions), two k-steps ahead, into one of three staged tiles.  Such a load puts the 16 bytes of lane
 //     L at (wave-uniform LDS base) + 16 L, so a wavefront fills 8 rows x 128 bytes with one instruction; the rows are
-//     not padded, instead the lane that fills chunk position p of row r fetches chunk p ^ (r & 7) of that row, and the
-//     readers (ds_read_b128, lane = row) apply the same XOR: conflict free.
+//     not padded, instead the lane that fills chunk position p of row r fetches chunk p ^ ((r >> 1) & 7) of that
+//     row, and the readers (ds_read_b128, lane = row) apply the same XOR.  The LDS serves such a read 16 lanes at a time from 64
+//     banks: 16 consecutive rows must start in 16 different 16-byte bank groups, and rows r, r+2, ... r+14 (same
+//     half of the 256 bytes that two rows span) get the 8 different chunk positions: conflict free.
 //   * B (weights) never touches LDS.  Lane (column j = lane%32, half kq = lane/32) of a wavefront loads, two steps
 //     ahead (each register is reloaded right after its last use, and the loop states its own exact waits: see
 //     LoadPlan), exactly the 8 bytes of packed weights it will feed to the matrix core: the two 32-bit words of its
@@ -280,8 +282,8 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // part of the uniform base, so a lane's offsets span at most 255 rows of A and 256 columns of weights: they fit
   // 32 bits for every M and N as long as 512 * lda does (mnb_gemm256_addressable).
   // Load i of a wavefront fills rows i * 64 + wave * 8 + [0, 8) of the staged tile; the lane at chunk position
-  // lane & 7 of row lane >> 3 fetches chunk (lane & 7) ^ (row & 7).
-  const int a_row = tid >> 3, a_kc = (tid & 7) ^ ((tid >> 3) & 7);
+  // lane & 7 of row lane >> 3 fetches chunk (lane & 7) ^ ((row >> 1) & 7).
+  const int a_row = tid >> 3, a_kc = (tid & 7) ^ ((tid >> 4) & 7);
   uint32_t a_off[A_LOADS];                     // byte offsets from a_tile + k0; set per tile (rows beyond M)
   // this lane's weight columns (one per column tile): its 8 bytes inside each 16-byte vector, and its meta entries.
   // The block of a lane's half vector is (k-group base >> bs_shift), plus kq when 4-bit blocks are 16 wide.
@@ -389,7 +391,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
     const int chunk = (BITS == 4) ? 4 * (kk >> 1) + 2 * kq + (kk & 1) : 2 * kk + kq;
-    a_rd[kk] = (uint32_t)((wm * 32 * TM + li) * ROW_BYTES + ((chunk ^ (li & 7)) * 16));
+    a_rd[kk] = (uint32_t)((wm * 32 * TM + li) * ROW_BYTES + ((chunk ^ ((li >> 1) & 7)) * 16));
   }
   auto read_a = [&](int stage_off, int kk, h8_t* FA) {
     const unsigned char* As = lds_bytes + stage_off + a_rd[kk];
