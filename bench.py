@@ -191,6 +191,8 @@ def main() -> int:
     ap.add_argument("--no-quantize", action="store_true", help="skip the blockwise quantiser (producer of the format)")
     ap.add_argument("--no-fused", action="store_true", help="skip the fused gate/up projection (MatMulNBitsMlp)")
     ap.add_argument("--no-sizes", action="store_true", help="skip the decode kernel on the larger gate+up matrices")
+    ap.add_argument("--no-int8", action="store_true",
+                    help="skip the int8-activation route (accuracy_level 4) beside the full-accuracy one")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -434,6 +436,32 @@ def main() -> int:
             del g5, p5
             torch.cuda.empty_cache()
         out["decode_sizes"] = rows
+
+    # ---- accuracy_level 4: int8 activations against the full-accuracy route on the same problems ----------------
+    if not args.no_int8:
+        rows = []
+        lib = _lib.load()
+        for label, M8, N8, K8, bs8 in (("configs[3] shape, block 32", 2048, 14336, 4096, 32),
+                                       ("configs[4] gate+up M=1024, block 128", 1024, 28672, 4096, 128),
+                                       ("the same with 256-wide blocks", 1024, 28672, 4096, 256)):
+            case = synthetic.make_case(M8, N8, K8, 4, bs8, np.float16, has_zp=True, seed=0)
+            p8 = Problem(case, 1, torch, _lib)
+            ms_full = time_steps(torch, p8.step, 20, 1, warm_ms=30.0)
+            need = lib.MnbGemmInt8WorkspaceSize(M8, N8, K8, 4, bs8, 1, _lib.DTYPE_FLOAT16)
+            ws8 = torch.empty(need, dtype=torch.uint8, device="cuda")
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+            def int8_step():
+                _lib.check(lib.MnbGemmInt8(M8, N8, K8, 4, bs8, 1, _lib.DTYPE_FLOAT16, _ptr(p8.a), K8, _ptr(p8.packed[0]),
+                                           None, _ptr(p8.y[0]), N8, _ptr(ws8), need, stream))
+            ms_int8 = time_steps(torch, int8_step, 20, 1, warm_ms=30.0)
+            rows.append({"workload": f"M={M8} K={K8} N={N8} int4 zero_points fp16, {label}",
+                         "full_accuracy_kernel": p8.kernel, "full_accuracy_ms": round(ms_full, 4),
+                         "int8_activations_ms": round(ms_int8, 4),
+                         "int8_over_full": round(ms_int8 / ms_full, 3)})
+            del p8, ws8
+            torch.cuda.empty_cache()
+        out["accuracy_level_4"] = rows
 
     # ---- the other configurations (not part of the JSON contract) ---------------------------------------------
     if args.sweep:

@@ -276,6 +276,22 @@ MNB_API int MnbVariantDequantize(float* dst_dev, const void* b_dev, const void* 
                                  const void* zero_points_dev, int zp_kind, const int32_t* g_idx_dev, size_t N,
                                  size_t K, int bits, int block_size, int a_dtype, void* stream);
 
+/* int8 activations (the reference's accuracy_level 4: SQ4BitGemm_CompInt8,
+ * onnxruntime/core/mlas/lib/qnbitgemm.cpp:883-1086, with the arithmetic of the scalar statement its kernels are
+ * tested against, onnxruntime/test/mlas/unittest/test_sqnbitgemm.cpp:94-170).  A is quantised per row and block of
+ * block_size elements (scale = max|a| / 127, round half away from zero), every block's dot product with the 4-bit
+ * weights is exact integer arithmetic, and Y = bias + sum over blocks of float(dot) * a_scale * b_scale in fp32,
+ * blocks in k order, narrowed once.  Same packed weights as MnbGemm.  Implemented for bits = 4, a_dtype float16 and
+ * block sizes 32 ... 256 (MNB_NOT_IMPLEMENTED otherwise).  accuracy_level is a permission, not a demand: MnbGemm
+ * computes the same nodes at full accuracy and is faster for every block size below 256, so nothing chooses this
+ * entry point by itself.  The workspace (16-byte aligned, MnbGemmInt8WorkspaceSize bytes, 0 = not implemented for
+ * these arguments) receives the quantised activations. */
+MNB_API size_t MnbGemmInt8WorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                                        int a_dtype);
+MNB_API int MnbGemmInt8(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                        const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev,
+                        size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* Name of the kernel MnbGemm would run for this problem (static string; for logs and profiles). */
 MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype);
 /* The same for activations with a row pitch of lda elements (MnbGemmKernelName assumes K rounded up to 8).  The tile

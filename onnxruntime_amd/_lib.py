@@ -92,6 +92,9 @@ SIGNATURES = {
                                c_size_t, c_void_p]),
     "MnbVariantDequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_size_t,
                                      c_int, c_int, c_int, c_void_p]),
+    "MnbGemmInt8WorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
+    "MnbGemmInt8": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
+                            c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
     "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
     "MnbGemmKernelNameStrided": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_size_t]),
 }

@@ -318,6 +318,49 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
                       c_dev, ldc, workspace_dev, workspace_bytes, stream);
 }
 
+size_t MnbGemmInt8WorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                                int a_dtype) {
+  if (check_config("MnbGemmInt8WorkspaceSize", bits, block_size, a_dtype) != MNB_OK || M == 0 || N == 0 || K == 0) return 0;
+  const MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  return mnb_gemm_i8_supported(L) ? mnb_gemm_i8_workspace_bytes(L, (int64_t)M) : 0;
+}
+
+int MnbGemmInt8(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev, size_t ldc,
+                void* workspace_dev, size_t workspace_bytes, void* stream) {
+  const char* fn = "MnbGemmInt8";
+  if (int rc = check_config(fn, bits, block_size, a_dtype)) return rc;
+  if (M == 0 || N == 0) return MNB_OK;
+  if (K == 0) return fail(MNB_INVALID_ARGUMENT, "%s: K must be positive", fn);
+  if (!a_dev || !packed_dev || !c_dev) return fail(MNB_INVALID_ARGUMENT, "%s: A, packed B and C must not be NULL", fn);
+  if (lda < K || ldc < N)
+    return fail(MNB_INVALID_ARGUMENT, "%s: lda (%zu) < K (%zu) or ldc (%zu) < N (%zu)", fn, lda, K, ldc, N);
+  if (M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff)
+    return fail(MNB_INVALID_ARGUMENT, "%s: M, N and K must fit in 31 bits", fn);
+  MnbGemmArgs a{};
+  a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  if (!mnb_gemm_i8_supported(a.L))
+    return fail(MNB_NOT_IMPLEMENTED,
+                "%s: int8 activations are implemented for 4-bit weights, float16 models and block sizes 32 to 256 "
+                "(got bits=%d, block_size=%d, a_dtype=%d); MnbGemm computes these at full accuracy",
+                fn, bits, block_size, a_dtype);
+  const size_t need = mnb_gemm_i8_workspace_bytes(a.L, (int64_t)M);
+  if (!workspace_dev || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0)
+    return fail(MNB_INVALID_ARGUMENT, "%s: a 16-byte aligned workspace of %zu bytes is needed (MnbGemmInt8WorkspaceSize), %zu given",
+                fn, need, workspace_dev ? workspace_bytes : (size_t)0);
+  a.M = (int64_t)M;
+  a.A = a_dev;
+  a.lda = (int64_t)lda;
+  a.packed = packed_dev;
+  a.bias = bias_dev;
+  a.C = c_dev;
+  a.ldc = (int64_t)ldc;
+  a.workspace = workspace_dev;
+  a.workspace_bytes = workspace_bytes;
+  const hipError_t e = mnb_launch_gemm_i8(a, (hipStream_t)stream);
+  return e == hipSuccess ? MNB_OK : hip_fail(e, fn);
+}
+
 }  // extern "C"
 
 // ---- the entry point that allocates nothing ---------------------------------------------------------------------------

@@ -56,7 +56,10 @@ class MatMulNBits:
 
     def __init__(self, K: int, N: int, bits: int = 4, block_size: int = 32, accuracy_level: int = 0,
                  dtype: torch.dtype = torch.float16, has_zero_points: bool = False, has_bias: bool = False,
-                 has_g_idx: bool = False, zero_points_dtype: torch.dtype = torch.uint8):
+                 has_g_idx: bool = False, zero_points_dtype: torch.dtype = torch.uint8,
+                 int8_activations: bool = False):
+        """``int8_activations``: take the permission that accuracy_level = 4 grants and quantise A blockwise to int8
+        (MnbGemmInt8) where that route exists; off by default, because the full-accuracy route is the faster one."""
         if bits not in (2, 4, 8):
             raise MnbError(_lib.INVALID_ARGUMENT, "Only 2b, 4b and 8b quantization is supported for MatMulNBits op, "
                                                   "additional bits support is planned.")
@@ -86,6 +89,7 @@ class MatMulNBits:
         self.packed: Optional[torch.Tensor] = None
         self.plan: Optional[_lib.MnbVariantPlan] = None
         self._workspace = {}
+        self.int8_activations = bool(int8_activations) and self.accuracy_level == 4 and not self.variant
 
     @property
     def zp_kind(self) -> int:
@@ -217,6 +221,15 @@ class MatMulNBits:
             _lib.check(self.lib.MnbVariantGemm(ctypes.byref(plan), M, _ptr(a2), lda, _ptr(packed), _ptr(bias),
                                                _ptr(y2), self.N, _ptr(ws), wsz, stream))
             return y
+        if self.packed is not None and self.int8_activations:
+            wsz = self.lib.MnbGemmInt8WorkspaceSize(M, self.N, self.K, self.bits, self.block_size,
+                                                    int(self.has_zero_points), dt)
+            if wsz:  # 0: no int8 route for this configuration, the full-accuracy one below takes it
+                ws = self._get_workspace(a.device, wsz)
+                _lib.check(self.lib.MnbGemmInt8(M, self.N, self.K, self.bits, self.block_size,
+                                                int(self.has_zero_points), dt, _ptr(a2), lda, _ptr(self.packed),
+                                                _ptr(bias), _ptr(y2), self.N, _ptr(ws), wsz, stream))
+                return y
         if self.packed is not None:
             wsz = self.lib.MnbGemmWorkspaceSize(M, self.N, self.K, self.bits, self.block_size,
                                                 int(self.has_zero_points), dt)

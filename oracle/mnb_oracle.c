@@ -2,8 +2,9 @@
  * TEST INFRASTRUCTURE ONLY -- CPU oracle for com.microsoft::MatMulNBits.
  *
  * A plain-C restatement of the reference's arithmetic contract for the op at
- * accuracy_level 0.  It is the checker used by tests/, __graft_entry__.smoke()
- * and the cpu_baseline leg of bench.py.  Nothing in the shipped library or the
+ * accuracy_level 0 (and, in a section of its own, of the int8-activation
+ * contract of accuracy_level 4).  It is the checker used by tests/,
+ * __graft_entry__.smoke() and the cpu_baseline leg of bench.py.  Nothing in the shipped library or the
  * Python host package may link, import or call it.
  *
  * What each function follows in the reference (onnxruntime 1.30.0):
@@ -307,6 +308,131 @@ void mnbo_matmul_f16(const uint16_t* A, const uint8_t* B, const uint16_t* scales
   mnbo_f16_to_f32_buffer(scales, s32, (size_t)(N * kbc));
   if (bias) mnbo_f16_to_f32_buffer(bias, b32, (size_t)N);
   mnbo_matmul_f32(a32, B, s32, zp, b32, y32, M, N, K, bits, bs, nthreads);
+  mnbo_f32_to_f16_buffer(y32, Y, (size_t)(M * N));
+  free(a32);
+  free(s32);
+  free(b32);
+  free(y32);
+}
+
+/* ------------------------------------------------------------------ int8 activations (accuracy_level 4)
+ *
+ * The reference's own scalar statement of the SQNBIT_CompInt8 contract, which its kernels are tested against
+ * (onnxruntime/test/mlas/unittest/test_sqnbitgemm.cpp:94-170, QuantizeA and CallReferenceGemm_CompInt8; the
+ * dispatcher is SQ4BitGemm_CompInt8, onnxruntime/core/mlas/lib/qnbitgemm.cpp:883-1086):
+ *   A, per row and block of bs elements along k (the weights' block size):
+ *       scale = max|a| / 127;  q = clamp(roundf(a * (scale != 0 ? 1 / scale : 0)), -128, 127)
+ *       (elements k >= K of the last block count as 0)
+ *   Y[m][n] = bias[n] (or 0);  for every block in k order:
+ *       qsum = sum_k qa * (qb - zp)           exact, int32
+ *       Y   += float(qsum) * a_scale * b_scale   evaluated left to right, every operation rounded to fp32
+ * 4-bit weights only (test_sqnbitgemm.cpp:160).  fp16 models widen A, scales and bias first and narrow Y once.
+ * Parity (tests/test_oracle_int8.py): the quantiser against hand-written integers on grids where the scale is a
+ * power of two (ties included: half away from zero); the product against numpy's exact int64 matmul where every
+ * scale is 1; against an independent numpy restatement that rounds to fp32 after every operation; against the
+ * accuracy_level-0 result within the analytic bound of the activation rounding, sum over blocks of
+ * (a_scale / 2) * sum |w|.
+ */
+void mnbo_quantize_a_int8(int8_t* qa, float* a_scale, const float* A, int64_t M, int64_t K, int64_t bs) {
+  int64_t kbc = k_blocks_of(K, bs);
+  for (int64_t m = 0; m < M; ++m) {
+    for (int64_t kb = 0; kb < kbc; ++kb) {
+      int64_t len = K - kb * bs < bs ? K - kb * bs : bs;
+      const float* a = A + m * K + kb * bs;
+      float amax = 0.0f;
+      for (int64_t r = 0; r < len; ++r) {
+        float v = fabsf(a[r]);
+        if (v > amax) amax = v;
+      }
+      const float scale = amax / 127.0f;
+      const float recip = scale != 0.0f ? 1.0f / scale : 0.0f;
+      a_scale[m * kbc + kb] = scale;
+      for (int64_t r = 0; r < bs; ++r) {
+        float q = r < len ? roundf(a[r] * recip) : 0.0f;
+        if (q < -128.0f) q = -128.0f;
+        if (q > 127.0f) q = 127.0f;
+        qa[(m * kbc + kb) * bs + r] = (int8_t)q;
+      }
+    }
+  }
+}
+
+typedef struct {
+  const int8_t* qa;
+  const float* a_scale;
+  const uint8_t* B;
+  const float* scales;
+  const uint8_t* zp;
+  const float* bias;
+  float* Y;
+  int64_t M, N, K, bs, n0, n1;
+} i8_job;
+
+static void* i8_worker(void* p) {
+  i8_job* j = (i8_job*)p;
+  int64_t kbc = k_blocks_of(j->K, j->bs);
+  for (int64_t m = 0; m < j->M; ++m) {
+    for (int64_t n = j->n0; n < j->n1; ++n) {
+      float sum = j->bias ? j->bias[n] : 0.0f;
+      for (int64_t kb = 0; kb < kbc; ++kb) {
+        int64_t len = j->K - kb * j->bs < j->bs ? j->K - kb * j->bs : j->bs;
+        const int z = zp_at(j->zp, n, kb, kbc, 4);
+        const int8_t* a = j->qa + (m * kbc + kb) * j->bs;
+        int32_t qsum = 0;
+        for (int64_t r = 0; r < len; ++r) qsum += (int32_t)a[r] * (q_at(j->B, n, kb * j->bs + r, kbc, j->bs, 4) - z);
+        float t = (float)qsum * j->a_scale[m * kbc + kb];
+        t = t * j->scales[n * kbc + kb];
+        sum = sum + t;
+      }
+      j->Y[m * j->N + n] = sum;
+    }
+  }
+  return NULL;
+}
+
+/* A fp32 [M][K]; 4-bit canonical B / scales / zero points; Y fp32 [M][N]. */
+void mnbo_matmul_int8_f32(const float* A, const uint8_t* B, const float* scales, const uint8_t* zp, const float* bias,
+                          float* Y, int64_t M, int64_t N, int64_t K, int64_t bs, int nthreads) {
+  int64_t kbc = k_blocks_of(K, bs);
+  int8_t* qa = (int8_t*)malloc((size_t)(M * kbc * bs));
+  float* as = (float*)malloc((size_t)(M * kbc) * sizeof(float));
+  mnbo_quantize_a_int8(qa, as, A, M, K, bs);
+  if (nthreads < 1) nthreads = 1;
+  if (nthreads > 256) nthreads = 256;
+  if ((int64_t)nthreads > N) nthreads = (int)(N > 0 ? N : 1);
+  pthread_t th[256];
+  i8_job jobs[256];
+  int64_t per = (N + nthreads - 1) / nthreads;
+  int started = 0;
+  for (int t = 0; t < nthreads; ++t) {
+    i8_job jb = {qa, as, B, scales, zp, bias, Y, M, N, K, bs, t * per, (t + 1) * per < N ? (t + 1) * per : N};
+    jobs[t] = jb;
+    if (jobs[t].n0 >= jobs[t].n1) break;
+    if (nthreads == 1) {
+      i8_worker(&jobs[t]);
+    } else {
+      pthread_create(&th[t], NULL, i8_worker, &jobs[t]);
+      ++started;
+    }
+  }
+  for (int t = 0; t < started; ++t) pthread_join(th[t], NULL);
+  free(qa);
+  free(as);
+}
+
+/* fp16 model: widen A, scales and bias, compute as above, narrow Y once (RNE). */
+void mnbo_matmul_int8_f16(const uint16_t* A, const uint8_t* B, const uint16_t* scales, const uint8_t* zp,
+                          const uint16_t* bias, uint16_t* Y, int64_t M, int64_t N, int64_t K, int64_t bs,
+                          int nthreads) {
+  int64_t kbc = k_blocks_of(K, bs);
+  float* a32 = (float*)malloc((size_t)(M * K) * sizeof(float));
+  float* s32 = (float*)malloc((size_t)(N * kbc) * sizeof(float));
+  float* b32 = bias ? (float*)malloc((size_t)N * sizeof(float)) : NULL;
+  float* y32 = (float*)malloc((size_t)(M * N) * sizeof(float));
+  mnbo_f16_to_f32_buffer(A, a32, (size_t)(M * K));
+  mnbo_f16_to_f32_buffer(scales, s32, (size_t)(N * kbc));
+  if (bias) mnbo_f16_to_f32_buffer(bias, b32, (size_t)N);
+  mnbo_matmul_int8_f32(a32, B, s32, zp, b32, y32, M, N, K, bs, nthreads);
   mnbo_f32_to_f16_buffer(y32, Y, (size_t)(M * N));
   free(a32);
   free(s32);

@@ -95,6 +95,13 @@ class _C:
             lib.mnbo_skip_simplified_layer_norm_f16.argtypes = [_u16p, _u16p, _u16p, _u16p, _i64, _u16p, _u16p,
                                                                 ctypes.c_float, _i64, _i64]
             lib.mnbo_skip_simplified_layer_norm_f16.restype = None
+            _i8p = ctypes.POINTER(ctypes.c_int8)
+            lib.mnbo_quantize_a_int8.argtypes = [_i8p, _f32p, _f32p, _i64, _i64, _i64]
+            lib.mnbo_quantize_a_int8.restype = None
+            lib.mnbo_matmul_int8_f32.argtypes = [_f32p, _u8p, _f32p, _u8p, _f32p, _f32p, _i64, _i64, _i64, _i64, _int]
+            lib.mnbo_matmul_int8_f32.restype = None
+            lib.mnbo_matmul_int8_f16.argtypes = [_u16p, _u8p, _u16p, _u8p, _u16p, _u16p, _i64, _i64, _i64, _i64, _int]
+            lib.mnbo_matmul_int8_f16.restype = None
             for f in (lib.mnbo_f16_to_f32_buffer, lib.mnbo_f32_to_f16_buffer, lib.mnbo_dequantize_f32,
                       lib.mnbo_dequantize_f16, lib.mnbo_matmul_f32, lib.mnbo_matmul_f64, lib.mnbo_matmul_f16,
                       lib.mnbo_quantize_f32):
@@ -173,6 +180,39 @@ class _C:
         y = np.empty((M, N), np.float32)
         self.lib.mnbo_matmul_f32(_ptr(a, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), _ptr(b, _f32p),
                                  _ptr(y, _f32p), M, N, K, bits, bs, nthreads)
+        return y.reshape(*lead, N)
+
+    # -- int8 activations (accuracy_level 4) ----------------------------------
+    def quantize_a_int8(self, A, bs):
+        """Blockwise int8 quantisation of the activations: returns (qa [M, k_blocks*bs] int8, scales [M, k_blocks])."""
+        a = np.ascontiguousarray(A.astype(np.float32))
+        M, K = a.shape
+        kb = -(-K // bs)
+        qa = np.empty((M, kb * bs), np.int8)
+        sc = np.empty((M, kb), np.float32)
+        self.lib.mnbo_quantize_a_int8(_ptr(qa, ctypes.POINTER(ctypes.c_int8)), _ptr(sc, _f32p), _ptr(a, _f32p), M, K, bs)
+        return qa, sc
+
+    def matmul_int8(self, A, B, scales, zp, bias, N, K, bs, nthreads=1) -> np.ndarray:
+        """Y = A x dequant(B)^T (+ bias) with A quantised blockwise to int8 first (4-bit weights), in the dtype of A."""
+        lead = A.shape[:-1]
+        M = int(np.prod(lead)) if lead else 1
+        B = np.ascontiguousarray(B, np.uint8)
+        zp = None if zp is None else np.ascontiguousarray(zp, np.uint8)
+        if A.dtype == np.float16:
+            a = np.ascontiguousarray(A).view(np.uint16)
+            s = np.ascontiguousarray(scales, np.float16).view(np.uint16)
+            b = None if bias is None else np.ascontiguousarray(bias, np.float16).view(np.uint16)
+            y = np.empty((M, N), np.uint16)
+            self.lib.mnbo_matmul_int8_f16(_ptr(a, _u16p), _ptr(B, _u8p), _ptr(s, _u16p), _ptr(zp, _u8p),
+                                          _ptr(b, _u16p), _ptr(y, _u16p), M, N, K, bs, nthreads)
+            return y.view(np.float16).reshape(*lead, N)
+        a = np.ascontiguousarray(A, np.float32)
+        s = np.ascontiguousarray(scales, np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+        y = np.empty((M, N), np.float32)
+        self.lib.mnbo_matmul_int8_f32(_ptr(a, _f32p), _ptr(B, _u8p), _ptr(s, _f32p), _ptr(zp, _u8p), _ptr(b, _f32p),
+                                      _ptr(y, _f32p), M, N, K, bs, nthreads)
         return y.reshape(*lead, N)
 
     def matmul_f64(self, A, B, scales, zp, bias, N, K, bits, bs, nthreads=1):
