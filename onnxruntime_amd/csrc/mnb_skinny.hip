@@ -437,6 +437,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   const int GK = L.group_k, CK = 4 * GK;
   const int chunks = (int)((L.K + CK - 1) / CK);
   pl.mode = (L.bs >= CK) ? 0 : 1;
+  if (const char* e = mnb_tuning_env("MNB_SKINNY_MODE")) pl.mode = e[0] == '1' ? 1 : pl.mode;  // calibration: exact halves
   pl.mtr = pow2_ceil((int)M);
   // workgroups: as many column slabs as fill the chip; wide slabs (T = 4) amortise the A operands best
   const int64_t tiles = (L.N + 15) / 16;
