@@ -184,22 +184,14 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
   return __builtin_bit_cast(h8_t, o);
 }
 
-// Scheduling pipeline of one slab section (NM MFMAs): after every MFMA a few of the other instructions of the
-// section, so they run in the MFMA's shadow.  The closing sched_barrier keeps the scheduler from mixing the MFMAs
-// of different slabs (they reuse the same accumulators).
-template <int NM, int LDS_READS, int VMEM, int VALU, int LDS_WRITE_EVERY>
-__device__ __forceinline__ void slab_pipeline() {
-#pragma unroll
-  for (int i = 0; i < NM; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                             // 1 MFMA
-    if (i < LDS_READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);          // 1 LDS read
-    if (i < VMEM) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);               // 2 VMEM reads
-    if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);  // VALU
-    if constexpr (LDS_WRITE_EVERY > 0) {
-      if (i % LDS_WRITE_EVERY == LDS_WRITE_EVERY - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // 1 LDS write
-    }
-  }
-  __builtin_amdgcn_sched_barrier(0);
+// End of one slab section (its matrix instructions, the LDS reads and the dequantisation of the next slab's operands,
+// a group of loads).  Inside a section the compiler's scheduler interleaves freely; it does that slightly better than
+// a hand-written order of "one MFMA, one LDS read, two loads, n VALU" per matrix instruction (measured: 1-2 % on every
+// shape).  A fence between sections keeps it from pulling the next slab's work forward, which pays everywhere (1-4 %)
+// except in the 256-row 4-bit kernel, where letting it mix the sections of a k-step is worth another 2 %.
+template <bool FENCE>
+__device__ __forceinline__ void slab_end() {
+  if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
 }
 
 // MPS: meta entries (scale, zero point) a lane keeps per k-step and column tile.  A k-step of 64 spans 64 / block_size
@@ -209,8 +201,7 @@ template <int BITS, bool HAS_ZP, int MPS, int TM>
 __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int BM = 64 * TM;                       // rows of the tile
   constexpr int STAGE_BYTES = BM * ROW_BYTES;       // one staged A tile
-  constexpr int NM = 2 * TM;                        // MFMAs per slab
-  constexpr int VALU_PER_MFMA = 32 / NM;            // the slab's dequantisation spread over its MFMAs
+  constexpr bool SLAB_FENCE = !(TM == 4 && (BITS == 4 || MPS == 4));  // (8-bit with four meta entries: fenced it spills)
   constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 16-byte activation loads per thread per k-step: TM
   // 4-bit: a 16-byte vector spans two slabs (one word each per lane); 8-bit: one slab (two words per lane)
   constexpr int VEC_PER_STEP = (BITS == 4) ? 2 : 4;  // 8-byte weight loads per lane, column tile and k-step
@@ -381,21 +372,21 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     make_b(1, Rc, FB1);
     mfma_slab(FA0, FB0);
     load_b_slot(ks + 2, Rc, 1);
-    slab_pipeline<NM, TM, (A_LOADS + Plan::size(1) + 1) / 2, VALU_PER_MFMA, 0>();
+    slab_end<SLAB_FENCE>();
     // slab 1: operands of slab 2
     read_a(cur, 2, FA0);
     if constexpr (Plan::slab_waits(2)) await_b(Slab<2>{}, Rc);
     make_b(2, Rc, FB0);
     mfma_slab(FA1, FB1);
     load_b_slot(ks + 2, Rc, 2);
-    slab_pipeline<NM, TM, (Plan::size(2) + 1) / 2, VALU_PER_MFMA, 0>();
+    slab_end<SLAB_FENCE>();
     // slab 2: operands of slab 3
     read_a(cur, 3, FA1);
     if constexpr (Plan::slab_waits(3)) await_b(Slab<3>{}, Rc);
     make_b(3, Rc, FB1);
     mfma_slab(FA0, FB0);
     load_b_slot(ks + 2, Rc, 3);
-    slab_pipeline<NM, TM, (Plan::size(3) + 1) / 2, VALU_PER_MFMA, 0>();
+    slab_end<SLAB_FENCE>();
     // The barrier of the step.  Before it a wavefront makes sure that its own part of A of step ks+1 has landed in
     // LDS (issued in slab 0 of step ks-1) and that the weights of slab 0 of step ks+1 are there; LoadPlan counts the
     // operations younger than both.  The wavefront's LDS reads have completed too, so the tile at `cur` may be
@@ -413,7 +404,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     make_b(0, Rn, FB0);
     mfma_slab(FA1, FB1);
     load_b_slot(ks + 3, Rn, 4);
-    slab_pipeline<NM, TM, (Plan::size(4) + 1) / 2, VALU_PER_MFMA, 0>();
+    slab_end<SLAB_FENCE>();
   };
 
   // ---- this workgroup's share of the units, walked from the top down
