@@ -73,7 +73,7 @@ struct Slab {
   static constexpr int value = KK;
 };
 
-template <int BITS, int MPS, int A_LOADS>
+template <int BITS, int MPS, int A_LOADS, int CT>
 struct LoadPlan {
   static constexpr int VPS = (BITS == 4) ? 2 : 4;
   static constexpr int slot_after(int kk) { return kk == 0 ? 4 : kk; }  // slot that follows make_b(kk)
@@ -84,8 +84,8 @@ struct LoadPlan {
   static constexpr int size(int q) {
     if (q == 0) return A_LOADS;
     int n = 0;
-    for (int v = 0; v < VPS; ++v) n += vec_slot(v) == q ? 2 : 0;
-    for (int e = 0; e < MPS; ++e) n += meta_slot(e) == q ? 2 : 0;
+    for (int v = 0; v < VPS; ++v) n += vec_slot(v) == q ? CT : 0;  // one load per column tile of the wavefront
+    for (int e = 0; e < MPS; ++e) n += meta_slot(e) == q ? CT : 0;
     return n;
   }
   static constexpr int before(int q) {  // operations of a step in front of slot q
@@ -197,35 +197,43 @@ __device__ __forceinline__ void slab_end() {
 // MPS: meta entries (scale, zero point) a lane keeps per k-step and column tile.  A k-step of 64 spans 64 / block_size
 // blocks; 4-bit vectors cover 32 k, so two entries serve every block size (16-wide blocks through the lane's half
 // kq); 8-bit vectors cover 16 k: 4 entries for blocks of 16, 2 for blocks of 32 and more.
-template <int BITS, bool HAS_ZP, int MPS, int TM>
+// WM: rows of the 2-D arrangement of the eight wavefronts over the tile.  WM = 2 (2 x 4): a wavefront owns
+// 32 TM rows x 64 columns, and the two wavefront rows dequantise the same columns.  WM = 1 (1 x 8): a wavefront owns
+// all 64 TM rows x 32 columns: every column is dequantised once per workgroup (half the vector instructions) and
+// every wavefront reads the whole staged A tile (twice the LDS reads).
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM>
 __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
+  constexpr int WN = 8 / WM;         // wavefront columns
+  constexpr int CT = WM;             // 32-column matrix-core tiles per wavefront: 256 / (32 WN)
+  constexpr int RT = 2 * TM / WM;    // 32-row matrix-core tiles per wavefront
+  constexpr int WCOLS = 32 * CT;     // columns of a wavefront
   constexpr int BM = 64 * TM;                       // rows of the tile
   constexpr int STAGE_BYTES = BM * ROW_BYTES;       // one staged A tile
   constexpr bool SLAB_FENCE = !(TM == 4 && (BITS == 4 || MPS == 4));  // (8-bit with four meta entries: fenced it spills)
   constexpr int A_LOADS = BM * (BK / 8) / THREADS;  // 16-byte activation loads per thread per k-step: TM
   // 4-bit: a 16-byte vector spans two slabs (one word each per lane); 8-bit: one slab (two words per lane)
   constexpr int VEC_PER_STEP = (BITS == 4) ? 2 : 4;  // 8-byte weight loads per lane, column tile and k-step
-  constexpr int ACC_PAIRS = TM * 2 * 8;              // 8-byte pairs of accumulators per lane
-  using Plan = LoadPlan<BITS, MPS, A_LOADS>;
+  constexpr int ACC_PAIRS = RT * CT * 8;             // 8-byte pairs of accumulators per lane
+  using Plan = LoadPlan<BITS, MPS, A_LOADS, CT>;
   extern __shared__ __align__(16) unsigned char lds_bytes[];
   _Float16* const lds = reinterpret_cast<_Float16*>(lds_bytes);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 wavefronts: rows wm*32*TM, columns wn*64
+  const int wm = wave / WN, wn = wave % WN;  // rows wm * 32 RT, columns wn * WCOLS
   const int li = lane & 31, kq = lane >> 5;
 
-  f16_t acc[TM][2];
+  f16_t acc[RT][CT];
 
   // Two register sets for the weight prefetch (distance: two k-steps); the activations need none.
   struct Stage {
-    u2_t b[VEC_PER_STEP][2];      // [vector of the k-step][column tile]
-    uint32_t m[MPS][2];           // meta entries of the blocks of the k-step (see m_off)
+    u2_t b[VEC_PER_STEP][CT];     // [vector of the k-step][column tile]
+    uint32_t m[MPS][CT];          // meta entries of the blocks of the k-step (see m_off)
   };
   Stage R0, R1;
-  h8_t FA0[TM], FA1[TM];  // A operands, double buffered over slabs
-  h8_t FB0[2], FB1[2];  // B operands, double buffered over slabs
+  h8_t FA0[RT], FA1[RT];  // A operands, double buffered over slabs
+  h8_t FB0[CT], FB1[CT];  // B operands, double buffered over slabs
 
   const UnpackConsts uc = make_unpack_consts();
 
@@ -246,10 +254,10 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // Without zero points an entry is a 16-bit scale.  A 16-bit load would be zero-extended, or packed with its
   // neighbour, right behind the load, which needs the data at once and defeats the prefetch: the lane loads the
   // aligned 32-bit word that holds its scale and shifts by m_shift (0 or 16) when it uses it.
-  uint32_t w_off[2], m_off[2], m_shift[2];
+  uint32_t w_off[CT], m_off[CT], m_shift[CT];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int col = wn * 64 + j * 32 + li;  // within the tile; tiles start at multiples of 256 columns
+  for (int j = 0; j < CT; ++j) {
+    const int col = wn * WCOLS + j * 32 + li;  // within the tile; tiles start at multiples of 256 columns
     w_off[j] = (uint32_t)(col * 16 + kq * 8);
     const uint32_t m_byte = (uint32_t)((mnb_meta_col(col) + (small_bs ? kq * p.Npad : 0)) * META_BYTES);
     m_off[j] = m_byte & ~3u;
@@ -282,7 +290,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       const int64_t kg = (int64_t)ks * VEC_PER_STEP + v;  // k-group of the vector
       const rsrc_t r = mnb_rsrc(w_tile + kg * vec_pitch);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) R.b[v][j] = mnb_buffer_load_b64(r, w_off[j]);
+      for (int j = 0; j < CT; ++j) R.b[v][j] = mnb_buffer_load_b64(r, w_off[j]);
     }
 #pragma unroll
     for (int e = 0; e < MPS; ++e) {
@@ -290,7 +298,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       const int64_t kb = ((int64_t)ks * BK + e * (BK / MPS)) >> p.bs_shift;  // block of the entry's first element
       const rsrc_t r = mnb_rsrc(meta_tile + kb * meta_pitch);
 #pragma unroll
-      for (int j = 0; j < 2; ++j) R.m[e][j] = mnb_buffer_load_b32(r, m_off[j]);
+      for (int j = 0; j < CT; ++j) R.m[e][j] = mnb_buffer_load_b32(r, m_off[j]);
     }
   };
   auto load_b = [&](int ks_raw, Stage& R) {
@@ -305,7 +313,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(vm));
     constexpr int v = Plan::vec_of_slab(kk), e = Plan::meta_of_slab(kk);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < CT; ++j) {
       asm volatile("; b %0" : "+v"(R.b[v][j]));
       asm volatile("; m %0" : "+v"(R.m[e][j]));
     }
@@ -325,7 +333,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // B operands of slab kk (0..3) of the k-step held in R
   auto make_b = [&](int kk, const Stage& R, h8_t* FB) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < CT; ++j) {
       h2_t s2;
       ZpH z;
       if constexpr (BITS == 4) {
@@ -345,19 +353,19 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
   for (int kk = 0; kk < 4; ++kk) {
     const int chunk = (BITS == 4) ? 4 * (kk >> 1) + 2 * kq + (kk & 1) : 2 * kk + kq;
-    a_rd[kk] = (uint32_t)((wm * 32 * TM + li) * ROW_BYTES + ((chunk ^ ((li >> 1) & 7)) * 16));
+    a_rd[kk] = (uint32_t)((wm * 32 * RT + li) * ROW_BYTES + ((chunk ^ ((li >> 1) & 7)) * 16));
   }
   auto read_a = [&](int stage_off, int kk, h8_t* FA) {
     const unsigned char* As = lds_bytes + stage_off + a_rd[kk];
 #pragma unroll
-    for (int t = 0; t < TM; ++t) FA[t] = *reinterpret_cast<const h8_t*>(As + t * 32 * ROW_BYTES);
+    for (int t = 0; t < RT; ++t) FA[t] = *reinterpret_cast<const h8_t*>(As + t * 32 * ROW_BYTES);
   };
 
   auto mfma_slab = [&](const h8_t* FA, const h8_t* FB) {
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < CT; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(FA[i], FB[j], acc[i][j], 0, 0, 0);
   };
 
@@ -445,7 +453,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
       for (int g = 0; g < ACC_PAIRS / 2; ++g) {
         const int pair = half * (ACC_PAIRS / 2) + g;
-        const int i = pair / 16, j = (pair / 8) % 2, q = pair % 8;
+        const int i = pair / 8 / CT, j = pair / 8 % CT, q = pair % 8;
         const float lo = __builtin_bit_cast(float, (uint32_t)t[g]), hi = __builtin_bit_cast(float, (uint32_t)(t[g] >> 32));
         acc[i][j][2 * q] = ok ? acc[i][j][2 * q] + lo : __builtin_nanf("");
         acc[i][j][2 * q + 1] = ok ? acc[i][j][2 * q + 1] + hi : __builtin_nanf("");
@@ -477,9 +485,9 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       a_off[i] = (uint32_t)(((int64_t)r * p.lda + a_kc * 8) * 2);
     }
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < CT; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -521,10 +529,10 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       asm volatile("" : "+v"(lane_here));
       uint64_t* dst = p.partials + (size_t)wg * SLOT_PAIRS + wave_pairs;
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          uint64_t* grp = dst + (size_t)((i * 2 + j) * 8) * 64;  // uniform
+        for (int j = 0; j < CT; ++j) {
+          uint64_t* grp = dst + (size_t)((i * CT + j) * 8) * 64;  // uniform
 #pragma unroll
           for (int q = 0; q < 8; ++q) {
             // (copies first: a bit cast applied to a vector element expression reads the vector's first element)
@@ -553,38 +561,42 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
     const int li_e = lane_e & 31, kq_e = lane_e >> 5;
-    float bcol[2];
+    float bcol[CT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn * 64 + j * 32 + li_e;
+    for (int j = 0; j < CT; ++j) {
+      const int n = n0 + wn * WCOLS + j * 32 + li_e;
       bcol[j] = (p.bias && n < p.N) ? (float)p.bias[n] : 0.f;
     }
     if (p.c_vec_ok) {
-      constexpr int EP_STRIDE = 72;  // halves per staged row: 16-byte aligned rows, conflict-free 16-byte reads
-      __syncthreads();               // every wavefront is done with the A tiles
+      // a wavefront stages 64 rows x WCOLS columns at a time
+      constexpr int EP_STRIDE = WCOLS + 8;  // halves per staged row: 16-byte aligned rows, conflict-free 16-byte reads
+      constexpr int LPR = WCOLS / 8;        // lanes per staged row in the plain store: 8 columns each
+      __syncthreads();                      // every wavefront is done with the A tiles
       _Float16* ep = lds + wave * (64 * EP_STRIDE);
-      const int erow = lane_e >> 3, ecol = (lane_e & 7) * 8;
-      const int n_out = n0 + wn * 64 + ecol;
+      const int erow = lane_e / LPR, ecol = (lane_e % LPR) * 8;
+      const int n_out = n0 + wn * WCOLS + ecol;
 #pragma unroll
-      for (int h = 0; h < TM / 2; ++h) {
+      for (int h = 0; h < RT / 2; ++h) {
 #pragma unroll
         for (int ii = 0; ii < 2; ++ii)
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
+          for (int j = 0; j < CT; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
               ep[(ii * 32 + (r >> 2) * 8 + kq_e * 4 + (r & 3)) * EP_STRIDE + j * 32 + li_e] =
                   (_Float16)(acc[2 * h + ii][j][r] + bcol[j]);
         // LDS operations of one wavefront complete in issue order: the reads below see the writes above
         if (p.epi_kind == kMnbFusedMlp) {
-          // a staged row is gate0 up0 gate1 up1 (16 columns each) = 32 output columns: four lanes per row, each reads
-          // its 8 gate and 8 up values (narrowed to fp16, as the two separate products would be) and writes 8 outputs
-          const int grow = lane_e >> 2, q = lane_e & 3;
+          // a staged row is gate0 up0 [gate1 up1] (16 columns each) = 16 CT output columns: 2 CT lanes per row, each
+          // reads its 8 gate and 8 up values (narrowed to fp16, as the two separate products would be) and writes 8
+          // outputs
+          constexpr int GL = 2 * CT;  // lanes per staged row
+          const int grow = lane_e / GL, q = lane_e % GL;
           const int gcol = (q >> 1) * 32 + (q & 1) * 8;
-          const int n_glu = ((n0 + wn * 64) >> 1) + q * 8;
+          const int n_glu = ((n0 + wn * WCOLS) >> 1) + q * 8;
 #pragma unroll
-          for (int ps = 0; ps < 4; ++ps) {
-            const int row = ps * 16 + grow;
+          for (int ps = 0; ps < GL; ++ps) {
+            const int row = ps * (64 / GL) + grow;
             const h8_t g = *reinterpret_cast<const h8_t*>(ep + row * EP_STRIDE + gcol);
             const h8_t u = *reinterpret_cast<const h8_t*>(ep + row * EP_STRIDE + gcol + 16);
             h8_t y;
@@ -593,7 +605,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
               const float gf = (float)g[e];
               y[e] = (_Float16)(gf / (1.0f + __expf(-gf)) * (float)u[e]);
             }
-            const int m = m0 + wm * 32 * TM + h * 64 + row;
+            const int m = m0 + wm * 32 * RT + h * 64 + row;
             if (m < p.M && n_glu < p.n_out0) *reinterpret_cast<h8_t*>(p.C + (int64_t)m * p.ldc + n_glu) = y;
           }
         } else {
@@ -610,24 +622,24 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
             }
           }
 #pragma unroll
-          for (int ps = 0; ps < 8; ++ps) {
-            const int row = ps * 8 + erow;
+          for (int ps = 0; ps < LPR; ++ps) {
+            const int row = ps * (64 / LPR) + erow;
             const u4_t v = *reinterpret_cast<const u4_t*>(ep + row * EP_STRIDE + ecol);
-            const int m = m0 + wm * 32 * TM + h * 64 + row;
+            const int m = m0 + wm * 32 * RT + h * 64 + row;
             if (m < p.M && n_loc < n_lim) *reinterpret_cast<u4_t*>(dst + (int64_t)m * ld + n_loc) = v;
           }
         }
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int n = n0 + wn * 64 + j * 32 + li_e;
+      for (int j = 0; j < CT; ++j) {
+        const int n = n0 + wn * WCOLS + j * 32 + li_e;
         if (n >= p.N) continue;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < RT; ++i) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int m = m0 + wm * 32 * TM + i * 32 + (r >> 2) * 8 + kq_e * 4 + (r & 3);
+            const int m = m0 + wm * 32 * RT + i * 32 + (r >> 2) * 8 + kq_e * 4 + (r & 3);
             if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + bcol[j]);
           }
         }
@@ -641,10 +653,10 @@ __global__ void __launch_bounds__(256) mnb_gemm256_clear_flags_kernel(uint32_t* 
   for (int i = threadIdx.x; i < n; i += 256) flags[i] = 0u;
 }
 
-template <int BITS, bool HAS_ZP, int MPS, int TM>
-hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM>
+hipError_t launch_wm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
   const size_t smem = (size_t)SMEM_BYTES;  // 98304 bytes
-  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM>;
+  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM>;
   // The attribute belongs to the function on the current device, so it is set on every launch (a host-side table
   // update, no device work): callers on several threads or devices need no shared flag.
   if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -653,6 +665,18 @@ hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
     return e;
   kernel<<<dim3(grid), dim3(THREADS), smem, s>>>(p);
   return hipGetLastError();
+}
+
+// The 1 x 8 arrangement of the wavefronts is faster on every shape and block size measured (0.84 ... 0.98 of the
+// 2 x 4 arrangement's time, bit-identical results): matrix and vector instructions hardly overlap on a SIMD, so the
+// halved dequantisation work counts in full.  The 2 x 4 arrangement is compiled into calibration builds only.
+template <int BITS, bool HAS_ZP, int MPS, int TM>
+hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
+#if defined(MNB_TUNING_HOOKS)
+  if (const char* e = mnb_tuning_env("MNB_GEMM256_WAVE_ROWS"); e != nullptr && e[0] == '2')
+    return launch_wm<BITS, HAS_ZP, MPS, TM, 2>(p, grid, s);
+#endif
+  return launch_wm<BITS, HAS_ZP, MPS, TM, 1>(p, grid, s);
 }
 
 template <int BITS, bool HAS_ZP, int MPS>
@@ -664,10 +688,9 @@ size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 
 }  // namespace
 
-// How the tile GEMM would run a problem: rows of the tile (the 128-row tile when its grid fills the compute units in
-// fewer, or at the kernel's step costs cheaper, rounds), the grid, whether tiles are split along K across workgroups
-// (only with a workspace, and only when the tiles leave at least half of the compute units idle), the workspace that
-// takes, and the estimated run time.  The kernel itself takes any division of the units into contiguous shares.
+// How the tile GEMM would run a problem: rows of the tile, the grid, whether tiles are split along K across
+// workgroups (only with a workspace), the workspace that takes, and the estimated run time.  The kernel itself takes
+// any division of the units into contiguous shares.
 // ---- the plan: tile height and split, from a cost model calibrated on the device
 // Measured behaviour (all shapes of M = 256 ... 4096, N = 4096 ... 28672, K = 4096 / 8192 / 14336, every tile height
 // and number of parts):

@@ -70,13 +70,14 @@ class Plan:
     """The issue order of a k-step, restated: slot 0 the activation loads, slots 1..3 the weight registers reloaded
     after the operands of slabs 1..3 were made, slot 4 those reloaded after slab 0's (behind the barrier)."""
 
-    def __init__(self, bits, mps, tm):
+    def __init__(self, bits, mps, tm, ct):
+        """ct: 32-column matrix-core tiles per wavefront = loads per weight vector and per meta entry."""
         self.bits, self.mps = bits, mps
         vps = 2 if bits == 4 else 4
         after = lambda kk: 4 if kk == 0 else kk  # noqa: E731
         self.vec_slot = [after(2 * v + 1 if bits == 4 else v) for v in range(vps)]
         self.meta_slot = [after(2 * e + 1 if bits == 4 else (e + 1) * 4 // mps - 1) for e in range(mps)]
-        self.size = [tm] + [2 * self.vec_slot.count(q) + 2 * self.meta_slot.count(q) for q in range(1, 5)]
+        self.size = [tm] + [ct * self.vec_slot.count(q) + ct * self.meta_slot.count(q) for q in range(1, 5)]
         self.per_step = sum(self.size)
 
     def before(self, q):
@@ -107,8 +108,8 @@ class Plan:
 def test_every_instantiation_issues_its_loads_and_waits_as_planned(kernels):
     assert len(kernels) == 12
     for name, lines in kernels.items():
-        bits, mps, tm = (int(x) for x in re.search(r"kernelILi(\d)ELb[01]ELi(\d)ELi(\d)E", name).groups())
-        plan = Plan(bits, mps, tm)
+        bits, mps, tm, wm = (int(x) for x in re.search(r"kernelILi(\d)ELb[01]ELi(\d)ELi(\d)ELi(\d)E", name).groups())
+        plan = Plan(bits, mps, tm, ct=wm)  # the wavefronts form wm x 8/wm: 256 / (32 * 8/wm) column tiles each
         loops = _hot_loops(lines)
         assert len(loops) == 1, name
         assert loops[0] == plan.step_tokens() * 2, (name, " ".join(loops[0]))
