@@ -695,9 +695,11 @@ size_t round256(size_t v) { return (v + 255) / 256 * 256; }
 // Measured behaviour (all shapes of M = 256 ... 4096, N = 4096 ... 28672, K = 4096 / 8192 / 14336, every tile height
 // and number of parts):
 //   * a workgroup that has its compute unit to itself on a chip at most half busy runs its k-steps at a fixed pace
-//     (kStepCycles), after a fixed start-up (kStartCycles: launch, prologue, epilogue);
+//     (step: 2530 cycles for a 256-row 4-bit tile, of which the 64 matrix instructions of a SIMD take 2048 and the
+//     vector instructions most of the rest -- the two hardly overlap on a SIMD), after a fixed start-up (start:
+//     launch, prologue, epilogue);
 //   * the chip is power-limited: with more than half of the compute units busy every workgroup slows down, by
-//     kLoad[...] at 3/4, 7/8 and all of them (a full chip does 1.3 times the work of half a chip per second, not 2);
+//     load[...] at 3/4, 7/8 and all of them (a full chip does 1.2 times the work of half a chip per second, not 2);
 //     kernels that are bound by the vector unit (8-bit weights, 128-row tiles) slow down less;
 //   * more workgroups than compute units run as rounds (128-row tiles share a compute unit in pairs, which costs
 //     what two rounds cost);
@@ -712,11 +714,11 @@ struct Variant {
   double full[2];     // slow-down of a full round when there are several
 };
 constexpr Variant kVariants[3] = {
-    {{16800, 15400}, {2850, 1860}, {{1.31, 1.43, 1.59}, {1.17, 1.28, 1.46}}, {1.59, 1.46}},
-    {{19200, 16800}, {2900, 2360}, {{1.28, 1.41, 1.58}, {1.06, 1.15, 1.24}}, {1.58, 1.35}},
-    {{19200, 16800}, {3820, 3460}, {{1.11, 1.20, 1.35}, {1.05, 1.10, 1.20}}, {1.35, 1.25}},
+    {{18000, 13440}, {2530, 1478}, {{1.31, 1.465, 1.66}, {1.216, 1.365, 1.535}}, {1.67, 1.57}},
+    {{18480, 15120}, {2545, 1582}, {{1.333, 1.48, 1.665}, {1.17, 1.313, 1.476}}, {1.69, 1.544}},
+    {{18480, 15120}, {3105, 1905}, {{1.16, 1.30, 1.47}, {1.10, 1.20, 1.35}}, {1.47, 1.37}},
 };
-constexpr double kFixCycles[2][2] = {{6000, 9400}, {2200, 6700}};  // [tile height][constant, per part]
+constexpr double kFixCycles[2][2] = {{3120, 9600}, {2400, 6720}};  // [tile height][constant, per part]
 
 inline double load_factor(const double (&at)[3], double busy) {  // busy: fraction of the compute units with a workgroup
   if (busy <= 0.5) return 1.0;
@@ -725,13 +727,14 @@ inline double load_factor(const double (&at)[3], double busy) {  // busy: fracti
   return at[1] + (at[2] - at[1]) * (busy > 1.0 ? 1.0 : (busy - 0.875) / 0.125);
 }
 
-// cycles for `grid` workgroups of `steps` k-steps each
+// cycles for `grid` workgroups of `steps` k-steps each (the finishing pass of a split does not slow down with load)
 inline double cycles(const Variant& v, int h, int64_t grid, int64_t steps, int parts, int64_t cus) {
-  const double part = (double)steps * v.step[h] + (parts > 1 ? kFixCycles[h][0] + parts * kFixCycles[h][1] : 0.0);
+  const double part = (double)steps * v.step[h];
+  const double fix = parts > 1 ? kFixCycles[h][0] + parts * kFixCycles[h][1] : 0.0;
   const int64_t rounds = grid / cus, rest = grid % cus;
   double t = v.start[h];
-  if (rounds > 0) t += (double)rounds * part * (rounds + (rest ? 1 : 0) > 1 ? v.full[h] : v.load[h][2]);
-  if (rest > 0) t += part * load_factor(v.load[h], (double)rest / (double)cus);
+  if (rounds > 0) t += (double)rounds * (part * (rounds + (rest ? 1 : 0) > 1 ? v.full[h] : v.load[h][2]) + fix);
+  if (rest > 0) t += part * load_factor(v.load[h], (double)rest / (double)cus) + fix;
   return t;
 }
 }  // namespace plan_model
