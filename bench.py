@@ -30,8 +30,8 @@ sys.path.insert(0, str(ROOT))
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000), and are copied here from the summary named in TRAFFIC_SOURCE (KiB per
 # dispatch as printed there).  Every `traffic` value in the output carries `traffic_source` beside it.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md (rocprofv3 --pmc; a constant, not this run)"
-PROFILED_TRAFFIC_BYTES = {"c2_decode": int((14858.3 * 2.0 + 28.0) * 1024), "c4_prefill": int((109756.6 * 2.0 + 57344.0) * 1024),
-                          "quantize": int((57399.0 * 2.0 + 30470.0) * 1024), "mlp_decode": int((29674.3 * 2.0 + 28.0) * 1024)}
+PROFILED_TRAFFIC_BYTES = {"c2_decode": int((14858.5 * 2.0 + 28.0) * 1024), "c4_prefill": int((109777.3 * 2.0 + 57344.0) * 1024),
+                          "quantize": int((57399.0 * 2.0 + 30511.9) * 1024), "mlp_decode": int((29675.0 * 2.0 + 28.0) * 1024)}
 # The reference's own MLAS kernel on the headline shape, timed by the survey on an 8-vCPU Sapphire-Rapids-class host
 # (standalone MLAS build, SQNBIT_CompFp32, N sliced over 8 threads): quoted beside the port so that the port's
 # figure is not read as the reference's.

@@ -205,8 +205,9 @@ constexpr double kMnbMidStartCycles = 19200.0;
 constexpr double kMnbMidFlopsPerCuCycle[2] = {1286.0, 1156.0};
 
 static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
-  if (M <= 128 || L.K % 128 != 0) return false;
+  if (L.K % 128 != 0) return false;
   if (const char* e = mnb_tuning_env("MNB_MID_MAX_M")) return M > (int64_t)atoll(e);  // calibration: M up to this streams
+  if (M <= 64) return false;  // (64-row tiles were measured: never ahead of the streaming kernel)
   const MnbDeviceInfo& dev = mnb_device_info();
   const double t_mid = (kMnbMidStartCycles + 2.0 * (double)M * (double)L.N * (double)L.K /
                                                  (kMnbMidFlopsPerCuCycle[L.bits == 4 ? 0 : 1] * dev.cus)) /
