@@ -35,6 +35,8 @@ struct MatMulNBitsKernel : OrtKernelImpl {
   OrtAllocator* packed_allocator = nullptr;
   int packed_dtype = 0;
   bool packed_has_zp = false;
+  // session configuration entry "ep.mi355x.int8_activations" = "1" and accuracy_level = 4: quantise A to int8
+  bool int8_activations = false;
 };
 
 MatMulNBitsKernel* Self(OrtKernelImpl* p) { return static_cast<MatMulNBitsKernel*>(p); }
@@ -382,10 +384,25 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
     if (dtype != k.packed_dtype) {
       return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A and scales must have the same element type");
     }
+    hipStream_t gs = static_cast<hipStream_t>(stream);
+    if (k.int8_activations) {
+      // accuracy_level 4 with the session's consent: the reference's int8-activation arithmetic, where implemented
+      const size_t ws8 = MnbGemmInt8WorkspaceSize(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype);
+      if (ws8 > 0) {
+        void* scratch8 = nullptr;
+        MI_RETURN_IF_HIP(a, hipMallocAsync(&scratch8, ws8, gs));
+        KernelTimer timer(gs, "MatMulNBits", "mnb_gemm_i8_kernel", M, k.N, k.K);
+        const int rc8 = MnbGemmInt8(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr, Nz,
+                                    scratch8, ws8, stream);
+        const hipError_t free8 = hipFreeAsync(scratch8, gs);
+        MI_RETURN_IF_ERROR(StatusFromMnb(a, rc8));
+        MI_RETURN_IF_HIP(a, free8);
+        return nullptr;
+      }
+    }
     // per-call scratch comes from the stream-ordered pool, so concurrent Run() calls never share it
     const size_t gemm_ws = MnbGemmWorkspaceSize(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype);
     void* gemm_scratch = nullptr;
-    hipStream_t gs = static_cast<hipStream_t>(stream);
     if (gemm_ws > 0) MI_RETURN_IF_HIP(a, hipMallocAsync(&gemm_scratch, gemm_ws, gs));
     KernelTimer timer(gs, "MatMulNBits", MnbGemmKernelName(Mz, Nz, Kz, bits, bs, dtype), M, k.N, k.K);
     const int gemm_rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr, Nz,
@@ -447,6 +464,18 @@ OrtStatus* ORT_API_CALL CreateMatMulNBits(void* state, const OrtKernelInfo* info
   if (OrtStatus* st = a.ort->KernelInfoGetAttribute_int64(info, "accuracy_level", &k->accuracy_level)) {
     a.ort->ReleaseStatus(st);
     k->accuracy_level = 0;
+  }
+  if (k->accuracy_level == 4 && a.ort->KernelInfo_GetConfigEntries != nullptr) {
+    // accuracy_level permits int8 activations, it does not ask for them, and the full-accuracy route is the faster
+    // one here: the int8 route is taken only when the session says so
+    OrtKeyValuePairs* entries = nullptr;
+    if (OrtStatus* st = a.ort->KernelInfo_GetConfigEntries(info, &entries)) {
+      a.ort->ReleaseStatus(st);
+    } else if (entries != nullptr) {
+      const char* v = a.ort->GetKeyValue(entries, "ep.mi355x.int8_activations");
+      k->int8_activations = v != nullptr && v[0] == '1' && v[1] == '\0';
+      a.ort->ReleaseKeyValuePairs(entries);
+    }
   }
   if (k->bits != 2 && k->bits != 4 && k->bits != 8) {
     return a.ort->CreateStatus(ORT_INVALID_ARGUMENT,

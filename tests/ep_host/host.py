@@ -82,6 +82,8 @@ def _load():
     lib.EpHostProbeFactory.restype = ctypes.c_int
     lib.EpHostProbeFactory.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t, ctypes.c_char_p,
                                        ctypes.c_size_t]
+    lib.EpHostSetSessionConfig.restype = None
+    lib.EpHostSetSessionConfig.argtypes = [ctypes.c_char_p, ctypes.c_char_p]
     lib.EpHostRunMatMulNBits.restype = ctypes.c_int
     lib.EpHostRunMatMulNBits.argtypes = [
         ctypes.c_char_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
@@ -204,6 +206,26 @@ def run_qkv(Nq, Nkv, K, bits, block_size, A, q, k, v, skip=None, norm_scale=None
                            [lead + (Nq,), lead + (Nkv,), lead + (Nkv,), A.shape], skipped=() if want_sum else (3,),
                            repeat=repeat)
     return outs[0], outs[1], outs[2], outs[3], trace
+
+
+class session_config:
+    """Context manager: session configuration entries (what OrtSessionOptions::AddConfigEntry sets) for the runs
+    inside the block."""
+
+    def __init__(self, **entries):
+        self.entries = {k.replace("__", "."): str(v) for k, v in entries.items()}
+
+    def __enter__(self):
+        lib = _load()
+        for k, v in self.entries.items():
+            lib.EpHostSetSessionConfig(k.encode(), v.encode())
+        return self
+
+    def __exit__(self, *exc):
+        lib = _load()
+        for k in self.entries:
+            lib.EpHostSetSessionConfig(k.encode(), None)
+        return False
 
 
 def probe_factory(offer_amd_gpu: bool = True) -> dict:

@@ -143,6 +143,9 @@ struct OrtKernelInfo {
   const OrtNode* node;
   std::map<size_t, const OrtValue*> constants;
 };
+struct OrtKeyValuePairs {
+  std::map<std::string, std::string> kv;
+};
 struct OrtSyncStream {
   OrtSyncStreamImpl* impl;
 };
@@ -157,6 +160,12 @@ struct OrtKernelContext {
 };
 
 namespace {
+
+// configuration entries of the (one) session this host stands for
+std::map<std::string, std::string>& SessionConfig() {
+  static std::map<std::string, std::string> config;
+  return config;
+}
 
 size_t ElemSize(ONNXTensorElementDataType t) {
   switch (t) {
@@ -260,6 +269,18 @@ void FillApisOnce() {
       }
     return MakeStatus(ORT_FAIL, (std::string("No attribute with name:'") + name + "'is defined.").c_str());
   };
+  // session configuration entries (OrtSessionOptions::AddConfigEntry in a real session; EpHostSetSessionConfig here)
+  g_ort.KernelInfo_GetConfigEntries = [](const OrtKernelInfo*, OrtKeyValuePairs** out) noexcept -> OrtStatus* {
+    auto* kv = new OrtKeyValuePairs();
+    kv->kv = SessionConfig();
+    *out = kv;
+    return nullptr;
+  };
+  g_ort.GetKeyValue = [](const OrtKeyValuePairs* kvps, const char* key) noexcept -> const char* {
+    auto it = kvps->kv.find(key);
+    return it == kvps->kv.end() ? nullptr : it->second.c_str();
+  };
+  g_ort.ReleaseKeyValuePairs = [](OrtKeyValuePairs* kvps) noexcept { delete kvps; };
   g_ort.KernelContext_GetOutputCount = [](const OrtKernelContext* c, size_t* out) noexcept -> OrtStatus* {
     *out = c->outputs.size();
     return nullptr;
@@ -680,6 +701,14 @@ enum {
   EP_HOST_PROTOCOL = -4,      // the plugin broke an expectation of the host
   EP_HOST_NOT_FUSED = -5      // a MatMulNBits + Add pair was offered and the plugin did not ask to fuse it
 };
+
+// Sets (value != NULL) or removes a session configuration entry for the sessions created afterwards.
+__attribute__((visibility("default"))) void EpHostSetSessionConfig(const char* key, const char* value) {
+  if (value != nullptr)
+    SessionConfig()[key] = value;
+  else
+    SessionConfig().erase(key);
+}
 
 // Factory-level queries that need no GPU. Writes "name|vendor|vendor_id|version|num_ep_devices" into `out`.
 __attribute__((visibility("default"))) int EpHostProbeFactory(const char* plugin_path, int offer_amd_gpu, char* out,

@@ -124,3 +124,30 @@ def test_shape_errors_carry_the_reference_messages():
     with pytest.raises(host.EpHostError) as e:   # A whose inner dimension is not K
         host.run_matmul_nbits(c.N, c.K, 4, 32, c.A[:, :-1], c.B, c.scales, c.zero_points)
     assert e.value.code == INVALID_ARGUMENT and "dimension mismatch" in e.value.message
+
+
+def test_accuracy_level_4_takes_int8_activations_only_with_the_sessions_consent(oracle):
+    """accuracy_level = 4 permits int8 activations.  Without the session configuration entry the node is computed at
+    full accuracy; with "ep.mi355x.int8_activations" = "1" it is computed with the reference's int8-activation
+    arithmetic (bit for bit the oracle's restatement); configurations without an int8 route keep full accuracy."""
+    M, N, K, bits, bs = 40, 192, 512, 4, 64
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, has_bias=True, seed=21)
+    want8 = oracle.C.matmul_int8(c.A, c.B, c.scales, c.zero_points, c.bias, N, K, bs)
+    want0 = oracle.C.matmul(c.A, c.B, c.scales, c.zero_points, c.bias, N, K, bits, bs)
+    y, _ = host.run_matmul_nbits(N, K, bits, bs, c.A, c.B, c.scales, c.zero_points, bias=c.bias, accuracy_level=4)
+    check_against_oracle(oracle, c, y)
+    assert not np.array_equal(y, want8)
+    with host.session_config(ep__mi355x__int8_activations=1):
+        y8, trace = host.run_matmul_nbits(N, K, bits, bs, c.A, c.B, c.scales, c.zero_points, bias=c.bias,
+                                          accuracy_level=4)
+        assert np.array_equal(y8, want8)
+        assert not np.array_equal(y8, want0)
+        # the entry does nothing for nodes that do not carry accuracy_level 4 ...
+        y0, _ = host.run_matmul_nbits(N, K, bits, bs, c.A, c.B, c.scales, c.zero_points, bias=c.bias, accuracy_level=0)
+        assert np.array_equal(y0, y)
+        # ... and nothing for configurations without an int8 route (8-bit weights)
+        c8 = make_case(M, N, K, 8, bs, np.float16, has_zp=True, seed=22)
+        y88, _ = host.run_matmul_nbits(N, K, 8, bs, c8.A, c8.B, c8.scales, c8.zero_points, accuracy_level=4)
+        check_against_oracle(oracle, c8, y88)
+    y_after, _ = host.run_matmul_nbits(N, K, bits, bs, c.A, c.B, c.scales, c.zero_points, bias=c.bias, accuracy_level=4)
+    assert np.array_equal(y_after, y)
