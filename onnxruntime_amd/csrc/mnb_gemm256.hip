@@ -3,14 +3,15 @@
 // Device counterpart of the reference's prefill loop (SQ4BitGemm_CompFp32, onnxruntime/core/mlas/lib/qnbitgemm.cpp:
 // 563-732: dequantise a strip of B, then run the float GEMM kernel over it).
 //
-// Eight wavefronts (2 x 4, two per SIMD), each owning a 128 x 64 block of the tile as 4 x 2
-// v_mfma_f32_32x32x16_f16 accumulators.  Per k-step of 64:
+// Eight wavefronts (1 x 8, two per SIMD), each owning all 256 rows and 32 columns of the tile as 8 x 1
+// v_mfma_f32_32x32x16_f16 accumulators (WM below; the 2 x 4 arrangement the kernel started with is kept for
+// calibration builds).  Per k-step of 64:
 //   * A (activations) goes from global memory straight into LDS (buffer_load_dwordx4 ... lds: no registers, no LDS
 //     store instructions), two k-steps ahead, into one of three staged tiles.  Such a load puts the 16 bytes of lane
 //     L at (wave-uniform LDS base) + 16 L, so a wavefront fills 8 rows x 128 bytes with one instruction; the rows are
 //     not padded, instead the lane that fills chunk position p of row r fetches chunk p ^ ((r >> 1) & 7) of that
-//     row, and the readers (ds_read_b128, lane = row) apply the same XOR.  The LDS serves such a read 16 lanes at a time from 64
-//     banks: 16 consecutive rows must start in 16 different 16-byte bank groups, and rows r, r+2, ... r+14 (same
+//     row, and the readers (ds_read_b128, lane = row) apply the same XOR.  The LDS serves such a read 16 lanes at a
+//     time from 64 banks: 16 consecutive rows must start in 16 different 16-byte bank groups, and rows r, r+2, ... r+14 (same
 //     half of the 256 bytes that two rows span) get the 8 different chunk positions: conflict free.
 //   * B (weights) never touches LDS.  Lane (column j = lane%32, half kq = lane/32) of a wavefront loads, two steps
 //     ahead (each register is reloaded right after its last use, and the loop states its own exact waits: see
@@ -19,9 +20,10 @@
 //     (q - zp), one rounding by the scale, bit-identical to the reference's fp16 dequantisation -- and IS the MFMA
 //     B operand of one k-slab.  (The contraction index of an MFMA may be permuted freely as long as A uses the same
 //     permutation: for 4-bit weights slab 2g takes k = 32g + 16kq + [0,8) and slab 2g+1 takes 32g + 16kq + [8,16).)
-//     LDS traffic is what bounded the design that staged a dequantised B tile in LDS (every wavefront re-read it);
-//     the price here is that the two wavefront rows dequantise the same columns.
-//   * one barrier per step; the dequantisation of slab s+1 and the A staging run in the shadow of slab s's MFMAs.
+//     LDS traffic is what bounded the design that staged a dequantised B tile in LDS (every wavefront re-read it).
+//     With the 1 x 8 arrangement every column is dequantised exactly once per workgroup.
+//   * one barrier per step; the dequantisation of slab s+1 is issued among slab s's MFMAs (on this hardware vector
+//     and matrix instructions of a SIMD overlap only partly: a k-step costs close to the sum of the two).
 // Bias add and the single fp32 -> fp16 narrowing happen in the epilogue.
 //
 // Work distribution ("stream-K").  The work of a problem is its tiles x k-steps, counted in units of two k-steps and
@@ -52,9 +54,9 @@ namespace {
 constexpr int BN = 256, BK = 64;
 constexpr int ROW_BYTES = BK * 2;  // bytes per staged A row (eight 16-byte chunks, XOR-swizzled with the row)
 constexpr int THREADS = 512;
-// Rows of the tile: 64 * TM, TM = 32-row matrix-core tiles per wavefront (4: 256 x 256, 2: 128 x 256 for grids that
-// leave most of the chip idle with the large tile).  The dynamic LDS allocation is that of TM = 4 for both: three
-// staged A tiles of 32 KiB; the epilogue stages 64 x 64 outputs per wavefront in it (72 KiB).
+// Rows of the tile: 64 * TM (TM = 4: 256 x 256; TM = 2: 128 x 256 for grids that leave most of the chip idle with
+// the large tile).  The dynamic LDS allocation is that of TM = 4 for both: three staged A tiles of 32 KiB; the
+// epilogue stages 64 rows of each wavefront's columns in it (40 KiB).
 constexpr int SMEM_BYTES = 3 * 256 * ROW_BYTES;
 // Order in which a wavefront issues its vector-memory operations in a k-step of the tile GEMM, and what each wait
 // of the step may leave outstanding.  The k-loop states its waits itself (the one in front of the barrier has to: the
