@@ -183,3 +183,27 @@ def test_tile_gemm_offsets_stay_below_four_gib():
     for lda in (limit + 8, limit + 4096, 1 << 24, 1 << 30):
         assert largest(lda) >= (1 << 32)
         assert name(2048, lda) != "mnb_gemm256_kernel"
+
+
+def test_dispatch_on_the_benchmark_layer_shapes():
+    """The kernel choice and the use of a split (workspace) for one Llama-3-8B layer: a guard for the calibrated plan.
+    The plan's inputs are the problem and the device's CU count and clock; without a device it assumes 256 CUs at
+    2.4 GHz, which is what it was calibrated on."""
+    lib = _lib.load()
+    if lib.MnbGetDeviceCount() > 0:
+        import pytest
+        pytest.skip("device properties replace the defaults the expectations below were written for")
+    from onnxruntime_amd.synthetic import C5_SHAPES
+    want = {  # M -> kernel, whether the tile GEMM splits tiles along K
+        "qkv": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
+        "o": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 1), 4096: ("gemm256", 0)},
+        "gate_up": {1: ("skinny", 0), 64: ("mid", 1), 256: ("gemm256", 0), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
+        "down": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 1), 4096: ("gemm256", 0)},
+    }
+    for bits, bs in ((4, 128), (8, 64)):
+        for name, (K, N) in C5_SHAPES.items():
+            for M, (kernel, ws) in want[name].items():
+                got = lib.MnbGemmKernelName(M, N, K, bits, bs, _lib.DTYPE_FLOAT16).decode()
+                assert got == f"mnb_{kernel}_kernel", (bits, name, M, got)
+                need = lib.MnbGemmWorkspaceSize(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16)
+                assert (need > 0) == bool(ws), (bits, name, M, need)
