@@ -19,6 +19,8 @@ pytestmark = pytest.mark.gpu
     (40, 384, 1024, 4, 32, np.float16),     # weight-streaming kernel (staging kernel + main kernel, workspace)
     (300, 512, 1024, 4, 64, np.float16),    # tile GEMM or streaming kernel, by the cost estimate
     (20, 100, 200, 4, 16, np.float32),      # generic kernel
+    (1024, 4096, 4096, 8, 64, np.float16),  # tile GEMM with tiles cut along K (flag-clearing kernel + main kernel)
+    (600, 1500, 512, 4, 128, np.float16),   # tile GEMM, ragged
 ])
 def test_gemm_replays_from_a_hip_graph(M, N, K, bits, bs, dtype):
     c = make_case(M, N, K, bits, bs, dtype, has_zp=True, has_bias=True, seed=M + N)
