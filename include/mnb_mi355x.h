@@ -229,6 +229,14 @@ MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* 
  *   typed zero points, bfloat16:  scales and zero points are widened to fp32 (exactly) and the fp32 kernels run on
  *                    a widened copy of the activations; the fp32 result plus bias is narrowed once.  This is the
  *                    reference's own arithmetic for these inputs (fp32 SGEMM on widened operands, :1336-1510).
+ *   bfloat16, more than 16 rows, packed_k a multiple of 128:  the tile GEMM runs on the same packed matrix with
+ *                    bfloat16 matrix-core operands: w = fma(float(q), scale, -zp * scale) in fp32, narrowed to bfloat16
+ *                    (round to nearest even), products accumulated in fp32, bias added and the sum narrowed in the
+ *                    epilogue.  This is what the reference's GPU provider multiplies for bfloat16 (B dequantised
+ *                    into the activation type, then a GEMM of that type:
+ *                    onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975); the CPU provider has no
+ *                    bfloat16 kernel.  Activations are read in place when 16-byte aligned with a pitch that is a
+ *                    multiple of 8 and no g_idx, else from a bfloat16 copy in the workspace.
  * Zero points are honoured together with g_idx for both zero-point types, as the schema defines; the reference's CPU
  * dequantiser reads uint8 zero points in that combination but then uses 8 (matmul_nbits_impl.cc:56-66).
  * Supported: g_idx with bits = 4; typed zero points with bits = 2 or 4 (the reference rejects 8, :1251-1252). */
@@ -268,6 +276,8 @@ MNB_API size_t MnbVariantGemmWorkspaceSize(const MnbVariantPlan* plan, size_t M)
 MNB_API int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size_t lda, const void* packed_dev,
                            const void* bias_dev, void* y_dev, size_t ldy, void* workspace_dev, size_t workspace_bytes,
                            void* stream);
+/* Name of the GEMM kernel MnbVariantGemm would run for M rows (static string; for logs and profiles). */
+MNB_API const char* MnbVariantGemmKernelName(const MnbVariantPlan* plan, size_t M);
 /* The reference's dequantiser for these inputs, dst_dev float[N][K] whatever a_dtype is
  * (Dequantize4BitsKernelReOrder, matmul_nbits_impl.cc:19-75; 2 bits: MlasDequantizeBlockwiseFpZeroPoint,
  * onnxruntime/core/mlas/lib/q4_dq.cpp:2187-2241): scales and zero points widened to fp32,

@@ -88,6 +88,7 @@ SIGNATURES = {
     "MnbVariantMakePlan": (c_int, [c_size_t, c_size_t, c_int, c_int, c_int, c_int, _I32_P, c_size_t, _PLAN_P]),
     "MnbVariantPack": (c_int, [_PLAN_P, c_void_p, c_void_p, c_void_p, _I32_P, c_size_t, c_void_p, c_void_p]),
     "MnbVariantGemmWorkspaceSize": (c_size_t, [_PLAN_P, c_size_t]),
+    "MnbVariantGemmKernelName": (c_char_p, [_PLAN_P, c_size_t]),
     "MnbVariantGemm": (c_int, [_PLAN_P, c_size_t, c_void_p, c_size_t, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p,
                                c_size_t, c_void_p]),
     "MnbVariantDequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_size_t,

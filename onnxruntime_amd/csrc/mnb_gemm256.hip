@@ -44,6 +44,7 @@
 // cache maintenance); the flags are cleared by a small kernel in front of the launch.
 // Without a workspace the grid is one workgroup per tile and nothing is split.
 #include <cstdlib>
+#include <type_traits>
 
 #include "mnb_buffer.hip.h"
 #include "mnb_device.hip.h"
@@ -186,6 +187,44 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
   return __builtin_bit_cast(h8_t, o);
 }
 
+// ---- bfloat16 models.  The packed matrix is the fp32 models' (meta entries {float scale[, float zero point]}, which
+// also holds zero points that are not integers); activations, bias and output are bfloat16.  A weight is
+// float(q) * scale - zp * scale in fp32 (one fused multiply-add), narrowed to bfloat16 (round to nearest even) as the
+// matrix core's operand; the products accumulate in fp32.
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
+  const bf2_t p = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, p);
+}
+__device__ __forceinline__ float bf16_widen(uint16_t bits) { return __builtin_bit_cast(float, (uint32_t)bits << 16); }
+
+// Packed weights of one lane and slab -> 8 bfloat16 weights in k order (s: scale, c: -zp * scale).
+template <int BITS>
+__device__ __forceinline__ h8_t dequant_word_bf16(uint32_t w0, uint32_t w1, float s, float c) {
+  uint32_t b0, b1;  // bytes: 4-bit e0 e4 e1 e5 | e2 e6 e3 e7 (the packed nibble order); 8-bit e0 e1 e2 e3 | e4 e5 e6 e7
+  if constexpr (BITS == 4) {
+    b0 = w0 & 0x0F0F0F0Fu;
+    b1 = (w0 >> 4) & 0x0F0F0F0Fu;
+  } else {
+    b0 = w0;
+    b1 = w1;
+  }
+  // opaque: otherwise the byte selects below are folded back into a shift and a mask per element
+  asm volatile("" : "+v"(b0), "+v"(b1));
+  auto f = [&](uint32_t b, int byte) { return __builtin_fmaf((float)((b >> (8 * byte)) & 0xffu), s, c); };
+  u4_t o;
+  if constexpr (BITS == 4) {
+    o = u4_t{bf16_pair(f(b0, 0), f(b0, 2)), bf16_pair(f(b1, 0), f(b1, 2)), bf16_pair(f(b0, 1), f(b0, 3)),
+             bf16_pair(f(b1, 1), f(b1, 3))};
+  } else {
+    o = u4_t{bf16_pair(f(b0, 0), f(b0, 1)), bf16_pair(f(b0, 2), f(b0, 3)), bf16_pair(f(b1, 0), f(b1, 1)),
+             bf16_pair(f(b1, 2), f(b1, 3))};
+  }
+  return __builtin_bit_cast(h8_t, o);
+}
+
 // End of one slab section (its matrix instructions, the LDS reads and the dequantisation of the next slab's operands,
 // a group of loads).  Inside a section the compiler's scheduler interleaves freely; it does that slightly better than
 // a hand-written order of "one MFMA, one LDS read, two loads, n VALU" per matrix instruction (measured: 1-2 % on every
@@ -203,7 +242,8 @@ __device__ __forceinline__ void slab_end() {
 // 32 TM rows x 64 columns, and the two wavefront rows dequantise the same columns.  WM = 1 (1 x 8): a wavefront owns
 // all 64 TM rows x 32 columns: every column is dequantised once per workgroup (half the vector instructions) and
 // every wavefront reads the whole staged A tile (twice the LDS reads).
-template <int BITS, bool HAS_ZP, int MPS, int TM, int WM>
+// DT: 0 = fp16 model (packed with fp16 meta entries), 1 = bfloat16 model (packed with fp32 meta entries).
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT>
 __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int WN = 8 / WM;         // wavefront columns
   constexpr int CT = WM;             // 32-column matrix-core tiles per wavefront: 256 / (32 WN)
@@ -229,9 +269,10 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   f16_t acc[RT][CT];
 
   // Two register sets for the weight prefetch (distance: two k-steps); the activations need none.
+  using meta_t = std::conditional_t<DT == 1 && HAS_ZP, u2_t, uint32_t>;  // fp16: {scale, zp} halves; bf16: floats
   struct Stage {
     u2_t b[VEC_PER_STEP][CT];     // [vector of the k-step][column tile]
-    uint32_t m[MPS][CT];          // meta entries of the blocks of the k-step (see m_off)
+    meta_t m[MPS][CT];            // meta entries of the blocks of the k-step (see m_off)
   };
   Stage R0, R1;
   h8_t FA0[RT], FA1[RT];  // A operands, double buffered over slabs
@@ -251,7 +292,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   uint32_t a_off[A_LOADS];                     // byte offsets from a_tile + k0; set per tile (rows beyond M)
   // this lane's weight columns (one per column tile): its 8 bytes inside each 16-byte vector, and its meta entries.
   // The block of a lane's half vector is (k-group base >> bs_shift), plus kq when 4-bit blocks are 16 wide.
-  constexpr int META_BYTES = HAS_ZP ? 4 : 2;
+  constexpr int META_BYTES = (DT == 1 ? 2 : 1) * (HAS_ZP ? 4 : 2);
   const bool small_bs = (BITS == 4) && p.bs_shift == 4;
   // Without zero points an entry is a 16-bit scale.  A 16-bit load would be zero-extended, or packed with its
   // neighbour, right behind the load, which needs the data at once and defeats the prefetch: the lane loads the
@@ -262,7 +303,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     const int col = wn * WCOLS + j * 32 + li;  // within the tile; tiles start at multiples of 256 columns
     w_off[j] = (uint32_t)(col * 16 + kq * 8);
     const uint32_t m_byte = (uint32_t)((mnb_meta_col(col) + (small_bs ? kq * p.Npad : 0)) * META_BYTES);
-    m_off[j] = m_byte & ~3u;
+    m_off[j] = DT == 1 ? m_byte : (m_byte & ~3u);
     m_shift[j] = (m_byte & 2u) * 8;
   }
   const int last_step = p.ksteps - 1;
@@ -300,7 +341,12 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       const int64_t kb = ((int64_t)ks * BK + e * (BK / MPS)) >> p.bs_shift;  // block of the entry's first element
       const rsrc_t r = mnb_rsrc(meta_tile + kb * meta_pitch);
 #pragma unroll
-      for (int j = 0; j < CT; ++j) R.m[e][j] = mnb_buffer_load_b32(r, m_off[j]);
+      for (int j = 0; j < CT; ++j) {
+        if constexpr (DT == 1 && HAS_ZP)
+          R.m[e][j] = mnb_buffer_load_b64(r, m_off[j]);
+        else
+          R.m[e][j] = mnb_buffer_load_b32(r, m_off[j]);
+      }
     }
   };
   auto load_b = [&](int ks_raw, Stage& R) {
@@ -321,7 +367,8 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     }
   };
 
-  auto decode = [&](uint32_t raw, int j, h2_t& s2, ZpH& z) {
+  auto decode = [&](auto raw_any, int j, h2_t& s2, ZpH& z) {  // fp16 models only
+    const uint32_t raw = (uint32_t)raw_any;
     if constexpr (HAS_ZP) {
       const h2_t m = mnb_as_h2(raw);
       s2 = mnb_h2(m.x);
@@ -336,15 +383,26 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   auto make_b = [&](int kk, const Stage& R, h8_t* FB) {
 #pragma unroll
     for (int j = 0; j < CT; ++j) {
-      h2_t s2;
-      ZpH z;
-      if constexpr (BITS == 4) {
-        const int v = kk >> 1;
-        decode(R.m[v][j], j, s2, z);
-        FB[j] = dequant_word<4>(R.b[v][j][kk & 1], 0u, uc, z, s2);
+      const int v = BITS == 4 ? kk >> 1 : kk;           // the vector of the slab
+      const int e = BITS == 4 ? kk >> 1 : kk * MPS / 4;  // its meta entry
+      const uint32_t w0 = BITS == 4 ? R.b[v][j][kk & 1] : R.b[v][j][0];
+      const uint32_t w1 = BITS == 4 ? 0u : R.b[v][j][1];
+      if constexpr (DT == 1) {
+        float sc, zp;
+        if constexpr (HAS_ZP) {
+          const uint32_t sc_bits = R.m[e][j][0], zp_bits = R.m[e][j][1];  // (a bit cast straight from a vector
+          sc = __builtin_bit_cast(float, sc_bits);                        // element reads element 0 for both)
+          zp = __builtin_bit_cast(float, zp_bits);
+        } else {
+          sc = __builtin_bit_cast(float, R.m[e][j]);
+          zp = (float)(1 << (BITS - 1));
+        }
+        FB[j] = dequant_word_bf16<BITS>(w0, w1, sc, -zp * sc);
       } else {
-        decode(R.m[kk * MPS / 4][j], j, s2, z);
-        FB[j] = dequant_word<8>(R.b[kk][j][0], R.b[kk][j][1], uc, z, s2);
+        h2_t s2;
+        ZpH z;
+        decode(R.m[e][j], j, s2, z);
+        FB[j] = dequant_word<BITS>(w0, w1, uc, z, s2);
       }
     }
   };
@@ -368,7 +426,14 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     for (int i = 0; i < RT; ++i)
 #pragma unroll
       for (int j = 0; j < CT; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(FA[i], FB[j], acc[i][j], 0, 0, 0);
+        if constexpr (DT == 1) {
+#if defined(__HIP_DEVICE_COMPILE__)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, FA[i]),
+                                                               __builtin_bit_cast(bf8_t, FB[j]), acc[i][j], 0, 0, 0);
+#endif
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(FA[i], FB[j], acc[i][j], 0, 0, 0);
+        }
   };
 
   // One k-step.  On entry: the staged tile at `cur` holds A of step ks, the one at `nxt` is receiving A of step ks+1,
@@ -415,6 +480,16 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     mfma_slab(FA1, FB1);
     load_b_slot(ks + 3, Rn, 4);
     slab_end<SLAB_FENCE>();
+  };
+
+  // bias and output in the model's 16-bit type (the pointers are typed _Float16 for both: bfloat16 travels as bits)
+  auto widen_elem = [](_Float16 v) {
+    if constexpr (DT == 1) return bf16_widen(__builtin_bit_cast(uint16_t, v));
+    else return (float)v;
+  };
+  auto narrow_elem = [](float v) {
+    if constexpr (DT == 1) return __builtin_bit_cast(_Float16, (__bf16)v);
+    else return (_Float16)v;
   };
 
   // ---- this workgroup's share of the units, walked from the top down
@@ -567,7 +642,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
     for (int j = 0; j < CT; ++j) {
       const int n = n0 + wn * WCOLS + j * 32 + li_e;
-      bcol[j] = (p.bias && n < p.N) ? (float)p.bias[n] : 0.f;
+      bcol[j] = (p.bias && n < p.N) ? widen_elem(p.bias[n]) : 0.f;
     }
     if (p.c_vec_ok) {
       // a wavefront stages 64 rows x WCOLS columns at a time
@@ -586,7 +661,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
             for (int r = 0; r < 16; ++r)
               ep[(ii * 32 + (r >> 2) * 8 + kq_e * 4 + (r & 3)) * EP_STRIDE + j * 32 + li_e] =
-                  (_Float16)(acc[2 * h + ii][j][r] + bcol[j]);
+                  narrow_elem(acc[2 * h + ii][j][r] + bcol[j]);
         // LDS operations of one wavefront complete in issue order: the reads below see the writes above
         if (p.epi_kind == kMnbFusedMlp) {
           // a staged row is gate0 up0 [gate1 up1] (16 columns each) = 16 CT output columns: 2 CT lanes per row, each
@@ -604,8 +679,8 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
             h8_t y;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const float gf = (float)g[e];
-              y[e] = (_Float16)(gf / (1.0f + __expf(-gf)) * (float)u[e]);
+              const float gf = widen_elem(g[e]);
+              y[e] = narrow_elem(gf / (1.0f + __expf(-gf)) * widen_elem(u[e]));
             }
             const int m = m0 + wm * 32 * RT + h * 64 + row;
             if (m < p.M && n_glu < p.n_out0) *reinterpret_cast<h8_t*>(p.C + (int64_t)m * p.ldc + n_glu) = y;
@@ -642,7 +717,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int m = m0 + wm * 32 * RT + i * 32 + (r >> 2) * 8 + kq_e * 4 + (r & 3);
-            if (m < p.M) p.C[(int64_t)m * p.ldc + n] = (_Float16)(acc[i][j][r] + bcol[j]);
+            if (m < p.M) p.C[(int64_t)m * p.ldc + n] = narrow_elem(acc[i][j][r] + bcol[j]);
           }
         }
       }
@@ -655,10 +730,10 @@ __global__ void __launch_bounds__(256) mnb_gemm256_clear_flags_kernel(uint32_t* 
   for (int i = threadIdx.x; i < n; i += 256) flags[i] = 0u;
 }
 
-template <int BITS, bool HAS_ZP, int MPS, int TM, int WM>
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT>
 hipError_t launch_wm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
   const size_t smem = (size_t)SMEM_BYTES;  // 98304 bytes
-  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM>;
+  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM, DT>;
   // The attribute belongs to the function on the current device, so it is set on every launch (a host-side table
   // update, no device work): callers on several threads or devices need no shared flag.
   if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -672,18 +747,27 @@ hipError_t launch_wm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
 // The 1 x 8 arrangement of the wavefronts is faster on every shape and block size measured (0.84 ... 0.98 of the
 // 2 x 4 arrangement's time, bit-identical results): matrix and vector instructions hardly overlap on a SIMD, so the
 // halved dequantisation work counts in full.  The 2 x 4 arrangement is compiled into calibration builds only.
-template <int BITS, bool HAS_ZP, int MPS, int TM>
+template <int BITS, bool HAS_ZP, int MPS, int TM, int DT>
 hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
 #if defined(MNB_TUNING_HOOKS)
   if (const char* e = mnb_tuning_env("MNB_GEMM256_WAVE_ROWS"); e != nullptr && e[0] == '2')
-    return launch_wm<BITS, HAS_ZP, MPS, TM, 2>(p, grid, s);
+    return launch_wm<BITS, HAS_ZP, MPS, TM, 2, DT>(p, grid, s);
 #endif
-  return launch_wm<BITS, HAS_ZP, MPS, TM, 1>(p, grid, s);
+  return launch_wm<BITS, HAS_ZP, MPS, TM, 1, DT>(p, grid, s);
 }
 
+// bfloat16 with four 8-byte meta entries per column and k-step (8-bit weights in blocks of 16 with zero points) does not
+// fit the register file at 256 rows: that model runs on 128-row tiles only (mnb_gemm256_plan knows).
+template <bool HAS_ZP, int MPS>
+constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
+
 template <int BITS, bool HAS_ZP, int MPS>
-hipError_t launch(const Gemm256Params& p, unsigned grid, hipStream_t s) {
-  return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4>(p, grid, s);
+hipError_t launch(const Gemm256Params& p, unsigned grid, bool bf16, hipStream_t s) {
+  if (bf16) {
+    if constexpr (!kBf16Has256Rows<HAS_ZP, MPS>) return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 1>(p, grid, s) : hipErrorInvalidValue;
+    else return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 1>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 1>(p, grid, s);
+  }
+  return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 0>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 0>(p, grid, s);
 }
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
@@ -747,9 +831,13 @@ MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspa
   const int64_t ksteps = L.K / BK, upt = ksteps / 2;
   const plan_model::Variant& v = plan_model::kVariants[L.bits == 4 ? 0 : (L.bs >= 32 ? 1 : 2)];
   const int64_t cus = dev.cus;
+  // a matrix packed for an fp32 model is run by the bfloat16 instantiations, whose 8-bit / block 16 / zero-point
+  // member has no 256-row form (see kBf16Has256Rows)
+  const bool only_128_rows = L.dtype == kMnbDtypeFloat && L.bits == 8 && L.bs < 32 && L.has_zp;
   MnbGemm256Plan best{};
   for (int h = 0; h < 2; ++h) {
     const int rows = h == 0 ? 256 : 128;
+    if (rows == 256 && only_128_rows) continue;
     const int64_t tiles = ((M + rows - 1) / rows) * tiles_n;
     for (int parts = 1; parts <= 8; ++parts) {
       // parts are whole units (two k-steps) of at least 16 k-steps, and never more than two rounds of workgroups:
@@ -767,7 +855,7 @@ MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspa
   }
   if (const char* e = mnb_tuning_env("MNB_GEMM256_PLAN")) {  // calibration: "<tile rows>,<parts>"
     int rows = 0, parts = 0;
-    if (sscanf(e, "%d,%d", &rows, &parts) == 2 && (rows == 128 || rows == 256) && parts >= 1 && parts <= 8 &&
+    if (sscanf(e, "%d,%d", &rows, &parts) == 2 && (rows == 128 || (rows == 256 && !only_128_rows)) && parts >= 1 && parts <= 8 &&
         upt % parts == 0 && (parts == 1 || with_workspace)) {
       const int64_t tiles = ((M + rows - 1) / rows) * tiles_n;
       best = MnbGemm256Plan{};
@@ -802,6 +890,9 @@ bool mnb_gemm256_fused_ok(const MnbEpilogue& e) {
 
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   if (!mnb_gemm256_addressable(a.lda, a.L.Npad)) return hipErrorInvalidValue;  // the dispatcher never sends these
+  // bfloat16 runs on a matrix packed for an fp32 model, fp16 on one packed for fp16; fused outputs are fp16 only
+  if ((a.io_bf16 != 0) != (a.L.dtype == kMnbDtypeFloat) || (a.io_bf16 && a.epi.kind != kMnbFusedNone))
+    return hipErrorInvalidValue;
   Gemm256Params p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
   p.W = reinterpret_cast<const uint8_t*>(a.packed);
@@ -854,9 +945,9 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
     p.ld1 = a.epi.ld[1];
     p.ld2 = a.epi.ld[2];
   }
-  if (a.L.bits == 4) return a.L.has_zp ? launch<4, true, 2>(p, grid, s) : launch<4, false, 2>(p, grid, s);
-  // 8-bit: two entries per k-step fit the register file without spills (also for blocks of 64 and more, where both
-  // entries name the same block); blocks of 16 need four and spill
-  if (a.L.bs >= 32) return a.L.has_zp ? launch<8, true, 2>(p, grid, s) : launch<8, false, 2>(p, grid, s);
-  return a.L.has_zp ? launch<8, true, 4>(p, grid, s) : launch<8, false, 4>(p, grid, s);
+  const bool bf16 = a.io_bf16 != 0;
+  if (a.L.bits == 4) return a.L.has_zp ? launch<4, true, 2>(p, grid, bf16, s) : launch<4, false, 2>(p, grid, bf16, s);
+  // 8-bit: two entries per k-step (also for blocks of 64 and more, where both name the same block); blocks of 16 need four
+  if (a.L.bs >= 32) return a.L.has_zp ? launch<8, true, 2>(p, grid, bf16, s) : launch<8, false, 2>(p, grid, bf16, s);
+  return a.L.has_zp ? launch<8, true, 4>(p, grid, bf16, s) : launch<8, false, 4>(p, grid, bf16, s);
 }

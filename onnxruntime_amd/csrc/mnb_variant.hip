@@ -14,11 +14,16 @@
 //     in the fp16 kernels' integer offset.  The fp32 kernels subtract a float zero point anyway: scales and zero
 //     points are widened to fp32, exactly, at pack time, activations are widened per call, and the fp32 result plus
 //     bias is narrowed once - the reference's own arithmetic for this input (fp32 SGEMM on widened operands).
-//   * bfloat16 activations take the same widened route.
+//   * bfloat16 activations take the same widened route for a few rows (the weight stream bounds those calls, whatever
+//     the arithmetic).  More rows go to the tile GEMM's bfloat16 form on the same packed matrix: weights dequantised
+//     in fp32 and narrowed to bfloat16 for the matrix cores (what the reference's GPU provider multiplies:
+//     onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975 dequantises B into the activation type and calls a
+//     GEMM of that type), fp32 accumulation, bias and narrowing in the epilogue.
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <vector>
 
 #include "../../include/mnb_mi355x.h"
@@ -155,6 +160,18 @@ __global__ void __launch_bounds__(256) mnb_variant_stage_a_kernel(const void* __
   if (j >= ld_out) return;
   const int64_t k = gather ? gather[j] : (j < K_in ? j : -1);
   out[m * ld_out + j] = k >= 0 ? (TO)widen(A, m * lda + k, in_kind) : (TO)0;
+}
+
+// The same for 16-bit activations that stay as they are (bfloat16 for the tile GEMM): a gathered or re-pitched copy.
+__global__ void __launch_bounds__(256) mnb_variant_stage_a16_kernel(const uint16_t* __restrict__ A, int64_t lda,
+                                                                    const int32_t* __restrict__ gather,
+                                                                    uint16_t* __restrict__ out, int64_t ld_out,
+                                                                    int64_t K_in) {
+  const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t m = blockIdx.y;
+  if (j >= ld_out) return;
+  const int64_t k = gather ? gather[j] : (j < K_in ? j : -1);
+  out[m * ld_out + j] = k >= 0 ? A[m * lda + k] : (uint16_t)0;
 }
 
 // Y[m][n] = narrow(Y32[m][n] + bias[n])
@@ -406,8 +423,32 @@ struct VariantWorkspace {
   size_t total() const { return staged + y32 + inner; }
 };
 
+// bfloat16 calls of more than this many rows run on the tile GEMM: measured 5 to 14 times faster than the widened route
+// from 17 rows up (a mostly empty 128-row tile still beats the fp32 matrix-core kernel between its two conversion
+// passes); up to 16 rows the fp32 kernel for few rows streams the weights once, which is all such a call costs
+constexpr size_t kTileBf16MinRows = 16;
+
+bool tile_bf16(const MnbVariantPlan& p, size_t M) {
+  size_t min_rows = kTileBf16MinRows;
+  if (const char* e = mnb_tuning_env("MNB_TILE_BF16_MIN_ROWS")) min_rows = (size_t)atoll(e);  // calibration
+  return p.a_dtype == MNB_DTYPE_BFLOAT16 && M > min_rows && p.packed_k % 128 == 0;
+}
+
+// The tile GEMM reads A through 16-byte loads at 32-bit offsets: a caller's A that is not aligned for that, or whose
+// columns have to be gathered, is copied first.
+bool tile_bf16_needs_copy(const MnbVariantPlan& p, const void* a, size_t lda) {
+  return p.has_g_idx || reinterpret_cast<uintptr_t>(a) % 16 != 0 || lda % 8 != 0 ||
+         !mnb_gemm256_addressable((int64_t)lda, packed_layout(p).Npad);
+}
+
 VariantWorkspace variant_workspace(const MnbVariantPlan& p, size_t M) {
   VariantWorkspace w{};
+  if (tile_bf16(p, M)) {
+    // room for the copy whether or not a call needs it: alignment and pitch are not known here
+    w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
+    w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
+    return w;
+  }
   const bool widened = p.compute_dtype != p.a_dtype;
   if (p.has_g_idx || widened) w.staged = round256(M * (size_t)staged_ld(p) * elem_size(p.compute_dtype));
   if (widened) w.y32 = round256(M * (size_t)p.N * sizeof(float));
@@ -448,6 +489,35 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
   const bool widened = p.compute_dtype != p.a_dtype;
   const int in_kind = src_kind(p.a_dtype);
 
+  if (tile_bf16(p, M)) {
+    MnbGemmArgs a{};
+    a.L = packed_layout(p);
+    a.io_bf16 = 1;
+    a.M = (int64_t)M;
+    a.A = a_dev;
+    a.lda = (int64_t)lda;
+    if (tile_bf16_needs_copy(p, a_dev, lda)) {
+      const int64_t ld = staged_ld(p);
+      const int32_t* gather =
+          p.has_g_idx ? reinterpret_cast<const int32_t*>(reinterpret_cast<const uint8_t*>(packed_dev) + p.gather_offset)
+                      : nullptr;
+      const dim3 grid((unsigned)((ld + 255) / 256), (unsigned)M), blk(256);
+      mnb_variant_stage_a16_kernel<<<grid, blk, 0, s>>>(reinterpret_cast<const uint16_t*>(a_dev), (int64_t)lda, gather,
+                                                        reinterpret_cast<uint16_t*>(ws), ld, p.K);
+      if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "MnbVariantGemm");
+      a.A = ws;
+      a.lda = ld;
+    }
+    a.packed = packed_dev;
+    a.bias = bias_dev;
+    a.C = y_dev;
+    a.ldc = (int64_t)ldy;
+    a.workspace = w.inner > 0 ? ws + w.staged : nullptr;
+    a.workspace_bytes = w.inner;
+    const hipError_t e = mnb_launch_gemm256(a, s);
+    return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbVariantGemm");
+  }
+
   const void* a_in = a_dev;
   size_t ld_in = lda;
   if (w.staged > 0) {
@@ -479,6 +549,13 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return hip_fail(e, "MnbVariantGemm");
   }
   return MNB_OK;
+}
+
+const char* MnbVariantGemmKernelName(const MnbVariantPlan* plan, size_t M) {
+  if (plan == nullptr || plan->packed_bytes == 0 || M == 0) return "none";
+  if (tile_bf16(*plan, M)) return "mnb_gemm256_kernel";
+  return MnbGemmKernelName(M, (size_t)plan->N, (size_t)plan->packed_k, plan->bits, plan->packed_block_size,
+                           plan->compute_dtype);
 }
 
 int MnbVariantDequantize(float* dst_dev, const void* b_dev, const void* scales_dev, const void* zero_points_dev,

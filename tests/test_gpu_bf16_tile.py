@@ -1,0 +1,95 @@
+"""bfloat16 calls with many rows: the tile GEMM on bfloat16 matrix-core operands (weights dequantised in fp32, narrowed
+to bfloat16, fp32 accumulation), through the C ABI's variant entry points and the host class.
+
+The reference's CPU provider has no bfloat16 kernel; its GPU provider dequantises B into bfloat16 and calls a bfloat16
+GEMM (contrib_ops/cuda/quantization/matmul_nbits.cc:844-975), which is the arithmetic here.  Gates: relative L2 <= 5e-3
+against a float64 product over the reference dequantiser's W (the operator's 16-bit tolerance), bit-exact recovery of W
+from unit-vector activations where no operation rounds, and bit-equal results between activations read in place and
+activations that go through the copy (misaligned base, odd pitch)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from onnxruntime_amd import MatMulNBits, _lib
+from oracle import oracle
+from test_gpu_variants import check, make, run_op, to_dev, to_host32, to_np_type
+
+pytestmark = pytest.mark.gpu
+C = oracle.C
+TILE = "mnb_gemm256_kernel"
+
+
+def kernel_name(op, M):
+    return op.lib.MnbVariantGemmKernelName(ctypes.byref(op.plan), M).decode()
+
+
+@pytest.mark.parametrize("bits,bs,zp_kind,g_kind", [
+    (4, 32, "none", "none"), (4, 32, "u8", "none"), (4, 32, "typed", "none"), (4, 128, "typed", "none"),
+    (4, 16, "u8", "none"), (4, 64, "u8", "act_order"), (4, 32, "typed", "act_order"),
+    (8, 32, "none", "none"), (8, 64, "u8", "none"), (8, 16, "u8", "none"), (8, 16, "none", "none"),
+    (2, 32, "u8", "none"), (2, 64, "typed", "none"), (2, 128, "none", "none")])
+@pytest.mark.parametrize("M", [17, 130, 300, 700])
+def test_gemm_against_float64(bits, bs, zp_kind, g_kind, M):
+    N, K = 300, 512
+    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=M + bits + bs, bias=M % 2 == 1)
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == TILE
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (M, N)
+    check("bf16", c, y, N, K, bits, bs)
+
+
+def test_tiles_cut_along_k_and_256_row_tiles():
+    """A deep K on few tiles makes the plan cut tiles along K (partial sums travel through the workspace); many rows
+    select 256-row tiles."""
+    for (M, N, K, bits, bs) in [(200, 256, 8192, 4, 64), (2048, 1024, 1024, 4, 32), (1500, 700, 2048, 8, 128)]:
+        c = make("bf16", N, K, bits, bs, "u8", "none", M, seed=M, bias=True)
+        y, op = run_op("bf16", c, N, K, bits, bs)
+        assert kernel_name(op, M) == TILE
+        check("bf16", c, y, N, K, bits, bs)
+
+
+@pytest.mark.parametrize("bits,bs,zp_kind,g_kind", [
+    (4, 32, "typed", "none"), (4, 32, "none", "none"), (4, 64, "u8", "act_order"), (4, 16, "u8", "none"),
+    (8, 32, "u8", "none"), (8, 16, "u8", "none"), (8, 64, "none", "none"), (2, 32, "typed", "none")])
+def test_unit_vectors_recover_w_exactly(bits, bs, zp_kind, g_kind):
+    """Power-of-two scales and (half-)integer zero points: q - zp has at most 8 significant bits, so neither the fp32
+    dequantisation nor the narrowing to bfloat16 rounds, and row k of I x W must be column k of the reference's W."""
+    N, K = 200, 256
+    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, K, seed=5, exact=True)
+    c["A"] = to_np_type(np.eye(K, dtype=np.float32), "bf16")
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    assert kernel_name(op, K) == TILE
+    w = C.variant_dequantize(c["B"], c["scales"], c["zp"], c["g"], N, K, bits, bs, honour_u8_zp_with_g_idx=True)
+    assert np.array_equal(to_host32(y), w.T)
+
+
+def test_activations_read_in_place_and_through_the_copy_agree():
+    N, K, bits, bs, M = 260, 384, 4, 32, 150
+    c = make("bf16", N, K, bits, bs, "u8", "none", M, seed=9, bias=True)
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    a = to_dev(c["A"])
+    bias = to_dev(c["bias"])
+    wide = torch.zeros(M, K + 3, dtype=torch.bfloat16, device=a.device)   # a pitch that is not a multiple of 8
+    wide[:, :K] = a
+    y2 = op.Compute(wide[:, :K], bias=bias)
+    flat = torch.zeros(M * K + 1, dtype=torch.bfloat16, device=a.device)  # a base that is not 16-byte aligned
+    flat[1:] = a.reshape(-1)
+    y3 = op.Compute(flat[1:].view(M, K), bias=bias)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    assert torch.equal(y.view(torch.int16), y3.view(torch.int16))
+
+
+def test_few_rows_and_other_k_keep_the_widened_route():
+    op = MatMulNBits(512, 300, bits=4, block_size=32, dtype=torch.bfloat16)
+    c = make("bf16", 300, 512, 4, 32, "none", "none", 4, seed=1)
+    d = {k: to_dev(v) for k, v in c.items()}
+    assert op.PrePack(d["B"], d["scales"], None, None)
+    assert kernel_name(op, 16) != TILE and kernel_name(op, 17) == TILE
+    op2 = MatMulNBits(416, 300, bits=4, block_size=32, dtype=torch.bfloat16)
+    c2 = make("bf16", 300, 416, 4, 32, "none", "none", 4, seed=1)
+    d2 = {k: to_dev(v) for k, v in c2.items()}
+    assert op2.PrePack(d2["B"], d2["scales"], None, None)
+    assert kernel_name(op2, 300) != TILE
