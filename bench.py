@@ -352,10 +352,20 @@ def main() -> int:
             mfma_const = v.value
             assert probe.MnbProbeMfmaRate(1, ctypes.byref(v)) == 0
             mfma_rand = v.value
+            # the same kernel, same launches, on activations that are all zero: the instruction stream is identical,
+            # only the switching activity of the operands (and with it the clock the power limit allows) differs
+            a_saved = p4.a.clone()
+            p4.a.zero_()
+            ms4_zero = time_steps(torch, p4.step, k4, max(1, args.warmup // 2), warm_ms=30.0) / 2
+            p4.a.copy_(a_saved)
+            del a_saved
+            tflops_zero = c4.flops() / (ms4_zero * 1e-3) / 1e12
             out["prefill"]["roofline"]["measured_ceiling"] = {
                 "mfma_only_loop_constant_operands_TFLOPs": round(mfma_const, 1),
                 "mfma_only_loop_random_operands_TFLOPs": round(mfma_rand, 1),
                 "frac_of_mfma_only_random": round(tflops / mfma_rand, 4) if mfma_rand > 0 else None,
+                "same_kernel_zero_activations_TFLOPs": round(tflops_zero, 1),
+                "same_kernel_zero_activations_ms_per_launch": round(ms4_zero, 4),
             }
         del p4
         torch.cuda.empty_cache()

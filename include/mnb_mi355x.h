@@ -229,7 +229,7 @@ MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* 
  *   typed zero points, bfloat16:  scales and zero points are widened to fp32 (exactly) and the fp32 kernels run on
  *                    a widened copy of the activations; the fp32 result plus bias is narrowed once.  This is the
  *                    reference's own arithmetic for these inputs (fp32 SGEMM on widened operands, :1336-1510).
- *   bfloat16, more than 16 rows, packed_k a multiple of 128:  the tile GEMM runs on the same packed matrix with
+ *   bfloat16, more than 8 rows, packed_k a multiple of 128:  the tile GEMM runs on the same packed matrix with
  *                    bfloat16 matrix-core operands: w = fma(float(q), scale, -zp * scale) in fp32, narrowed to bfloat16
  *                    (round to nearest even), products accumulated in fp32, bias added and the sum narrowed in the
  *                    epilogue.  This is what the reference's GPU provider multiplies for bfloat16 (B dequantised

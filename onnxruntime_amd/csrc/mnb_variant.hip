@@ -425,8 +425,9 @@ struct VariantWorkspace {
 
 // bfloat16 calls of more than this many rows run on the tile GEMM: measured 5 to 14 times faster than the widened route
 // from 17 rows up (a mostly empty 128-row tile still beats the fp32 matrix-core kernel between its two conversion
-// passes); up to 16 rows the fp32 kernel for few rows streams the weights once, which is all such a call costs
-constexpr size_t kTileBf16MinRows = 16;
+// passes), and ahead of the fp32 kernel for few rows from 9 rows up, where that kernel needs a second pass; up to 8
+// rows the fp32 kernel streams the weights once and is the faster one (14.7 us against 32 us at one row)
+constexpr size_t kTileBf16MinRows = 8;
 
 bool tile_bf16(const MnbVariantPlan& p, size_t M) {
   size_t min_rows = kTileBf16MinRows;
