@@ -26,7 +26,7 @@ struct MnbGemmArgs {
   void* workspace;
   size_t workspace_bytes;
   MnbEpilogue epi;  // kind != kMnbFusedNone: C / ldc are unused, bias is indexed by packed column
-  int io_bf16 = 0;  // tile GEMM only: A, bias and C are bfloat16 and L describes a matrix packed for an fp32 model
+  int io_bf16 = 0;  // tile GEMM and decode kernel: A, bias and C are bfloat16, L describes a matrix packed for an fp32 model
 };
 
 enum MnbKernelKind {

@@ -2,6 +2,7 @@
 // registers (mnb_skinny.hip for M <= 16, mnb_mid.hip for 16 < M): kernel parameters, the nibble/byte to "magic half"
 // conversion, the per-chunk register block with its loads, and the constant operands of the correction MFMAs.
 #pragma once
+#include "mnb_bf16.hip.h"
 #include "mnb_device.hip.h"
 #include "mnb_internal.h"
 
@@ -30,6 +31,7 @@ struct SkinnyParams {
   int phase_chunks; // chunks staged in LDS at a time
   int mtr;          // rows of A staged (power of two >= M, <= 16)
   int a_vec_ok;     // A allows 16-byte loads
+  int io_bf16;      // A, bias and C hold bfloat16 bits (MODE 2: the matrix is packed with fp32 meta entries)
   EpiParams epi;
 };
 
@@ -78,6 +80,8 @@ struct ChunkRegs {
   uint4 w[T];
   uint32_t m0[T];  // meta entry of the lane's (first) block: raw bits (32 with zero points, else 16)
   uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
+  uint32_t z0[T];  // MODE 2: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
+  uint32_t z1[T];
 };
 
 // T adjacent meta entries (2 or 4 bytes each) with one load; dst holds the raw bits of each entry
@@ -108,6 +112,36 @@ __device__ __forceinline__ void load_meta_vec(const uint8_t* __restrict__ meta, 
   }
 }
 
+// The same for a matrix packed with fp32 entries ({scale, zero point}: 8 bytes, or {scale}: 4 bytes).
+template <bool HAS_ZP, int T>
+__device__ __forceinline__ void load_meta_vec_f32(const uint8_t* __restrict__ meta, int64_t first, uint32_t* s,
+                                                  uint32_t* z) {
+  if constexpr (HAS_ZP) {
+    const uint2* q = reinterpret_cast<const uint2*>(meta) + first;
+    if constexpr (T == 4) {
+      const uint4 v0 = *reinterpret_cast<const uint4*>(q), v1 = *reinterpret_cast<const uint4*>(q + 2);
+      s[0] = v0.x, z[0] = v0.y, s[1] = v0.z, z[1] = v0.w, s[2] = v1.x, z[2] = v1.y, s[3] = v1.z, z[3] = v1.w;
+    } else if constexpr (T == 2) {
+      const uint4 v = *reinterpret_cast<const uint4*>(q);
+      s[0] = v.x, z[0] = v.y, s[1] = v.z, z[1] = v.w;
+    } else {
+      const uint2 v = *q;
+      s[0] = v.x, z[0] = v.y;
+    }
+  } else {
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(meta) + first;
+    if constexpr (T == 4) {
+      const uint4 v = *reinterpret_cast<const uint4*>(q);
+      s[0] = v.x, s[1] = v.y, s[2] = v.z, s[3] = v.w;
+    } else if constexpr (T == 2) {
+      const uint2 v = *reinterpret_cast<const uint2*>(q);
+      s[0] = v.x, s[1] = v.y;
+    } else {
+      s[0] = *q;
+    }
+  }
+}
+
 // col0 = first column of the workgroup + j; the T tiles of a lane are columns col0 + 16 t.
 template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq, int64_t col0, ChunkRegs<BITS, T>& R) {
@@ -118,6 +152,10 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
   if constexpr (MODE == 0) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
+  } else if constexpr (MODE == 2) {
+    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
+    load_meta_vec_f32<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0, R.z0);
+    if constexpr (BITS == 4) load_meta_vec_f32<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1, R.z1);
   } else {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
     load_meta_vec<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0);
@@ -138,6 +176,14 @@ __device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, in
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
     for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t]);
+  } else if constexpr (MODE == 2) {
+    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      load_meta_vec_f32<HAS_ZP, 1>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol[t], &R.m0[t], &R.z0[t]);
+      if constexpr (BITS == 4)
+        load_meta_vec_f32<HAS_ZP, 1>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol[t], &R.m1[t], &R.z1[t]);
+    }
   } else {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
 #pragma unroll
@@ -195,6 +241,7 @@ __device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, co
     for (int w2 = 0; w2 < NW; ++w2) sum += red[(w2 * T * 4 + tr) * 64 + l];
     return sum;
   };
+  const bool bf16 = p.io_bf16 != 0;
   if (p.epi.kind == kMnbFusedMlp) {
     // adjacent tiles (2u, 2u + 1) are gate and up of output columns [n0 / 2 + 16 u, +16)
     if constexpr (T >= 2) {
@@ -205,9 +252,9 @@ __device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, co
         const int64_t n_out = (n0 >> 1) + u * 16 + (l & 15);
         if (m >= p.M || n_out >= p.epi.n0) continue;
         const int64_t ng = n0 + u * 32 + (l & 15);
-        const float g = total((2 * u) * 4 + r, l) + (float)p.bias[ng];
-        const float up = total((2 * u + 1) * 4 + r, l) + (float)p.bias[ng + 16];
-        p.C[(int64_t)m * p.ldc + n_out] = (_Float16)(g / (1.0f + __expf(-g)) * up);
+        const float g = total((2 * u) * 4 + r, l) + widen16(p.bias[ng], bf16);
+        const float up = total((2 * u + 1) * 4 + r, l) + widen16(p.bias[ng + 16], bf16);
+        p.C[(int64_t)m * p.ldc + n_out] = narrow16(g / (1.0f + __expf(-g)) * up, bf16);
       }
     }
     return;
@@ -219,17 +266,17 @@ __device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, co
     const int64_t n = n0 + t * 16 + (l & 15);
     if (m >= p.M || n >= p.N) continue;
     float sum = total(tr, l);
-    if (p.bias) sum += (float)p.bias[n];
+    if (p.bias) sum += widen16(p.bias[n], bf16);
     if (p.epi.kind == kMnbFusedQkv) {
       if (n >= p.epi.start2) {
-        if (n - p.epi.start2 < p.epi.n2) p.epi.out2[(int64_t)m * p.epi.ld2 + (n - p.epi.start2)] = (_Float16)sum;
+        if (n - p.epi.start2 < p.epi.n2) p.epi.out2[(int64_t)m * p.epi.ld2 + (n - p.epi.start2)] = narrow16(sum, bf16);
       } else if (n >= p.epi.start1) {
-        if (n - p.epi.start1 < p.epi.n1) p.epi.out1[(int64_t)m * p.epi.ld1 + (n - p.epi.start1)] = (_Float16)sum;
+        if (n - p.epi.start1 < p.epi.n1) p.epi.out1[(int64_t)m * p.epi.ld1 + (n - p.epi.start1)] = narrow16(sum, bf16);
       } else if (n < p.epi.n0) {
-        p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
+        p.C[(int64_t)m * p.ldc + n] = narrow16(sum, bf16);
       }
     } else {
-      p.C[(int64_t)m * p.ldc + n] = (_Float16)sum;
+      p.C[(int64_t)m * p.ldc + n] = narrow16(sum, bf16);
     }
   }
 }

@@ -14,11 +14,12 @@
 //     in the fp16 kernels' integer offset.  The fp32 kernels subtract a float zero point anyway: scales and zero
 //     points are widened to fp32, exactly, at pack time, activations are widened per call, and the fp32 result plus
 //     bias is narrowed once - the reference's own arithmetic for this input (fp32 SGEMM on widened operands).
-//   * bfloat16 activations take the same widened route for a few rows (the weight stream bounds those calls, whatever
-//     the arithmetic).  More rows go to the tile GEMM's bfloat16 form on the same packed matrix: weights dequantised
-//     in fp32 and narrowed to bfloat16 for the matrix cores (what the reference's GPU provider multiplies:
-//     onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975 dequantises B into the activation type and calls a
-//     GEMM of that type), fp32 accumulation, bias and narrowing in the epilogue.
+//   * bfloat16 activations use the same packed matrix (fp32 scales and zero points), but the matrix-core kernels run
+//     on it in bfloat16: the decode kernel up to 16 rows, the tile GEMM beyond (k extents that are multiples of 128;
+//     others take the widened route).  Weights are dequantised in fp32 and narrowed to bfloat16 for the matrix cores
+//     (what the reference's GPU provider multiplies: onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975
+//     dequantises B into the activation type and calls a GEMM of that type), fp32 accumulation, bias and narrowing
+//     in the epilogue.
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -423,31 +424,37 @@ struct VariantWorkspace {
   size_t total() const { return staged + y32 + inner; }
 };
 
-// bfloat16 calls of more than this many rows run on the tile GEMM: measured 5 to 14 times faster than the widened route
-// from 17 rows up (a mostly empty 128-row tile still beats the fp32 matrix-core kernel between its two conversion
-// passes), and ahead of the fp32 kernel for few rows from 9 rows up, where that kernel needs a second pass; up to 8
-// rows the fp32 kernel streams the weights once and is the faster one (14.7 us against 32 us at one row)
-constexpr size_t kTileBf16MinRows = 8;
+// bfloat16 runs on the matrix cores in its own type (weights dequantised in fp32 and narrowed to bfloat16): up to 16
+// rows on the decode kernel (any K), beyond on the tile GEMM, which needs a k extent that is a multiple of 128.  What
+// is left (more than 16 rows on another k extent) takes the widened route.  Measured against the widened route on
+// (N, K) = (14336, 4096): 5 to 14 times faster from 17 rows up.
+enum Bf16Route { kBf16None, kBf16Decode, kBf16Tile };
 
-bool tile_bf16(const MnbVariantPlan& p, size_t M) {
-  size_t min_rows = kTileBf16MinRows;
-  if (const char* e = mnb_tuning_env("MNB_TILE_BF16_MIN_ROWS")) min_rows = (size_t)atoll(e);  // calibration
-  return p.a_dtype == MNB_DTYPE_BFLOAT16 && M > min_rows && p.packed_k % 128 == 0;
+Bf16Route bf16_route(const MnbVariantPlan& p, size_t M) {
+  if (p.a_dtype != MNB_DTYPE_BFLOAT16) return kBf16None;
+  if (const char* e = mnb_tuning_env("MNB_BF16_ROUTE")) {  // calibration: "wide" switches the native kernels off
+    if (e[0] == 'w') return kBf16None;
+    if (e[0] == 't' && p.packed_k % 128 == 0) return kBf16Tile;
+  }
+  if (M <= 16) return kBf16Decode;
+  return p.packed_k % 128 == 0 ? kBf16Tile : kBf16None;
 }
 
-// The tile GEMM reads A through 16-byte loads at 32-bit offsets: a caller's A that is not aligned for that, or whose
-// columns have to be gathered, is copied first.
-bool tile_bf16_needs_copy(const MnbVariantPlan& p, const void* a, size_t lda) {
-  return p.has_g_idx || reinterpret_cast<uintptr_t>(a) % 16 != 0 || lda % 8 != 0 ||
+// The tile GEMM reads A through 16-byte loads at 32-bit offsets: a caller's A that is not aligned for that is copied
+// first.  (The decode kernel takes any alignment.)  Columns that have to be gathered are copied for both.
+bool bf16_needs_copy(const MnbVariantPlan& p, Bf16Route route, const void* a, size_t lda) {
+  if (p.has_g_idx) return true;
+  if (route != kBf16Tile) return false;
+  return reinterpret_cast<uintptr_t>(a) % 16 != 0 || lda % 8 != 0 ||
          !mnb_gemm256_addressable((int64_t)lda, packed_layout(p).Npad);
 }
 
 VariantWorkspace variant_workspace(const MnbVariantPlan& p, size_t M) {
   VariantWorkspace w{};
-  if (tile_bf16(p, M)) {
-    // room for the copy whether or not a call needs it: alignment and pitch are not known here
-    w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
-    w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
+  if (const Bf16Route route = bf16_route(p, M); route != kBf16None) {
+    // the tile GEMM gets room for the copy whether or not a call needs it: alignment and pitch are not known here
+    if (route == kBf16Tile || p.has_g_idx) w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
+    if (route == kBf16Tile) w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
     return w;
   }
   const bool widened = p.compute_dtype != p.a_dtype;
@@ -490,14 +497,14 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
   const bool widened = p.compute_dtype != p.a_dtype;
   const int in_kind = src_kind(p.a_dtype);
 
-  if (tile_bf16(p, M)) {
+  if (const Bf16Route route = bf16_route(p, M); route != kBf16None) {
     MnbGemmArgs a{};
     a.L = packed_layout(p);
     a.io_bf16 = 1;
     a.M = (int64_t)M;
     a.A = a_dev;
     a.lda = (int64_t)lda;
-    if (tile_bf16_needs_copy(p, a_dev, lda)) {
+    if (bf16_needs_copy(p, route, a_dev, lda)) {
       const int64_t ld = staged_ld(p);
       const int32_t* gather =
           p.has_g_idx ? reinterpret_cast<const int32_t*>(reinterpret_cast<const uint8_t*>(packed_dev) + p.gather_offset)
@@ -515,7 +522,7 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
     a.ldc = (int64_t)ldy;
     a.workspace = w.inner > 0 ? ws + w.staged : nullptr;
     a.workspace_bytes = w.inner;
-    const hipError_t e = mnb_launch_gemm256(a, s);
+    const hipError_t e = route == kBf16Tile ? mnb_launch_gemm256(a, s) : mnb_launch_skinny(a, s);
     return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbVariantGemm");
   }
 
@@ -554,7 +561,8 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
 
 const char* MnbVariantGemmKernelName(const MnbVariantPlan* plan, size_t M) {
   if (plan == nullptr || plan->packed_bytes == 0 || M == 0) return "none";
-  if (tile_bf16(*plan, M)) return "mnb_gemm256_kernel";
+  if (const Bf16Route route = bf16_route(*plan, M); route != kBf16None)
+    return route == kBf16Tile ? "mnb_gemm256_kernel" : "mnb_skinny_kernel";
   return MnbGemmKernelName(M, (size_t)plan->N, (size_t)plan->packed_k, plan->bits, plan->packed_block_size,
                            plan->compute_dtype);
 }

@@ -1,5 +1,6 @@
-"""bfloat16 calls with many rows: the tile GEMM on bfloat16 matrix-core operands (weights dequantised in fp32, narrowed
-to bfloat16, fp32 accumulation), through the C ABI's variant entry points and the host class.
+"""bfloat16 on the matrix cores in its own type (weights dequantised in fp32, narrowed to bfloat16, fp32
+accumulation): the decode kernel up to 16 rows, the tile GEMM beyond, through the C ABI's variant entry points and the
+host class.
 
 The reference's CPU provider has no bfloat16 kernel; its GPU provider dequantises B into bfloat16 and calls a bfloat16
 GEMM (contrib_ops/cuda/quantization/matmul_nbits.cc:844-975), which is the arithmetic here.  Gates: relative L2 <= 5e-3
@@ -19,6 +20,7 @@ from test_gpu_variants import check, make, run_op, to_dev, to_host32, to_np_type
 pytestmark = pytest.mark.gpu
 C = oracle.C
 TILE = "mnb_gemm256_kernel"
+DECODE = "mnb_skinny_kernel"
 
 
 def kernel_name(op, M):
@@ -30,12 +32,12 @@ def kernel_name(op, M):
     (4, 16, "u8", "none"), (4, 64, "u8", "act_order"), (4, 32, "typed", "act_order"),
     (8, 32, "none", "none"), (8, 64, "u8", "none"), (8, 16, "u8", "none"), (8, 16, "none", "none"),
     (2, 32, "u8", "none"), (2, 64, "typed", "none"), (2, 128, "none", "none")])
-@pytest.mark.parametrize("M", [9, 130, 300, 700])
+@pytest.mark.parametrize("M", [1, 3, 8, 11, 16, 17, 130, 300, 700])
 def test_gemm_against_float64(bits, bs, zp_kind, g_kind, M):
     N, K = 300, 512
     c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=M + bits + bs, bias=M % 2 == 1)
     y, op = run_op("bf16", c, N, K, bits, bs)
-    assert kernel_name(op, M) == TILE
+    assert kernel_name(op, M) == (DECODE if M <= 16 else TILE)
     assert y.dtype == torch.bfloat16 and tuple(y.shape) == (M, N)
     check("bf16", c, y, N, K, bits, bs)
 
@@ -65,6 +67,55 @@ def test_unit_vectors_recover_w_exactly(bits, bs, zp_kind, g_kind):
     assert np.array_equal(to_host32(y), w.T)
 
 
+@pytest.mark.parametrize("N,K,bits,bs,zp_kind,g_kind", [
+    (14336, 4096, 4, 128, "none", "none"),    # the decode benchmark's shape: everything loaded up front
+    (4096, 14336, 4, 32, "u8", "none"),       # general chunk loop
+    (6144, 4096, 8, 64, "u8", "none"),        # three-tile slabs
+    (1000, 416, 4, 32, "typed", "none"),      # K that is not a whole number of chunks: activations staged in LDS
+    (520, 1000, 8, 16, "u8", "none"),
+    (300, 640, 4, 16, "typed", "ragged"),     # gathered columns, blocks of 16
+    (300, 640, 2, 32, "typed", "none")])
+@pytest.mark.parametrize("M", [1, 4, 7, 16])
+def test_decode_shapes_against_float64(N, K, bits, bs, zp_kind, g_kind, M):
+    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=M + N, bias=M % 2 == 0)
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == DECODE
+    check("bf16", c, y, N, K, bits, bs)
+
+
+@pytest.mark.parametrize("bits,bs,zp_kind,g_kind", [
+    (4, 32, "typed", "none"), (4, 128, "none", "none"), (4, 64, "u8", "act_order"), (4, 16, "u8", "none"),
+    (8, 32, "u8", "none"), (8, 16, "none", "none"), (2, 32, "typed", "none")])
+def test_decode_unit_rows_recover_columns_of_w_exactly(bits, bs, zp_kind, g_kind):
+    """Sixteen unit-vector rows e_k: row m of the product must be column k_m of the reference's W, bit for bit
+    (power-of-two scales and (half-)integer zero points: nothing rounds)."""
+    N, K, M = 520, 1024, 16
+    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=6, exact=True)
+    ks = np.random.default_rng(1).choice(K, size=M, replace=False)
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), ks] = 1.0
+    c["A"] = to_np_type(a, "bf16")
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == DECODE
+    w = C.variant_dequantize(c["B"], c["scales"], c["zp"], c["g"], N, K, bits, bs, honour_u8_zp_with_g_idx=True)
+    assert np.array_equal(to_host32(y), w[:, ks].T)
+
+
+def test_decode_misaligned_activations_agree_with_aligned():
+    N, K, bits, bs, M = 520, 1024, 4, 64, 6
+    c = make("bf16", N, K, bits, bs, "u8", "none", M, seed=4, bias=True)
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    a, bias = to_dev(c["A"]), to_dev(c["bias"])
+    flat = torch.zeros(M * (K + 3) + 1, dtype=torch.bfloat16, device=a.device)
+    view = flat[1:].view(M, K + 3)[:, :K]    # odd base, odd pitch: the kernel stages the rows itself
+    view.copy_(a)
+    y2 = op.Compute(view, bias=bias)
+    torch.cuda.synchronize()
+    # the staged kernel splits K over its wavefronts differently: equal up to the rounding of the fp32 sums
+    assert torch.allclose(y.float(), y2.float(), rtol=2e-2, atol=1e-3)
+    check("bf16", c, y2, N, K, bits, bs)
+
+
 def test_activations_read_in_place_and_through_the_copy_agree():
     N, K, bits, bs, M = 260, 384, 4, 32, 150
     c = make("bf16", N, K, bits, bs, "u8", "none", M, seed=9, bias=True)
@@ -82,14 +133,14 @@ def test_activations_read_in_place_and_through_the_copy_agree():
     assert torch.equal(y.view(torch.int16), y3.view(torch.int16))
 
 
-def test_few_rows_and_other_k_keep_the_widened_route():
+def test_route_by_rows_and_k():
     op = MatMulNBits(512, 300, bits=4, block_size=32, dtype=torch.bfloat16)
     c = make("bf16", 300, 512, 4, 32, "none", "none", 4, seed=1)
     d = {k: to_dev(v) for k, v in c.items()}
     assert op.PrePack(d["B"], d["scales"], None, None)
-    assert kernel_name(op, 8) != TILE and kernel_name(op, 9) == TILE
+    assert kernel_name(op, 16) == DECODE and kernel_name(op, 17) == TILE
     op2 = MatMulNBits(416, 300, bits=4, block_size=32, dtype=torch.bfloat16)
     c2 = make("bf16", 300, 416, 4, 32, "none", "none", 4, seed=1)
     d2 = {k: to_dev(v) for k, v in c2.items()}
     assert op2.PrePack(d2["B"], d2["scales"], None, None)
-    assert kernel_name(op2, 300) != TILE
+    assert kernel_name(op2, 16) == DECODE and kernel_name(op2, 300) not in (TILE, DECODE)   # the widened route
