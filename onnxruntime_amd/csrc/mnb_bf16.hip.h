@@ -1,4 +1,5 @@
-// bfloat16 models on the matrix cores (tile GEMM: mnb_gemm256.hip, few rows: mnb_skinny.hip).
+// 16-bit models on a matrix packed with fp32 meta entries - bfloat16 models, and fp16 models whose zero points are in
+// the activation type - on the matrix cores (tile GEMM: mnb_gemm256.hip, few rows: mnb_skinny.hip).
 #pragma once
 #include "mnb_buffer.hip.h"
 #include "mnb_device.hip.h"
@@ -18,9 +19,16 @@ __device__ __forceinline__ uint32_t bf16_pair(float lo, float hi) {
 }
 __device__ __forceinline__ float bf16_widen(uint16_t bits) { return __builtin_bit_cast(float, (uint32_t)bits << 16); }
 
-// Packed weights of one lane and slab -> 8 bfloat16 weights in k order (s: scale, c: -zp * scale).
-template <int BITS>
-__device__ __forceinline__ h8_t dequant_word_bf16(uint32_t w0, uint32_t w1, float s, float c) {
+__device__ __forceinline__ uint32_t f16_pair(float lo, float hi) {
+  const h2_t p = {(_Float16)lo, (_Float16)hi};  // one v_cvt_pk_f16_f32, round to nearest even
+  return __builtin_bit_cast(uint32_t, p);
+}
+
+// Packed weights of one lane and slab -> 8 weights in k order, fma(float(q), s, c) with c = -zp * s, narrowed to
+// bfloat16 (BF16) or fp16.
+template <int BITS, bool BF16>
+__device__ __forceinline__ h8_t dequant_word_wide(uint32_t w0, uint32_t w1, float s, float c) {
+  auto pair = [](float lo, float hi) { return BF16 ? bf16_pair(lo, hi) : f16_pair(lo, hi); };
   uint32_t b0, b1;  // bytes: 4-bit e0 e4 e1 e5 | e2 e6 e3 e7 (the packed nibble order); 8-bit e0 e1 e2 e3 | e4 e5 e6 e7
   if constexpr (BITS == 4) {
     b0 = w0 & 0x0F0F0F0Fu;
@@ -34,11 +42,9 @@ __device__ __forceinline__ h8_t dequant_word_bf16(uint32_t w0, uint32_t w1, floa
   auto f = [&](uint32_t b, int byte) { return __builtin_fmaf((float)((b >> (8 * byte)) & 0xffu), s, c); };
   u4_t o;
   if constexpr (BITS == 4) {
-    o = u4_t{bf16_pair(f(b0, 0), f(b0, 2)), bf16_pair(f(b1, 0), f(b1, 2)), bf16_pair(f(b0, 1), f(b0, 3)),
-             bf16_pair(f(b1, 1), f(b1, 3))};
+    o = u4_t{pair(f(b0, 0), f(b0, 2)), pair(f(b1, 0), f(b1, 2)), pair(f(b0, 1), f(b0, 3)), pair(f(b1, 1), f(b1, 3))};
   } else {
-    o = u4_t{bf16_pair(f(b0, 0), f(b0, 1)), bf16_pair(f(b0, 2), f(b0, 3)), bf16_pair(f(b1, 0), f(b1, 1)),
-             bf16_pair(f(b1, 2), f(b1, 3))};
+    o = u4_t{pair(f(b0, 0), f(b0, 1)), pair(f(b0, 2), f(b0, 3)), pair(f(b1, 0), f(b1, 1)), pair(f(b1, 2), f(b1, 3))};
   }
   return __builtin_bit_cast(h8_t, o);
 }

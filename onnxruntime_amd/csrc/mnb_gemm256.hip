@@ -205,7 +205,8 @@ __device__ __forceinline__ void slab_end() {
 // 32 TM rows x 64 columns, and the two wavefront rows dequantise the same columns.  WM = 1 (1 x 8): a wavefront owns
 // all 64 TM rows x 32 columns: every column is dequantised once per workgroup (half the vector instructions) and
 // every wavefront reads the whole staged A tile (twice the LDS reads).
-// DT: 0 = fp16 model (packed with fp16 meta entries), 1 = bfloat16 model (packed with fp32 meta entries).
+// DT: 0 = fp16 model (packed with fp16 meta entries); on a matrix packed with fp32 meta entries: 1 = bfloat16 model,
+// 2 = fp16 model with zero points in the activation type.
 template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT>
 __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int WN = 8 / WM;         // wavefront columns
@@ -232,7 +233,8 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   f16_t acc[RT][CT];
 
   // Two register sets for the weight prefetch (distance: two k-steps); the activations need none.
-  using meta_t = std::conditional_t<DT == 1 && HAS_ZP, u2_t, uint32_t>;  // fp16: {scale, zp} halves; bf16: floats
+  constexpr bool WIDE = DT != 0;                                          // fp32 meta entries
+  using meta_t = std::conditional_t<WIDE && HAS_ZP, u2_t, uint32_t>;  // fp16 entries: {scale, zp} halves; fp32: floats
   struct Stage {
     u2_t b[VEC_PER_STEP][CT];     // [vector of the k-step][column tile]
     meta_t m[MPS][CT];            // meta entries of the blocks of the k-step (see m_off)
@@ -255,7 +257,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   uint32_t a_off[A_LOADS];                     // byte offsets from a_tile + k0; set per tile (rows beyond M)
   // this lane's weight columns (one per column tile): its 8 bytes inside each 16-byte vector, and its meta entries.
   // The block of a lane's half vector is (k-group base >> bs_shift), plus kq when 4-bit blocks are 16 wide.
-  constexpr int META_BYTES = (DT == 1 ? 2 : 1) * (HAS_ZP ? 4 : 2);
+  constexpr int META_BYTES = (WIDE ? 2 : 1) * (HAS_ZP ? 4 : 2);
   const bool small_bs = (BITS == 4) && p.bs_shift == 4;
   // Without zero points an entry is a 16-bit scale.  A 16-bit load would be zero-extended, or packed with its
   // neighbour, right behind the load, which needs the data at once and defeats the prefetch: the lane loads the
@@ -266,7 +268,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     const int col = wn * WCOLS + j * 32 + li;  // within the tile; tiles start at multiples of 256 columns
     w_off[j] = (uint32_t)(col * 16 + kq * 8);
     const uint32_t m_byte = (uint32_t)((mnb_meta_col(col) + (small_bs ? kq * p.Npad : 0)) * META_BYTES);
-    m_off[j] = DT == 1 ? m_byte : (m_byte & ~3u);
+    m_off[j] = WIDE ? m_byte : (m_byte & ~3u);
     m_shift[j] = (m_byte & 2u) * 8;
   }
   const int last_step = p.ksteps - 1;
@@ -305,7 +307,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       const rsrc_t r = mnb_rsrc(meta_tile + kb * meta_pitch);
 #pragma unroll
       for (int j = 0; j < CT; ++j) {
-        if constexpr (DT == 1 && HAS_ZP)
+        if constexpr (WIDE && HAS_ZP)
           R.m[e][j] = mnb_buffer_load_b64(r, m_off[j]);
         else
           R.m[e][j] = mnb_buffer_load_b32(r, m_off[j]);
@@ -350,7 +352,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
       const int e = BITS == 4 ? kk >> 1 : kk * MPS / 4;  // its meta entry
       const uint32_t w0 = BITS == 4 ? R.b[v][j][kk & 1] : R.b[v][j][0];
       const uint32_t w1 = BITS == 4 ? 0u : R.b[v][j][1];
-      if constexpr (DT == 1) {
+      if constexpr (WIDE) {
         float sc, zp;
         if constexpr (HAS_ZP) {
           const uint32_t sc_bits = R.m[e][j][0], zp_bits = R.m[e][j][1];  // (a bit cast straight from a vector
@@ -360,7 +362,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
           sc = __builtin_bit_cast(float, R.m[e][j]);
           zp = (float)(1 << (BITS - 1));
         }
-        FB[j] = dequant_word_bf16<BITS>(w0, w1, sc, -zp * sc);
+        FB[j] = dequant_word_wide<BITS, DT == 1>(w0, w1, sc, -zp * sc);
       } else {
         h2_t s2;
         ZpH z;
@@ -725,8 +727,14 @@ template <bool HAS_ZP, int MPS>
 constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
 
 template <int BITS, bool HAS_ZP, int MPS>
-hipError_t launch(const Gemm256Params& p, unsigned grid, bool bf16, hipStream_t s) {
-  if (bf16) {
+hipError_t launch(const Gemm256Params& p, unsigned grid, int io, hipStream_t s) {
+  if (io == kMnbIoF16Wide) {  // zero points in the activation type exist for 4-bit (and 2-bit, packed as 4-bit) only
+    if constexpr (BITS == 4 && HAS_ZP)
+      return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 2>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 2>(p, grid, s);
+    else
+      return hipErrorInvalidValue;
+  }
+  if (io == kMnbIoBf16) {
     if constexpr (!kBf16Has256Rows<HAS_ZP, MPS>) return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 1>(p, grid, s) : hipErrorInvalidValue;
     else return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 1>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 1>(p, grid, s);
   }
@@ -853,8 +861,8 @@ bool mnb_gemm256_fused_ok(const MnbEpilogue& e) {
 
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   if (!mnb_gemm256_addressable(a.lda, a.L.Npad)) return hipErrorInvalidValue;  // the dispatcher never sends these
-  // bfloat16 runs on a matrix packed for an fp32 model, fp16 on one packed for fp16; fused outputs are fp16 only
-  if ((a.io_bf16 != 0) != (a.L.dtype == kMnbDtypeFloat) || (a.io_bf16 && a.epi.kind != kMnbFusedNone))
+  // a matrix packed for an fp32 model is run in a 16-bit type named by a.io; fused outputs exist for fp16 models only
+  if ((a.io != kMnbIoModel) != (a.L.dtype == kMnbDtypeFloat) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone))
     return hipErrorInvalidValue;
   Gemm256Params p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
@@ -908,9 +916,8 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
     p.ld1 = a.epi.ld[1];
     p.ld2 = a.epi.ld[2];
   }
-  const bool bf16 = a.io_bf16 != 0;
-  if (a.L.bits == 4) return a.L.has_zp ? launch<4, true, 2>(p, grid, bf16, s) : launch<4, false, 2>(p, grid, bf16, s);
+  if (a.L.bits == 4) return a.L.has_zp ? launch<4, true, 2>(p, grid, a.io, s) : launch<4, false, 2>(p, grid, a.io, s);
   // 8-bit: two entries per k-step (also for blocks of 64 and more, where both name the same block); blocks of 16 need four
-  if (a.L.bs >= 32) return a.L.has_zp ? launch<8, true, 2>(p, grid, bf16, s) : launch<8, false, 2>(p, grid, bf16, s);
-  return a.L.has_zp ? launch<8, true, 4>(p, grid, bf16, s) : launch<8, false, 4>(p, grid, bf16, s);
+  if (a.L.bs >= 32) return a.L.has_zp ? launch<8, true, 2>(p, grid, a.io, s) : launch<8, false, 2>(p, grid, a.io, s);
+  return a.L.has_zp ? launch<8, true, 4>(p, grid, a.io, s) : launch<8, false, 4>(p, grid, a.io, s);
 }

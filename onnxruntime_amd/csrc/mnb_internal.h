@@ -14,6 +14,11 @@ struct MnbEpilogue {
   int64_t ld[3];
 };
 
+// Element type of A, bias and C when it is not the packed matrix's own (MnbGemmArgs::io).
+constexpr int kMnbIoModel = 0;    // L.dtype
+constexpr int kMnbIoBf16 = 1;     // bfloat16 on a matrix packed with fp32 {scale, zero point} entries
+constexpr int kMnbIoF16Wide = 2;  // fp16 on such a matrix (zero points in the activation type: 4-bit with zero points)
+
 struct MnbGemmArgs {
   MnbLayout L;
   int64_t M;
@@ -26,7 +31,8 @@ struct MnbGemmArgs {
   void* workspace;
   size_t workspace_bytes;
   MnbEpilogue epi;  // kind != kMnbFusedNone: C / ldc are unused, bias is indexed by packed column
-  int io_bf16 = 0;  // tile GEMM and decode kernel: A, bias and C are bfloat16, L describes a matrix packed for an fp32 model
+  int io = 0;       // tile GEMM and decode kernel: kMnbIoModel, or A, bias and C in a 16-bit type on a matrix packed for
+                    // an fp32 model (L.dtype is float): kMnbIoBf16, kMnbIoF16Wide
 };
 
 enum MnbKernelKind {

@@ -31,7 +31,7 @@ struct SkinnyParams {
   int phase_chunks; // chunks staged in LDS at a time
   int mtr;          // rows of A staged (power of two >= M, <= 16)
   int a_vec_ok;     // A allows 16-byte loads
-  int io_bf16;      // A, bias and C hold bfloat16 bits (MODE 2: the matrix is packed with fp32 meta entries)
+  int io_bf16;      // A, bias and C hold bfloat16 bits (MODE 2)
   EpiParams epi;
 };
 
@@ -80,7 +80,7 @@ struct ChunkRegs {
   uint4 w[T];
   uint32_t m0[T];  // meta entry of the lane's (first) block: raw bits (32 with zero points, else 16)
   uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
-  uint32_t z0[T];  // MODE 2: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
+  uint32_t z0[T];  // MODE 2 and 3: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
   uint32_t z1[T];
 };
 
@@ -152,7 +152,7 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
   if constexpr (MODE == 0) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
-  } else if constexpr (MODE == 2) {
+  } else if constexpr (MODE >= 2) {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
     load_meta_vec_f32<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0, R.z0);
     if constexpr (BITS == 4) load_meta_vec_f32<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1, R.z1);
@@ -176,7 +176,7 @@ __device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, in
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
     for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t]);
-  } else if constexpr (MODE == 2) {
+  } else if constexpr (MODE >= 2) {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
 #pragma unroll
     for (int t = 0; t < T; ++t) {

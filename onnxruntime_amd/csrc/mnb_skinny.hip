@@ -21,6 +21,8 @@
 //  * MODE 2 (bfloat16 models, whose matrix is packed with fp32 {scale, zero point} entries): weights dequantised in
 //    fp32, fma(float(q), scale, -zp * scale), narrowed to bfloat16 and multiplied by v_mfma_f32_16x16x32_bf16; A,
 //    bias and Y hold bfloat16 bits.
+//  * MODE 3 (fp16 models with zero points in the activation type, packed the same way): as MODE 2 with the weights
+//    narrowed to fp16 and the fp16 matrix instruction.
 //  * The A operands come straight from global memory (L2 hits after the first workgroup) when the rows of A are
 //    16-byte aligned -- every load of a wavefront's first two chunks is issued before anything is waited for;
 //    otherwise the rows are staged in LDS phase by phase (zero-filled beyond K, any alignment).
@@ -74,7 +76,7 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
         for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, d[r], y[t][r]);
       }
     }
-  } else if constexpr (MODE == 2) {
+  } else if constexpr (MODE >= 2) {
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
@@ -85,9 +87,12 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const bool second = (BITS == 4) && i >= 2;
-        const h8_t b = BITS == 4 ? dequant_word_bf16<BITS>(wd[i], 0u, second ? s1 : s0, second ? c1 : c0)
-                                 : dequant_word_bf16<BITS>(wd[(2 * i) & 3], wd[(2 * i + 1) & 3], s0, c0);
-        y[t] = mfma16_bf16(af[i], b, y[t]);
+        const h8_t b = BITS == 4 ? dequant_word_wide<BITS, MODE == 2>(wd[i], 0u, second ? s1 : s0, second ? c1 : c0)
+                                 : dequant_word_wide<BITS, MODE == 2>(wd[(2 * i) & 3], wd[(2 * i + 1) & 3], s0, c0);
+        if constexpr (MODE == 2)
+          y[t] = mfma16_bf16(af[i], b, y[t]);
+        else
+          y[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], b, y[t], 0, 0, 0);
       }
     }
   } else {
@@ -451,13 +456,13 @@ int pow2_ceil(int v) {
   return r;
 }
 
-SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
+SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int min_t) {
   SkinnyPlan pl;
   const int GK = L.group_k, CK = 4 * GK;
   const int chunks = (int)((L.K + CK - 1) / CK);
   pl.mode = (L.bs >= CK) ? 0 : 1;
   if (const char* e = mnb_tuning_env("MNB_SKINNY_MODE")) pl.mode = e[0] == '1' ? 1 : pl.mode;  // calibration: exact halves
-  if (L.dtype == kMnbDtypeFloat) pl.mode = 2;  // bfloat16 model
+  if (io != kMnbIoModel) pl.mode = io == kMnbIoBf16 ? 2 : 3;  // fp32 meta entries
   pl.mtr = pow2_ceil((int)M);
   // workgroups: as many column slabs as fill the chip; wide slabs (T = 4) amortise the A operands best
   const int64_t tiles = (L.N + 15) / 16;
@@ -483,8 +488,8 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int64_t M, bool direct, int min_t) {
   const bool up_front = chunks == pl.nw || chunks == 2 * pl.nw;  // everything loaded before the first wait
   pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4);
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
-  // the fp32 dequantisation of bfloat16 models does not fit the 128 registers of sixteen wavefronts in the general loop
-  if (pl.mode == 2 && !up_front && pl.nw == 16) pl.nw = 8;
+  // the fp32 dequantisation of modes 2 and 3 does not fit the 128 registers of sixteen wavefronts in the general loop
+  if (pl.mode >= 2 && !up_front && pl.nw == 16) pl.nw = 8;
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
   pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
@@ -506,7 +511,7 @@ hipError_t launch_slab(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
   const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
   // the plan never asks for the LDS route in the general loop of sixteen wavefronts on 4-bit weights: not instantiated
   if (pl.a_lds && cpw == 0 && BITS == 4 && pl.nw == 16) return hipErrorInvalidConfiguration;
-  if (MODE == 2 && cpw == 0 && pl.nw == 16) return hipErrorInvalidConfiguration;  // (nor bfloat16 there at all)
+  if (MODE >= 2 && cpw == 0 && pl.nw == 16) return hipErrorInvalidConfiguration;  // (nor the fp32-entry modes at all)
 #define MNB_SLAB_LAUNCH(NW_, CPW_, LDS_) \
   mnb_skinny_slab_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_>                  \
       <<<grid, dim3(NW_ * 64), pl.smem, s>>>(MNB_SKINNY_HOT_ARGS(p), p)
@@ -524,7 +529,7 @@ hipError_t launch_slab(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
         MNB_SLAB_LAUNCH(NW_, 1, false);                             \
       else if (cpw == 2)                                            \
         MNB_SLAB_LAUNCH(NW_, 2, false);                             \
-      else if constexpr (!(MODE == 2 && NW_ == 16))                 \
+      else if constexpr (!(MODE >= 2 && NW_ == 16))                 \
         MNB_SLAB_LAUNCH(NW_, 0, false);                             \
     }                                                               \
   } while (0)
@@ -545,7 +550,7 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
     const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
     // not instantiated, never planned: LDS route in the general loop of four-tile slabs or of sixteen 4-bit wavefronts
     if (pl.a_lds && cpw == 0 && (T == 4 || (BITS == 4 && pl.nw == 16))) return hipErrorInvalidConfiguration;
-    if (MODE == 2 && cpw == 0 && pl.nw == 16) return hipErrorInvalidConfiguration;  // (nor bfloat16 there at all)
+    if (MODE >= 2 && cpw == 0 && pl.nw == 16) return hipErrorInvalidConfiguration;  // (nor the fp32-entry modes at all)
 #define MNB_SKINNY_LAUNCH(NW_, CPW_, LDS_) \
   mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_>                \
       <<<grid, dim3(NW_ * 64), pl.smem, s>>>(MNB_SKINNY_HOT_ARGS(p), p)
@@ -563,7 +568,7 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
         MNB_SKINNY_LAUNCH(NW_, 1, false);                           \
       else if (cpw == 2)                                            \
         MNB_SKINNY_LAUNCH(NW_, 2, false);                           \
-      else if constexpr (!(MODE == 2 && NW_ == 16))                 \
+      else if constexpr (!(MODE >= 2 && NW_ == 16))                 \
         MNB_SKINNY_LAUNCH(NW_, 0, false);                           \
     }                                                               \
   } while (0)
@@ -594,22 +599,26 @@ hipError_t launch_mode(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
 template <int BITS, bool HAS_ZP>
 hipError_t launch_zp(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
   if (pl.mode == 2) return launch_mode<BITS, HAS_ZP, 2>(p, pl, s);
+  if (pl.mode == 3) {
+    if constexpr (BITS == 4 && HAS_ZP) return launch_mode<BITS, HAS_ZP, 3>(p, pl, s);
+    else return hipErrorInvalidValue;  // zero points in the activation type: 4-bit with zero points
+  }
   return pl.mode == 0 ? launch_mode<BITS, HAS_ZP, 0>(p, pl, s) : launch_mode<BITS, HAS_ZP, 1>(p, pl, s);
 }
 
 }  // namespace
 
 bool mnb_skinny_applicable(const MnbGemmArgs& a) {
-  // fp16 models, and bfloat16 ones (io_bf16) on a matrix packed with fp32 meta entries
-  return (a.io_bf16 ? a.L.dtype == kMnbDtypeFloat : a.L.dtype == kMnbDtypeFloat16) && a.M >= 1 && a.M <= 16;
+  // fp16 models, and 16-bit ones (a.io) on a matrix packed with fp32 meta entries
+  return (a.io != kMnbIoModel ? a.L.dtype == kMnbDtypeFloat : a.L.dtype == kMnbDtypeFloat16) && a.M >= 1 && a.M <= 16;
 }
 
 hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
-  if (!mnb_skinny_applicable(a) || (a.io_bf16 && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
+  if (!mnb_skinny_applicable(a) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
   // direct variant: 16-byte loads of whole chunks of A
   const bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
-  SkinnyPlan pl = skinny_plan(L, a.M, a_vec_ok, a.epi.kind == kMnbFusedMlp ? 2 : 1);
+  SkinnyPlan pl = skinny_plan(L, a.io, a.M, a_vec_ok, a.epi.kind == kMnbFusedMlp ? 2 : 1);
   SkinnyParams p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
   p.W = reinterpret_cast<const uint4*>(a.packed);
@@ -628,7 +637,7 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   p.phase_chunks = pl.phase_chunks;
   p.mtr = pl.mtr;
   p.a_vec_ok = a_vec_ok;
-  p.io_bf16 = a.io_bf16;
+  p.io_bf16 = a.io == kMnbIoBf16;
   p.epi.kind = a.epi.kind;
   if (a.epi.kind != kMnbFusedNone) {
     p.C = reinterpret_cast<_Float16*>(a.epi.out[0]);

@@ -11,15 +11,16 @@
 //     order once; per call the activation columns are gathered into the same order, with zeros in the padding (so
 //     the padded weights never count).
 //   * zero points in the activation type are not integers (HQQ-style quantisers produce them), so they cannot ride
-//     in the fp16 kernels' integer offset.  The fp32 kernels subtract a float zero point anyway: scales and zero
-//     points are widened to fp32, exactly, at pack time, activations are widened per call, and the fp32 result plus
-//     bias is narrowed once - the reference's own arithmetic for this input (fp32 SGEMM on widened operands).
-//   * bfloat16 activations use the same packed matrix (fp32 scales and zero points), but the matrix-core kernels run
-//     on it in bfloat16: the decode kernel up to 16 rows, the tile GEMM beyond (k extents that are multiples of 128;
-//     others take the widened route).  Weights are dequantised in fp32 and narrowed to bfloat16 for the matrix cores
-//     (what the reference's GPU provider multiplies: onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975
-//     dequantises B into the activation type and calls a GEMM of that type), fp32 accumulation, bias and narrowing
-//     in the epilogue.
+//     in the fp16 kernels' integer offset: scales and zero points are widened to fp32, exactly, at pack time (the
+//     matrix is packed as an fp32 model's).  fp32 models run the fp32 kernels on it.  The widened route for 16-bit
+//     models does the same on a widened copy of the activations and narrows the fp32 result plus bias once - the
+//     reference's own arithmetic for this input (fp32 SGEMM on widened operands).
+//   * 16-bit models on such a matrix - bfloat16 (always packed this way), fp16 with zero points in the activation
+//     type - normally skip the widened route: the decode kernel (up to 16 rows) and the tile GEMM (beyond, for k
+//     extents that are multiples of 128) dequantise the weights in fp32, narrow them to the activation type for the
+//     matrix cores (what the reference's GPU provider multiplies:
+//     onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975 dequantises B into the activation type and
+//     calls a GEMM of that type), accumulate in fp32, and add bias and narrow in the epilogue.
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -424,37 +425,45 @@ struct VariantWorkspace {
   size_t total() const { return staged + y32 + inner; }
 };
 
-// bfloat16 runs on the matrix cores in its own type (weights dequantised in fp32 and narrowed to bfloat16): up to 16
-// rows on the decode kernel (any K), beyond on the tile GEMM, which needs a k extent that is a multiple of 128.  What
-// is left (more than 16 rows on another k extent) takes the widened route.  Measured against the widened route on
-// (N, K) = (14336, 4096): 5 to 14 times faster from 17 rows up.
-enum Bf16Route { kBf16None, kBf16Decode, kBf16Tile };
+// 16-bit activations on a matrix packed with fp32 entries - bfloat16 models, and fp16 models whose zero points are in
+// the activation type - run on the matrix cores in their own type (weights dequantised in fp32 and narrowed): up to
+// 16 rows on the decode kernel (any K), beyond on the tile GEMM, which needs a k extent that is a multiple of 128.
+// What is left (more than 16 rows on another k extent) takes the widened route.  Measured against the widened route
+// on (N, K) = (14336, 4096), bfloat16: 5 to 14 times faster from 17 rows up, 1.4 to 6 times up to 16 rows.
+enum NativeRoute { kNativeNone, kNativeDecode, kNativeTile };
 
-Bf16Route bf16_route(const MnbVariantPlan& p, size_t M) {
-  if (p.a_dtype != MNB_DTYPE_BFLOAT16) return kBf16None;
-  if (const char* e = mnb_tuning_env("MNB_BF16_ROUTE")) {  // calibration: "wide" switches the native kernels off
-    if (e[0] == 'w') return kBf16None;
-    if (e[0] == 't' && p.packed_k % 128 == 0) return kBf16Tile;
+// kMnbIoModel when the plan's kernels run in the compute type (fp32 models, fp16 models with integer zero points)
+int native_io(const MnbVariantPlan& p) {
+  if (p.a_dtype == MNB_DTYPE_BFLOAT16) return kMnbIoBf16;
+  if (p.a_dtype == MNB_DTYPE_FLOAT16 && p.compute_dtype == MNB_DTYPE_FLOAT) return kMnbIoF16Wide;  // typed zero points
+  return kMnbIoModel;
+}
+
+NativeRoute native_route(const MnbVariantPlan& p, size_t M) {
+  if (native_io(p) == kMnbIoModel) return kNativeNone;
+  if (const char* e = mnb_tuning_env("MNB_NATIVE_ROUTE")) {  // calibration: "wide" switches the native kernels off
+    if (e[0] == 'w') return kNativeNone;
+    if (e[0] == 't' && p.packed_k % 128 == 0) return kNativeTile;
   }
-  if (M <= 16) return kBf16Decode;
-  return p.packed_k % 128 == 0 ? kBf16Tile : kBf16None;
+  if (M <= 16) return kNativeDecode;
+  return p.packed_k % 128 == 0 ? kNativeTile : kNativeNone;
 }
 
 // The tile GEMM reads A through 16-byte loads at 32-bit offsets: a caller's A that is not aligned for that is copied
 // first.  (The decode kernel takes any alignment.)  Columns that have to be gathered are copied for both.
-bool bf16_needs_copy(const MnbVariantPlan& p, Bf16Route route, const void* a, size_t lda) {
+bool native_needs_copy(const MnbVariantPlan& p, NativeRoute route, const void* a, size_t lda) {
   if (p.has_g_idx) return true;
-  if (route != kBf16Tile) return false;
+  if (route != kNativeTile) return false;
   return reinterpret_cast<uintptr_t>(a) % 16 != 0 || lda % 8 != 0 ||
          !mnb_gemm256_addressable((int64_t)lda, packed_layout(p).Npad);
 }
 
 VariantWorkspace variant_workspace(const MnbVariantPlan& p, size_t M) {
   VariantWorkspace w{};
-  if (const Bf16Route route = bf16_route(p, M); route != kBf16None) {
+  if (const NativeRoute route = native_route(p, M); route != kNativeNone) {
     // the tile GEMM gets room for the copy whether or not a call needs it: alignment and pitch are not known here
-    if (route == kBf16Tile || p.has_g_idx) w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
-    if (route == kBf16Tile) w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
+    if (route == kNativeTile || p.has_g_idx) w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
+    if (route == kNativeTile) w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
     return w;
   }
   const bool widened = p.compute_dtype != p.a_dtype;
@@ -497,14 +506,14 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
   const bool widened = p.compute_dtype != p.a_dtype;
   const int in_kind = src_kind(p.a_dtype);
 
-  if (const Bf16Route route = bf16_route(p, M); route != kBf16None) {
+  if (const NativeRoute route = native_route(p, M); route != kNativeNone) {
     MnbGemmArgs a{};
     a.L = packed_layout(p);
-    a.io_bf16 = 1;
+    a.io = native_io(p);
     a.M = (int64_t)M;
     a.A = a_dev;
     a.lda = (int64_t)lda;
-    if (bf16_needs_copy(p, route, a_dev, lda)) {
+    if (native_needs_copy(p, route, a_dev, lda)) {
       const int64_t ld = staged_ld(p);
       const int32_t* gather =
           p.has_g_idx ? reinterpret_cast<const int32_t*>(reinterpret_cast<const uint8_t*>(packed_dev) + p.gather_offset)
@@ -522,7 +531,7 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
     a.ldc = (int64_t)ldy;
     a.workspace = w.inner > 0 ? ws + w.staged : nullptr;
     a.workspace_bytes = w.inner;
-    const hipError_t e = route == kBf16Tile ? mnb_launch_gemm256(a, s) : mnb_launch_skinny(a, s);
+    const hipError_t e = route == kNativeTile ? mnb_launch_gemm256(a, s) : mnb_launch_skinny(a, s);
     return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbVariantGemm");
   }
 
@@ -561,8 +570,8 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
 
 const char* MnbVariantGemmKernelName(const MnbVariantPlan* plan, size_t M) {
   if (plan == nullptr || plan->packed_bytes == 0 || M == 0) return "none";
-  if (const Bf16Route route = bf16_route(*plan, M); route != kBf16None)
-    return route == kBf16Tile ? "mnb_gemm256_kernel" : "mnb_skinny_kernel";
+  if (const NativeRoute route = native_route(*plan, M); route != kNativeNone)
+    return route == kNativeTile ? "mnb_gemm256_kernel" : "mnb_skinny_kernel";
   return MnbGemmKernelName(M, (size_t)plan->N, (size_t)plan->packed_k, plan->bits, plan->packed_block_size,
                            plan->compute_dtype);
 }

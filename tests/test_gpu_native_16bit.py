@@ -1,6 +1,6 @@
-"""bfloat16 on the matrix cores in its own type (weights dequantised in fp32, narrowed to bfloat16, fp32
-accumulation): the decode kernel up to 16 rows, the tile GEMM beyond, through the C ABI's variant entry points and the
-host class.
+"""16-bit models on a matrix packed with fp32 scales and zero points - bfloat16, and fp16 with zero points in the
+activation type - on the matrix cores in their own type (weights dequantised in fp32, narrowed, fp32 accumulation): the
+decode kernel up to 16 rows, the tile GEMM beyond, through the C ABI's variant entry points and the host class.
 
 The reference's CPU provider has no bfloat16 kernel; its GPU provider dequantises B into bfloat16 and calls a bfloat16
 GEMM (contrib_ops/cuda/quantization/matmul_nbits.cc:844-975), which is the arithmetic here.  Gates: relative L2 <= 5e-3
@@ -144,3 +144,43 @@ def test_route_by_rows_and_k():
     d2 = {k: to_dev(v) for k, v in c2.items()}
     assert op2.PrePack(d2["B"], d2["scales"], None, None)
     assert kernel_name(op2, 16) == DECODE and kernel_name(op2, 300) not in (TILE, DECODE)   # the widened route
+
+
+# ---- fp16 activations with zero points in the activation type (4- and 2-bit): the same two kernels, fp16 operands
+@pytest.mark.parametrize("bits,bs,g_kind", [(4, 32, "none"), (4, 128, "none"), (4, 16, "none"), (4, 64, "act_order"),
+                                            (4, 32, "ragged"), (2, 32, "none"), (2, 64, "none")])
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 130, 600])
+def test_f16_typed_zero_points_against_float64(bits, bs, g_kind, M):
+    N, K = 300, 512
+    c = make("f16", N, K, bits, bs, "typed", g_kind, M, seed=M + bits + bs, bias=M % 2 == 1)
+    y, op = run_op("f16", c, N, K, bits, bs)
+    if M <= 16:
+        assert kernel_name(op, M) == DECODE
+    elif op.plan.packed_k % 128 == 0:    # ragged groups are padded: the packed k extent need not stay a multiple of 128
+        assert kernel_name(op, M) == TILE
+    assert y.dtype == torch.float16 and tuple(y.shape) == (M, N)
+    check("f16", c, y, N, K, bits, bs)
+
+
+@pytest.mark.parametrize("bits,bs", [(4, 32), (4, 16), (2, 64)])
+@pytest.mark.parametrize("rows", ["decode", "tile"])
+def test_f16_typed_zero_points_unit_rows_recover_w_exactly(bits, bs, rows):
+    N, K = 200, 256
+    M = 16 if rows == "decode" else K
+    c = make("f16", N, K, bits, bs, "typed", "none", M, seed=7, exact=True)
+    ks = np.random.default_rng(2).choice(K, size=M, replace=False)
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), ks] = 1.0
+    c["A"] = to_np_type(a, "f16")
+    y, op = run_op("f16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == (DECODE if rows == "decode" else TILE)
+    w = C.variant_dequantize(c["B"], c["scales"], c["zp"], None, N, K, bits, bs)
+    assert np.array_equal(to_host32(y), w[:, ks].T)
+
+
+def test_f16_prefill_shape_with_typed_zero_points():
+    M, N, K, bits, bs = 1024, 2048, 4096, 4, 32
+    c = make("f16", N, K, bits, bs, "typed", "none", M, seed=3, bias=True)
+    y, op = run_op("f16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == TILE
+    check("f16", c, y, N, K, bits, bs)

@@ -107,8 +107,9 @@ class Plan:
 
 def test_every_instantiation_issues_its_loads_and_waits_as_planned(kernels):
     # {4-bit, 8-bit with 2 or 4 entries} x {zp, none} x {128, 256 rows} x {fp16, bfloat16}, less the one that does not
-    # fit the register file (bfloat16, four entries with zero points, 256 rows: never launched)
-    assert len(kernels) == 23
+    # fit the register file (bfloat16, four entries with zero points, 256 rows: never launched), plus fp16 on fp32
+    # meta entries (zero points in the activation type: 4-bit with zero points) x {128, 256 rows}
+    assert len(kernels) == 25
     for name, lines in kernels.items():
         bits, mps, tm, wm = (int(x) for x in re.search(r"kernelILi(\d)ELb[01]ELi(\d)ELi(\d)ELi(\d)E", name).groups())
         plan = Plan(bits, mps, tm, ct=wm)  # the wavefronts form wm x 8/wm: 256 / (32 * 8/wm) column tiles each
