@@ -226,18 +226,19 @@ MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* 
  *                    block size 16 and every group padded to a multiple of 16.  The activation columns are gathered
  *                    into that order (zeros in the padding) in front of every GEMM.  A g_idx equal to
  *                    k / block_size is recognised and dropped.
- *   typed zero points:  scales and zero points are widened to fp32 (exactly) and the fp32 kernels run on a widened
- *                    copy of the activations; the fp32 result plus bias is narrowed once.  This is the reference's
- *                    own arithmetic for these inputs (fp32 SGEMM on widened operands, :1336-1510).
- *   bfloat16:        the same packed matrix, multiplied on the matrix cores in bfloat16 - up to 16 rows by the
- *                    decode kernel (any K), beyond by the tile GEMM when packed_k is a multiple of 128 (other k
- *                    extents take the widened route above):  w = fma(float(q), scale, -zp * scale) in fp32, narrowed
- *                    to bfloat16 (round to nearest even), products accumulated in fp32, bias added and the sum
- *                    narrowed in the epilogue.  This is what the reference's GPU provider multiplies for bfloat16 (B
- *                    dequantised into the activation type, then a GEMM of that type:
- *                    onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975); the CPU provider has no
- *                    bfloat16 kernel.  The tile GEMM reads activations in place when they are 16-byte aligned with a
- *                    pitch that is a multiple of 8 and there is no g_idx, else from a bfloat16 copy in the workspace.
+ *   typed zero points:  scales and zero points are widened to fp32 (exactly) at pack time and the matrix is packed
+ *                    as an fp32 model's; fp32 models run the fp32 kernels on it (the reference's own arithmetic for
+ *                    these inputs: fp32 SGEMM on dequantised operands, :1336-1510).
+ *   16-bit models on such a matrix (bfloat16, always packed this way; fp16 with typed zero points):  the matrix-core
+ *                    kernels run on it in the activation type instead - the decode kernel up to 16 rows, the
+ *                    streaming kernel or the tile GEMM beyond, chosen as for fp16 models:
+ *                    w = fma(float(q), scale, -zp * scale) in fp32, narrowed to the activation type (round to nearest
+ *                    even), products accumulated in fp32, bias added and the sum narrowed in the epilogue.  This is
+ *                    what the reference's GPU provider multiplies (B dequantised into the activation type, then a
+ *                    GEMM of that type: onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975); the CPU
+ *                    provider has no bfloat16 kernel.  The tile GEMM reads activations in place when they are 16-byte
+ *                    aligned with a pitch that is a multiple of 8 and there is no g_idx, else from a copy in the
+ *                    workspace; the other two take any alignment.
  * Zero points are honoured together with g_idx for both zero-point types, as the schema defines; the reference's CPU
  * dequantiser reads uint8 zero points in that combination but then uses 8 (matmul_nbits_impl.cc:56-66).
  * Supported: g_idx with bits = 4; typed zero points with bits = 2 or 4 (the reference rejects 8, :1251-1252). */

@@ -204,7 +204,7 @@ const MnbDeviceInfo& mnb_device_info() {
 constexpr double kMnbMidStartCycles = 19200.0;
 constexpr double kMnbMidFlopsPerCuCycle[2] = {1286.0, 1156.0};
 
-static bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
+bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M) {
   if (L.K % 128 != 0) return false;
   if (const char* e = mnb_tuning_env("MNB_MID_MAX_M")) return M > (int64_t)atoll(e);  // calibration: M up to this streams
   if (M <= 64) return false;  // (64-row tiles were measured: never ahead of the streaming kernel)

@@ -9,6 +9,10 @@
 // reference's fp16 dequantisation bit for bit) and the matrix cores accumulate across blocks; the VALU cost of the
 // dequantisation is amortised over MT * 4 matrix instructions per word.
 //
+// 16-bit models on a matrix packed with fp32 meta entries (IO = kMnbIoBf16, kMnbIoF16Wide: bfloat16, and fp16 with zero
+// points in the activation type) run the same kernel: the weights are dequantised in fp32, fma(float(q), scale,
+// -zp * scale), narrowed to the activation type, and multiplied by the matrix instruction of that type.
+//
 // The A operand of lane (j, kq) is 16 bytes of row j at a 64-byte stride between lanes -- read from the row-major
 // activations, one load instruction would touch 64 cache lines.  A small staging kernel therefore first rewrites A
 // into operand order in the caller's workspace, [chunk][word i][row tile][kq][j] in 16-byte units (zero-filled beyond
@@ -88,7 +92,7 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
 // three quarters of a chunk ahead without a second register set.  NEXT_A is a compile-time flag on purpose: a load
 // under a run-time condition makes the number of outstanding loads unknown to the compiler at the join, and every
 // later wait then degenerates to "wait for all loads", the weight prefetch issued just before included.
-template <int BITS, bool HAS_ZP, int T, int MT, bool NEXT_A>
+template <int BITS, bool HAS_ZP, int T, int MT, bool NEXT_A, int IO>
 __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h8_t (*af)[(128 / BITS) / 8],
                                                   const uint4* a_next, int64_t a_step, const UnpackConsts& uc,
                                                   f4_t (*y)[T]) {
@@ -99,15 +103,28 @@ __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
-      _Float16 sc, nz;
-      decode_meta<BITS, HAS_ZP>(second ? R.m1[t] : R.m0[t], sc, nz);
-      const h2_t s2 = mnb_h2(sc);
-      const h2_t z_lo = mnb_h2(nz);                     // -(1024 + zp)
-      const h2_t z_hi = mnb_h2(nz + (_Float16)960.0f);  // -(64 + zp), exact
-      const h8_t b = BITS == 4 ? dequant_word<4>(wd[i], 0u, uc, z_lo, z_hi, s2)
-                               : dequant_word<8>(wd[(2 * i) & 3], wd[(2 * i + 1) & 3], uc, z_lo, z_hi, s2);
+      h8_t b;
+      if constexpr (IO != kMnbIoModel) {
+        const float sc = __uint_as_float(second ? R.m1[t] : R.m0[t]);
+        const float zp = HAS_ZP ? __uint_as_float(second ? R.z1[t] : R.z0[t]) : (float)(1 << (BITS - 1));
+        b = BITS == 4 ? dequant_word_wide<BITS, IO == kMnbIoBf16>(wd[i], 0u, sc, -zp * sc)
+                      : dequant_word_wide<BITS, IO == kMnbIoBf16>(wd[(2 * i) & 3], wd[(2 * i + 1) & 3], sc, -zp * sc);
+      } else {
+        _Float16 sc, nz;
+        decode_meta<BITS, HAS_ZP>(second ? R.m1[t] : R.m0[t], sc, nz);
+        const h2_t s2 = mnb_h2(sc);
+        const h2_t z_lo = mnb_h2(nz);                     // -(1024 + zp)
+        const h2_t z_hi = mnb_h2(nz + (_Float16)960.0f);  // -(64 + zp), exact
+        b = BITS == 4 ? dequant_word<4>(wd[i], 0u, uc, z_lo, z_hi, s2)
+                      : dequant_word<8>(wd[(2 * i) & 3], wd[(2 * i + 1) & 3], uc, z_lo, z_hi, s2);
+      }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) y[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][i], b, y[mt][t], 0, 0, 0);
+      for (int mt = 0; mt < MT; ++mt) {
+        if constexpr (IO == kMnbIoBf16)
+          y[mt][t] = mfma16_bf16(af[mt][i], b, y[mt][t]);
+        else
+          y[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[mt][i], b, y[mt][t], 0, 0, 0);
+      }
     }
     // Nothing moves across the end of a word step: loads hoisted above the matrix instructions that still read
     // af[.][i] would need a second register set, and so would dequantised operands prepared steps ahead.
@@ -122,7 +139,7 @@ __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h
 
 // What a wavefront needs to issue its first loads comes as leading scalar kernel arguments, which the build asks the
 // compiler to have preloaded into SGPRs at wavefront start; the parameter block carries the rest.
-template <int BITS, bool HAS_ZP, int T, int MT, int NW>
+template <int BITS, bool HAS_ZP, int T, int MT, int NW, int IO>
 __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, int64_t hot_Npad, const uint4* hot_As,
                                                           const uint8_t* hot_meta, int hot_row_tiles, int hot_chunks,
                                                           int hot_bs_shift, MidParams rest) {
@@ -137,6 +154,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, in
   const SkinnyParams& p = mp.s;
   constexpr int GK = 128 / BITS;
   constexpr int NI = GK / 8;
+  constexpr int LOAD_MODE = IO == kMnbIoModel ? 1 : 2;  // which meta entries a chunk's loads fetch (load_chunk)
   extern __shared__ __align__(16) unsigned char smem[];
   float* red = reinterpret_cast<float*>(smem);
   const int lane = threadIdx.x & 63;
@@ -173,19 +191,19 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, in
   ChunkRegs<BITS, T> R0, R1;
   const int last = p.chunks - 1;
   int c = wave;
-  load_chunk<BITS, HAS_ZP, 1, T>(p, min(c, last), kq, col0, R0);
+  load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c, last), kq, col0, R0);
   load_a(min(c, last));
-  load_chunk<BITS, HAS_ZP, 1, T>(p, min(c + NW, last), kq, col0, R1);
+  load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + NW, last), kq, col0, R1);
   __builtin_amdgcn_sched_barrier(0);
   for (; c + NW < p.chunks; c += 2 * NW) {
-    mid_compute_chunk<BITS, HAS_ZP, T, MT, true>(R0, af, a_of(c + NW), a_step, uc, y);
-    load_chunk<BITS, HAS_ZP, 1, T>(p, min(c + 2 * NW, last), kq, col0, R0);
+    mid_compute_chunk<BITS, HAS_ZP, T, MT, true, IO>(R0, af, a_of(c + NW), a_step, uc, y);
+    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 2 * NW, last), kq, col0, R0);
     __builtin_amdgcn_sched_barrier(0);
-    mid_compute_chunk<BITS, HAS_ZP, T, MT, true>(R1, af, a_of(min(c + 2 * NW, last)), a_step, uc, y);
-    load_chunk<BITS, HAS_ZP, 1, T>(p, min(c + 3 * NW, last), kq, col0, R1);
+    mid_compute_chunk<BITS, HAS_ZP, T, MT, true, IO>(R1, af, a_of(min(c + 2 * NW, last)), a_step, uc, y);
+    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 3 * NW, last), kq, col0, R1);
     __builtin_amdgcn_sched_barrier(0);
   }
-  if (c < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false>(R0, af, nullptr, a_step, uc, y);
+  if (c < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false, IO>(R0, af, nullptr, a_step, uc, y);
 
   // reduce over the wavefronts, one row tile at a time: lane (j, kq), register r of y[mt][t] holds
   // row m0 + 16 mt + 4 kq + r, column n0 + 16 t + j
@@ -250,39 +268,52 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   return pl;
 }
 
-template <int BITS, bool HAS_ZP, int T, int MT>
+template <int BITS, bool HAS_ZP, int T, int MT, int IO>
 hipError_t launch_nw(const MidParams& mp, const MidPlan& pl, hipStream_t s) {
   const SkinnyParams& p = mp.s;
   dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)));
   const size_t smem = (size_t)pl.nw * T * 4 * 64 * sizeof(float);
   if (pl.nw == 8)
-    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8><<<grid, dim3(512), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8, IO><<<grid, dim3(512), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
                                                                         p.chunks, p.bs_shift, mp);
   else
-    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4><<<grid, dim3(256), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4, IO><<<grid, dim3(256), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
                                                                         p.chunks, p.bs_shift, mp);
   return hipGetLastError();
 }
 
-template <int BITS, bool HAS_ZP, int T>
+template <int BITS, bool HAS_ZP, int T, int IO>
 hipError_t launch_mt(const MidParams& p, const MidPlan& pl, hipStream_t s) {
-  return pl.mt == 2 ? launch_nw<BITS, HAS_ZP, T, 2>(p, pl, s) : launch_nw<BITS, HAS_ZP, T, 4>(p, pl, s);
+  return pl.mt == 2 ? launch_nw<BITS, HAS_ZP, T, 2, IO>(p, pl, s) : launch_nw<BITS, HAS_ZP, T, 4, IO>(p, pl, s);
+}
+
+template <int BITS, bool HAS_ZP, int IO>
+hipError_t launch_t(const MidParams& p, const MidPlan& pl, hipStream_t s) {
+  switch (pl.t) {
+    case 4: return launch_mt<BITS, HAS_ZP, 4, IO>(p, pl, s);
+    case 2: return launch_mt<BITS, HAS_ZP, 2, IO>(p, pl, s);
+    default: return launch_mt<BITS, HAS_ZP, 1, IO>(p, pl, s);
+  }
 }
 
 template <int BITS, bool HAS_ZP>
-hipError_t launch_t(const MidParams& p, const MidPlan& pl, hipStream_t s) {
-  switch (pl.t) {
-    case 4: return launch_mt<BITS, HAS_ZP, 4>(p, pl, s);
-    case 2: return launch_mt<BITS, HAS_ZP, 2>(p, pl, s);
-    default: return launch_mt<BITS, HAS_ZP, 1>(p, pl, s);
+hipError_t launch_io(const MidParams& p, const MidPlan& pl, int io, hipStream_t s) {
+  if (io == kMnbIoBf16) return launch_t<BITS, HAS_ZP, kMnbIoBf16>(p, pl, s);
+  if (io == kMnbIoF16Wide) {  // zero points in the activation type: 4-bit with zero points
+    if constexpr (BITS == 4 && HAS_ZP) return launch_t<BITS, HAS_ZP, kMnbIoF16Wide>(p, pl, s);
+    else return hipErrorInvalidValue;
   }
+  return launch_t<BITS, HAS_ZP, kMnbIoModel>(p, pl, s);
 }
 
 int mid_row_tiles(int64_t M, int mt) { return (int)((M + 16 * mt - 1) / (16 * mt)) * mt; }
 
 }  // namespace
 
-bool mnb_mid_applicable(const MnbGemmArgs& a) { return a.L.dtype == kMnbDtypeFloat16 && a.M >= 1; }
+bool mnb_mid_applicable(const MnbGemmArgs& a) {
+  // fp16 models, and 16-bit ones (a.io) on a matrix packed with fp32 meta entries
+  return (a.io != kMnbIoModel ? a.L.dtype == kMnbDtypeFloat : a.L.dtype == kMnbDtypeFloat16) && a.M >= 1;
+}
 
 // bytes of the staged copy of A
 size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
@@ -293,6 +324,7 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
 
 hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
+  if (!mnb_mid_applicable(a) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
   const MidPlan pl = mid_plan(L, a.M, a.epi.kind == kMnbFusedMlp ? 2 : 1);
   const int CK = 4 * L.group_k;
   MidParams mp{};
@@ -310,6 +342,7 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   p.K = (int)L.K;
   p.bs_shift = mnb_log2i(L.bs);
   p.chunks = (int)((L.K + CK - 1) / CK);
+  p.io_bf16 = a.io == kMnbIoBf16;
   p.epi.kind = a.epi.kind;
   if (a.epi.kind != kMnbFusedNone) {
     p.C = reinterpret_cast<_Float16*>(a.epi.out[0]);
@@ -335,6 +368,6 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   else
     mnb_mid_stage_a_kernel<8><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
   if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-  if (L.bits == 4) return L.has_zp ? launch_t<4, true>(mp, pl, s) : launch_t<4, false>(mp, pl, s);
-  return L.has_zp ? launch_t<8, true>(mp, pl, s) : launch_t<8, false>(mp, pl, s);
+  if (L.bits == 4) return L.has_zp ? launch_io<4, true>(mp, pl, a.io, s) : launch_io<4, false>(mp, pl, a.io, s);
+  return L.has_zp ? launch_io<8, true>(mp, pl, a.io, s) : launch_io<8, false>(mp, pl, a.io, s);
 }

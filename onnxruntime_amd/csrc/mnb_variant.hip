@@ -16,8 +16,8 @@
 //     models does the same on a widened copy of the activations and narrows the fp32 result plus bias once - the
 //     reference's own arithmetic for this input (fp32 SGEMM on widened operands).
 //   * 16-bit models on such a matrix - bfloat16 (always packed this way), fp16 with zero points in the activation
-//     type - normally skip the widened route: the decode kernel (up to 16 rows) and the tile GEMM (beyond, for k
-//     extents that are multiples of 128) dequantise the weights in fp32, narrow them to the activation type for the
+//     type - skip the widened route: the decode kernel (up to 16 rows), the streaming kernel and the tile GEMM
+//     (beyond) dequantise the weights in fp32, narrow them to the activation type for the
 //     matrix cores (what the reference's GPU provider multiplies:
 //     onnxruntime/contrib_ops/cuda/quantization/matmul_nbits.cc:844-975 dequantises B into the activation type and
 //     calls a GEMM of that type), accumulate in fp32, and add bias and narrow in the epilogue.
@@ -427,10 +427,10 @@ struct VariantWorkspace {
 
 // 16-bit activations on a matrix packed with fp32 entries - bfloat16 models, and fp16 models whose zero points are in
 // the activation type - run on the matrix cores in their own type (weights dequantised in fp32 and narrowed): up to
-// 16 rows on the decode kernel (any K), beyond on the tile GEMM, which needs a k extent that is a multiple of 128.
-// What is left (more than 16 rows on another k extent) takes the widened route.  Measured against the widened route
-// on (N, K) = (14336, 4096), bfloat16: 5 to 14 times faster from 17 rows up, 1.4 to 6 times up to 16 rows.
-enum NativeRoute { kNativeNone, kNativeDecode, kNativeTile };
+// 16 rows on the decode kernel, beyond on the streaming kernel or the tile GEMM, chosen as for fp16 models.  The
+// widened route is left to fp32 models.  Measured against the widened route on (N, K) = (14336, 4096), bfloat16:
+// 5 to 14 times faster from 17 rows up, 1.4 to 6 times up to 16 rows.
+enum NativeRoute { kNativeNone, kNativeDecode, kNativeMid, kNativeTile };
 
 // kMnbIoModel when the plan's kernels run in the compute type (fp32 models, fp16 models with integer zero points)
 int native_io(const MnbVariantPlan& p) {
@@ -444,13 +444,14 @@ NativeRoute native_route(const MnbVariantPlan& p, size_t M) {
   if (const char* e = mnb_tuning_env("MNB_NATIVE_ROUTE")) {  // calibration: "wide" switches the native kernels off
     if (e[0] == 'w') return kNativeNone;
     if (e[0] == 't' && p.packed_k % 128 == 0) return kNativeTile;
+    if (e[0] == 'm') return kNativeMid;
   }
   if (M <= 16) return kNativeDecode;
-  return p.packed_k % 128 == 0 ? kNativeTile : kNativeNone;
+  return mnb_prefer_gemm256(packed_layout(p), (int64_t)M) ? kNativeTile : kNativeMid;  // (false unless k % 128 == 0)
 }
 
 // The tile GEMM reads A through 16-byte loads at 32-bit offsets: a caller's A that is not aligned for that is copied
-// first.  (The decode kernel takes any alignment.)  Columns that have to be gathered are copied for both.
+// first.  (The other two kernels take any alignment.)  Columns that have to be gathered are copied for all three.
 bool native_needs_copy(const MnbVariantPlan& p, NativeRoute route, const void* a, size_t lda) {
   if (p.has_g_idx) return true;
   if (route != kNativeTile) return false;
@@ -464,6 +465,7 @@ VariantWorkspace variant_workspace(const MnbVariantPlan& p, size_t M) {
     // the tile GEMM gets room for the copy whether or not a call needs it: alignment and pitch are not known here
     if (route == kNativeTile || p.has_g_idx) w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
     if (route == kNativeTile) w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
+    if (route == kNativeMid) w.inner = round256(mnb_mid_workspace_bytes(packed_layout(p), (int64_t)M));
     return w;
   }
   const bool widened = p.compute_dtype != p.a_dtype;
@@ -531,7 +533,9 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
     a.ldc = (int64_t)ldy;
     a.workspace = w.inner > 0 ? ws + w.staged : nullptr;
     a.workspace_bytes = w.inner;
-    const hipError_t e = route == kNativeTile ? mnb_launch_gemm256(a, s) : mnb_launch_skinny(a, s);
+    const hipError_t e = route == kNativeTile  ? mnb_launch_gemm256(a, s)
+                         : route == kNativeMid ? mnb_launch_mid(a, s)
+                                               : mnb_launch_skinny(a, s);
     return e == hipSuccess ? MNB_OK : hip_fail(e, "MnbVariantGemm");
   }
 
@@ -571,7 +575,7 @@ int MnbVariantGemm(const MnbVariantPlan* plan, size_t M, const void* a_dev, size
 const char* MnbVariantGemmKernelName(const MnbVariantPlan* plan, size_t M) {
   if (plan == nullptr || plan->packed_bytes == 0 || M == 0) return "none";
   if (const NativeRoute route = native_route(*plan, M); route != kNativeNone)
-    return route == kNativeTile ? "mnb_gemm256_kernel" : "mnb_skinny_kernel";
+    return route == kNativeTile ? "mnb_gemm256_kernel" : route == kNativeMid ? "mnb_mid_kernel" : "mnb_skinny_kernel";
   return MnbGemmKernelName(M, (size_t)plan->N, (size_t)plan->packed_k, plan->bits, plan->packed_block_size,
                            plan->compute_dtype);
 }

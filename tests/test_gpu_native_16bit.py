@@ -1,6 +1,7 @@
 """16-bit models on a matrix packed with fp32 scales and zero points - bfloat16, and fp16 with zero points in the
 activation type - on the matrix cores in their own type (weights dequantised in fp32, narrowed, fp32 accumulation): the
-decode kernel up to 16 rows, the tile GEMM beyond, through the C ABI's variant entry points and the host class.
+decode kernel up to 16 rows, the streaming kernel or the tile GEMM beyond (chosen as for fp16 models: the tile GEMM
+takes the large problems), through the C ABI's variant entry points and the host class.
 
 The reference's CPU provider has no bfloat16 kernel; its GPU provider dequantises B into bfloat16 and calls a bfloat16
 GEMM (contrib_ops/cuda/quantization/matmul_nbits.cc:844-975), which is the arithmetic here.  Gates: relative L2 <= 5e-3
@@ -21,6 +22,8 @@ pytestmark = pytest.mark.gpu
 C = oracle.C
 TILE = "mnb_gemm256_kernel"
 DECODE = "mnb_skinny_kernel"
+MID = "mnb_mid_kernel"
+BIG = (1024, 4096, 4096)   # M, N, K of a problem the tile GEMM takes
 
 
 def kernel_name(op, M):
@@ -32,39 +35,60 @@ def kernel_name(op, M):
     (4, 16, "u8", "none"), (4, 64, "u8", "act_order"), (4, 32, "typed", "act_order"),
     (8, 32, "none", "none"), (8, 64, "u8", "none"), (8, 16, "u8", "none"), (8, 16, "none", "none"),
     (2, 32, "u8", "none"), (2, 64, "typed", "none"), (2, 128, "none", "none")])
-@pytest.mark.parametrize("M", [1, 3, 8, 11, 16, 17, 130, 300, 700])
+@pytest.mark.parametrize("M", [1, 3, 8, 11, 16, 17, 40, 130, 300, 700])
 def test_gemm_against_float64(bits, bs, zp_kind, g_kind, M):
     N, K = 300, 512
     c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=M + bits + bs, bias=M % 2 == 1)
     y, op = run_op("bf16", c, N, K, bits, bs)
-    assert kernel_name(op, M) == (DECODE if M <= 16 else TILE)
+    assert kernel_name(op, M) == (DECODE if M <= 16 else MID)
     assert y.dtype == torch.bfloat16 and tuple(y.shape) == (M, N)
     check("bf16", c, y, N, K, bits, bs)
 
 
-def test_tiles_cut_along_k_and_256_row_tiles():
-    """A deep K on few tiles makes the plan cut tiles along K (partial sums travel through the workspace); many rows
-    select 256-row tiles."""
-    for (M, N, K, bits, bs) in [(200, 256, 8192, 4, 64), (2048, 1024, 1024, 4, 32), (1500, 700, 2048, 8, 128)]:
+@pytest.mark.parametrize("bits,bs,zp_kind,g_kind", [
+    (4, 32, "u8", "none"), (4, 128, "typed", "none"), (4, 16, "none", "none"), (4, 64, "u8", "act_order"),
+    (8, 64, "u8", "none"), (8, 16, "u8", "none"), (8, 32, "none", "none"), (2, 32, "typed", "none")])
+def test_tile_gemm_against_float64(bits, bs, zp_kind, g_kind):
+    M, N, K = BIG
+    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=bits + bs, bias=True)
+    y, op = run_op("bf16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == TILE
+    check("bf16", c, y, N, K, bits, bs)
+
+
+def test_tiles_cut_along_k_and_ragged_tiles():
+    """A deep K on few tiles makes the plan cut tiles along K (partial sums travel through the workspace); M and N that
+    are not multiples of the tile leave ragged tiles."""
+    for (M, N, K, bits, bs) in [(512, 8192, 8192, 4, 64), (1024, 4096, 8192, 8, 64), (1000, 4000, 8192, 4, 32)]:
         c = make("bf16", N, K, bits, bs, "u8", "none", M, seed=M, bias=True)
         y, op = run_op("bf16", c, N, K, bits, bs)
         assert kernel_name(op, M) == TILE
         check("bf16", c, y, N, K, bits, bs)
 
 
+def unit_rows(M, K, seed):
+    ks = np.random.default_rng(seed).choice(K, size=M, replace=False)
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), ks] = 1.0
+    return a, ks
+
+
 @pytest.mark.parametrize("bits,bs,zp_kind,g_kind", [
-    (4, 32, "typed", "none"), (4, 32, "none", "none"), (4, 64, "u8", "act_order"), (4, 16, "u8", "none"),
-    (8, 32, "u8", "none"), (8, 16, "u8", "none"), (8, 64, "none", "none"), (2, 32, "typed", "none")])
-def test_unit_vectors_recover_w_exactly(bits, bs, zp_kind, g_kind):
+    (4, 32, "typed", "none"), (4, 64, "u8", "act_order"), (4, 16, "u8", "none"), (8, 16, "u8", "none"),
+    (8, 64, "none", "none"), (2, 32, "typed", "none")])
+@pytest.mark.parametrize("rows", ["mid", "tile"])
+def test_unit_rows_recover_columns_of_w_exactly(bits, bs, zp_kind, g_kind, rows):
     """Power-of-two scales and (half-)integer zero points: q - zp has at most 8 significant bits, so neither the fp32
-    dequantisation nor the narrowing to bfloat16 rounds, and row k of I x W must be column k of the reference's W."""
-    N, K = 200, 256
-    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, K, seed=5, exact=True)
-    c["A"] = to_np_type(np.eye(K, dtype=np.float32), "bf16")
+    dequantisation nor the narrowing to bfloat16 rounds, and a unit-vector row e_k of A must produce column k of the
+    reference's W, bit for bit."""
+    M, N, K = BIG if rows == "tile" else (200, 200, 256)
+    c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=5, exact=True)
+    a, ks = unit_rows(M, K, 1)
+    c["A"] = to_np_type(a, "bf16")
     y, op = run_op("bf16", c, N, K, bits, bs)
-    assert kernel_name(op, K) == TILE
+    assert kernel_name(op, M) == (TILE if rows == "tile" else MID)
     w = C.variant_dequantize(c["B"], c["scales"], c["zp"], c["g"], N, K, bits, bs, honour_u8_zp_with_g_idx=True)
-    assert np.array_equal(to_host32(y), w.T)
+    assert np.array_equal(to_host32(y), w[:, ks].T)
 
 
 @pytest.mark.parametrize("N,K,bits,bs,zp_kind,g_kind", [
@@ -91,9 +115,7 @@ def test_decode_unit_rows_recover_columns_of_w_exactly(bits, bs, zp_kind, g_kind
     (power-of-two scales and (half-)integer zero points: nothing rounds)."""
     N, K, M = 520, 1024, 16
     c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=6, exact=True)
-    ks = np.random.default_rng(1).choice(K, size=M, replace=False)
-    a = np.zeros((M, K), np.float32)
-    a[np.arange(M), ks] = 1.0
+    a, ks = unit_rows(M, K, 1)
     c["A"] = to_np_type(a, "bf16")
     y, op = run_op("bf16", c, N, K, bits, bs)
     assert kernel_name(op, M) == DECODE
@@ -116,10 +138,11 @@ def test_decode_misaligned_activations_agree_with_aligned():
     check("bf16", c, y2, N, K, bits, bs)
 
 
-def test_activations_read_in_place_and_through_the_copy_agree():
-    N, K, bits, bs, M = 260, 384, 4, 32, 150
+def test_tile_gemm_activations_read_in_place_and_through_the_copy_agree():
+    (M, N, K), bits, bs = BIG, 4, 32
     c = make("bf16", N, K, bits, bs, "u8", "none", M, seed=9, bias=True)
     y, op = run_op("bf16", c, N, K, bits, bs)
+    assert kernel_name(op, M) == TILE
     a = to_dev(c["A"])
     bias = to_dev(c["bias"])
     wide = torch.zeros(M, K + 3, dtype=torch.bfloat16, device=a.device)   # a pitch that is not a multiple of 8
@@ -138,12 +161,17 @@ def test_route_by_rows_and_k():
     c = make("bf16", 300, 512, 4, 32, "none", "none", 4, seed=1)
     d = {k: to_dev(v) for k, v in c.items()}
     assert op.PrePack(d["B"], d["scales"], None, None)
-    assert kernel_name(op, 16) == DECODE and kernel_name(op, 17) == TILE
+    assert kernel_name(op, 16) == DECODE and kernel_name(op, 17) == MID and kernel_name(op, 700) == MID
     op2 = MatMulNBits(416, 300, bits=4, block_size=32, dtype=torch.bfloat16)
     c2 = make("bf16", 300, 416, 4, 32, "none", "none", 4, seed=1)
     d2 = {k: to_dev(v) for k, v in c2.items()}
     assert op2.PrePack(d2["B"], d2["scales"], None, None)
-    assert kernel_name(op2, 16) == DECODE and kernel_name(op2, 300) not in (TILE, DECODE)   # the widened route
+    assert kernel_name(op2, 16) == DECODE and kernel_name(op2, 300) == MID
+    big = MatMulNBits(4096, 4096, bits=4, block_size=32, dtype=torch.bfloat16)
+    cb = make("bf16", 4096, 4096, 4, 32, "none", "none", 1, seed=1)
+    db = {k: to_dev(v) for k, v in cb.items()}
+    assert big.PrePack(db["B"], db["scales"], None, None)
+    assert kernel_name(big, 64) == MID and kernel_name(big, 1024) == TILE
 
 
 # ---- fp16 activations with zero points in the activation type (4- and 2-bit): the same two kernels, fp16 operands
@@ -154,32 +182,26 @@ def test_f16_typed_zero_points_against_float64(bits, bs, g_kind, M):
     N, K = 300, 512
     c = make("f16", N, K, bits, bs, "typed", g_kind, M, seed=M + bits + bs, bias=M % 2 == 1)
     y, op = run_op("f16", c, N, K, bits, bs)
-    if M <= 16:
-        assert kernel_name(op, M) == DECODE
-    elif op.plan.packed_k % 128 == 0:    # ragged groups are padded: the packed k extent need not stay a multiple of 128
-        assert kernel_name(op, M) == TILE
+    assert kernel_name(op, M) == (DECODE if M <= 16 else MID)
     assert y.dtype == torch.float16 and tuple(y.shape) == (M, N)
     check("f16", c, y, N, K, bits, bs)
 
 
 @pytest.mark.parametrize("bits,bs", [(4, 32), (4, 16), (2, 64)])
-@pytest.mark.parametrize("rows", ["decode", "tile"])
+@pytest.mark.parametrize("rows", ["decode", "mid", "tile"])
 def test_f16_typed_zero_points_unit_rows_recover_w_exactly(bits, bs, rows):
-    N, K = 200, 256
-    M = 16 if rows == "decode" else K
+    M, N, K = {"decode": (16, 200, 256), "mid": (200, 200, 256), "tile": BIG}[rows]
     c = make("f16", N, K, bits, bs, "typed", "none", M, seed=7, exact=True)
-    ks = np.random.default_rng(2).choice(K, size=M, replace=False)
-    a = np.zeros((M, K), np.float32)
-    a[np.arange(M), ks] = 1.0
+    a, ks = unit_rows(M, K, 2)
     c["A"] = to_np_type(a, "f16")
     y, op = run_op("f16", c, N, K, bits, bs)
-    assert kernel_name(op, M) == (DECODE if rows == "decode" else TILE)
+    assert kernel_name(op, M) == {"decode": DECODE, "mid": MID, "tile": TILE}[rows]
     w = C.variant_dequantize(c["B"], c["scales"], c["zp"], None, N, K, bits, bs)
     assert np.array_equal(to_host32(y), w[:, ks].T)
 
 
 def test_f16_prefill_shape_with_typed_zero_points():
-    M, N, K, bits, bs = 1024, 2048, 4096, 4, 32
+    (M, N, K), bits, bs = BIG, 4, 32
     c = make("f16", N, K, bits, bs, "typed", "none", M, seed=3, bias=True)
     y, op = run_op("f16", c, N, K, bits, bs)
     assert kernel_name(op, M) == TILE
