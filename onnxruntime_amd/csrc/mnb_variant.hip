@@ -14,7 +14,8 @@
 //     in the fp16 kernels' integer offset: scales and zero points are widened to fp32, exactly, at pack time (the
 //     matrix is packed as an fp32 model's).  fp32 models run the fp32 kernels on it.  The widened route for 16-bit
 //     models does the same on a widened copy of the activations and narrows the fp32 result plus bias once - the
-//     reference's own arithmetic for this input (fp32 SGEMM on widened operands).
+//     reference's own arithmetic for this input (fp32 SGEMM on widened operands).  It is the yardstick the
+//     matrix-core routes below were measured against and runs in calibration builds only (MNB_NATIVE_ROUTE=wide).
 //   * 16-bit models on such a matrix - bfloat16 (always packed this way), fp16 with zero points in the activation
 //     type - skip the widened route: the decode kernel (up to 16 rows), the streaming kernel and the tile GEMM
 //     (beyond) dequantise the weights in fp32, narrow them to the activation type for the
@@ -428,7 +429,7 @@ struct VariantWorkspace {
 // 16-bit activations on a matrix packed with fp32 entries - bfloat16 models, and fp16 models whose zero points are in
 // the activation type - run on the matrix cores in their own type (weights dequantised in fp32 and narrowed): up to
 // 16 rows on the decode kernel, beyond on the streaming kernel or the tile GEMM, chosen as for fp16 models.  The
-// widened route is left to fp32 models.  Measured against the widened route on (N, K) = (14336, 4096), bfloat16:
+// widened route serves calibration builds only.  Measured against it on (N, K) = (14336, 4096), bfloat16:
 // 5 to 14 times faster from 17 rows up, 1.4 to 6 times up to 16 rows.
 enum NativeRoute { kNativeNone, kNativeDecode, kNativeMid, kNativeTile };
 
