@@ -21,7 +21,7 @@ CSRC = PKG / "csrc"
 LIB = PKG / "libmnb_mi355x.so"
 OBJ_DIR = PKG / "build"
 
-SOURCES = ["mnb_api.hip", "mnb_pack.hip", "mnb_quant.hip", "mnb_gemv.hip", "mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_gemm_i8.hip", "mnb_gemm32.hip", "mnb_fused.hip", "mnb_variant.hip"]
+SOURCES = ["mnb_api.hip", "mnb_pack.hip", "mnb_quant.hip", "mnb_gemv.hip", "mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_gemm_i8.hip", "mnb_gemm32.hip", "mnb_rows16_f32.hip", "mnb_fused.hip", "mnb_variant.hip"]
 PROBE_LIB = PKG / "libmnb_probe.so"
 PROBE_SOURCES = ["mnb_probe.hip"]
 

@@ -226,6 +226,7 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
     if (!direct && a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;
     return kMnbKernelSkinny;
   }
+  if (mnb_rows16_f32_applicable(a)) return kMnbKernelRows16F32;
   if (mnb_gemv_applicable(a)) return kMnbKernelGemv;
   if (mnb_gemm32_applicable(a)) return kMnbKernelGemm32;
   if (a.L.dtype == kMnbDtypeFloat16) {
@@ -247,6 +248,7 @@ const char* mnb_kernel_name(MnbKernelKind k, const MnbLayout&) {
     case kMnbKernelMid: return "mnb_mid_kernel";
     case kMnbKernelGemm256: return "mnb_gemm256_kernel";
     case kMnbKernelGemm32: return "mnb_gemm32_kernel";
+    case kMnbKernelRows16F32: return "mnb_rows16_f32_kernel";
     case kMnbKernelGemmGeneric: return "mnb_gemm_generic_kernel";
     default: return "none";
   }
@@ -307,6 +309,7 @@ static int gemm_checked(const char* fn, size_t M, size_t N, size_t K, int bits, 
     }
     case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
     case kMnbKernelGemm32: e = mnb_launch_gemm32(a, s); break;
+    case kMnbKernelRows16F32: e = mnb_launch_rows16_f32(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }
   return e == hipSuccess ? MNB_OK : hip_fail(e, fn);
@@ -569,6 +572,7 @@ int fused_gemm(const char* fn, const MnbFusedLayout& F, size_t M, const void* a_
     case kMnbKernelMid: e = mnb_launch_mid(a, s); break;
     case kMnbKernelGemm256: e = mnb_launch_gemm256(a, s); break;
     case kMnbKernelGemm32: e = mnb_launch_gemm32(a, s); break;
+    case kMnbKernelRows16F32: e = mnb_launch_rows16_f32(a, s); break;
     default: e = mnb_launch_gemm_generic(a, s); break;
   }
   if (e != hipSuccess) return hip_fail(e, fn);

@@ -41,7 +41,8 @@ enum MnbKernelKind {
   kMnbKernelGemv,       // fp32, M <= 16: dequantising GEMV (VALU dot products, activations in SGPRs)
   kMnbKernelMid,        // fp16, M > 16: weights from registers to the matrix cores, K split over waves (any shape)
   kMnbKernelGemm256,    // fp16, MFMA GEMM with 256 x 256 tiles: large M, enough tiles to fill the chip
-  kMnbKernelGemm32,     // fp32, M > 16: tile GEMM on the fp32 matrix cores
+  kMnbKernelGemm32,     // fp32, many rows: tile GEMM on the fp32 matrix cores
+  kMnbKernelRows16F32,  // fp32, 5 <= M <= 64: weights from registers to the fp32 matrix cores, K split over waves
   kMnbKernelGemmGeneric // any shape: simple tile kernel (fallback)
 };
 
@@ -67,6 +68,8 @@ bool mnb_skinny_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s);
 bool mnb_mid_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s);
+bool mnb_rows16_f32_applicable(const MnbGemmArgs& a);
+hipError_t mnb_launch_rows16_f32(const MnbGemmArgs& a, hipStream_t s);
 size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M);  // staged copy of A
 // 16 < M: whether the tile GEMM's plan beats the streaming kernel's estimate for this shape (needs K % 128 == 0)
 bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M);
