@@ -211,6 +211,7 @@ def main() -> int:
     ap.add_argument("--no-quantize", action="store_true", help="skip the blockwise quantiser (producer of the format)")
     ap.add_argument("--no-fused", action="store_true", help="skip the fused gate/up projection (MatMulNBitsMlp)")
     ap.add_argument("--no-sizes", action="store_true", help="skip the decode kernel on the larger gate+up matrices")
+    ap.add_argument("--no-bf16", action="store_true", help="skip the bfloat16 rows")
     ap.add_argument("--no-int8", action="store_true",
                     help="skip the int8-activation route (accuracy_level 4) beside the full-accuracy one")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
@@ -500,6 +501,50 @@ def main() -> int:
             del p8, ws8
             torch.cuda.empty_cache()
         out["accuracy_level_4"] = rows
+
+    # ---- bfloat16 models: configs[1]'s and configs[3]'s shapes through the variant entry points --------------------
+    if not args.no_bf16:
+        from onnxruntime_amd.matmul_nbits import MatMulNBits
+        lib = _lib.load()
+        rows = []
+        for label, case, copies in (("configs[1] shape (M=1, int4 bs128 symmetric)", c2, 16),
+                                    ("configs[3] shape (M=2048, int4 bs32 zero_points bias)",
+                                     synthetic.config_c4(seed=0), 2)):
+            dev = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).cuda()
+            b, z = dev(case.B), dev(case.zero_points)
+            sc = dev(case.scales.astype(np.float32)).to(torch.bfloat16)
+            a = dev(case.A.reshape(-1, case.K).astype(np.float32)).to(torch.bfloat16)
+            bias = None if case.bias is None else dev(case.bias.astype(np.float32)).to(torch.bfloat16)
+            ops = []
+            for i in range(copies):
+                op = MatMulNBits(case.K, case.N, case.bits, case.block_size, dtype=torch.bfloat16,
+                                 has_zero_points=z is not None, has_bias=bias is not None)
+                assert op.PrePack(torch.roll(b, i, 0) if i else b, sc, z, None)
+                ops.append(op)
+            Mb = a.shape[0]
+            ys = [torch.empty(Mb, case.N, dtype=torch.bfloat16, device="cuda") for _ in ops]
+
+            def bstep():
+                for op, y in zip(ops, ys):
+                    op.Compute(a, bias=bias, out=y)
+            bstep()
+            if Mb <= 16:
+                g = graph_of(torch, bstep)
+                ms_b = time_steps(torch, g.replay, max(4, args.steps // 2), 2) / copies
+            else:
+                ms_b = time_steps(torch, bstep, 50, 2, warm_ms=30.0) / copies
+            # algorithmic bytes: the packed matrix carries fp32 scales (and zero points) for bfloat16 models
+            kb = case.k_blocks
+            abytes = case.N * kb * (case.block_size * case.bits // 8) + case.N * kb * (8 if z is not None else 4) + \
+                Mb * case.K * 2 + Mb * case.N * 2 + (case.N * 2 if bias is not None else 0)
+            rows.append({"workload": f"bfloat16, {label}",
+                         "kernel": lib.MnbVariantGemmKernelName(ctypes.byref(ops[0].plan), Mb).decode(),
+                         "us_per_launch": round(ms_b * 1e3, 3),
+                         "GBs": round(abytes / (ms_b * 1e-3) / 1e9, 1),
+                         "TFLOPs": round(2.0 * Mb * case.N * case.K / (ms_b * 1e-3) / 1e12, 1)})
+            del ops, ys
+            torch.cuda.empty_cache()
+        out["bfloat16"] = rows
 
     # ---- the other configurations (not part of the JSON contract) ---------------------------------------------
     if args.sweep:
