@@ -80,7 +80,7 @@ struct ChunkRegs {
   uint4 w[T];
   uint32_t m0[T];  // meta entry of the lane's (first) block: raw bits (32 with zero points, else 16)
   uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
-  uint32_t z0[T];  // MODE 2 and 3: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
+  uint32_t z0[T];  // MODE 2, 3 and 4: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
   uint32_t z1[T];
 };
 
@@ -152,6 +152,9 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
   if constexpr (MODE == 0) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
+  } else if constexpr (MODE == 4) {
+    const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
+    load_meta_vec_f32<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0, R.z0);
   } else if constexpr (MODE >= 2) {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
     load_meta_vec_f32<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0, R.z0);
@@ -176,6 +179,10 @@ __device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, in
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
     for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t]);
+  } else if constexpr (MODE == 4) {
+    const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
+#pragma unroll
+    for (int t = 0; t < T; ++t) load_meta_vec_f32<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t], &R.z0[t]);
   } else if constexpr (MODE >= 2) {
     const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
 #pragma unroll
@@ -227,6 +234,30 @@ __device__ __forceinline__ BConst make_bconst() {
   bc.off = h8_t{lo, lo, hi, hi, lo, lo, hi, hi};
   bc.one = h8_t{m1, m1, m1, m1, m1, m1, m1, m1};
   return bc;
+}
+
+// The same for bfloat16 models (MODE 4): every raw operand is the bfloat16 128 + q (see raw4_bf16).
+template <bool HAS_ZP>
+__device__ __forceinline__ BConst make_bconst_bf16() {
+  const float zp = HAS_ZP ? 0.f : 8.f;
+  const uint32_t off2 = bf16_pair(-(128.0f + zp), -(128.0f + zp)), one2 = bf16_pair(-1.0f, -1.0f);  // exact
+  const u4_t off = {off2, off2, off2, off2}, one = {one2, one2, one2, one2};
+  BConst bc;
+  bc.off = __builtin_bit_cast(h8_t, off);
+  bc.one = __builtin_bit_cast(h8_t, one);
+  return bc;
+}
+
+// raw bfloat16 operands of one 4-bit word: 128 + e0 ... 128 + e7 in k order.  bfloat16 keeps 8 significant bits: 128 + q
+// is exact for q < 128, and a nibble fits the mantissa only at bit 0 of a half, hence the shifts (7 operations per 8
+// weights; 8-bit weights do not fit at all and take MODE 2).
+__device__ __forceinline__ h8_t raw4_bf16(uint32_t w, const UnpackConsts& u, uint32_t magic) {
+  u4_t r;
+  r[0] = (w & u.mask_lo) | magic;
+  r[1] = ((w >> 4) & u.mask_lo) | magic;
+  r[2] = ((w >> 8) & u.mask_lo) | magic;
+  r[3] = ((w >> 12) & u.mask_lo) | magic;
+  return __builtin_bit_cast(h8_t, r);
 }
 
 // Sum the per-wavefront partial tiles (red[(w * T * 4 + t * 4 + r) * 64 + lane], written by NW wavefronts) in

@@ -23,6 +23,8 @@
 //    bias and Y hold bfloat16 bits.
 //  * MODE 3 (fp16 models with zero points in the activation type, packed the same way): as MODE 2 with the weights
 //    narrowed to fp16 and the fp16 matrix instruction.
+//  * MODE 4 (bfloat16 models, 4-bit weights, block_size >= chunk): MODE 0's scheme on bfloat16 - the raw operand is
+//    the bfloat16 128 + q, exact in its 8 significant bits.
 //  * The A operands come straight from global memory (L2 hits after the first workgroup) when the rows of A are
 //    16-byte aligned -- every load of a wavefront's first two chunks is issued before anything is waited for;
 //    otherwise the rows are staged in LDS phase by phase (zero-filled beyond K, any alignment).
@@ -34,6 +36,12 @@
 #include "mnb_mfma16_common.hip.h"
 
 namespace {
+
+template <int BITS, bool HAS_ZP, int MODE>
+__device__ __forceinline__ BConst bconst_of_mode() {
+  if constexpr (MODE == 4) return make_bconst_bf16<HAS_ZP>();
+  else return make_bconst<BITS, HAS_ZP>();
+}
 
 // One chunk: T column tiles x (4 k-groups) against the 16-row A operands af[].
 template <int BITS, bool HAS_ZP, int MODE, int T>
@@ -69,6 +77,35 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
       }
       if constexpr (HAS_ZP) {
         const float zp = -(float)nz - 1024.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, __builtin_fmaf(zp, nc2[r], d[r]), y[t][r]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, d[r], y[t][r]);
+      }
+    }
+  } else if constexpr (MODE == 4) {
+    // MODE 0 on bfloat16: raw operands 128 + q, offsets and zero points removed through the correction MFMAs
+    static_assert(MODE != 4 || BITS == 4, "8-bit weights do not fit a bfloat16 mantissa");
+    const f4_t zero = f4_t{0.f, 0.f, 0.f, 0.f};
+    f4_t init = zero, nc2 = zero;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) init = mfma16_bf16(af[i], bc.off, init);
+    if constexpr (HAS_ZP) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) nc2 = mfma16_bf16(af[i], bc.one, nc2);
+    }
+    uint32_t magic;
+    asm("v_mov_b32 %0, 0x43004300" : "=v"(magic));  // two bfloat16 128.0 (held in a register: see UnpackConsts)
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const float sf = __uint_as_float(R.m0[t]);
+      const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
+      f4_t d = init;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) d = mfma16_bf16(af[i], raw4_bf16(wd[i], uc, magic), d);
+      if constexpr (HAS_ZP) {
+        const float zp = __uint_as_float(R.z0[t]);
 #pragma unroll
         for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, __builtin_fmaf(zp, nc2[r], d[r]), y[t][r]);
       } else {
@@ -208,7 +245,7 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
   const int arow = j < p.M ? j : p.M - 1;  // rows >= M of the MFMA A operand re-read row M-1: they are never stored
   const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
   h8_t* mine = reinterpret_cast<h8_t*>(smem) + wave * (16 * AStage<BITS>::PIECES);  // A_LDS only
-  const BConst bconst = make_bconst<BITS, HAS_ZP>();
+  const BConst bconst = bconst_of_mode<BITS, HAS_ZP, MODE>();
   const UnpackConsts uc = make_unpack_consts();
 
   // the activation loads of chunk c: the operands themselves, or the row-contiguous pieces that pass through LDS
@@ -408,7 +445,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
   f4_t y[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
-  const BConst bconst = make_bconst<BITS, HAS_ZP>();
+  const BConst bconst = bconst_of_mode<BITS, HAS_ZP, MODE>();
   const UnpackConsts uc = make_unpack_consts();
 
   for (int ph0 = 0; ph0 < p.chunks; ph0 += p.phase_chunks) {
@@ -462,7 +499,8 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   const int chunks = (int)((L.K + CK - 1) / CK);
   pl.mode = (L.bs >= CK) ? 0 : 1;
   if (const char* e = mnb_tuning_env("MNB_SKINNY_MODE")) pl.mode = e[0] == '1' ? 1 : pl.mode;  // calibration: exact halves
-  if (io != kMnbIoModel) pl.mode = io == kMnbIoBf16 ? 2 : 3;  // fp32 meta entries
+  if (io != kMnbIoModel) pl.mode = io == kMnbIoBf16 ? (L.bits == 4 && L.bs >= CK ? 4 : 2) : 3;  // fp32 meta entries
+  if (const char* e = mnb_tuning_env("MNB_SKINNY_BF16_EXACT")) pl.mode = (pl.mode == 4 && e[0] == '1') ? 2 : pl.mode;
   pl.mtr = pow2_ceil((int)M);
   // workgroups: as many column slabs as fill the chip; wide slabs (T = 4) amortise the A operands best
   const int64_t tiles = (L.N + 15) / 16;
@@ -488,7 +526,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   const bool up_front = chunks == pl.nw || chunks == 2 * pl.nw;  // everything loaded before the first wait
   pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4);
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
-  // the fp32 dequantisation of modes 2 and 3 does not fit the 128 registers of sixteen wavefronts in the general loop
+  // the fp32 scales and zero points of modes 2 to 4 do not fit the 128 registers of sixteen wavefronts in the general loop
   if (pl.mode >= 2 && !up_front && pl.nw == 16) pl.nw = 8;
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
@@ -598,6 +636,10 @@ hipError_t launch_mode(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
 
 template <int BITS, bool HAS_ZP>
 hipError_t launch_zp(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
+  if (pl.mode == 4) {
+    if constexpr (BITS == 4) return launch_mode<BITS, HAS_ZP, 4>(p, pl, s);
+    else return hipErrorInvalidValue;
+  }
   if (pl.mode == 2) return launch_mode<BITS, HAS_ZP, 2>(p, pl, s);
   if (pl.mode == 3) {
     if constexpr (BITS == 4 && HAS_ZP) return launch_mode<BITS, HAS_ZP, 3>(p, pl, s);

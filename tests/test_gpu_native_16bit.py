@@ -92,7 +92,9 @@ def test_unit_rows_recover_columns_of_w_exactly(bits, bs, zp_kind, g_kind, rows)
 
 
 @pytest.mark.parametrize("N,K,bits,bs,zp_kind,g_kind", [
-    (14336, 4096, 4, 128, "none", "none"),    # the decode benchmark's shape: everything loaded up front
+    (14336, 4096, 4, 128, "none", "none"),    # the decode benchmark's shape: everything loaded up front; raw operands
+    (4096, 4096, 4, 128, "typed", "none"),    # raw bfloat16 operands (blocks of 128 and more), zero points removed after
+    (6144, 4096, 4, 256, "u8", "none"),       # the same on three-tile slabs
     (4096, 14336, 4, 32, "u8", "none"),       # general chunk loop
     (6144, 4096, 8, 64, "u8", "none"),        # three-tile slabs
     (1000, 416, 4, 32, "typed", "none"),      # K that is not a whole number of chunks: activations staged in LDS
@@ -109,7 +111,8 @@ def test_decode_shapes_against_float64(N, K, bits, bs, zp_kind, g_kind, M):
 
 @pytest.mark.parametrize("bits,bs,zp_kind,g_kind", [
     (4, 32, "typed", "none"), (4, 128, "none", "none"), (4, 64, "u8", "act_order"), (4, 16, "u8", "none"),
-    (8, 32, "u8", "none"), (8, 16, "none", "none"), (2, 32, "typed", "none")])
+    (8, 32, "u8", "none"), (8, 16, "none", "none"), (2, 32, "typed", "none"), (4, 128, "u8", "none"),
+    (4, 256, "typed", "none"), (2, 128, "u8", "none")])
 def test_decode_unit_rows_recover_columns_of_w_exactly(bits, bs, zp_kind, g_kind):
     """Sixteen unit-vector rows e_k: row m of the product must be column k_m of the reference's W, bit for bit
     (power-of-two scales and (half-)integer zero points: nothing rounds)."""
