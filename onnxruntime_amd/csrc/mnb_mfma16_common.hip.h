@@ -80,7 +80,7 @@ struct ChunkRegs {
   uint4 w[T];
   uint32_t m0[T];  // meta entry of the lane's (first) block: raw bits (32 with zero points, else 16)
   uint32_t m1[T];  // MODE 1, 4-bit only: entry of the second half vector (differs when block_size is 16)
-  uint32_t z0[T];  // MODE 2, 3 and 4: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
+  uint32_t z0[T];  // MODE 2 to 5: m0 / m1 hold the bits of the fp32 scale, z0 / z1 those of the fp32 zero point
   uint32_t z1[T];
 };
 
@@ -152,7 +152,7 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
   if constexpr (MODE == 0) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
-  } else if constexpr (MODE == 4) {
+  } else if constexpr (MODE == 4 || MODE == 5) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec_f32<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0, R.z0);
   } else if constexpr (MODE >= 2) {
@@ -179,7 +179,7 @@ __device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, in
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
     for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t]);
-  } else if constexpr (MODE == 4) {
+  } else if constexpr (MODE == 4 || MODE == 5) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
     for (int t = 0; t < T; ++t) load_meta_vec_f32<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t], &R.z0[t]);

@@ -25,6 +25,8 @@
 //    narrowed to fp16 and the fp16 matrix instruction.
 //  * MODE 4 (bfloat16 models, 4-bit weights, block_size >= chunk): MODE 0's scheme on bfloat16 - the raw operand is
 //    the bfloat16 128 + q, exact in its 8 significant bits.
+//  * MODE 5 (fp16 models with zero points in the activation type, block_size >= chunk): MODE 0 with the block's
+//    fp32 scale and zero point - the zero point enters the fp32 correction unrounded.
 //  * The A operands come straight from global memory (L2 hits after the first workgroup) when the rows of A are
 //    16-byte aligned -- every load of a wavefront's first two chunks is issued before anything is waited for;
 //    otherwise the rows are staged in LDS phase by phase (zero-filled beyond K, any alignment).
@@ -48,7 +50,7 @@ template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t* af, const BConst& bc,
                                               const UnpackConsts& uc, f4_t* y) {
   constexpr int NI = (128 / BITS) / 8;
-  if constexpr (MODE == 0) {
+  if constexpr (MODE == 0 || MODE == 5) {
     // init[m] = -sum_k (off_k + zp) a[m][k] (no zero points) or -sum_k off_k a[m][k]; nc2[m] = -sum_k a[m][k].
     // The constant operands are the same in every lane, so every lane receives the value of its own rows.
     const f4_t zero = f4_t{0.f, 0.f, 0.f, 0.f};
@@ -61,9 +63,16 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
     }
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      _Float16 s, nz;
-      decode_meta<BITS, HAS_ZP>(R.m0[t], s, nz);
-      const float sf = (float)s;
+      float sf, zp;  // scale and zero point of the chunk's block
+      if constexpr (MODE == 5) {
+        sf = __uint_as_float(R.m0[t]);
+        zp = __uint_as_float(R.z0[t]);
+      } else {
+        _Float16 s, nz;
+        decode_meta<BITS, HAS_ZP>(R.m0[t], s, nz);
+        sf = (float)s;
+        zp = -(float)nz - 1024.0f;
+      }
       const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
       f4_t d = init;
 #pragma unroll
@@ -76,7 +85,6 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
         d = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], b, d, 0, 0, 0);
       }
       if constexpr (HAS_ZP) {
-        const float zp = -(float)nz - 1024.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, __builtin_fmaf(zp, nc2[r], d[r]), y[t][r]);
       } else {
@@ -499,8 +507,12 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   const int chunks = (int)((L.K + CK - 1) / CK);
   pl.mode = (L.bs >= CK) ? 0 : 1;
   if (const char* e = mnb_tuning_env("MNB_SKINNY_MODE")) pl.mode = e[0] == '1' ? 1 : pl.mode;  // calibration: exact halves
-  if (io != kMnbIoModel) pl.mode = io == kMnbIoBf16 ? (L.bits == 4 && L.bs >= CK ? 4 : 2) : 3;  // fp32 meta entries
-  if (const char* e = mnb_tuning_env("MNB_SKINNY_BF16_EXACT")) pl.mode = (pl.mode == 4 && e[0] == '1') ? 2 : pl.mode;
+  if (io != kMnbIoModel) {  // fp32 meta entries: raw operands where a chunk lies inside a block, else exact weights
+    const bool raw = L.bits == 4 && L.bs >= CK;
+    pl.mode = io == kMnbIoBf16 ? (raw ? 4 : 2) : (raw ? 5 : 3);
+    if (const char* e = mnb_tuning_env("MNB_SKINNY_WIDE_EXACT"))  // calibration: exact weights everywhere
+      if (e[0] == '1') pl.mode = io == kMnbIoBf16 ? 2 : 3;
+  }
   pl.mtr = pow2_ceil((int)M);
   // workgroups: as many column slabs as fill the chip; wide slabs (T = 4) amortise the A operands best
   const int64_t tiles = (L.N + 15) / 16;
@@ -638,6 +650,10 @@ template <int BITS, bool HAS_ZP>
 hipError_t launch_zp(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) {
   if (pl.mode == 4) {
     if constexpr (BITS == 4) return launch_mode<BITS, HAS_ZP, 4>(p, pl, s);
+    else return hipErrorInvalidValue;
+  }
+  if (pl.mode == 5) {
+    if constexpr (BITS == 4 && HAS_ZP) return launch_mode<BITS, HAS_ZP, 5>(p, pl, s);
     else return hipErrorInvalidValue;
   }
   if (pl.mode == 2) return launch_mode<BITS, HAS_ZP, 2>(p, pl, s);

@@ -190,7 +190,7 @@ def test_f16_typed_zero_points_against_float64(bits, bs, g_kind, M):
     check("f16", c, y, N, K, bits, bs)
 
 
-@pytest.mark.parametrize("bits,bs", [(4, 32), (4, 16), (2, 64)])
+@pytest.mark.parametrize("bits,bs", [(4, 32), (4, 16), (2, 64), (4, 128), (2, 256)])
 @pytest.mark.parametrize("rows", ["decode", "mid", "tile"])
 def test_f16_typed_zero_points_unit_rows_recover_w_exactly(bits, bs, rows):
     M, N, K = {"decode": (16, 200, 256), "mid": (200, 200, 256), "tile": BIG}[rows]
