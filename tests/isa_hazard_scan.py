@@ -5,12 +5,12 @@ Why it exists: the compiler's own hazard handling lost track of a matrix instruc
 behind the branches of a loop (single-tile decode kernel: rows 4 kq + 3 came out wrong).  The kernels now avoid the
 pattern; this check keeps it from coming back unnoticed.  One instruction = one wait state, `s_nop N` = N + 1, as in
 the compiler's own model; the thresholds are the ones the compiler applies in straight-line code on this target
-(4-pass 16x16x32: 8, 8-pass 32x32x16: 12).  A dependent MFMA that takes the result as its C operand is interlocked
+(4-pass 16x16x32: 8, 8-pass 32x32x16: 12, the 8-pass fp32 16x16x4 outside the dense-math pipe: 10).  A dependent MFMA that takes the result as its C operand is interlocked
 by the hardware and is not a finding."""
 import re
 
 _REG = re.compile(r'\b([av])\[(\d+):(\d+)\]|\b([av])(\d+)\b')
-NEED = {"16x16x32": 8, "32x32x16": 12}
+NEED = {"16x16x32": 8, "32x32x16": 12, "16x16x4_f32": 10}
 
 
 def _regs(tok):

@@ -1,5 +1,5 @@
 """The generated code of the matrix-core kernels never reads an MFMA result before it is there (see
-isa_hazard_scan.py).  Compiles the three sources to assembly with the flags of the build; no GPU needed."""
+isa_hazard_scan.py).  Compiles the sources to assembly with the flags of the build; no GPU needed."""
 import shutil
 import subprocess
 import tempfile
@@ -14,7 +14,7 @@ HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
 @pytest.mark.skipif(not Path(HIPCC).exists(), reason="hipcc not available")
-@pytest.mark.parametrize("source", ["mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip"])
+@pytest.mark.parametrize("source", ["mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_rows16_f32.hip"])
 def test_no_early_read_of_mfma_results(source):
     from onnxruntime_amd.build import HIPCC_FLAGS
     with tempfile.TemporaryDirectory() as tmp:
