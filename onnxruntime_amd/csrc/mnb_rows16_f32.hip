@@ -239,8 +239,10 @@ hipError_t mnb_launch_rows16_f32(const MnbGemmArgs& a, hipStream_t s) {
   if (tiles * row_blocks >= 4 * 224) t = 4;
   else if (tiles * row_blocks >= 2 * 224) t = 2;
   if (const char* e = mnb_tuning_env("MNB_ROWS16_T")) t = atoi(e) == 4 ? 4 : atoi(e) == 2 ? 2 : 1;  // calibration
-  // wavefronts: at least two chunks each
-  int nw = p.chunks >= 32 ? 16 : p.chunks >= 16 ? 8 : 4;
+  // wavefronts: at least four chunks each (measured: sixteen wavefronts pay only for K beyond 8192 or so), and four
+  // when the grid brings several workgroups per compute unit anyway
+  int nw = p.chunks >= 64 ? 16 : p.chunks >= 16 ? 8 : 4;
+  if (((tiles + t - 1) / t) * row_blocks >= 512) nw = 4;
   if (const char* e = mnb_tuning_env("MNB_ROWS16_NW")) nw = atoi(e) == 16 ? 16 : atoi(e) == 8 ? 8 : 4;
   if (L.bits == 4) return L.has_zp ? launch_bs<4, true>(p, L.bs, t, nw, s) : launch_bs<4, false>(p, L.bs, t, nw, s);
   return L.has_zp ? launch_bs<8, true>(p, L.bs, t, nw, s) : launch_bs<8, false>(p, L.bs, t, nw, s);
