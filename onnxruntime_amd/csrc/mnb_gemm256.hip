@@ -726,19 +726,26 @@ hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
 template <bool HAS_ZP, int MPS>
 constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
 
+// 128- or 256-row tiles of element type DT (HAS_256: whether the 256-row member exists)
+template <int BITS, bool HAS_ZP, int MPS, int DT, bool HAS_256 = true>
+hipError_t launch_rows(const Gemm256Params& p, unsigned grid, hipStream_t s) {
+  if (p.tile_rows == 128) return launch_tm<BITS, HAS_ZP, MPS, 2, DT>(p, grid, s);
+  if constexpr (HAS_256)
+    return launch_tm<BITS, HAS_ZP, MPS, 4, DT>(p, grid, s);
+  else
+    return hipErrorInvalidValue;
+}
+
 template <int BITS, bool HAS_ZP, int MPS>
 hipError_t launch(const Gemm256Params& p, unsigned grid, int io, hipStream_t s) {
   if (io == kMnbIoF16Wide) {  // zero points in the activation type exist for 4-bit (and 2-bit, packed as 4-bit) only
     if constexpr (BITS == 4 && HAS_ZP)
-      return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 2>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 2>(p, grid, s);
+      return launch_rows<BITS, HAS_ZP, MPS, 2>(p, grid, s);
     else
       return hipErrorInvalidValue;
   }
-  if (io == kMnbIoBf16) {
-    if constexpr (!kBf16Has256Rows<HAS_ZP, MPS>) return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 1>(p, grid, s) : hipErrorInvalidValue;
-    else return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 1>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 1>(p, grid, s);
-  }
-  return p.tile_rows == 128 ? launch_tm<BITS, HAS_ZP, MPS, 2, 0>(p, grid, s) : launch_tm<BITS, HAS_ZP, MPS, 4, 0>(p, grid, s);
+  if (io == kMnbIoBf16) return launch_rows<BITS, HAS_ZP, MPS, 1, kBf16Has256Rows<HAS_ZP, MPS>>(p, grid, s);
+  return launch_rows<BITS, HAS_ZP, MPS, 0>(p, grid, s);
 }
 
 size_t round256(size_t v) { return (v + 255) / 256 * 256; }
