@@ -312,6 +312,11 @@ MNB_API const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, in
  * most; pitches beyond that range select the streaming kernel, whose addressing is 64-bit. */
 MNB_API const char* MnbGemmKernelNameStrided(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype,
                                              size_t lda);
+/* How the tile GEMM would cut this problem when MnbGemm runs it with the workspace MnbGemmWorkspaceSize asks for: rows and
+ * columns of a tile (256 x 256, 128 x 256 or 128 x 128) and the number of parts a tile is cut into along K; zeros when
+ * another kernel takes the problem.  For logs, profiles and tests. */
+MNB_API int MnbGemmTilePlan(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                            int* tile_rows, int* tile_cols, int* parts);
 
 #ifdef __cplusplus
 }

@@ -98,6 +98,8 @@ SIGNATURES = {
                             c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
     "MnbGemmKernelName": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int]),
     "MnbGemmKernelNameStrided": (c_char_p, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_size_t]),
+    "MnbGemmTilePlan": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int),
+                                ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
 }
 
 _lib = None

@@ -756,4 +756,20 @@ const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_
   return MnbGemmKernelNameStrided(M, N, K, bits, block_size, a_dtype, (K + 7) / 8 * 8);  // the usual aligned rows
 }
 
+int MnbGemmTilePlan(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                    int* tile_rows, int* tile_cols, int* parts) {
+  if (tile_rows) *tile_rows = 0;
+  if (tile_cols) *tile_cols = 0;
+  if (parts) *parts = 0;
+  if (!supported(bits, block_size, a_dtype) || M == 0 || N == 0 || K == 0) return MNB_OK;
+  if (std::string(MnbGemmKernelName(M, N, K, bits, block_size, a_dtype)) != "mnb_gemm256_kernel") return MNB_OK;
+  const MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  const MnbGemm256Plan pl = mnb_gemm256_plan(L, (int64_t)M, true);
+  const int64_t tiles = (((int64_t)M + pl.tile_rows - 1) / pl.tile_rows) * (((int64_t)N + pl.tile_cols - 1) / pl.tile_cols);
+  if (tile_rows) *tile_rows = pl.tile_rows;
+  if (tile_cols) *tile_cols = pl.tile_cols;
+  if (parts) *parts = (int)(pl.grid / tiles);
+  return MNB_OK;
+}
+
 }  // extern "C"

@@ -53,9 +53,8 @@
 
 namespace {
 
-constexpr int BN = 256, BK = 64;
+constexpr int BK = 64;
 constexpr int ROW_BYTES = BK * 2;  // bytes per staged A row (eight 16-byte chunks, XOR-swizzled with the row)
-constexpr int THREADS = 512;
 // Rows of the tile: 64 * TM (TM = 4: 256 x 256; TM = 2: 128 x 256 for grids that leave most of the chip idle with
 // the large tile).  The dynamic LDS allocation is that of TM = 4 for both: three staged A tiles of 32 KiB; the
 // epilogue stages 64 rows of each wavefront's columns in it (40 KiB).
@@ -131,11 +130,12 @@ struct Gemm256Params {
   int ksteps;
   int tiles_m, tiles_n;
   int tile_rows;  // 256 or 128
+  int tile_cols;  // 256, or 128 with 128 rows
   // work distribution: `units` = tiles x ksteps / 2 split over the grid; workgroup w takes
   // [w * share_q + min(w, share_r), (w + 1) * share_q + min(w + 1, share_r))
   int upt;                  // units per tile
   int64_t share_q, share_r;
-  uint64_t* partials;       // one slot of tile_rows x 256 floats per workgroup (NULL: grid == tiles, nothing is split)
+  uint64_t* partials;       // one slot of tile_rows x tile_cols floats per workgroup (NULL: grid == tiles, nothing is split)
   uint32_t* flags;          // one word per workgroup and wavefront, zero when the kernel starts
   int spin_limit;           // polls of a flag before the wait gives up and the tile is poisoned with NaN
   int c_vec_ok;  // C allows 16-byte stores of 8 columns: aligned base and pitch, N a multiple of 8
@@ -207,10 +207,15 @@ __device__ __forceinline__ void slab_end() {
 // every wavefront reads the whole staged A tile (twice the LDS reads).
 // DT: 0 = fp16 model (packed with fp16 meta entries); on a matrix packed with fp32 meta entries: 1 = bfloat16 model,
 // 2 = fp16 model with zero points in the activation type.
-template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT>
-__global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p) {
-  constexpr int WN = 8 / WM;         // wavefront columns
-  constexpr int CT = WM;             // 32-column matrix-core tiles per wavefront: 256 / (32 WN)
+// NWV: wavefronts of the workgroup, 8 (256 columns) or 4 (128 columns: twice the tiles for problems whose 256-column
+// tiles leave compute units idle; same work per wavefront).
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV>
+__global__ void __launch_bounds__(64 * NWV, 2) mnb_gemm256_kernel(Gemm256Params p) {
+  constexpr int THREADS = 64 * NWV;
+  constexpr int WN = NWV / WM;       // wavefront columns
+  constexpr int CT = WM;             // 32-column matrix-core tiles per wavefront
+  constexpr int BN = 32 * CT * WN;   // columns of the tile
+  constexpr int ROWS_PER_LOAD = THREADS / 8;  // rows of A one load instruction of the workgroup stages
   constexpr int RT = 2 * TM / WM;    // 32-row matrix-core tiles per wavefront
   constexpr int WCOLS = 32 * CT;     // columns of a wavefront
   constexpr int BM = 64 * TM;                       // rows of the tile
@@ -251,7 +256,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
   // one of them; with the buffer form its waits are exact.)  The tile's first row and column are
   // part of the uniform base, so a lane's offsets span at most 255 rows of A and 256 columns of weights: they fit
   // 32 bits for every M and N as long as 512 * lda does (mnb_gemm256_addressable).
-  // Load i of a wavefront fills rows i * 64 + wave * 8 + [0, 8) of the staged tile; the lane at chunk position
+  // Load i of a wavefront fills rows i * ROWS_PER_LOAD + wave * 8 + [0, 8) of the staged tile; the lane at chunk position
   // lane & 7 of row lane >> 3 fetches chunk (lane & 7) ^ ((row >> 1) & 7).
   const int a_row = tid >> 3, a_kc = (tid & 7) ^ ((tid >> 4) & 7);
   uint32_t a_off[A_LOADS];                     // byte offsets from a_tile + k0; set per tile (rows beyond M)
@@ -287,7 +292,8 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
     const rsrc_t r = mnb_rsrc(a_tile + (int64_t)ks * BK);
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i)
-      mnb_buffer_load_lds_b128(r, a_off[i], (lds_ptr_t)(lds_bytes + stage_off + (i * 64 + wave * 8) * ROW_BYTES));
+      mnb_buffer_load_lds_b128(r, a_off[i],
+                               (lds_ptr_t)(lds_bytes + stage_off + (i * ROWS_PER_LOAD + wave * 8) * ROW_BYTES));
   };
   // One issue group of the weight prefetch: the loads of issue slot `slot` (see LoadPlan) for k-step ks_raw.
   auto load_b_slot = [&](int ks_raw, Stage& R, int slot) {
@@ -522,7 +528,7 @@ __global__ void __launch_bounds__(THREADS, 2) mnb_gemm256_kernel(Gemm256Params p
 #pragma unroll
     for (int i = 0; i < A_LOADS; ++i) {
       // rows beyond M re-read row M-1 and are never stored (a predicated load would serialise the loop)
-      int r = a_row + i * 64;
+      int r = a_row + i * ROWS_PER_LOAD;
       r = m0 + r < p.M ? r : p.M - 1 - m0;
       a_off[i] = (uint32_t)(((int64_t)r * p.lda + a_kc * 8) * 2);
     }
@@ -695,17 +701,19 @@ __global__ void __launch_bounds__(256) mnb_gemm256_clear_flags_kernel(uint32_t* 
   for (int i = threadIdx.x; i < n; i += 256) flags[i] = 0u;
 }
 
-template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT>
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV = 8>
 hipError_t launch_wm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
-  const size_t smem = (size_t)SMEM_BYTES;  // 98304 bytes
-  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM, DT>;
+  // eight wavefronts: 98304 bytes whatever the tile height (one workgroup per compute unit either way); four: the
+  // three staged tiles of the 128-row tile, so that three workgroups share a compute unit
+  const size_t smem = NWV == 8 ? (size_t)SMEM_BYTES : (size_t)3 * 64 * TM * ROW_BYTES;
+  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM, DT, NWV>;
   // The attribute belongs to the function on the current device, so it is set on every launch (a host-side table
   // update, no device work): callers on several threads or devices need no shared flag.
   if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
       e != hipSuccess)
     return e;
-  kernel<<<dim3(grid), dim3(THREADS), smem, s>>>(p);
+  kernel<<<dim3(grid), dim3(64 * NWV), smem, s>>>(p);
   return hipGetLastError();
 }
 
@@ -726,9 +734,16 @@ hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
 template <bool HAS_ZP, int MPS>
 constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
 
-// 128- or 256-row tiles of element type DT (HAS_256: whether the 256-row member exists)
+// 128- or 256-row tiles of element type DT (HAS_256: whether the 256-row member exists); 128 x 128 tiles for fp16
+// models
 template <int BITS, bool HAS_ZP, int MPS, int DT, bool HAS_256 = true>
 hipError_t launch_rows(const Gemm256Params& p, unsigned grid, hipStream_t s) {
+  if (p.tile_cols == 128) {
+    if constexpr (DT == 0)
+      return p.tile_rows == 128 ? launch_wm<BITS, HAS_ZP, MPS, 2, 1, DT, 4>(p, grid, s) : hipErrorInvalidValue;
+    else
+      return hipErrorInvalidValue;
+  }
   if (p.tile_rows == 128) return launch_tm<BITS, HAS_ZP, MPS, 2, DT>(p, grid, s);
   if constexpr (HAS_256)
     return launch_tm<BITS, HAS_ZP, MPS, 4, DT>(p, grid, s);
@@ -801,47 +816,77 @@ inline double cycles(const Variant& v, int h, int64_t grid, int64_t steps, int p
   if (rest > 0) t += part * load_factor(v.load[h], (double)rest / (double)cus) + fix;
   return t;
 }
+// 128 x 128 tiles (four wavefronts).  Measured: a workgroup alone on its compute unit (one wavefront per SIMD) needs
+// 1100 cycles per k-step (4-bit) and slows down by only 1.19 when every compute unit has one - a single wavefront
+// per SIMD does not draw the power two do; k workgroups on a compute unit share its matrix cores, k x 1222 cycles per
+// step with the chip full, less when only some compute units hold k.  They pay exactly where the 256-column tiles
+// leave half the chip idle and a split along K would need its finishing pass: 5 to 11 % on those shapes.
+constexpr double kNarrowStart[3] = {12000, 13000, 13000};
+constexpr double kNarrowStepAlone[3] = {1100, 1166, 1289};
+constexpr double kNarrowLoad[3] = {1.06, 1.12, 1.19};
+constexpr double kNarrowStepShared[3] = {1222, 1282, 1410};
+inline double cycles_narrow(int vi, int64_t grid, int64_t steps, int64_t cus) {
+  const int64_t k = (grid + cus - 1) / cus;
+  double step;
+  if (k <= 1)
+    step = kNarrowStepAlone[vi] * load_factor(kNarrowLoad, (double)grid / (double)cus);
+  else
+    step = (double)k * kNarrowStepShared[vi] * (0.5 + 0.5 * (double)grid / (double)(k * cus));
+  return kNarrowStart[vi] + (double)steps * step;
+}
 }  // namespace plan_model
+
+namespace {
+size_t split_workspace_bytes(int64_t grid, int rows, int cols) {
+  return round256((size_t)grid * 8 * sizeof(uint32_t)) + (size_t)grid * rows * cols * sizeof(float);
+}
+}  // namespace
 
 MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace) {
   const MnbDeviceInfo& dev = mnb_device_info();
-  const int64_t tiles_n = (L.N + BN - 1) / BN;
   const int64_t ksteps = L.K / BK, upt = ksteps / 2;
-  const plan_model::Variant& v = plan_model::kVariants[L.bits == 4 ? 0 : (L.bs >= 32 ? 1 : 2)];
+  const int vi = L.bits == 4 ? 0 : (L.bs >= 32 ? 1 : 2);
+  const plan_model::Variant& v = plan_model::kVariants[vi];
   const int64_t cus = dev.cus;
   // a matrix packed for an fp32 model is run by the bfloat16 instantiations, whose 8-bit / block 16 / zero-point
   // member has no 256-row form (see kBf16Has256Rows)
   const bool only_128_rows = L.dtype == kMnbDtypeFloat && L.bits == 8 && L.bs < 32 && L.has_zp;
+  const bool narrow_ok = L.dtype == kMnbDtypeFloat16;  // 128 x 128 tiles exist for fp16 models
+  auto tiles_of = [&](int rows, int cols) { return ((M + rows - 1) / rows) * ((L.N + cols - 1) / cols); };
   MnbGemm256Plan best{};
-  for (int h = 0; h < 2; ++h) {
-    const int rows = h == 0 ? 256 : 128;
-    if (rows == 256 && only_128_rows) continue;
-    const int64_t tiles = ((M + rows - 1) / rows) * tiles_n;
+  for (int h = 0; h < 3; ++h) {
+    const int rows = h == 0 ? 256 : 128, cols = h == 2 ? 128 : 256;
+    if ((rows == 256 && only_128_rows) || (h == 2 && !narrow_ok)) continue;
+    const int64_t tiles = tiles_of(rows, cols);
     for (int parts = 1; parts <= 8; ++parts) {
       // parts are whole units (two k-steps) of at least 16 k-steps, and never more than two rounds of workgroups:
       // a part waits for the parts below it, which must not sit in a later round than the model assumes
       if (upt % parts != 0 || (parts > 1 && (!with_workspace || ksteps / parts < 16 || tiles * parts > 2 * cus))) continue;
+      if (h == 2 && parts > 1) continue;  // narrow tiles are the alternative to a split, not its companion
       MnbGemm256Plan pl{};
       pl.tile_rows = rows;
+      pl.tile_cols = cols;
       pl.grid = tiles * parts;
       pl.split = parts > 1;
-      pl.seconds = plan_model::cycles(v, h, pl.grid, ksteps / parts, parts, cus) / dev.clock_hz;
-      if (pl.split)
-        pl.workspace_bytes = round256((size_t)pl.grid * 8 * sizeof(uint32_t)) + (size_t)pl.grid * rows * BN * sizeof(float);
+      pl.seconds = (h == 2 ? plan_model::cycles_narrow(vi, pl.grid, ksteps, cus)
+                           : plan_model::cycles(v, h, pl.grid, ksteps / parts, parts, cus)) /
+                   dev.clock_hz;
+      if (pl.split) pl.workspace_bytes = split_workspace_bytes(pl.grid, rows, cols);
       if (best.grid == 0 || pl.seconds < best.seconds) best = pl;
     }
   }
-  if (const char* e = mnb_tuning_env("MNB_GEMM256_PLAN")) {  // calibration: "<tile rows>,<parts>"
-    int rows = 0, parts = 0;
-    if (sscanf(e, "%d,%d", &rows, &parts) == 2 && (rows == 128 || (rows == 256 && !only_128_rows)) && parts >= 1 && parts <= 8 &&
-        upt % parts == 0 && (parts == 1 || with_workspace)) {
-      const int64_t tiles = ((M + rows - 1) / rows) * tiles_n;
+  if (const char* e = mnb_tuning_env("MNB_GEMM256_PLAN")) {  // calibration: "<tile rows>,<parts>[,<tile columns>]"
+    int rows = 0, parts = 0, cols = 256;
+    const int got = sscanf(e, "%d,%d,%d", &rows, &parts, &cols);
+    if (got >= 2 && (rows == 128 || (rows == 256 && !only_128_rows)) && parts >= 1 && parts <= 8 &&
+        upt % parts == 0 && (parts == 1 || with_workspace) &&
+        (cols == 256 || (cols == 128 && rows == 128 && narrow_ok))) {
       best = MnbGemm256Plan{};
       best.tile_rows = rows;
-      best.grid = tiles * parts;
+      best.tile_cols = cols;
+      best.grid = tiles_of(rows, cols) * parts;
       best.split = parts > 1;
-      best.workspace_bytes =
-          parts > 1 ? round256((size_t)best.grid * 8 * sizeof(uint32_t)) + (size_t)best.grid * rows * BN * sizeof(float) : 0;
+      best.workspace_bytes = parts > 1 ? split_workspace_bytes(best.grid, rows, cols) : 0;
     }
   }
   return best;
@@ -890,8 +935,9 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
                      reinterpret_cast<uintptr_t>(a.workspace) % 8 == 0;
   const MnbGemm256Plan plan = ws_ok ? plan_ws : mnb_gemm256_plan(a.L, a.M, false);
   p.tile_rows = plan.tile_rows;
+  p.tile_cols = plan.tile_cols;
   p.tiles_m = (int)((a.M + p.tile_rows - 1) / p.tile_rows);
-  p.tiles_n = (int)((a.L.N + BN - 1) / BN);
+  p.tiles_n = (int)((a.L.N + p.tile_cols - 1) / p.tile_cols);
   p.upt = p.ksteps / 2;
   const int64_t units = (int64_t)p.tiles_m * p.tiles_n * p.upt;
   if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff) return hipErrorInvalidValue;

@@ -93,6 +93,7 @@ const MnbDeviceInfo& mnb_device_info();
 // how the tile GEMM would run a problem (mnb_gemm256.hip)
 struct MnbGemm256Plan {
   int tile_rows;           // 256 or 128
+  int tile_cols;           // 256, or 128 (with 128 rows, fp16 models)
   int64_t grid;            // workgroups: the tiles, or one per compute unit when tiles are split along K
   bool split;              // tiles are computed in parts by several workgroups (needs workspace_bytes of scratch)
   size_t workspace_bytes;  // flags + one partial tile per workgroup; 0 without a split

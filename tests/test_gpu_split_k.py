@@ -35,7 +35,7 @@ def _gemm(case, op, a, bias, with_workspace):
 
 
 # M, N, K, bits, block size: two and four parts, 128- and 256-row tiles, ragged M / N, 8-bit weights
-SHAPES = [(1024, 4096, 4096, 8, 64), (1000, 4000, 8192, 4, 32), (512, 8192, 8192, 4, 64), (1024, 4096, 14336, 4, 128),
+SHAPES = [(768, 4096, 4096, 8, 64), (1000, 4000, 8192, 4, 32), (512, 8192, 8192, 4, 64), (1024, 4096, 14336, 4, 128),
           (1024, 4096, 8192, 8, 64), (1000, 4090, 14336, 8, 32), (512, 4096, 14336, 8, 64)]
 
 
@@ -96,3 +96,43 @@ def test_fused_gate_up_through_the_split(oracle):
     want = oracle.C.mlp(g.A[rows], (g.B, g.scales, g.bias), (u.B, u.scales, u.bias), N, K, bits, bs).astype(np.float64)
     assert np.linalg.norm(y[rows] - want) / np.linalg.norm(want) <= FP16_GATE
     assert np.isfinite(y).all()
+
+
+def _tile_plan(M, N, K, bits, bs):
+    lib = _lib.load()
+    r, c, p = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    _lib.check(lib.MnbGemmTilePlan(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16, ctypes.byref(r), ctypes.byref(c),
+                                   ctypes.byref(p)))
+    return r.value, c.value, p.value
+
+
+def test_the_shapes_above_are_cut_along_k():
+    for (M, N, K, bits, bs) in SHAPES:
+        rows, cols, parts = _tile_plan(M, N, K, bits, bs)
+        assert cols == 256 and parts > 1, (M, N, K, bits, bs, rows, cols, parts)
+
+
+# problems whose 256-column tiles would leave half of the compute units idle: 128 x 128 tiles of four wavefronts
+NARROW = [(1024, 4096, 4096, 4, 128), (512, 6144, 4096, 4, 32), (1000, 4000, 4096, 8, 64), (1024, 4096, 4096, 8, 16),
+          (250, 14300, 4096, 4, 64)]
+
+
+@pytest.mark.parametrize("M,N,K,bits,bs", NARROW)
+def test_narrow_tiles_against_the_oracle_and_unit_vectors(oracle, M, N, K, bits, bs):
+    assert _tile_plan(M, N, K, bits, bs) == (128, 128, 1)
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, has_bias=True, seed=M + N)
+    op = MatMulNBits(K, N, bits, bs, dtype=torch.float16, has_zero_points=True, has_bias=True)
+    assert op.PrePack(dev(c.B), dev(c.scales), dev(c.zero_points))
+    y, need = _gemm(c, op, dev(c.A), dev(c.bias), True)
+    assert need == 0 and not torch.isnan(y).any()
+    rows = np.unique(np.concatenate([np.linspace(0, M - 1, 7).astype(int), [127, 128, M - 1]]))
+    y64, _ = oracle.C.matmul_f64(c.A[rows], c.B, c.scales, c.zero_points, c.bias, N, K, bits, bs, nthreads=8)
+    got = y[torch.from_numpy(rows).cuda()].cpu().numpy().astype(np.float64)
+    assert np.linalg.norm(got - y64) / np.linalg.norm(y64) <= FP16_GATE
+    # unit-vector rows: column k(m) of the dequantised weights, bit for bit
+    ks = (np.arange(M) * 37 + 5) % K
+    A = np.zeros((M, K), np.float16)
+    A[np.arange(M), ks] = 1
+    y1, _ = _gemm(c, op, dev(A), None, True)
+    w = oracle.C.dequantize(c.B, c.scales, c.zero_points, N, K, bits, bs)
+    assert np.array_equal(y1.cpu().numpy().view(np.uint16), np.ascontiguousarray(w[:, ks].T).view(np.uint16))

@@ -70,14 +70,15 @@ class Plan:
     """The issue order of a k-step, restated: slot 0 the activation loads, slots 1..3 the weight registers reloaded
     after the operands of slabs 1..3 were made, slot 4 those reloaded after slab 0's (behind the barrier)."""
 
-    def __init__(self, bits, mps, tm, ct):
-        """ct: 32-column matrix-core tiles per wavefront = loads per weight vector and per meta entry."""
+    def __init__(self, bits, mps, a_loads, ct):
+        """a_loads: activation loads per thread and k-step (tile rows x 8 / threads); ct: 32-column matrix-core tiles
+        per wavefront = loads per weight vector and per meta entry."""
         self.bits, self.mps = bits, mps
         vps = 2 if bits == 4 else 4
         after = lambda kk: 4 if kk == 0 else kk  # noqa: E731
         self.vec_slot = [after(2 * v + 1 if bits == 4 else v) for v in range(vps)]
         self.meta_slot = [after(2 * e + 1 if bits == 4 else (e + 1) * 4 // mps - 1) for e in range(mps)]
-        self.size = [tm] + [ct * self.vec_slot.count(q) + ct * self.meta_slot.count(q) for q in range(1, 5)]
+        self.size = [a_loads] + [ct * self.vec_slot.count(q) + ct * self.meta_slot.count(q) for q in range(1, 5)]
         self.per_step = sum(self.size)
 
     def before(self, q):
@@ -108,11 +109,14 @@ class Plan:
 def test_every_instantiation_issues_its_loads_and_waits_as_planned(kernels):
     # {4-bit, 8-bit with 2 or 4 entries} x {zp, none} x {128, 256 rows} x {fp16, bfloat16}, less the one that does not
     # fit the register file (bfloat16, four entries with zero points, 256 rows: never launched), plus fp16 on fp32
-    # meta entries (zero points in the activation type: 4-bit with zero points) x {128, 256 rows}
-    assert len(kernels) == 25
+    # meta entries (zero points in the activation type: 4-bit with zero points) x {128, 256 rows}, plus the 128 x 128
+    # tiles of four wavefronts for fp16 models ({4-bit, 8-bit with 2 or 4 entries} x {zp, none})
+    assert len(kernels) == 31
     for name, lines in kernels.items():
-        bits, mps, tm, wm = (int(x) for x in re.search(r"kernelILi(\d)ELb[01]ELi(\d)ELi(\d)ELi(\d)E", name).groups())
-        plan = Plan(bits, mps, tm, ct=wm)  # the wavefronts form wm x 8/wm: 256 / (32 * 8/wm) column tiles each
+        bits, mps, tm, wm, nwv = (int(x) for x in re.search(
+            r"kernelILi(\d)ELb[01]ELi(\d)ELi(\d)ELi(\d)ELi\dELi(\d)E", name).groups())
+        # nwv wavefronts form wm x nwv/wm; 64 tm rows x 8 chunks are loaded by 64 nwv threads
+        plan = Plan(bits, mps, a_loads=64 * tm * 8 // (64 * nwv), ct=wm)
         loops = _hot_loops(lines)
         assert len(loops) == 1, name
         assert loops[0] == plan.step_tokens() * 2, (name, " ".join(loops[0]))
