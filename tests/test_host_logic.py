@@ -196,7 +196,8 @@ def test_dispatch_on_the_benchmark_layer_shapes():
     from onnxruntime_amd.synthetic import C5_SHAPES
     want = {  # M -> kernel, whether the tile GEMM splits tiles along K
         "qkv": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
-        "o": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 1), 4096: ("gemm256", 0)},
+        # (o at M = 1024: 128 x 128 tiles, one per compute unit, instead of a cut along K)
+        "o": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
         "gate_up": {1: ("skinny", 0), 64: ("mid", 1), 256: ("gemm256", 0), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
         "down": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 1), 4096: ("gemm256", 0)},
     }
@@ -207,3 +208,11 @@ def test_dispatch_on_the_benchmark_layer_shapes():
                 assert got == f"mnb_{kernel}_kernel", (bits, name, M, got)
                 need = lib.MnbGemmWorkspaceSize(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16)
                 assert (need > 0) == bool(ws), (bits, name, M, need)
+    import ctypes
+    r, c, p = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    plan = lambda M, N, K: (lib.MnbGemmTilePlan(M, N, K, 4, 128, 1, _lib.DTYPE_FLOAT16, ctypes.byref(r), ctypes.byref(c),
+                                                ctypes.byref(p)), r.value, c.value, p.value)[1:]
+    assert plan(1024, 4096, 4096) == (128, 128, 1)      # o
+    assert plan(1024, 4096, 14336) == (128, 256, 2)     # down
+    assert plan(4096, 28672, 4096) == (256, 256, 1)     # gate_up
+    assert plan(64, 4096, 4096) == (0, 0, 0)            # another kernel
