@@ -734,12 +734,12 @@ hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
 template <bool HAS_ZP, int MPS>
 constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
 
-// 128- or 256-row tiles of element type DT (HAS_256: whether the 256-row member exists); 128 x 128 tiles for fp16
-// models
+// 128- or 256-row tiles of element type DT (HAS_256: whether the 256-row member exists); 128 x 128 tiles for fp16 and
+// bfloat16 models
 template <int BITS, bool HAS_ZP, int MPS, int DT, bool HAS_256 = true>
 hipError_t launch_rows(const Gemm256Params& p, unsigned grid, hipStream_t s) {
   if (p.tile_cols == 128) {
-    if constexpr (DT == 0)
+    if constexpr (DT == 0 || DT == 1)
       return p.tile_rows == 128 ? launch_wm<BITS, HAS_ZP, MPS, 2, 1, DT, 4>(p, grid, s) : hipErrorInvalidValue;
     else
       return hipErrorInvalidValue;
@@ -842,7 +842,7 @@ size_t split_workspace_bytes(int64_t grid, int rows, int cols) {
 }
 }  // namespace
 
-MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace) {
+MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace, int io) {
   const MnbDeviceInfo& dev = mnb_device_info();
   const int64_t ksteps = L.K / BK, upt = ksteps / 2;
   const int vi = L.bits == 4 ? 0 : (L.bs >= 32 ? 1 : 2);
@@ -851,7 +851,9 @@ MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspa
   // a matrix packed for an fp32 model is run by the bfloat16 instantiations, whose 8-bit / block 16 / zero-point
   // member has no 256-row form (see kBf16Has256Rows)
   const bool only_128_rows = L.dtype == kMnbDtypeFloat && L.bits == 8 && L.bs < 32 && L.has_zp;
-  const bool narrow_ok = L.dtype == kMnbDtypeFloat16;  // 128 x 128 tiles exist for fp16 models
+  // 128 x 128 tiles exist for fp16 and bfloat16 models; a matrix packed with fp32 entries may also belong to an fp16
+  // model with zero points in the activation type (4-bit with zero points), which has none
+  const bool narrow_ok = L.dtype == kMnbDtypeFloat16 || io == kMnbIoBf16;
   auto tiles_of = [&](int rows, int cols) { return ((M + rows - 1) / rows) * ((L.N + cols - 1) / cols); };
   MnbGemm256Plan best{};
   for (int h = 0; h < 3; ++h) {
@@ -930,10 +932,10 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.K = (int)a.L.K;
   p.bs_shift = mnb_log2i(a.L.bs);
   p.ksteps = (int)(a.L.K / BK);  // K is a multiple of 2 * BK
-  const MnbGemm256Plan plan_ws = mnb_gemm256_plan(a.L, a.M, true);
+  const MnbGemm256Plan plan_ws = mnb_gemm256_plan(a.L, a.M, true, a.io);
   const bool ws_ok = plan_ws.split && a.workspace != nullptr && a.workspace_bytes >= plan_ws.workspace_bytes &&
                      reinterpret_cast<uintptr_t>(a.workspace) % 8 == 0;
-  const MnbGemm256Plan plan = ws_ok ? plan_ws : mnb_gemm256_plan(a.L, a.M, false);
+  const MnbGemm256Plan plan = ws_ok ? plan_ws : mnb_gemm256_plan(a.L, a.M, false, a.io);
   p.tile_rows = plan.tile_rows;
   p.tile_cols = plan.tile_cols;
   p.tiles_m = (int)((a.M + p.tile_rows - 1) / p.tile_rows);

@@ -99,7 +99,8 @@ struct MnbGemm256Plan {
   size_t workspace_bytes;  // flags + one partial tile per workgroup; 0 without a split
   double seconds;          // estimate, for the choice between kernels
 };
-MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace);
+// io: element type of the activations when it is not the packed matrix's own (MnbGemmArgs::io)
+MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace, int io = kMnbIoModel);
 bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
 // the tile GEMM's 32-bit per-lane offsets reach every element of this problem
 uint64_t mnb_gemm256_max_lane_offset(int64_t lda);

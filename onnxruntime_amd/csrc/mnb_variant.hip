@@ -465,7 +465,8 @@ VariantWorkspace variant_workspace(const MnbVariantPlan& p, size_t M) {
   if (const NativeRoute route = native_route(p, M); route != kNativeNone) {
     // the tile GEMM gets room for the copy whether or not a call needs it: alignment and pitch are not known here
     if (route == kNativeTile || p.has_g_idx) w.staged = round256(M * (size_t)staged_ld(p) * sizeof(uint16_t));
-    if (route == kNativeTile) w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true).workspace_bytes);
+    if (route == kNativeTile)
+      w.inner = round256(mnb_gemm256_plan(packed_layout(p), (int64_t)M, true, native_io(p)).workspace_bytes);
     if (route == kNativeMid) w.inner = round256(mnb_mid_workspace_bytes(packed_layout(p), (int64_t)M));
     return w;
   }

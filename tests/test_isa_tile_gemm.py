@@ -110,8 +110,8 @@ def test_every_instantiation_issues_its_loads_and_waits_as_planned(kernels):
     # {4-bit, 8-bit with 2 or 4 entries} x {zp, none} x {128, 256 rows} x {fp16, bfloat16}, less the one that does not
     # fit the register file (bfloat16, four entries with zero points, 256 rows: never launched), plus fp16 on fp32
     # meta entries (zero points in the activation type: 4-bit with zero points) x {128, 256 rows}, plus the 128 x 128
-    # tiles of four wavefronts for fp16 models ({4-bit, 8-bit with 2 or 4 entries} x {zp, none})
-    assert len(kernels) == 31
+    # tiles of four wavefronts for fp16 and bfloat16 models ({4-bit, 8-bit with 2 or 4 entries} x {zp, none} each)
+    assert len(kernels) == 37
     for name, lines in kernels.items():
         bits, mps, tm, wm, nwv = (int(x) for x in re.search(
             r"kernelILi(\d)ELb[01]ELi(\d)ELi(\d)ELi(\d)ELi\dELi(\d)E", name).groups())
