@@ -22,6 +22,7 @@ pytestmark = pytest.mark.gpu
     (1024, 4096, 4096, 8, 64, np.float16),  # tile GEMM with tiles cut along K (flag-clearing kernel + main kernel)
     (600, 1500, 512, 4, 128, np.float16),   # tile GEMM, ragged
     (24, 700, 1024, 4, 32, np.float32),     # fp32 rows through the fp32 matrix cores
+    (1024, 4096, 4096, 4, 128, np.float16),  # tile GEMM on 128 x 128 tiles of four wavefronts
 ])
 def test_gemm_replays_from_a_hip_graph(M, N, K, bits, bs, dtype):
     c = make_case(M, N, K, bits, bs, dtype, has_zp=True, has_bias=True, seed=M + N)
