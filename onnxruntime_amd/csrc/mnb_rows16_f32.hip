@@ -1,4 +1,4 @@
-// fp32 models with 5 <= M <= 64 rows on the fp32 matrix cores.
+// fp32 models with few rows (5 <= M <= 64, and beyond while the tile GEMM's grid stays small) on the fp32 matrix cores.
 //
 // Between the VALU kernel for very few rows (mnb_gemv.hip: the rows of A ride in scalar registers, which run out
 // beyond eight rows) and the tile GEMM for many (mnb_gemm32.hip: 64 x 128 tiles, N / 128 workgroups - a chip mostly
@@ -203,10 +203,14 @@ hipError_t launch_bs(const Rows16Params& p, int bs, int t, int nw, hipStream_t s
 
 }  // namespace
 
-// Rows of A 16-byte aligned, K a whole number of k-groups; 5 <= M <= 64 (fewer rows: the VALU kernel streams the
-// weights as fast and wastes no matrix-core rows; more: the tile GEMM).
+// Rows of A 16-byte aligned, K a whole number of k-groups; from 5 rows (fewer: the VALU kernel streams the weights as
+// fast and wastes no matrix-core rows) up to where the tile GEMM's 64 x 128 tiles fill the chip: both kernels run the
+// fp32 matrix cores at the same rate once busy (measured 87-89 TFLOP/s), but the tile GEMM pays a whole round of
+// workgroups (183 us at K = 4096) however few of them there are; the two meet at about one and a half rounds.
 bool mnb_rows16_f32_applicable(const MnbGemmArgs& a) {
   int64_t min_m = 5, max_m = 64;
+  const int64_t tile_gemm_wgs = ((a.M + 63) / 64) * ((a.L.N + 127) / 128);
+  if (tile_gemm_wgs * 2 <= (int64_t)mnb_device_info().cus * 3) max_m = a.M;
   if (const char* e = mnb_tuning_env("MNB_ROWS16_M")) {  // calibration: "<min>,<max>"
     long long lo = 0, hi = 0;
     if (sscanf(e, "%lld,%lld", &lo, &hi) == 2) min_m = lo, max_m = hi;

@@ -132,7 +132,7 @@ def test_gemm_parity(oracle, dtype, bits, bs, zp, bias):
 
 
 @pytest.mark.parametrize("bits,bs,zp", [(4, 32, True), (4, 16, False), (8, 64, True), (2, 32, True)])
-@pytest.mark.parametrize("M,N,K,offset", [(1100, 2100, 160, 0), (1100, 2100, 100, 0), (700, 4100, 93, 1)])
+@pytest.mark.parametrize("M,N,K,offset", [(1500, 2100, 160, 0), (1100, 2100, 100, 0), (700, 4100, 93, 1)])
 def test_fp32_matrix_core_gemm_with_128_row_tiles(oracle, bits, bs, zp, M, N, K, offset):
     """fp32 problems whose 64-row tiles no longer fit the chip in one round run 128 x 128 tiles; K that is not a
     multiple of the 32-deep step (tail guarded), A that is not 16-byte aligned (element-wise loads), and unit-vector

@@ -1,4 +1,4 @@
-"""fp32 models with 5 <= M <= 64 rows: the kernel that feeds packed weights from registers to the fp32 matrix cores
+"""fp32 models with few rows (from 5, up to where the tile GEMM's grid fills the chip): the kernel that feeds packed weights from registers to the fp32 matrix cores
 (mnb_rows16_f32.hip), through the C ABI, against the CPU oracle (reference semantics, fp32 tolerance
 |err| <= 1e-4 * sum|a * w|) and bit-exactly on unit-vector rows (the weights are dequantised as (q - zp) * scale, the
 reference's fp32 dequantisation)."""
@@ -20,7 +20,7 @@ def kernel_name(M, N, K, bits, bs):
 # N selects the column tiles per workgroup (one, two, four), K the wavefronts per workgroup (4, 8, 16) and whether the
 # last chunk of four k-groups is partly empty
 SHAPES = [(5, 70, 96), (16, 300, 512), (17, 1000, 1024), (33, 4096, 2048), (64, 520, 4096), (48, 7200, 1056),
-          (9, 14336, 4096), (64, 14336, 512), (40, 3600, 8192), (12, 64, 160)]
+          (9, 14336, 4096), (64, 14336, 512), (40, 3600, 8192), (12, 64, 160), (300, 1000, 512), (130, 4096, 1024)]
 
 
 @pytest.mark.parametrize("bits,bs,zp,bias", [(4, 32, True, True), (4, 128, False, False), (4, 16, True, False),
@@ -51,5 +51,6 @@ def test_unit_rows_recover_the_dequantised_weights(oracle, bits, bs, N, K):
 
 def test_rows_and_k_outside_its_range_take_the_other_kernels():
     assert kernel_name(4, 4096, 4096, 4, 32) == "mnb_gemv_kernel"
-    assert kernel_name(65, 4096, 4096, 4, 32) == "mnb_gemm32_kernel"
+    assert kernel_name(512, 4096, 4096, 4, 32) == KERNEL             # the tile GEMM's grid would be one round
+    assert kernel_name(2048, 4096, 4096, 4, 32) == "mnb_gemm32_kernel"
     assert kernel_name(16, 4096, 4100, 4, 32) != KERNEL   # K is not a whole number of k-groups
