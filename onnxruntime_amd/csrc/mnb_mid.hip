@@ -139,7 +139,13 @@ __device__ __forceinline__ void mid_compute_chunk(const ChunkRegs<BITS, T>& R, h
 
 // What a wavefront needs to issue its first loads comes as leading scalar kernel arguments, which the build asks the
 // compiler to have preloaded into SGPRs at wavefront start; the parameter block carries the rest.
-template <int BITS, bool HAS_ZP, int T, int MT, int NW, int IO>
+// DIRECT: the activations are read from the caller's row-major A (16-byte aligned rows, K a whole number of chunks) and
+// brought into operand order inside the kernel, so the staging pass and its launch drop out: a wavefront reads its
+// chunk of a 16-row tile row-contiguously (64 lanes x 16 bytes = 4 rows x 256 bytes with 4-bit weights: 8 cache lines
+// per instruction), passes it through a private 4 KiB of LDS and picks its operands up from there, tile after tile (LDS
+// executes a wavefront's accesses in order: no barrier).  The loads of the next chunk are issued before the current one
+// is computed and wait in registers (MT x NI vectors).
+template <int BITS, bool HAS_ZP, int T, int MT, int NW, int IO, bool DIRECT>
 __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, int64_t hot_Npad, const uint4* hot_As,
                                                           const uint8_t* hot_meta, int hot_row_tiles, int hot_chunks,
                                                           int hot_bs_shift, MidParams rest) {
@@ -182,6 +188,36 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, in
       for (int i = 0; i < NI; ++i)
         af[mt][i] = __builtin_bit_cast(h8_t, a_lane[((int64_t)c * NI + i) * a_step + mt * 64]);
   };
+  // DIRECT: 16-byte pieces of a chunk's row: PIECES; rows one load instruction covers: RPI (16 / RPI == NI instructions
+  // per 16-row tile).  Pieces are XOR-swizzled with the row so that neither the row-contiguous writes nor the operand
+  // reads conflict on LDS banks.
+  constexpr int PIECES = 4 * NI, RPI = 64 / PIECES;
+  const int piece = lane % PIECES, r0 = lane / PIECES;
+  auto swz = [](int row) { return PIECES == 16 ? row : (row >> 1); };
+  h8_t* const mine = reinterpret_cast<h8_t*>(smem + (size_t)NW * T * 4 * 64 * sizeof(float)) + wave * (16 * PIECES);
+  h8_t g[MT][NI];  // the next chunk's activations on their way (DIRECT)
+  auto fetch_a = [&](int c) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int I = 0; I < NI; ++I) {
+        int row = m0 + mt * 16 + I * RPI + r0;
+        row = row < p.M ? row : p.M - 1;  // rows beyond M re-read the last row and are never stored
+        g[mt][I] = *reinterpret_cast<const h8_t*>(p.A + (int64_t)row * p.lda + (int64_t)c * 4 * GK + piece * 8);
+      }
+  };
+  auto pass_a = [&]() {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+      for (int I = 0; I < NI; ++I) {
+        const int row = I * RPI + r0;
+        mine[row * PIECES + (piece ^ swz(row))] = g[mt][I];
+      }
+#pragma unroll
+      for (int i = 0; i < NI; ++i) af[mt][i] = mine[j * PIECES + ((kq * NI + i) ^ swz(j))];
+    }
+  };
 
   // Weights two chunks ahead (double buffer), activations reloaded word step by word step inside the chunk.  No load
   // of the loop sits under a condition, so every wait counts exactly the loads it needs and leaves the younger
@@ -191,19 +227,43 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, in
   ChunkRegs<BITS, T> R0, R1;
   const int last = p.chunks - 1;
   int c = wave;
-  load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c, last), kq, col0, R0);
-  load_a(min(c, last));
-  load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + NW, last), kq, col0, R1);
-  __builtin_amdgcn_sched_barrier(0);
-  for (; c + NW < p.chunks; c += 2 * NW) {
-    mid_compute_chunk<BITS, HAS_ZP, T, MT, true, IO>(R0, af, a_of(c + NW), a_step, uc, y);
-    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 2 * NW, last), kq, col0, R0);
+  if constexpr (DIRECT) {
+    // weights two chunks ahead, activations one: fetched into g before a chunk is computed, passed through LDS after
+    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c, last), kq, col0, R0);
+    fetch_a(min(c, last));
+    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + NW, last), kq, col0, R1);
+    pass_a();
     __builtin_amdgcn_sched_barrier(0);
-    mid_compute_chunk<BITS, HAS_ZP, T, MT, true, IO>(R1, af, a_of(min(c + 2 * NW, last)), a_step, uc, y);
-    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 3 * NW, last), kq, col0, R1);
+    for (; c + NW < p.chunks; c += 2 * NW) {
+      fetch_a(c + NW);
+      __builtin_amdgcn_sched_barrier(0);
+      mid_compute_chunk<BITS, HAS_ZP, T, MT, false, IO>(R0, af, nullptr, a_step, uc, y);
+      load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 2 * NW, last), kq, col0, R0);
+      __builtin_amdgcn_sched_barrier(0);
+      pass_a();
+      fetch_a(min(c + 2 * NW, last));
+      __builtin_amdgcn_sched_barrier(0);
+      mid_compute_chunk<BITS, HAS_ZP, T, MT, false, IO>(R1, af, nullptr, a_step, uc, y);
+      load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 3 * NW, last), kq, col0, R1);
+      __builtin_amdgcn_sched_barrier(0);
+      pass_a();
+    }
+    if (c < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false, IO>(R0, af, nullptr, a_step, uc, y);
+  } else {
+    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c, last), kq, col0, R0);
+    load_a(min(c, last));
+    load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + NW, last), kq, col0, R1);
     __builtin_amdgcn_sched_barrier(0);
+    for (; c + NW < p.chunks; c += 2 * NW) {
+      mid_compute_chunk<BITS, HAS_ZP, T, MT, true, IO>(R0, af, a_of(c + NW), a_step, uc, y);
+      load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 2 * NW, last), kq, col0, R0);
+      __builtin_amdgcn_sched_barrier(0);
+      mid_compute_chunk<BITS, HAS_ZP, T, MT, true, IO>(R1, af, a_of(min(c + 2 * NW, last)), a_step, uc, y);
+      load_chunk<BITS, HAS_ZP, LOAD_MODE, T>(p, min(c + 3 * NW, last), kq, col0, R1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (c < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false, IO>(R0, af, nullptr, a_step, uc, y);
   }
-  if (c < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false, IO>(R0, af, nullptr, a_step, uc, y);
 
   // reduce over the wavefronts, one row tile at a time: lane (j, kq), register r of y[mt][t] holds
   // row m0 + 16 mt + 4 kq + r, column n0 + 16 t + j
@@ -268,42 +328,59 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   return pl;
 }
 
+// whether the direct form of an instantiation exists: the widest tiles have no registers left for the activations in
+// flight
+template <int BITS, int T, int MT>
+constexpr bool kMidHasDirect = !(MT == 4 && T == 4);
+
 template <int BITS, bool HAS_ZP, int T, int MT, int IO>
-hipError_t launch_nw(const MidParams& mp, const MidPlan& pl, hipStream_t s) {
+hipError_t launch_nw(const MidParams& mp, const MidPlan& pl, bool direct, hipStream_t s) {
   const SkinnyParams& p = mp.s;
   dim3 grid((unsigned)((p.N + 16 * T - 1) / (16 * T)), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)));
-  const size_t smem = (size_t)pl.nw * T * 4 * 64 * sizeof(float);
+  const size_t red = (size_t)pl.nw * T * 4 * 64 * sizeof(float);
+  if constexpr (kMidHasDirect<BITS, T, MT>) {
+    if (direct) {
+      const size_t smem = red + (size_t)pl.nw * 16 * (128 / BITS / 2) * 16;  // + 16 rows of one chunk per wavefront
+      if (pl.nw == 8)
+        mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8, IO, true><<<grid, dim3(512), smem, s>>>(
+            p.W, p.Npad, mp.As, p.meta, mp.row_tiles, p.chunks, p.bs_shift, mp);
+      else
+        mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4, IO, true><<<grid, dim3(256), smem, s>>>(
+            p.W, p.Npad, mp.As, p.meta, mp.row_tiles, p.chunks, p.bs_shift, mp);
+      return hipGetLastError();
+    }
+  }
   if (pl.nw == 8)
-    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8, IO><<<grid, dim3(512), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
-                                                                        p.chunks, p.bs_shift, mp);
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 8, IO, false><<<grid, dim3(512), red, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
+                                                                               p.chunks, p.bs_shift, mp);
   else
-    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4, IO><<<grid, dim3(256), smem, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
-                                                                        p.chunks, p.bs_shift, mp);
+    mnb_mid_kernel<BITS, HAS_ZP, T, MT, 4, IO, false><<<grid, dim3(256), red, s>>>(p.W, p.Npad, mp.As, p.meta, mp.row_tiles,
+                                                                               p.chunks, p.bs_shift, mp);
   return hipGetLastError();
 }
 
 template <int BITS, bool HAS_ZP, int T, int IO>
-hipError_t launch_mt(const MidParams& p, const MidPlan& pl, hipStream_t s) {
-  return pl.mt == 2 ? launch_nw<BITS, HAS_ZP, T, 2, IO>(p, pl, s) : launch_nw<BITS, HAS_ZP, T, 4, IO>(p, pl, s);
+hipError_t launch_mt(const MidParams& p, const MidPlan& pl, bool direct, hipStream_t s) {
+  return pl.mt == 2 ? launch_nw<BITS, HAS_ZP, T, 2, IO>(p, pl, direct, s) : launch_nw<BITS, HAS_ZP, T, 4, IO>(p, pl, direct, s);
 }
 
 template <int BITS, bool HAS_ZP, int IO>
-hipError_t launch_t(const MidParams& p, const MidPlan& pl, hipStream_t s) {
+hipError_t launch_t(const MidParams& p, const MidPlan& pl, bool direct, hipStream_t s) {
   switch (pl.t) {
-    case 4: return launch_mt<BITS, HAS_ZP, 4, IO>(p, pl, s);
-    case 2: return launch_mt<BITS, HAS_ZP, 2, IO>(p, pl, s);
-    default: return launch_mt<BITS, HAS_ZP, 1, IO>(p, pl, s);
+    case 4: return launch_mt<BITS, HAS_ZP, 4, IO>(p, pl, direct, s);
+    case 2: return launch_mt<BITS, HAS_ZP, 2, IO>(p, pl, direct, s);
+    default: return launch_mt<BITS, HAS_ZP, 1, IO>(p, pl, direct, s);
   }
 }
 
 template <int BITS, bool HAS_ZP>
-hipError_t launch_io(const MidParams& p, const MidPlan& pl, int io, hipStream_t s) {
-  if (io == kMnbIoBf16) return launch_t<BITS, HAS_ZP, kMnbIoBf16>(p, pl, s);
+hipError_t launch_io(const MidParams& p, const MidPlan& pl, int io, bool direct, hipStream_t s) {
+  if (io == kMnbIoBf16) return launch_t<BITS, HAS_ZP, kMnbIoBf16>(p, pl, direct, s);
   if (io == kMnbIoF16Wide) {  // zero points in the activation type: 4-bit with zero points
-    if constexpr (BITS == 4 && HAS_ZP) return launch_t<BITS, HAS_ZP, kMnbIoF16Wide>(p, pl, s);
+    if constexpr (BITS == 4 && HAS_ZP) return launch_t<BITS, HAS_ZP, kMnbIoF16Wide>(p, pl, direct, s);
     else return hipErrorInvalidValue;
   }
-  return launch_t<BITS, HAS_ZP, kMnbIoModel>(p, pl, s);
+  return launch_t<BITS, HAS_ZP, kMnbIoModel>(p, pl, direct, s);
 }
 
 int mid_row_tiles(int64_t M, int mt) { return (int)((M + 16 * mt - 1) / (16 * mt)) * mt; }
@@ -360,14 +437,21 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   mp.As = reinterpret_cast<const uint4*>(a.workspace);
   mp.row_tiles = mid_row_tiles(a.M, pl.mt);
   const int vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
-  const int64_t units = (int64_t)p.chunks * (L.group_k / 8) * mp.row_tiles * 64;
-  const dim3 sgrid((unsigned)((units + 255) / 256));
-  uint4* staged = reinterpret_cast<uint4*>(a.workspace);
+  // Activations straight from A when its rows allow 16-byte loads and K is a whole number of chunks (the kernel then
+  // reorders them itself); otherwise, and for the widest tiles, a staging pass writes them in operand order first.
+  bool direct = vec_ok && L.K % CK == 0 && !(pl.mt == 4 && pl.t == 4);
+  if (const char* e = mnb_tuning_env("MNB_MID_DIRECT")) direct = direct && e[0] != '0';  // calibration
+  if (!direct) {
+    const int64_t units = (int64_t)p.chunks * (L.group_k / 8) * mp.row_tiles * 64;
+    const dim3 sgrid((unsigned)((units + 255) / 256));
+    uint4* staged = reinterpret_cast<uint4*>(a.workspace);
+    if (L.bits == 4)
+      mnb_mid_stage_a_kernel<4><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
+    else
+      mnb_mid_stage_a_kernel<8><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+  }
   if (L.bits == 4)
-    mnb_mid_stage_a_kernel<4><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
-  else
-    mnb_mid_stage_a_kernel<8><<<sgrid, dim3(256), 0, s>>>(p.A, p.lda, p.M, p.K, p.chunks, mp.row_tiles, vec_ok, staged);
-  if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
-  if (L.bits == 4) return L.has_zp ? launch_io<4, true>(mp, pl, a.io, s) : launch_io<4, false>(mp, pl, a.io, s);
-  return L.has_zp ? launch_io<8, true>(mp, pl, a.io, s) : launch_io<8, false>(mp, pl, a.io, s);
+    return L.has_zp ? launch_io<4, true>(mp, pl, a.io, direct, s) : launch_io<4, false>(mp, pl, a.io, direct, s);
+  return L.has_zp ? launch_io<8, true>(mp, pl, a.io, direct, s) : launch_io<8, false>(mp, pl, a.io, direct, s);
 }
