@@ -223,7 +223,7 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
     // any alignment) is the faster route whenever the caller's workspace allows it.
     const bool direct = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) &&
                         (a.L.K % (4 * a.L.group_k) == 0);
-    if (!direct && a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;
+    if (!direct && a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;  // (staged there too)
     return kMnbKernelSkinny;
   }
   if (mnb_rows16_f32_applicable(a)) return kMnbKernelRows16F32;
@@ -236,7 +236,8 @@ MnbKernelKind mnb_select_kernel(const MnbGemmArgs& a) {
                          mnb_gemm256_addressable(a.lda, a.L.Npad);
     if (aligned && mnb_prefer_gemm256(a.L, a.M)) return kMnbKernelGemm256;
     // the workspace is sized for the streaming kernel only when the shape alone selects it
-    if (!mnb_prefer_gemm256(a.L, a.M) || a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M)) return kMnbKernelMid;
+    if (!mnb_prefer_gemm256(a.L, a.M) || a.workspace_bytes >= mnb_mid_workspace_bytes(a.L, a.M) || mnb_mid_direct(a))
+      return kMnbKernelMid;
   }
   return kMnbKernelGemmGeneric;
 }
@@ -301,7 +302,7 @@ static int gemm_checked(const char* fn, size_t M, size_t N, size_t K, int bits, 
     case kMnbKernelGemv: e = mnb_launch_gemv(a, s); break;
     case kMnbKernelMid: {
       const size_t need = mnb_mid_workspace_bytes(a.L, a.M);
-      if (a.workspace_bytes < need)
+      if (a.workspace_bytes < need && !mnb_mid_direct(a))  // (aligned activations are read in place)
         return fail(MNB_INVALID_ARGUMENT, "%s: workspace of %zu bytes needed (MnbGemmWorkspaceSize), %zu given", fn, need,
                     a.workspace_bytes);
       e = mnb_launch_mid(a, s);

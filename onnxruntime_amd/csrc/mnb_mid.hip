@@ -399,6 +399,17 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
   return (size_t)chunks * (L.group_k / 8) * mid_row_tiles(M, 4) * 64 * 16;  // the larger of the two row blockings
 }
 
+// Activations straight from A when its rows allow 16-byte loads and K is a whole number of chunks (the kernel then
+// reorders them itself, and no workspace is touched); otherwise, and for the widest tiles, a staging pass writes them
+// in operand order first.
+bool mnb_mid_direct(const MnbGemmArgs& a) {
+  const MidPlan pl = mid_plan(a.L, a.M, a.epi.kind == kMnbFusedMlp ? 2 : 1);
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
+  bool direct = vec_ok && a.L.K % (4 * a.L.group_k) == 0 && !(pl.mt == 4 && pl.t == 4);
+  if (const char* e = mnb_tuning_env("MNB_MID_DIRECT")) direct = direct && e[0] != '0';  // calibration
+  return direct;
+}
+
 hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
   if (!mnb_mid_applicable(a) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
@@ -437,11 +448,9 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
   mp.As = reinterpret_cast<const uint4*>(a.workspace);
   mp.row_tiles = mid_row_tiles(a.M, pl.mt);
   const int vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
-  // Activations straight from A when its rows allow 16-byte loads and K is a whole number of chunks (the kernel then
-  // reorders them itself); otherwise, and for the widest tiles, a staging pass writes them in operand order first.
-  bool direct = vec_ok && L.K % CK == 0 && !(pl.mt == 4 && pl.t == 4);
-  if (const char* e = mnb_tuning_env("MNB_MID_DIRECT")) direct = direct && e[0] != '0';  // calibration
+  const bool direct = mnb_mid_direct(a);
   if (!direct) {
+    if (a.workspace == nullptr || a.workspace_bytes < mnb_mid_workspace_bytes(L, a.M)) return hipErrorInvalidValue;
     const int64_t units = (int64_t)p.chunks * (L.group_k / 8) * mp.row_tiles * 64;
     const dim3 sgrid((unsigned)((units + 255) / 256));
     uint4* staged = reinterpret_cast<uint4*>(a.workspace);

@@ -226,3 +226,36 @@ def test_deterministic_run_to_run():
     y0 = op.Compute(a).clone()
     for _ in range(3):
         assert torch.equal(op.Compute(a), y0)
+
+
+def test_streaming_kernel_needs_no_workspace_when_a_is_aligned(oracle):
+    """16 < M with aligned rows and K a whole number of chunks: the streaming kernel reads A in place, so a call without
+    the workspace MnbGemmWorkspaceSize names is served (bit-identical to the call with it); a misaligned A still needs
+    the staged copy and is refused without room for it."""
+    import ctypes
+    from onnxruntime_amd import _lib
+    lib = _lib.load()
+    M, N, K, bits, bs = 40, 384, 1024, 4, 32
+    assert lib.MnbGemmKernelName(M, N, K, bits, bs, _lib.DTYPE_FLOAT16).decode() == "mnb_mid_kernel"
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, has_bias=True, seed=5)
+    op = make_op(c)
+    a, bias = dev(c.A), dev(c.bias)
+    ptr = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    need = lib.MnbGemmWorkspaceSize(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ys = []
+    for w, nbytes in ((ws, need), (None, 0)):
+        y = torch.empty(M, N, dtype=torch.float16, device="cuda")
+        _lib.check(lib.MnbGemm(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16, ptr(a), K, ptr(op.packed), ptr(bias), ptr(y), N,
+                               ptr(w), nbytes, None))
+        torch.cuda.synchronize()
+        ys.append(y)
+    assert torch.equal(ys[0].view(torch.int16), ys[1].view(torch.int16))
+    check_against_oracle(oracle, c, ys[1].cpu().numpy())
+    flat = torch.zeros(M * K + 1, dtype=torch.float16, device="cuda")
+    flat[1:] = a.reshape(-1)
+    y = torch.empty(M, N, dtype=torch.float16, device="cuda")
+    rc = lib.MnbGemm(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16, ptr(flat[1:]), K, ptr(op.packed), ptr(bias), ptr(y), N,
+                     None, 0, None)
+    assert rc == _lib.INVALID_ARGUMENT and "workspace of" in _lib.last_error()
