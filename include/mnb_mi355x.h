@@ -97,8 +97,9 @@ MNB_API int MnbPackQuantBData(size_t N, size_t K, int bits, int block_size, int 
  * this problem.  Non-zero only for fp16 activations: (a) shapes that select the weight-streaming kernel (M > 16 below
  * the tile GEMM's range, or M <= 16 with K not a multiple of 128 (4-bit) / 64 (8-bit)): a copy of A in matrix-core
  * operand order, about M*K*2 bytes, which that kernel needs unless A is 16-byte aligned with a pitch that is a
- * multiple of 8 and K is a whole number of 128 (4-bit) / 64 (8-bit) elements - such activations are read in place and
- * the call is served without the scratch; (b) tall problems with few output tiles on
+ * multiple of 8 and K is a whole number of 128 (4-bit) / 64 (8-bit) elements - such activations are read in place
+ * (except by the widest tile, 64 rows x 64 columns, which large N with more than 32 rows selects) and the call is
+ * then served without the scratch; (b) tall problems with few output tiles on
  * the tile GEMM, which then cuts every tile along K across workgroups: flags plus one fp32 partial tile per workgroup,
  * up to about 64 MiB.  Without (or with less than) the scratch of (b) the tile GEMM runs uncut. */
 MNB_API size_t MnbGemmWorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
