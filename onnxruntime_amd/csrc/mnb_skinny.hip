@@ -519,6 +519,21 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   pl.t = tiles >= 800 ? 4 : tiles >= 320 ? 2 : 1;  // measured: N = 6144 prefers 2 (192 workgroups), N = 4096 prefers 1
   // wavefronts per workgroup: aim for >= 2 chunks per wavefront
   pl.nw = chunks >= 32 ? 16 : chunks >= 16 ? 8 : 4;
+  // More four-tile slabs than compute units: sixteen-wavefront workgroups run one per unit, in rounds that each pay
+  // their own first-load latency and reduction, and the last round is partly empty.  Smaller workgroups share a unit
+  // and overlap these (measured at K = 4096 and 8192, N = 20480 ... 57344, M = 1, 8, 16: 3-26 % faster; 4-bit
+  // prefers four wavefronts with the general loop, 8-bit eight; up to 1.6 rounds two-tile slabs balance best).
+  const int64_t slabs4 = (tiles + 3) / 4, cus = mnb_device_info().cus;
+  if (direct && pl.nw == 16 && slabs4 > cus) {
+    if (slabs4 * 5 <= cus * 8) {
+      pl.t = 2;
+      pl.nw = M >= 9 ? 4 : 8;
+    } else {
+      pl.nw = L.bits == 4 ? 4 : 8;
+    }
+  }
+  // 8-bit weights over a long K on single-tile slabs: eight wavefronts of twice the chunks (measured, K >= 8192, M = 1 and 8: 4-7 %)
+  if (direct && L.bits == 8 && pl.t == 1 && chunks >= 128 && M <= 8) pl.nw = 8;
   static const char* const plan_override = mnb_tuning_env("MNB_SKINNY_PLAN");  // tuning override "<T>,<NW>", read once
   if (const char* e = plan_override) {
     int t = 0, nw = 0;

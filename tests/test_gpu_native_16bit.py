@@ -100,7 +100,11 @@ def test_unit_rows_recover_columns_of_w_exactly(bits, bs, zp_kind, g_kind, rows)
     (1000, 416, 4, 32, "typed", "none"),      # K that is not a whole number of chunks: activations staged in LDS
     (520, 1000, 8, 16, "u8", "none"),
     (300, 640, 4, 16, "typed", "ragged"),     # gathered columns, blocks of 16
-    (300, 640, 2, 32, "typed", "none")])
+    (300, 640, 2, 32, "typed", "none"),
+    (20480, 4096, 4, 128, "typed", "none"),   # more slabs than compute units: two-tile slabs of eight (four) wavefronts
+    (28672, 4096, 4, 32, "u8", "none"),       # four-tile slabs of four wavefronts, exact weights
+    (28672, 4096, 4, 128, "u8", "none"),      # the same with raw operands
+    (28680, 2048, 8, 64, "u8", "none")])      # 8-bit: eight wavefronts
 @pytest.mark.parametrize("M", [1, 4, 7, 16])
 def test_decode_shapes_against_float64(N, K, bits, bs, zp_kind, g_kind, M):
     c = make("bf16", N, K, bits, bs, zp_kind, g_kind, M, seed=M + N, bias=M % 2 == 0)
@@ -201,6 +205,15 @@ def test_f16_typed_zero_points_unit_rows_recover_w_exactly(bits, bs, rows):
     assert kernel_name(op, M) == {"decode": DECODE, "mid": MID, "tile": TILE}[rows]
     w = C.variant_dequantize(c["B"], c["scales"], c["zp"], None, N, K, bits, bs)
     assert np.array_equal(to_host32(y), w[:, ks].T)
+
+
+@pytest.mark.parametrize("N,K,bs", [(20480, 4096, 128), (28672, 4096, 32), (28672, 4096, 256)])
+@pytest.mark.parametrize("M", [1, 8, 16])
+def test_f16_typed_zero_points_decode_with_more_slabs_than_compute_units(N, K, bs, M):
+    c = make("f16", N, K, 4, bs, "typed", "none", M, seed=M + N, bias=True)
+    y, op = run_op("f16", c, N, K, 4, bs)
+    assert kernel_name(op, M) == DECODE
+    check("f16", c, y, N, K, 4, bs)
 
 
 def test_f16_prefill_shape_with_typed_zero_points():

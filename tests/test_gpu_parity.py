@@ -192,6 +192,25 @@ def test_decode_with_activations_through_lds(oracle, bits, bs, zp, N, K, M):
         assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
 
 
+@pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (8, 64, True), (8, 16, False)])
+@pytest.mark.parametrize("N,K,M", [(20480, 4096, 1), (20490, 4096, 8), (24576, 4096, 16), (28672, 4096, 1),
+                                   (28672, 4096, 9), (33000, 8192, 3), (4096, 8192, 2), (4096, 11008, 8)])
+def test_decode_with_more_slabs_than_compute_units(oracle, bits, bs, zp, N, K, M):
+    """More four-tile slabs than compute units (N > 16384 on 256 units) with a K deep enough for sixteen wavefronts:
+    the decode kernel runs smaller workgroups instead - two-tile slabs up to 1.6 slabs per unit, four or eight
+    wavefronts with the general chunk loop beyond - and 8-bit weights over K >= 8192 run eight wavefronts on
+    single-tile slabs.  Every row of Y against the oracle; unit-vector rows return columns of W bit for bit."""
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + M)
+    check_against_oracle(oracle, c, run_case(c))
+    if K == 4096 and M >= 8:
+        ks = np.random.default_rng(N).choice(K, size=M, replace=False)
+        eye = np.zeros((M, K), np.float16)
+        eye[np.arange(M), ks] = 1
+        c0 = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + M)
+        w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
+        assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+
+
 def test_unpacked_route_matches_packed():
     for dtype in (np.float16, np.float32):
         for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128)]:
