@@ -10,11 +10,13 @@
 // stored scale, the zero point from the unrounded one.  Output is the canonical operand layout of the operator.
 // Positions k >= K of the last block (left unwritten by the reference) receive the zero point: they dequantise to 0.
 //
-// A workgroup owns 64 neighbouring columns and the 8/bits consecutive blocks that share one zero-point byte.  Each
-// block is first copied to LDS with 16-byte loads (rows of the source are contiguous across the 64 columns), so the
+// A workgroup owns 128 neighbouring columns and the 8/bits consecutive blocks that share one zero-point byte.  Each
+// block is first copied to LDS with 16-byte loads (rows of the source are contiguous across the 128 columns: 256-byte
+// pieces of fp16 rows; 128-byte pieces - 64 columns - were measured 8 % slower, 512-byte pieces 20 % slower), so the
 // source is read from HBM exactly once.  Four threads per column take one quarter of the block each: a thread reads
-// its quarter from LDS once, keeps it widened to fp32 in registers across the range scan, and quantises from there
-// (the block size is a template parameter for that reason).  (Reading a thread's elements straight from global
+// its quarter from LDS, keeps it widened to fp32 in registers across the range scan, and quantises from there
+// (the block size is a template parameter for that reason; quarters of 16 and more elements are read a second time
+// instead).  Whole blocks - all but a ragged last one - run without per-element conditions.  (Reading a thread's elements straight from global
 // memory into registers - no LDS tile, one barrier per block - was measured at less than half the speed: 2-byte
 // loads per lane put too few bytes in flight.)
 #include <hip/hip_runtime.h>
@@ -23,7 +25,7 @@
 
 namespace {
 
-constexpr int kCols = 64;      // columns per workgroup
+constexpr int kCols = 128;     // columns per workgroup
 constexpr int kQuarters = 4;   // threads per column (each takes one quarter of the block)
 
 // QROWS = block size / 4: the elements of a thread's quarter.  A compile-time constant so that the quarter, widened
@@ -100,17 +102,35 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
     __syncthreads();
     // range of this thread's quarter, then of the whole block
     const int mine = rows - q0 < QROWS ? rows - q0 : QROWS;  // rows of the quarter that exist (may be <= 0)
-    float held[QROWS];
+    const bool whole = rows == bs;  // every block but a ragged last one: no per-element conditions (uniform)
+    // blocks of 64 and more elements read the tile a second time when they quantise instead of holding their
+    // quarter in registers (which, with the registers of the load in flight, keeps wavefronts off the SIMD)
+    constexpr bool kHold = QROWS < 16;
+    float held[kHold ? QROWS : 1];
     float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+    if (whole) {
 #pragma unroll
-    for (int e = 0; e < QROWS; ++e) {
-      float v = 0.f;
-      if (e < mine) {
-        v = (float)tile[(q0 + e) * kCols + c];
-        mn = v < mn ? v : mn;
-        mx = v > mx ? v : mx;
+      for (int e = 0; e < QROWS; ++e) {
+        const float v = (float)tile[(q0 + e) * kCols + c];
+        mn = __builtin_fminf(v, mn);  // one instruction each; like the comparisons below they skip a NaN
+        mx = __builtin_fmaxf(v, mx);
+        if constexpr (kHold) held[e] = v;
       }
-      held[e] = v;
+      // The reference's scan (if (v < min) min = v) keeps the first zero it meets, whatever its sign, where the
+      // minimum instruction prefers -0.  Only an all-zero block shows it (the sign of its stored scale, taken from
+      // the block's first element): restore the first element there.
+      if (mn == 0.f && mx == 0.f) mn = mx = (float)tile[q0 * kCols + c];
+    } else {
+#pragma unroll
+      for (int e = 0; e < QROWS; ++e) {
+        float v = 0.f;
+        if (e < mine) {
+          v = (float)tile[(q0 + e) * kCols + c];
+          mn = v < mn ? v : mn;
+          mx = v > mx ? v : mx;
+        }
+        if constexpr (kHold) held[e] = v;
+      }
     }
     red[qr * kCols + c] = mn;
     red[(kQuarters + qr) * kCols + c] = mx;
@@ -153,21 +173,29 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
       uint32_t word[QWORDS];
 #pragma unroll
       for (int w = 0; w < QWORDS; ++w) word[w] = 0;
+      // clamp(roundf(t), 0, MAXQ), roundf rounding halves away from zero: for t >= 0 that is trunc(t + 0.49999997f)
+      // (the largest float below one half: a sum that lands exactly between two floats rounds to the even one,
+      // which is the integer, only when t itself is a tie), everything below 0.5 ends at 0 either way, and the clamp
+      // commutes with the truncation because its bounds are integers.
+      auto quantise = [&](float v) -> uint32_t {
+        float t = v * rscale;  // separate statements: the product is rounded before the addition
+        t = t + zf32;
+        t = t + 0.49999997f;
+        t = __builtin_amdgcn_fmed3f(t, 0.f, (float)MAXQ);
+        return (uint32_t)t;
+      };
+      if (whole) {
 #pragma unroll
-      for (int e = 0; e < QROWS; ++e) {
-        uint32_t q = (uint32_t)z;
-        if (e < mine) {
-          float t = held[e] * rscale;  // separate statements: the product is rounded before the addition
-          t = t + zf32;
-          // clamp(roundf(t), 0, MAXQ), roundf rounding halves away from zero: for t >= 0 that is
-          // trunc(t + 0.49999997f) (the largest float below one half: a sum that lands exactly between two floats
-          // rounds to the even one, which is the integer, only when t itself is a tie), everything below 0.5 ends
-          // at 0 either way, and the clamp commutes with the truncation because its bounds are integers.
-          t = t + 0.49999997f;
-          t = __builtin_amdgcn_fmed3f(t, 0.f, (float)MAXQ);
-          q = (uint32_t)t;
+        for (int e = 0; e < QROWS; ++e) {
+          const float v = kHold ? held[e] : (float)tile[(q0 + e) * kCols + c];
+          word[(e * BITS) / 32] |= quantise(v) << ((e * BITS) % 32);
         }
-        word[(e * BITS) / 32] |= q << ((e * BITS) % 32);
+      } else {
+#pragma unroll
+        for (int e = 0; e < QROWS; ++e) {
+          const uint32_t q = e < mine ? quantise(kHold ? held[e] : (float)tile[(q0 + e) * kCols + c]) : (uint32_t)z;
+          word[(e * BITS) / 32] |= q << ((e * BITS) % 32);
+        }
       }
       uint8_t* out = B + (n * kbc + kb) * blob + qr * (QBITS / 8);
       if constexpr (QBITS == 8) {
@@ -200,8 +228,8 @@ hipError_t launch_k(void* B, void* scales, void* zp, const void* src, int64_t K,
   }
   const int64_t kbc = (K + bs - 1) / bs;
   // Blocks per workgroup: the 8/bits blocks of one zero-point byte when zero points are written, else one.  Many
-  // small workgroups beat few long ones here: [4096, 14336] fp16 to 4 bits, blocks of 128, takes 36 us with one
-  // block per workgroup (7168 workgroups), 41 us with two and 44-46 us with four to eight.
+  // small workgroups beat few long ones here: [4096, 14336] fp16 to 4 bits, blocks of 128, took 36 us with one
+  // block per workgroup, 41 us with two and 44-46 us with four to eight (64-column workgroups).
   const int nsub = zp ? 8 / BITS : 1;
   const int64_t strips = (N + kCols - 1) / kCols;
   dim3 grid((unsigned)strips, (unsigned)((kbc + nsub - 1) / nsub)), blk(kCols * kQuarters);

@@ -40,6 +40,43 @@ def test_identical_to_oracle(oracle, dtype, bits, bs, symmetric):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bs", [16, 64, 128])
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_signed_zeros_and_nans_follow_the_sequential_scan(oracle, dtype, bs, symmetric):
+    """The reference scans a block with `if (v < min) min = v; if (v > max) max = v` (q4_dq.cpp:513-516): among equal
+    values the first one met stays, so the symmetric scale of an all-zero block takes its sign from the block's first
+    element (+0 -> scale -0, -0 -> scale +0), zeros of either sign inside an ordinary block change nothing, and a NaN
+    never enters the range.  Whole blocks and a ragged last block, every quarter of a block starting with either
+    zero."""
+    K, N = 3 * bs + bs // 2, 140
+    rng = np.random.default_rng(bs)
+    W = np.zeros((K, N), dtype)
+    signs = rng.integers(0, 2, size=(K, N)).astype(bool)
+    W[signs] = -0.0                                       # columns 0..69: nothing but zeros of random sign
+    W[:, 70:] = rng.standard_normal((K, N - 70)).astype(dtype)
+    zero_at = rng.integers(0, 4, size=(K, N - 70)) == 0   # columns 70..: ordinary values with zeros of both signs
+    W[:, 70:][zero_at] = np.where(rng.integers(0, 2, size=int(zero_at.sum())).astype(bool), -0.0, 0.0).astype(dtype)
+    W[0, :35], W[0, 35:70] = 0.0, -0.0                    # both first elements, also for the later blocks' quarters
+    for q in range(1, 14):
+        W[q * bs // 4, q % 2:70:2] = -0.0
+    Wn = W.copy()
+    Wn[1::7, 100:] = np.nan                               # NaNs are skipped by both comparisons
+    for src in (W, Wn):
+        Bq, s, z = oracle.C.quantize(src, 4, bs, symmetric)
+        b, sc, zp = quantize_blockwise(dev(src), 4, bs, symmetric)
+        torch.cuda.synchronize()
+        assert np.array_equal(_bits(sc.cpu().numpy()), _bits(s))
+        if not symmetric:
+            assert np.array_equal(zp.cpu().numpy(), z)
+        if src is W:                                      # (a NaN element itself converts to an unspecified integer)
+            assert np.array_equal(b.cpu().numpy(), Bq)
+    if symmetric:
+        s_bits = _bits(s)[:70, 0]
+        sign = np.uint32(1) << np.uint32(8 * s.dtype.itemsize - 1)
+        assert np.array_equal((s_bits & sign) != 0, np.arange(70) < 35)   # +0 first -> scale -0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("bits", [2, 4, 8])
 @pytest.mark.parametrize("bs", [16, 64])
 @pytest.mark.parametrize("symmetric", [False, True])
