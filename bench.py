@@ -31,7 +31,7 @@ sys.path.insert(0, str(ROOT))
 # dispatch as printed there).  Every `traffic` value in the output carries `traffic_source` beside it.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_skinny_c2_gemm256_c4_quantize.md (rocprofv3 --pmc; a constant, not this run)"
 PROFILED_TRAFFIC_BYTES = {"c2_decode": int((14858.5 * 2.0 + 28.0) * 1024), "c4_prefill": int((109777.3 * 2.0 + 57344.0) * 1024),
-                          "quantize": int((57399.0 * 2.0 + 30511.9) * 1024), "mlp_decode": int((29675.0 * 2.0 + 28.0) * 1024)}
+                          "quantize": int((57412.5 * 2.0 + 36364.4) * 1024), "mlp_decode": int((29675.0 * 2.0 + 28.0) * 1024)}
 # The reference's own MLAS kernel on the headline shape, timed by the survey on an 8-vCPU Sapphire-Rapids-class host
 # (standalone MLAS build, SQNBIT_CompFp32, N sliced over 8 threads): quoted beside the port so that the port's
 # figure is not read as the reference's.
