@@ -223,10 +223,9 @@ __global__ void __launch_bounds__(kCols * kQuarters) mnb_quantize_kernel(uint8_t
 // block of 64), so blocks of up to 32 need no exchange of ranges at all, the source is still read in 256-byte pieces
 // of 64 or 128 rows, a column's BPW blobs are contiguous in B, and the zero points of the blocks that share a byte
 // meet in LDS.  One pass per workgroup; the arithmetic is that of the kernel above, statement for statement.
-constexpr int kSlots = 4;  // threads per column
-
-template <typename T, int BITS, int BS, int TPB>
-__global__ void __launch_bounds__(kCols * kSlots) mnb_quantize_small_kernel(uint8_t* __restrict__ B, T* __restrict__ scales,
+// SLOTS = threads per column
+template <typename T, int BITS, int BS, int TPB, int SLOTS>
+__global__ void __launch_bounds__(kCols * SLOTS) mnb_quantize_small_kernel(uint8_t* __restrict__ B, T* __restrict__ scales,
                                                                             uint8_t* __restrict__ zp,
                                                                             const T* __restrict__ src, int64_t K,
                                                                             int64_t N, int64_t ld, int vec_ok) {
@@ -235,7 +234,7 @@ __global__ void __launch_bounds__(kCols * kSlots) mnb_quantize_small_kernel(uint
   constexpr int MID = 1 << (BITS - 1);
   constexpr int VEC = 16 / (int)sizeof(T);
   constexpr int EPT = BS / TPB;        // elements per thread
-  constexpr int BPW = kSlots / TPB;    // blocks per workgroup
+  constexpr int BPW = SLOTS / TPB;    // blocks per workgroup
   constexpr int ROWS = BPW * BS;
   constexpr int blob = BS * BITS / 8;
   constexpr int QWORDS = EPT * BITS / 32;
@@ -243,8 +242,8 @@ __global__ void __launch_bounds__(kCols * kSlots) mnb_quantize_small_kernel(uint
                 "a thread writes whole words; a zero-point byte stays in one workgroup");
   extern __shared__ __align__(16) unsigned char smem[];
   T* tile = reinterpret_cast<T*>(smem);                                              // [ROWS][kCols]
-  float* red = reinterpret_cast<float*>(smem + (size_t)ROWS * kCols * sizeof(T));    // [2][kSlots][kCols]
-  uint32_t* zs = reinterpret_cast<uint32_t*>(red + 2 * kSlots * kCols);              // [BPW][kCols]
+  float* red = reinterpret_cast<float*>(smem + (size_t)ROWS * kCols * sizeof(T));    // [2][SLOTS][kCols]
+  uint32_t* zs = reinterpret_cast<uint32_t*>(red + 2 * SLOTS * kCols);              // [BPW][kCols]
 
   const int tid = threadIdx.x;
   const int c = tid % kCols, slot = tid / kCols;
@@ -260,22 +259,22 @@ __global__ void __launch_bounds__(kCols * kSlots) mnb_quantize_small_kernel(uint
 
   if (vec_ok && n0 + kCols <= N) {
     constexpr int CH = kCols / VEC;                       // 16-byte chunks per row
-    constexpr int PRE = ROWS * CH / (kCols * kSlots);     // chunks per thread
-    static_assert(ROWS * CH % (kCols * kSlots) == 0, "whole chunks per thread");
+    constexpr int PRE = ROWS * CH / (kCols * SLOTS);     // chunks per thread
+    static_assert(ROWS * CH % (kCols * SLOTS) == 0, "whole chunks per thread");
     uint4 pre[PRE];
 #pragma unroll
     for (int u = 0; u < PRE; ++u) {
-      const int i = tid + u * kCols * kSlots;
+      const int i = tid + u * kCols * SLOTS;
       const int r = i / CH < rows ? i / CH : rows - 1;    // rows beyond K re-read the last one and are never used
       pre[u] = *reinterpret_cast<const uint4*>(src + (k0 + r) * ld + n0 + (i % CH) * VEC);
     }
 #pragma unroll
     for (int u = 0; u < PRE; ++u) {
-      const int i = tid + u * kCols * kSlots;
+      const int i = tid + u * kCols * SLOTS;
       *reinterpret_cast<uint4*>(tile + (i / CH) * kCols + (i % CH) * VEC) = pre[u];
     }
   } else {
-    for (int i = tid; i < rows * kCols; i += kCols * kSlots) {
+    for (int i = tid; i < rows * kCols; i += kCols * SLOTS) {
       const int r = i / kCols, cc = i % kCols;
       tile[r * kCols + cc] = n0 + cc < N ? src[(k0 + r) * ld + n0 + cc] : (T)0.0f;
     }
@@ -307,11 +306,11 @@ __global__ void __launch_bounds__(kCols * kSlots) mnb_quantize_small_kernel(uint
   }
   if constexpr (TPB > 1) {
     red[slot * kCols + c] = mn;
-    red[(kSlots + slot) * kCols + c] = mx;
+    red[(SLOTS + slot) * kCols + c] = mx;
     __syncthreads();
 #pragma unroll
     for (int q2 = 0; q2 < TPB; ++q2) {
-      const float a = red[(bi * TPB + q2) * kCols + c], b = red[(kSlots + bi * TPB + q2) * kCols + c];
+      const float a = red[(bi * TPB + q2) * kCols + c], b = red[(SLOTS + bi * TPB + q2) * kCols + c];
       mn = a < mn ? a : mn;
       mx = b > mx ? b : mx;
     }
@@ -388,16 +387,17 @@ template <typename T, int BITS, int BS>
 hipError_t launch_small(void* B, void* scales, void* zp, const void* src, int64_t K, int64_t N, int64_t ld,
                         hipStream_t s) {
   constexpr int TPB = (BS == 64 && BITS != 2) ? 2 : 1;  // 2-bit blocks of 64: four blocks share a zero-point byte
-  constexpr int BPW = kSlots / TPB, ROWS = BPW * BS;
-  const auto kernel = mnb_quantize_small_kernel<T, BITS, BS, TPB>;
-  const size_t smem = (size_t)ROWS * kCols * sizeof(T) + 2 * kSlots * kCols * sizeof(float) + (size_t)BPW * kCols * 4;
+  constexpr int SLOTS = 4;  // (eight for blocks of 16 - 128 rows again - was measured: no difference)
+  constexpr int BPW = SLOTS / TPB, ROWS = BPW * BS;
+  const auto kernel = mnb_quantize_small_kernel<T, BITS, BS, TPB, SLOTS>;
+  const size_t smem = (size_t)ROWS * kCols * sizeof(T) + 2 * SLOTS * kCols * sizeof(float) + (size_t)BPW * kCols * 4;
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)smem);
     if (e != hipSuccess) return e;
   }
   const int64_t kbc = (K + BS - 1) / BS;
-  dim3 grid((unsigned)((N + kCols - 1) / kCols), (unsigned)((kbc + BPW - 1) / BPW)), blk(kCols * kSlots);
+  dim3 grid((unsigned)((N + kCols - 1) / kCols), (unsigned)((kbc + BPW - 1) / BPW)), blk(kCols * SLOTS);
   const int vec_ok = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (ld % (16 / sizeof(T)) == 0);
   kernel<<<grid, blk, smem, s>>>((uint8_t*)B, (T*)scales, (uint8_t*)zp, (const T*)src, K, N, ld, vec_ok);
   return hipGetLastError();
