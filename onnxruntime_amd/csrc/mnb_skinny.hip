@@ -532,9 +532,6 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
       pl.nw = L.bits == 4 ? 4 : 8;
     }
   }
-  // 8-bit weights over a long K on single-tile slabs: eight wavefronts of twice the chunks (measured, K >= 8192,
-  // M = 1 and 8: 4-7 %)
-  if (direct && L.bits == 8 && pl.t == 1 && chunks >= 128 && M <= 8) pl.nw = 8;
   static const char* const plan_override = mnb_tuning_env("MNB_SKINNY_PLAN");  // tuning override "<T>,<NW>", read once
   if (const char* e = plan_override) {
     int t = 0, nw = 0;
@@ -546,12 +543,20 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   if (pl.t < min_t) pl.t = min_t;  // gate/up pairs live in one workgroup
   // three tiles per workgroup (slab kernel): one round of at most 256 workgroups where two tiles would need up to 384
   if (direct && min_t == 1 && tiles > 512 && tiles <= 768 && plan_override == nullptr) pl.t = 3;
-  // 4-bit weights as raw operands on slabs of two or four tiles: five to eight rows of A read straight from memory
-  // (two cache lines per row and load), and K >= 8192, run better on eight wavefronts of twice the chunks (measured
-  // N = 8192 ... 16384: 0-11 %, most with zero points; exact operands, blocks of 64 at N = 6144, do not gain)
-  if (plan_override == nullptr && direct && L.bits == 4 && pl.mode == 0 && pl.nw == 16 && (pl.t == 2 || pl.t == 4) &&
-      M <= 8 && (M >= 5 || (pl.t == 4 && chunks >= 64)))
-    pl.nw = 8;
+  // Eight wavefronts of twice the chunks instead of sixteen (fp16 models; measured on K = 4096 ... 14336):
+  //  * single-tile slabs (N < 5120), up to eight rows or K up to 64 chunks: 2-9 % (N = K = 4096 int4 M = 1:
+  //    4.5 -> 4.1 us; 8-bit K >= 8192: 4-7 %);
+  //  * two-tile slabs with K up to 64 chunks, 8-bit weights or raw 4-bit operands: 1-6 %, M = 1 even;
+  //  * raw 4-bit operands on slabs of two or four tiles with five to eight rows of A read straight from memory (two
+  //    cache lines per row and load), and four-tile slabs with K >= 8192: 0-11 %, most with zero points.
+  // Exact 4-bit operands (blocks of 32 and 64) on two-tile slabs do not gain.
+  if (plan_override == nullptr && direct && pl.nw == 16 && pl.mode <= 1) {
+    const bool raw4 = L.bits == 4 && pl.mode == 0;
+    if (pl.t == 1 ? (M <= 8 || chunks <= 64)
+                  : (pl.t == 2 && chunks <= 64 && (L.bits == 8 || raw4)) ||
+                        (raw4 && (pl.t == 2 || pl.t == 4) && M <= 8 && (M >= 5 || (pl.t == 4 && chunks >= 64))))
+      pl.nw = 8;
+  }
   // Activations through LDS (see AStage) pay from nine rows on, for single-tile slabs from five (measured: at
   // M = 8 the wider slabs gain or lose a few per cent either way; at M = 16 everything gains 10-35 % except the
   // general loop of four-tile slabs).  The general loop needs one more operand set for it, which sixteen wavefronts
