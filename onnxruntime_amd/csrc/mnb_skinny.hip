@@ -546,16 +546,22 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   // Eight wavefronts of twice the chunks instead of sixteen (fp16 models; measured on K = 4096 ... 14336):
   //  * single-tile slabs (N < 5120), up to eight rows or K up to 64 chunks: 2-9 % (N = K = 4096 int4 M = 1:
   //    4.5 -> 4.1 us; 8-bit K >= 8192: 4-7 %);
-  //  * two-tile slabs with K up to 64 chunks, 8-bit weights or raw 4-bit operands: 1-6 %, M = 1 even;
+  //  * two-tile slabs at K = 4096, 8-bit weights or raw 4-bit operands: 1-6 %, M = 1 even; three-tile slabs of raw
+  //    4-bit operands at K = 4096 from four rows on: 0-10 % (at K = 8192 they lose 1-4 %);
   //  * raw 4-bit operands on slabs of two or four tiles with five to eight rows of A read straight from memory (two
   //    cache lines per row and load), and four-tile slabs with K >= 8192: 0-11 %, most with zero points.
   // Exact 4-bit operands (blocks of 32 and 64) on two-tile slabs do not gain.
   if (plan_override == nullptr && direct && pl.nw == 16 && pl.mode <= 1) {
     const bool raw4 = L.bits == 4 && pl.mode == 0;
     if (pl.t == 1 ? (M <= 8 || chunks <= 64)
-                  : (pl.t == 2 && chunks <= 64 && (L.bits == 8 || raw4)) ||
+                  : (pl.t == 2 && ((L.bits == 8 && chunks <= 64) || (raw4 && chunks <= 32))) ||
+                        (pl.t == 3 && raw4 && chunks <= 32 && M >= 4) ||
                         (raw4 && (pl.t == 2 || pl.t == 4) && M <= 8 && (M >= 5 || (pl.t == 4 && chunks >= 64))))
       pl.nw = 8;
+  }
+  if (const char* e = mnb_tuning_env("MNB_SKINNY_NW")) {  // tuning override of the wavefront count alone
+    const int nw = atoi(e);
+    if (nw == 4 || nw == 8 || nw == 16) pl.nw = nw;
   }
   // Activations through LDS (see AStage) pay from nine rows on, for single-tile slabs from five (measured: at
   // M = 8 the wider slabs gain or lose a few per cent either way; at M = 16 everything gains 10-35 % except the
