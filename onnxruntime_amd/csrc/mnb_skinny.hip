@@ -559,6 +559,11 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
                         (raw4 && (pl.t == 2 || pl.t == 4) && M <= 8 && (M >= 5 || (pl.t == 4 && chunks >= 64))))
       pl.nw = 8;
   }
+  // 16-bit models on fp32 entries: only raw operands on single-tile slabs with up to four rows gain (N = K = 4096
+  // M = 1: 5.0 -> 4.6 us); every other shape of the sweep was equal or slower with eight wavefronts
+  if (plan_override == nullptr && direct && pl.nw == 16 && (pl.mode == 4 || pl.mode == 5) && pl.t == 1 && M <= 4 &&
+      chunks <= 32)
+    pl.nw = 8;
   if (const char* e = mnb_tuning_env("MNB_SKINNY_NW")) {  // tuning override of the wavefront count alone
     const int nw = atoi(e);
     if (nw == 4 || nw == 8 || nw == 16) pl.nw = nw;
