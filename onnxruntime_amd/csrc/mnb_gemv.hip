@@ -456,7 +456,13 @@ template <int BITS, bool HAS_ZP, bool SMALL_BS, int MT>
 hipError_t launch_gemv16_nw(const GemvParams& p, hipStream_t s) {
   dim3 grid((unsigned)((p.N + 15) / 16));
   const int chunks = (p.KG + 3) / 4;
-  if (chunks >= 32) {
+  // K split over 4, 8 or 16 wavefronts; sixteen while the grid has at most two workgroups per compute unit (measured:
+  // N = K = 4096 M = 1/2/4: 7.1 -> 6.8, 8.5 -> 7.6, 11.3 -> 9.6 us; K = 14336: 20.4 -> 16.3 us; N = 11008: 11.1 -> 12.0)
+  int nw = chunks >= 32 ? (grid.x <= 2u * (unsigned)mnb_device_info().cus ? 16 : 8) : 4;
+  if (const char* e = mnb_tuning_env("MNB_GEMV16_NW")) nw = atoi(e);
+  if (nw == 16) {
+    mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 16><<<grid, dim3(1024), 0, s>>>(MNB_GEMV_HOT_ARGS(p), p);
+  } else if (nw == 8) {
     mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 8><<<grid, dim3(512), 0, s>>>(MNB_GEMV_HOT_ARGS(p), p);
   } else {
     mnb_gemv16_kernel<BITS, HAS_ZP, SMALL_BS, MT, 4><<<grid, dim3(256), 0, s>>>(MNB_GEMV_HOT_ARGS(p), p);

@@ -211,6 +211,23 @@ def test_decode_with_more_slabs_than_compute_units(oracle, bits, bs, zp, N, K, M
         assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
 
 
+@pytest.mark.parametrize("bits,bs,zp", [(4, 32, True), (4, 128, False), (4, 16, True), (8, 64, True)])
+@pytest.mark.parametrize("N,K", [(300, 4096), (4100, 8192), (1000, 14336), (8200, 4096)])
+@pytest.mark.parametrize("M", [1, 2, 4])
+def test_fp32_few_rows_with_k_split_over_sixteen_wavefronts(oracle, bits, bs, zp, N, K, M):
+    """fp32 models, up to four rows, K of 32 chunks and more on grids of up to two workgroups per compute unit: the
+    16-column kernel splits K over sixteen wavefronts (eight on larger grids: N = 8200 here).  Against the oracle, and
+    unit-vector rows return columns of W bit for bit."""
+    c = make_case(M, N, K, bits, bs, np.float32, has_zp=zp, has_bias=True, seed=N + K + M)
+    check_against_oracle(oracle, c, run_case(c))
+    ks = np.random.default_rng(K + M).choice(K, size=M, replace=False)
+    eye = np.zeros((M, K), np.float32)
+    eye[np.arange(M), ks] = 1
+    c0 = make_case(M, N, K, bits, bs, np.float32, has_zp=zp, seed=N + K + M)
+    w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
+    assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+
+
 def test_unpacked_route_matches_packed():
     for dtype in (np.float16, np.float32):
         for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128)]:
