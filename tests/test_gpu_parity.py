@@ -154,11 +154,12 @@ def test_fp32_matrix_core_gemm_with_128_row_tiles(oracle, bits, bs, zp, M, N, K,
 
 @pytest.mark.parametrize("bits,bs,zp", [(4, 128, False), (4, 128, True), (4, 32, True), (8, 64, True), (8, 16, False)])
 @pytest.mark.parametrize("N,K,M", [(8200, 512, 1), (9000, 1024, 5), (12288, 2048, 16), (11008, 4096, 1),
-                                   (12281, 640, 3)])
+                                   (12281, 640, 3), (9216, 4096, 8), (11008, 4096, 16)])
 def test_decode_with_three_tile_slabs(oracle, bits, bs, zp, N, K, M):
     """513..768 column tiles: the decode kernel cuts N into slabs of 48 columns that do not start at multiples of 64
     (tiles addressed one by one); every chunk schedule (one, two, many chunks per wavefront), both dequantisation
-    modes, ragged N, and unit vectors that recover W bit for bit across slab boundaries."""
+    modes, ragged N, eight wavefronts instead of sixteen for raw 4-bit operands from four rows on (the last two
+    shapes), and unit vectors that recover W bit for bit across slab boundaries."""
     c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + bits)
     y = run_case(c)
     check_against_oracle(oracle, c, y)
