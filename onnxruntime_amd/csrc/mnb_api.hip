@@ -489,9 +489,14 @@ FusedWorkspace fused_workspace(const MnbFusedLayout& F, size_t M, int has_norm) 
     // fp16: the decode and streaming kernels write the operator's outputs themselves, and so does the tile GEMM when
     // the outputs allow 16-byte stores.  Where the shape selects the tile GEMM, the streaming kernel's scratch is
     // reserved as well: it takes over when the caller's pointers turn out not to be aligned.
-    const bool tile_gemm = M > 16 && w.inner == 0;
-    if (tile_gemm && widths_allow_vector_stores(F)) w.inner = mnb_mid_workspace_bytes(L, (int64_t)M);
-    w.tmp = (tile_gemm && w.inner == 0) ? round256(M * (size_t)L.N * elem_size(L.dtype)) : 0;
+    // (The shape alone decides: MnbGemmWorkspaceSize is non-zero for the tile GEMM too, when its plan cuts tiles
+    // along K, so its value says nothing about which kernel runs.)
+    const bool tile_gemm = M > 16 && mnb_prefer_gemm256(L, (int64_t)M);
+    if (tile_gemm && widths_allow_vector_stores(F)) {
+      const size_t mid = mnb_mid_workspace_bytes(L, (int64_t)M);
+      if (w.inner < mid) w.inner = mid;
+    }
+    w.tmp = (tile_gemm && !widths_allow_vector_stores(F)) ? round256(M * (size_t)L.N * elem_size(L.dtype)) : 0;
   } else {
     w.tmp = round256(M * (size_t)L.N * elem_size(L.dtype));
   }

@@ -265,3 +265,39 @@ def test_fused_argument_errors():
     assert lib.MnbMlpPackSize(64, 256, 3, 32, _lib.DTYPE_FLOAT16) == 0  # 3-bit: no such format
     # empty batch
     assert tuple(op.Compute(torch.empty(0, 256, dtype=torch.float16, device="cuda")).shape) == (0, 64)
+
+
+def test_split_shape_with_misaligned_pointers_takes_the_streaming_kernel(oracle):
+    """A shape whose tile-GEMM plan cuts tiles along K (its own workspace is then non-zero): with an A or a Y that
+    does not allow 16-byte accesses the streaming kernel takes over, inside the workspace the contract reserves.
+    Checked against the aligned call (tile GEMM) and, on sampled rows, against the oracle."""
+    import ctypes
+    lib = _lib.load()
+    M, N, K, bits, bs = 2048, 512, 14336, 4, 128
+    r, c, p = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    lib.MnbGemmTilePlan(M, 2 * N, K, bits, bs, 0, _lib.DTYPE_FLOAT16, ctypes.byref(r), ctypes.byref(c), ctypes.byref(p))
+    assert p.value > 1, "the case is meant to be a split shape"
+    g, _ = _mats(M, N, K, bits, bs, np.float16, True, 61)
+    u, _ = _mats(M, N, K, bits, bs, np.float16, False, 62)
+    op = MatMulNBitsMlp(K, N, bits, bs)
+    op.PrePack(dev(g.B), dev(g.scales), dev(g.bias), dev(u.B), dev(u.scales), None)
+    a = dev(g.A)
+    y_ref = op.Compute(a)
+    wsz = lib.MnbMlpWorkspaceSize(M, N, K, bits, bs, _lib.DTYPE_FLOAT16, 0)
+    ws = torch.empty(wsz, dtype=torch.uint8, device="cuda")
+    a_raw = torch.zeros(M * K + 4, dtype=torch.float16, device="cuda")
+    a_off = a_raw[4:].view(M, K)
+    a_off.copy_(a)
+    y_raw = torch.zeros(M * N + 4, dtype=torch.float16, device="cuda")
+    y_off = y_raw[4:].view(M, N)
+    y_al = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    rows = np.array([0, 1, 255, 256, 1000, 2047])
+    for a_t, y_t in ((a_off, y_al), (a, y_off), (a_off, y_off)):
+        y_t.zero_()
+        _lib.check(lib.MnbMlpGemm(M, N, K, bits, bs, _lib.DTYPE_FLOAT16, a_t.data_ptr(), K, None,
+                                  op.packed.data_ptr(), 0, y_t.data_ptr(), N, ws.data_ptr(), wsz, None))
+        torch.cuda.synchronize()
+        assert not y_raw[:4].any()
+        d = (y_t.float() - y_ref.float()).abs()
+        assert float(d.max()) <= 4e-3 * float(y_ref.float().abs().max())
+        _check_mlp(oracle, y_t.cpu().numpy()[rows], g.A[rows], g, u, N, K, bits, bs, np.float16)

@@ -216,3 +216,30 @@ def test_dispatch_on_the_benchmark_layer_shapes():
     assert plan(1024, 4096, 14336) == (128, 256, 2)     # down
     assert plan(4096, 28672, 4096) == (256, 256, 1)     # gate_up
     assert plan(64, 4096, 4096) == (0, 0, 0)            # another kernel
+
+
+def test_fused_workspace_covers_the_streaming_kernel_on_split_shapes():
+    """Where the tile GEMM's plan cuts tiles along K its own workspace is non-zero; the fused operators' workspace
+    must still hold the streaming kernel's copy of A, which takes over when pointers turn out to be misaligned."""
+    import ctypes
+    lib = _lib.load()
+    # the streaming kernel's copy of A (4-bit weights): chunks of 128 k, 16-row tiles in blocks of four, 4 KiB each
+    mid_bytes = lambda M, K: -(-K // 128) * 4 * (-(-M // 64) * 4) * 64 * 16  # noqa: E731
+    assert lib.MnbGemmKernelName(64, 256, 4096, 4, 128, _lib.DTYPE_FLOAT16) == b"mnb_mid_kernel"
+    assert lib.MnbGemmWorkspaceSize(64, 256, 4096, 4, 128, 0, _lib.DTYPE_FLOAT16) == mid_bytes(64, 4096)
+    r, c, p = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    seen = 0
+    for M in (512, 1024, 2048, 4096):
+        for N in (256, 512, 1024, 2048):
+            for K in (8192, 14336):
+                Np = 2 * N
+                lib.MnbGemmTilePlan(M, Np, K, 4, 128, 0, _lib.DTYPE_FLOAT16, ctypes.byref(r), ctypes.byref(c),
+                                    ctypes.byref(p))
+                if p.value <= 1:
+                    continue
+                seen += 1
+                split = lib.MnbGemmWorkspaceSize(M, Np, K, 4, 128, 0, _lib.DTYPE_FLOAT16)
+                mid = mid_bytes(M, K)
+                need = lib.MnbMlpWorkspaceSize(M, N, K, 4, 128, _lib.DTYPE_FLOAT16, 0)
+                assert split > 0 and need >= max(split, mid), (M, N, K, split, mid, need)
+    assert seen >= 8
