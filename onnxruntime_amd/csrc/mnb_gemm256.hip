@@ -209,11 +209,19 @@ __device__ __forceinline__ void slab_end() {
 // 2 = fp16 model with zero points in the activation type.
 // NWV: wavefronts of the workgroup, 8 (256 columns) or 4 (128 columns: twice the tiles for problems whose 256-column
 // tiles leave compute units idle; same work per wavefront).
-template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV>
-__global__ void __launch_bounds__(64 * NWV, 2) mnb_gemm256_kernel(Gemm256Params p) {
+// CTW: 32-column matrix-core tiles per wavefront.  WM for the eight-wavefront arrangements; 2 with four wavefronts side by
+// side (1 x 4: a wavefront owns all 64 TM rows x 64 columns, one wavefront per SIMD with the accumulators in the
+// second half of its register file: every column is still dequantised once, and the staged A tile is read four times
+// instead of eight).  The 1 x 4 arrangement exists in calibration builds only: bit-identical results, half the LDS
+// reads (4.66 M instead of 8.34 M per launch of M = 2048, N = 14336, K = 4096), but a single wavefront per SIMD leaves
+// the matrix pipe idle while it issues its own vector instructions: 3217 cycles per k-step against 2460, 231.5 us
+// against 212.0 us on the same box although the power limit then allows 2.10 instead of 1.82 GHz; with the order inside a
+// slab section stated by hand (one matrix instruction, two vector instructions, one LDS read, one load) 244.7 us.
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV, int CTW = WM>
+__global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 : 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int THREADS = 64 * NWV;
   constexpr int WN = NWV / WM;       // wavefront columns
-  constexpr int CT = WM;             // 32-column matrix-core tiles per wavefront
+  constexpr int CT = CTW;            // 32-column matrix-core tiles per wavefront
   constexpr int BN = 32 * CT * WN;   // columns of the tile
   constexpr int ROWS_PER_LOAD = THREADS / 8;  // rows of A one load instruction of the workgroup stages
   constexpr int RT = 2 * TM / WM;    // 32-row matrix-core tiles per wavefront
@@ -701,12 +709,12 @@ __global__ void __launch_bounds__(256) mnb_gemm256_clear_flags_kernel(uint32_t* 
   for (int i = threadIdx.x; i < n; i += 256) flags[i] = 0u;
 }
 
-template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV = 8>
+template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV = 8, int CTW = WM>
 hipError_t launch_wm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
   // eight wavefronts: 98304 bytes whatever the tile height (one workgroup per compute unit either way); four: the
   // three staged tiles of the 128-row tile, so that three workgroups share a compute unit
   const size_t smem = NWV == 8 ? (size_t)SMEM_BYTES : (size_t)3 * 64 * TM * ROW_BYTES;
-  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM, DT, NWV>;
+  auto kernel = mnb_gemm256_kernel<BITS, HAS_ZP, MPS, TM, WM, DT, NWV, CTW>;
   // The attribute belongs to the function on the current device, so it is set on every launch (a host-side table
   // update, no device work): callers on several threads or devices need no shared flag.
   if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -725,6 +733,9 @@ hipError_t launch_tm(const Gemm256Params& p, unsigned grid, hipStream_t s) {
 #if defined(MNB_TUNING_HOOKS)
   if (const char* e = mnb_tuning_env("MNB_GEMM256_WAVE_ROWS"); e != nullptr && e[0] == '2')
     return launch_wm<BITS, HAS_ZP, MPS, TM, 2, DT>(p, grid, s);
+  if constexpr (TM == 4 && DT == 0 && BITS == 4)
+    if (const char* e = mnb_tuning_env("MNB_GEMM256_WAVES"); e != nullptr && e[0] == '4')
+      return launch_wm<BITS, HAS_ZP, MPS, TM, 1, DT, 4, 2>(p, grid, s);  // 1 x 4, one wavefront per SIMD
 #endif
   return launch_wm<BITS, HAS_ZP, MPS, TM, 1, DT>(p, grid, s);
 }
