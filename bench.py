@@ -214,6 +214,7 @@ def main() -> int:
     ap.add_argument("--no-bf16", action="store_true", help="skip the bfloat16 rows")
     ap.add_argument("--no-int8", action="store_true",
                     help="skip the int8-activation route (accuracy_level 4) beside the full-accuracy one")
+    ap.add_argument("--no-plugin", action="store_true", help="skip the leg through the plugin-EP boundary")
     ap.add_argument("--sweep", action="store_true", help="also time the other configurations (printed to stderr)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -545,6 +546,62 @@ def main() -> int:
             del ops, ys
             torch.cuda.empty_cache()
         out["bfloat16"] = rows
+
+    # ---- the same decode call through the plugin-EP boundary ---------------------------------------------------
+    # Everything above enters the library at MnbGemm (ctypes).  ONNX Runtime enters at OrtKernelImpl::Compute
+    # (plugin_ep/ep_kernel_registration.cc:78-80): input and shape queries through the C API, output allocation from
+    # the session's arena, the workspace request, then the same MnbGemm.  The host test double plays ONNX Runtime's
+    # part (tests/ep_host): CreateEpFactories -> ... -> PrePackWeight -> Compute, called back to back on one
+    # device-resident activation, one packed matrix (which therefore stays in the Infinity Cache: compare with
+    # us_per_launch_weights_in_infinity_cache, not with the headline).
+    if not args.no_plugin:
+        sys.path.insert(0, str(ROOT / "tests"))
+        try:
+            from ep_host import host
+            have_host = host.available()
+        except Exception:  # noqa: BLE001 - the leg is optional
+            have_host = False
+        if have_host:
+            rows = {}
+            for label, case in (("decode M=1 (configs[1])", c2), ("M=64 K=4100 N=6144 int4 bs128 zp (staged activations: a workspace per call)",
+                                                                   synthetic.make_case(64, 6144, 4100, 4, 128, np.float16, has_zp=True, seed=3))):  # (K not a whole number of chunks)
+                host.time_next_run(50, 400)
+                _, trace = host.run_matmul_nbits(case.N, case.K, case.bits, case.block_size, case.A, case.B,
+                                                 case.scales, case.zero_points, None, case.bias)
+                st = host.last_run_stats()
+                # the eager ctypes call on the same problem, for the difference
+                op = Problem(case, 1, torch, _lib)
+                for _ in range(50):
+                    op.launch(0)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t0 = time.perf_counter()
+                e0.record()
+                for _ in range(400):
+                    op.launch(0)
+                e1.record()
+                t1 = time.perf_counter()
+                torch.cuda.synchronize()
+                rows[label] = {
+                    "kernel": op.kernel,
+                    "compute_calls_timed": int(st["timed_computes"]),
+                    "host_us_per_Compute": round(st["host_us_per_compute"], 2),
+                    "device_us_per_Compute": round(st["device_us_per_compute"], 2),
+                    "wall_us_per_Compute": round(st["wall_us_per_compute"], 2),
+                    "scratch_requests_served_by_session": int(st["scratch_served"]),
+                    "provider_allocations_while_timed": 0 if "ep_allocs_while_timed=0" in trace else None,
+                    "ctypes_MnbGemm_host_us_per_call": round((t1 - t0) / 400 * 1e6, 2),
+                    "ctypes_MnbGemm_device_us_per_call": round(e0.elapsed_time(e1) / 400 * 1e3, 2),
+                }
+                del op
+            out["plugin_boundary"] = {
+                "path": "tests/ep_host host double: CreateEpFactories -> CreateEp -> kernel registry -> PrePackWeight -> "
+                        "OrtKernelImpl::Compute, back to back on one stream, outputs and workspace from the "
+                        "session's arena (KernelContext_GetOutput / KernelContext_GetScratchBuffer)",
+                "rows": rows,
+            }
+        else:
+            out["plugin_boundary"] = None
 
     # ---- the other configurations (not part of the JSON contract) ---------------------------------------------
     if args.sweep:

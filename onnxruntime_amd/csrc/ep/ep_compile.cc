@@ -83,12 +83,12 @@ OrtStatus* ORT_API_CALL ComputeImpl(OrtNodeComputeInfo* this_ptr, void* /*comput
   const size_t Mz = static_cast<size_t>(M), Nz = static_cast<size_t>(k.N), Kz = static_cast<size_t>(k.K);
   const int bits = static_cast<int>(k.bits), bs = static_cast<int>(k.block_size);
   const size_t ws_bytes = MnbGemmWorkspaceSize(Mz, Nz, Kz, bits, bs, k.has_zp, k.dtype);
-  void* ws = nullptr;
-  if (ws_bytes > 0) MI_RETURN_IF_HIP(a, hipMallocAsync(&ws, ws_bytes, hs));  // per call: concurrent runs never share it
+  CallScratch ws;  // per call: concurrent runs never share it
+  MI_RETURN_IF_ERROR(ws.Acquire(a, ctx, y, ws_bytes, hs));
   KernelTimer timer(hs, "MatMulNBits+Add", MnbGemmKernelName(Mz, Nz, Kz, bits, bs, k.dtype), M, k.N, k.K);
-  const int rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.has_zp, k.dtype, a_ptr, Kz, k.packed, k.bias, y_ptr, Nz, ws, ws_bytes,
-                         stream);
-  const hipError_t free_err = ws != nullptr ? hipFreeAsync(ws, hs) : hipSuccess;
+  const int rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.has_zp, k.dtype, a_ptr, Kz, k.packed, k.bias, y_ptr, Nz, ws.get(),
+                         ws_bytes, stream);
+  const hipError_t free_err = ws.Release();
   MI_RETURN_IF_ERROR(StatusFromMnb(a, rc));
   MI_RETURN_IF_HIP(a, free_err);
   return nullptr;

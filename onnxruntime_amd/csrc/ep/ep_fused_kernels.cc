@@ -185,6 +185,7 @@ OrtStatus* ORT_API_CALL FusedCompute(OrtKernelImpl* this_ptr, OrtKernelContext* 
   // outputs
   const int nout = k.is_qkv ? 3 : 1;
   void* out_ptr[3] = {nullptr, nullptr, nullptr};
+  const OrtValue* first_output = nullptr;  // names the device memory the call's scratch comes from
   int64_t out_elems = 0;
   for (int o = 0; o < nout; ++o) {
     std::vector<int64_t> dims(ad.dims.begin(), ad.dims.end() - 1);
@@ -193,6 +194,7 @@ OrtStatus* ORT_API_CALL FusedCompute(OrtKernelImpl* this_ptr, OrtKernelContext* 
     MI_RETURN_IF_ERROR(a.ort->KernelContext_GetOutput(ctx, static_cast<size_t>(o), dims.data(), dims.size(), &y));
     if (y == nullptr) return invalid(std::string(k.op()) + ": an output is missing");
     MI_RETURN_IF_ERROR(a.ort->GetTensorMutableData(y, &out_ptr[o]));
+    if (o == 0) first_output = y;
     out_elems += M * k.n[o];
   }
   if (num_outputs > static_cast<size_t>(nout)) {
@@ -239,9 +241,10 @@ OrtStatus* ORT_API_CALL FusedCompute(OrtKernelImpl* this_ptr, OrtKernelContext* 
   }
   const size_t ws_bytes = k.is_qkv ? MnbQkvWorkspaceSize(Mz, n0, n1, Kz, bits, bs, dtype, has_norm)
                                    : MnbMlpWorkspaceSize(Mz, n0, Kz, bits, bs, dtype, has_norm);
-  char* scratch = nullptr;
-  if (pack_bytes + ws_bytes > 0)
-    MI_RETURN_IF_HIP(a, hipMallocAsync(reinterpret_cast<void**>(&scratch), pack_bytes + ws_bytes, hs));
+  pack_bytes = (pack_bytes + 255) / 256 * 256;  // the workspace behind it is 256-byte aligned
+  CallScratch call_scratch;
+  MI_RETURN_IF_ERROR(call_scratch.Acquire(a, ctx, first_output, pack_bytes + ws_bytes, hs));
+  char* scratch = static_cast<char*>(call_scratch.get());
   int rc = MNB_OK;
   const void* packed = k.packed;
   if (k.packed == nullptr) {
@@ -259,7 +262,7 @@ OrtStatus* ORT_API_CALL FusedCompute(OrtKernelImpl* this_ptr, OrtKernelContext* 
       rc = MnbMlpGemm(Mz, n0, Kz, bits, bs, dtype, a_ptr, Kz, has_norm ? &norm : nullptr, packed, MNB_ACTIVATION_SILU,
                       out_ptr[0], n0, ws, ws_bytes, stream);
   }
-  const hipError_t free_err = scratch != nullptr ? hipFreeAsync(scratch, hs) : hipSuccess;
+  const hipError_t free_err = call_scratch.Release();
   MI_RETURN_IF_ERROR(StatusFromMnb(a, rc));
   MI_RETURN_IF_HIP(a, free_err);
   return nullptr;

@@ -76,6 +76,80 @@ class DeviceView {
   void* owned_ = nullptr;
 };
 
+// Device scratch that lives for one Compute call.  It comes from the session's allocator for the device that holds
+// `like` (the node's output), the way the reference's own GPU providers take theirs: KernelContext_GetScratchBuffer
+// (onnxruntime_c_api.h:5269), handed back through the allocator of KernelContext_GetAllocator (:4929) once the call's
+// kernels are enqueued -- the arena keeps the chunk with the compute stream.  A host that offers neither call (an
+// ONNX Runtime older than the calls, or one whose allocator declines) is served from HIP's stream-ordered pool.
+class CallScratch {
+ public:
+  CallScratch() = default;
+  CallScratch(const CallScratch&) = delete;
+  CallScratch& operator=(const CallScratch&) = delete;
+  ~CallScratch() { (void)Release(); }
+
+  // bytes == 0 leaves get() NULL.  `alignment`: what the consumer of the buffer demands of its address.
+  OrtStatus* Acquire(const Apis& a, OrtKernelContext* ctx, const OrtValue* like, size_t bytes, hipStream_t stream,
+                     size_t alignment = 256) {
+    (void)Release();
+    apis_ = &a;
+    stream_ = stream;
+    if (bytes == 0) return nullptr;
+    if (ctx != nullptr && like != nullptr && a.ort->KernelContext_GetScratchBuffer != nullptr &&
+        a.ort->KernelContext_GetAllocator != nullptr && a.ort->GetTensorMemoryInfo != nullptr &&
+        a.ort->ReleaseAllocator != nullptr) {
+      const OrtMemoryInfo* mem = nullptr;
+      OrtStatus* st = a.ort->GetTensorMemoryInfo(like, &mem);
+      if (st == nullptr && mem != nullptr) st = a.ort->KernelContext_GetAllocator(ctx, mem, &allocator_);
+      void* p = nullptr;
+      if (st == nullptr && allocator_ != nullptr) st = a.ort->KernelContext_GetScratchBuffer(ctx, mem, bytes, &p);
+      if (st != nullptr) {  // the host declined: not an error of the node
+        a.ort->ReleaseStatus(st);
+        p = nullptr;
+      }
+      if (p != nullptr && reinterpret_cast<uintptr_t>(p) % alignment != 0) {
+        allocator_->Free(allocator_, p);
+        p = nullptr;
+      }
+      if (p != nullptr) {
+        ptr_ = p;
+        return nullptr;
+      }
+      if (allocator_ != nullptr) a.ort->ReleaseAllocator(allocator_);
+      allocator_ = nullptr;
+    }
+    MI_RETURN_IF_HIP(a, hipMallocAsync(&ptr_, bytes, stream));
+    pooled_ = true;
+    return nullptr;
+  }
+
+  // Hands the buffer back; the work that uses it has been enqueued on the stream by then.
+  hipError_t Release() {
+    hipError_t e = hipSuccess;
+    if (ptr_ != nullptr) {
+      if (pooled_)
+        e = hipFreeAsync(ptr_, stream_);
+      else
+        allocator_->Free(allocator_, ptr_);
+    }
+    if (allocator_ != nullptr) apis_->ort->ReleaseAllocator(allocator_);
+    ptr_ = nullptr;
+    allocator_ = nullptr;
+    pooled_ = false;
+    return e;
+  }
+
+  void* get() const { return ptr_; }
+  bool from_session() const { return ptr_ != nullptr && !pooled_; }
+
+ private:
+  const Apis* apis_ = nullptr;
+  OrtAllocator* allocator_ = nullptr;
+  void* ptr_ = nullptr;
+  hipStream_t stream_ = nullptr;
+  bool pooled_ = false;
+};
+
 inline bool InputExists(const Apis& a, const OrtKernelInfo* info, size_t index, size_t count) {
   if (index >= count) return false;
   size_t size = 0;

@@ -194,7 +194,8 @@ OrtStatus* VariantCompute(MatMulNBitsKernel& k, OrtKernelContext* ctx) {
   MI_RETURN_IF_ERROR(a.ort->KernelContext_GetGPUComputeStream(ctx, &stream));
   hipStream_t hs = static_cast<hipStream_t>(stream);
 
-  // operands fed per run (or prepacking disabled): plan and pack per call into stream-ordered memory
+  // operands fed per run (or prepacking disabled): plan and pack per call into scratch memory of the session
+  CallScratch pack_scratch, gemm_scratch;
   MnbVariantPlan call_plan{};
   const MnbVariantPlan* plan = &k.plan;
   void* call_packed = nullptr;
@@ -204,14 +205,11 @@ OrtStatus* VariantCompute(MatMulNBitsKernel& k, OrtKernelContext* ctx) {
       return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: B and scales are required when B was not prepacked");
     }
     auto alloc = [&](size_t bytes, void** out) -> OrtStatus* {
-      MI_RETURN_IF_HIP(a, hipMallocAsync(out, bytes, hs));
+      MI_RETURN_IF_ERROR(pack_scratch.Acquire(a, ctx, y, bytes, hs));
+      *out = pack_scratch.get();
       return nullptr;
     };
-    OrtStatus* st = VariantPack(k, in[kB], in[kScales], in[kZeroPoints], in[kGIdx], hs, alloc, &call_plan, &call_packed);
-    if (st != nullptr) {
-      if (call_packed != nullptr) (void)hipFreeAsync(call_packed, hs);
-      return st;
-    }
+    MI_RETURN_IF_ERROR(VariantPack(k, in[kB], in[kScales], in[kZeroPoints], in[kGIdx], hs, alloc, &call_plan, &call_packed));
     plan = &call_plan;
     packed = call_packed;
   }
@@ -228,22 +226,17 @@ OrtStatus* VariantCompute(MatMulNBitsKernel& k, OrtKernelContext* ctx) {
     if (result == nullptr) {
       const size_t Mz = static_cast<size_t>(M);
       const size_t ws_bytes = MnbVariantGemmWorkspaceSize(plan, Mz);
-      void* ws = nullptr;
-      hipError_t e = ws_bytes > 0 ? hipMallocAsync(&ws, ws_bytes, hs) : hipSuccess;
-      if (e != hipSuccess) {
-        result = a.ort->CreateStatus(ORT_EP_FAIL, hipGetErrorString(e));
-      } else {
+      result = gemm_scratch.Acquire(a, ctx, y, ws_bytes, hs);
+      if (result == nullptr) {
         KernelTimer timer(hs, "MatMulNBits", plan->has_g_idx ? "gather + MatMulNBits" : "MatMulNBits (widened)", M,
                           k.N, k.K);
         const int rc = MnbVariantGemm(plan, Mz, a_ptr, static_cast<size_t>(k.K), packed, bias_ptr, y_ptr,
-                                      static_cast<size_t>(k.N), ws, ws_bytes, stream);
-        if (ws != nullptr) (void)hipFreeAsync(ws, hs);
+                                      static_cast<size_t>(k.N), gemm_scratch.get(), ws_bytes, stream);
         result = StatusFromMnb(a, rc);
       }
     }
   }
-  if (call_packed != nullptr) (void)hipFreeAsync(call_packed, hs);
-  return result;
+  return result;  // (the scratch objects hand their buffers back)
 }
 
 // PrePack(B) folds the constant scales and zero points into one device buffer in the gfx950 layout, the way the
@@ -389,32 +382,32 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
       // accuracy_level 4 with the session's consent: the reference's int8-activation arithmetic, where implemented
       const size_t ws8 = MnbGemmInt8WorkspaceSize(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype);
       if (ws8 > 0) {
-        void* scratch8 = nullptr;
-        MI_RETURN_IF_HIP(a, hipMallocAsync(&scratch8, ws8, gs));
+        CallScratch scratch8;
+        MI_RETURN_IF_ERROR(scratch8.Acquire(a, ctx, y, ws8, gs));
         KernelTimer timer(gs, "MatMulNBits", "mnb_gemm_i8_kernel", M, k.N, k.K);
         const int rc8 = MnbGemmInt8(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr, Nz,
-                                    scratch8, ws8, stream);
-        const hipError_t free8 = hipFreeAsync(scratch8, gs);
+                                    scratch8.get(), ws8, stream);
+        const hipError_t free8 = scratch8.Release();
         MI_RETURN_IF_ERROR(StatusFromMnb(a, rc8));
         MI_RETURN_IF_HIP(a, free8);
         return nullptr;
       }
     }
-    // per-call scratch comes from the stream-ordered pool, so concurrent Run() calls never share it
+    // per-call scratch: concurrent Run() calls never share it (CallScratch)
     const size_t gemm_ws = MnbGemmWorkspaceSize(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype);
-    void* gemm_scratch = nullptr;
-    if (gemm_ws > 0) MI_RETURN_IF_HIP(a, hipMallocAsync(&gemm_scratch, gemm_ws, gs));
+    CallScratch gemm_scratch;
+    MI_RETURN_IF_ERROR(gemm_scratch.Acquire(a, ctx, y, gemm_ws, gs));
     KernelTimer timer(gs, "MatMulNBits", MnbGemmKernelName(Mz, Nz, Kz, bits, bs, dtype), M, k.N, k.K);
     const int gemm_rc = MnbGemm(Mz, Nz, Kz, bits, bs, k.packed_has_zp, dtype, a_ptr, Kz, k.packed, bias_ptr, y_ptr, Nz,
-                                gemm_scratch, gemm_ws, stream);
-    const hipError_t gemm_free = gemm_scratch != nullptr ? hipFreeAsync(gemm_scratch, gs) : hipSuccess;
+                                gemm_scratch.get(), gemm_ws, stream);
+    const hipError_t gemm_free = gemm_scratch.Release();
     MI_RETURN_IF_ERROR(StatusFromMnb(a, gemm_rc));
     MI_RETURN_IF_HIP(a, gemm_free);
     return nullptr;
   }
 
   // B was not packed at session initialisation (prepacking disabled, or B / scales / zero points are not constant
-  // initializers): pack into stream-ordered scratch memory, then run the same kernels (matmul_nbits.cc:1184-1333).
+  // initializers): pack into per-call scratch memory, then run the same kernels (matmul_nbits.cc:1184-1333).
   if (in[kB] == nullptr) return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: input B is missing");
   if (static_cast<int>(d[kScales].type) != dtype) {
     return a.ort->CreateStatus(ORT_INVALID_ARGUMENT, "MatMulNBits: A and scales must have the same element type");
@@ -430,13 +423,13 @@ OrtStatus* ORT_API_CALL MatMulNBitsCompute(OrtKernelImpl* this_ptr, OrtKernelCon
   if (in[kZeroPoints] != nullptr) MI_RETURN_IF_ERROR(a.ort->GetTensorData(in[kZeroPoints], &z_ptr));
   const size_t ws_bytes = MnbGemmUnpackedWorkspaceSize(Mz, Nz, Kz, bits, bs, z_ptr != nullptr, dtype);
   if (ws_bytes == 0) return a.ort->CreateStatus(ORT_NOT_IMPLEMENTED, "MatMulNBits: configuration has no MI355X kernel");
-  void* ws = nullptr;
   hipStream_t hs = static_cast<hipStream_t>(stream);
-  MI_RETURN_IF_HIP(a, hipMallocAsync(&ws, ws_bytes, hs));
+  CallScratch ws;
+  MI_RETURN_IF_ERROR(ws.Acquire(a, ctx, y, ws_bytes, hs));
   KernelTimer timer(hs, "MatMulNBits", "pack + MatMulNBits", M, k.N, k.K);
-  int rc = MnbGemmUnpacked(Mz, Nz, Kz, bits, bs, dtype, a_ptr, Kz, b_ptr, s_ptr, z_ptr, bias_ptr, y_ptr, Nz, ws,
+  int rc = MnbGemmUnpacked(Mz, Nz, Kz, bits, bs, dtype, a_ptr, Kz, b_ptr, s_ptr, z_ptr, bias_ptr, y_ptr, Nz, ws.get(),
                            ws_bytes, stream);
-  hipError_t free_err = hipFreeAsync(ws, hs);
+  hipError_t free_err = ws.Release();
   MI_RETURN_IF_ERROR(StatusFromMnb(a, rc));
   MI_RETURN_IF_HIP(a, free_err);
   return nullptr;

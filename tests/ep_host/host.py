@@ -73,6 +73,52 @@ class profiled:
         return False
 
 
+class EpHostRunStats(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint64) for n in ("scratch_requests", "scratch_served", "scratch_bytes_max",
+                                                "allocator_requests", "allocators_released", "scratch_freed",
+                                                "ep_allocs", "arena_allocs")] + \
+               [(n, ctypes.c_double) for n in ("host_us_per_compute", "wall_us_per_compute",
+                                               "device_us_per_compute")] + [("timed_computes", ctypes.c_uint64)]
+
+
+def last_run_stats() -> dict:
+    """Allocator / scratch statistics (and timing figures, when asked for) of the last run_* call on this thread."""
+    lib = _load()
+    lib.EpHostLastRunStats.restype = None
+    lib.EpHostLastRunStats.argtypes = [ctypes.POINTER(EpHostRunStats)]
+    st = EpHostRunStats()
+    lib.EpHostLastRunStats(ctypes.byref(st))
+    return {n: getattr(st, n) for n, _ in EpHostRunStats._fields_}
+
+
+class scratch_mode:
+    """Context manager: how the host answers KernelContext_GetScratchBuffer inside it (0 serve, 1 fail with a status,
+    2 succeed with NULL, 3 return a buffer that is only 64-byte aligned)."""
+
+    def __init__(self, mode: int):
+        self.mode = mode
+
+    def __enter__(self):
+        lib = _load()
+        lib.EpHostSetScratchMode.restype = None
+        lib.EpHostSetScratchMode.argtypes = [ctypes.c_int]
+        lib.EpHostSetScratchMode(self.mode)
+        return self
+
+    def __exit__(self, *exc):
+        _load().EpHostSetScratchMode(0)
+        return False
+
+
+def time_next_run(warmup: int, iters: int) -> None:
+    """The next run_* call on this thread ends with ``warmup`` untimed and ``iters`` timed Compute calls on
+    device-resident inputs; ``last_run_stats()`` then reports host / wall / device microseconds per call."""
+    lib = _load()
+    lib.EpHostTimeNextRun.restype = None
+    lib.EpHostTimeNextRun.argtypes = [ctypes.c_int, ctypes.c_int]
+    lib.EpHostTimeNextRun(warmup, iters)
+
+
 def available() -> bool:
     return SHIM.exists() and PLUGIN.exists()
 

@@ -14,6 +14,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <chrono>
 #include <cstring>
 #include <map>
 #include <memory>
@@ -149,6 +150,101 @@ struct OrtKeyValuePairs {
 struct OrtSyncStream {
   OrtSyncStreamImpl* impl;
 };
+// What the session's allocator and the scratch calls saw during the last run on this thread (EpHostLastRunStats).
+struct EpHostRunStats {
+  uint64_t scratch_requests;     // KernelContext_GetScratchBuffer calls
+  uint64_t scratch_served;       // ... that returned memory
+  uint64_t scratch_bytes_max;    // largest request
+  uint64_t allocator_requests;   // KernelContext_GetAllocator calls
+  uint64_t allocators_released;  // ReleaseAllocator calls on those allocators
+  uint64_t scratch_freed;        // scratch buffers handed back through such an allocator
+  uint64_t ep_allocs;            // Alloc calls that reached the plugin's own OrtAllocator (arena misses)
+  uint64_t arena_allocs;         // Alloc calls on the session's arena (outputs, scratch, PrePack)
+  double host_us_per_compute;    // timing mode: host time of one Compute call (mean), stream kept busy
+  double wall_us_per_compute;    // ... wall time per call including the final stream flush
+  double device_us_per_compute;  // ... device time per call between two events on the compute stream (-1: no HIP)
+  uint64_t timed_computes;
+};
+thread_local EpHostRunStats tl_stats{};
+// 0: scratch requests are served from the arena; 1: KernelContext_GetScratchBuffer fails with a status;
+// 2: it succeeds with a NULL buffer; 3: it returns memory that is only 64-byte aligned
+thread_local int tl_scratch_mode = 0;
+
+// The session's device allocator: ONNX Runtime puts an arena in front of the provider's OrtAllocator, so in steady
+// state an output or a scratch buffer of a size seen before costs no call into the provider.  Modelled as exact-size
+// free lists over 256-byte multiples.
+struct ArenaAllocator : OrtAllocator {
+  OrtAllocator* inner = nullptr;
+  std::mutex mutex;
+  std::map<size_t, std::vector<void*>> free_lists;
+  std::map<void*, size_t> live;
+  explicit ArenaAllocator(OrtAllocator* ep_allocator) : inner(ep_allocator) {
+    version = ORT_API_VERSION;
+    Alloc = [](OrtAllocator* self, size_t size) noexcept -> void* {
+      auto* a = static_cast<ArenaAllocator*>(self);
+      const size_t rounded = (size + 255) / 256 * 256;
+      std::lock_guard<std::mutex> lock(a->mutex);
+      ++tl_stats.arena_allocs;
+      void* p = nullptr;
+      auto& fl = a->free_lists[rounded];
+      if (!fl.empty()) {
+        p = fl.back();
+        fl.pop_back();
+      } else {
+        ++tl_stats.ep_allocs;
+        p = a->inner->Alloc(a->inner, rounded);
+      }
+      if (p != nullptr) a->live[p] = rounded;
+      return p;
+    };
+    Free = [](OrtAllocator* self, void* p) noexcept {
+      if (p == nullptr) return;
+      auto* a = static_cast<ArenaAllocator*>(self);
+      std::lock_guard<std::mutex> lock(a->mutex);
+      auto it = a->live.find(p);
+      if (it == a->live.end()) return;  // not ours: a protocol error the tests see as a leak of `live`
+      a->free_lists[it->second].push_back(p);
+      a->live.erase(it);
+    };
+    Info = [](const OrtAllocator* self) noexcept -> const OrtMemoryInfo* {
+      auto* a = static_cast<const ArenaAllocator*>(self);
+      return a->inner->Info(a->inner);
+    };
+    Reserve = nullptr;
+    GetStats = nullptr;
+    AllocOnStream = nullptr;
+  }
+  ~ArenaAllocator() {
+    for (auto& kv : free_lists)
+      for (void* p : kv.second) inner->Free(inner, p);
+    for (auto& kv : live) inner->Free(inner, kv.first);
+  }
+};
+
+// What KernelContext_GetAllocator hands out: a handle onto the session's arena that ReleaseAllocator deletes.
+struct AllocatorHandle : OrtAllocator {
+  OrtAllocator* arena = nullptr;
+  explicit AllocatorHandle(OrtAllocator* a) : arena(a) {
+    version = ORT_API_VERSION;
+    Alloc = [](OrtAllocator* self, size_t size) noexcept -> void* {
+      auto* h = static_cast<AllocatorHandle*>(self);
+      return h->arena->Alloc(h->arena, size);
+    };
+    Free = [](OrtAllocator* self, void* p) noexcept {
+      auto* h = static_cast<AllocatorHandle*>(self);
+      if (p != nullptr) ++tl_stats.scratch_freed;
+      h->arena->Free(h->arena, p);
+    };
+    Info = [](const OrtAllocator* self) noexcept -> const OrtMemoryInfo* {
+      auto* h = static_cast<const AllocatorHandle*>(self);
+      return h->arena->Info(h->arena);
+    };
+    Reserve = nullptr;
+    GetStats = nullptr;
+    AllocOnStream = nullptr;
+  }
+};
+
 struct OrtKernelContext {
   std::vector<const OrtValue*> inputs;
   std::vector<std::unique_ptr<OrtValue>> outputs;
@@ -378,6 +474,52 @@ void FillApisOnce() {
       c->outputs[index] = std::move(v);
     }
     *out = c->outputs[index].get();
+    return nullptr;
+  };
+  g_ort.GetTensorMemoryInfo = [](const OrtValue* v, const OrtMemoryInfo** out) noexcept -> OrtStatus* {
+    *out = v->mem;
+    return nullptr;
+  };
+  // custom_ops.cc:219-232: the session's allocator for the device of mem_info, wrapped; the caller releases the wrapper
+  g_ort.KernelContext_GetAllocator = [](const OrtKernelContext* c, const OrtMemoryInfo* mem,
+                                        OrtAllocator** out) noexcept -> OrtStatus* {
+    ++tl_stats.allocator_requests;
+    *out = nullptr;
+    const OrtMemoryInfo* dev = c->device_allocator->Info(c->device_allocator);
+    if (mem == nullptr || mem->dev.type != dev->dev.type || mem->dev.device_id != dev->dev.device_id ||
+        mem->dev.mem_type != dev->dev.mem_type)
+      return MakeStatus(ORT_INVALID_ARGUMENT, "No requested allocator available");
+    *out = new AllocatorHandle(c->device_allocator);
+    return nullptr;
+  };
+  g_ort.ReleaseAllocator = [](OrtAllocator* a) noexcept {
+    ++tl_stats.allocators_released;
+    delete static_cast<AllocatorHandle*>(a);
+  };
+  // custom_ops.cc:901-913: a buffer from that allocator, tied to the compute stream; the caller frees it through the
+  // allocator.  A request for 0 bytes yields NULL.
+  g_ort.KernelContext_GetScratchBuffer = [](const OrtKernelContext* c, const OrtMemoryInfo* mem, size_t bytes,
+                                            void** out) noexcept -> OrtStatus* {
+    ++tl_stats.scratch_requests;
+    if (bytes > tl_stats.scratch_bytes_max) tl_stats.scratch_bytes_max = bytes;
+    *out = nullptr;
+    if (bytes == 0) return nullptr;
+    const OrtMemoryInfo* dev = c->device_allocator->Info(c->device_allocator);
+    if (mem == nullptr || mem->dev.type != dev->dev.type || mem->dev.device_id != dev->dev.device_id ||
+        mem->dev.mem_type != dev->dev.mem_type)
+      return MakeStatus(ORT_INVALID_ARGUMENT, "No requested allocator available");
+    if (tl_scratch_mode == 1) return MakeStatus(ORT_FAIL, "the host declines scratch requests (test mode)");
+    if (tl_scratch_mode == 2) return nullptr;
+    if (tl_scratch_mode == 3) {
+      // a misaligned address inside a block the arena never sees again until the session ends (freed as not-ours)
+      char* block = static_cast<char*>(c->device_allocator->Alloc(c->device_allocator, bytes + 256));
+      *out = block ? block + 64 : nullptr;
+      if (block) ++tl_stats.scratch_served;
+      return nullptr;
+    }
+    *out = c->device_allocator->Alloc(c->device_allocator, bytes);
+    if (*out == nullptr) return MakeStatus(ORT_FAIL, "device allocation of a scratch buffer failed");
+    ++tl_stats.scratch_served;
     return nullptr;
   };
   g_ort.KernelContext_GetGPUComputeStream = [](const OrtKernelContext* c, void** out) noexcept -> OrtStatus* {
@@ -668,6 +810,36 @@ Plugin* LoadPlugin(const char* path, std::string* error) {
 // session profiling does and writes one line per reported event into the buffer.
 thread_local char* tl_profile_buf = nullptr;
 thread_local size_t tl_profile_len = 0;
+// Set by EpHostTimeNextRun: after its functional repeats the next RunNode on this thread calls Compute `warmup` +
+// `iters` more times on the same device inputs and reports what one call costs (EpHostLastRunStats).
+thread_local int tl_timing_iters = 0;
+thread_local int tl_timing_warmup = 0;
+
+// HIP events for the device-side figure of the timing mode, looked up at run time so that this host double links
+// against nothing of the GPU stack.
+struct HipEvents {
+  using Create = int (*)(void**);
+  using Record = int (*)(void*, void*);
+  using Sync = int (*)(void*);
+  using Elapsed = int (*)(float*, void*, void*);
+  using Destroy = int (*)(void*);
+  Create create = nullptr;
+  Record record = nullptr;
+  Sync sync = nullptr;
+  Elapsed elapsed = nullptr;
+  Destroy destroy = nullptr;
+  bool ok = false;
+  HipEvents() {
+    void* h = dlopen("libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
+    if (h == nullptr) return;
+    create = reinterpret_cast<Create>(dlsym(h, "hipEventCreate"));
+    record = reinterpret_cast<Record>(dlsym(h, "hipEventRecord"));
+    sync = reinterpret_cast<Sync>(dlsym(h, "hipEventSynchronize"));
+    elapsed = reinterpret_cast<Elapsed>(dlsym(h, "hipEventElapsedTime"));
+    destroy = reinterpret_cast<Destroy>(dlsym(h, "hipEventDestroy"));
+    ok = create && record && sync && elapsed && destroy;
+  }
+};
 constexpr int64_t kProfilingStartOffsetNs = 5000000;  // pretend ORT's profiling began 5 ms before the EP's
 
 int Fail(OrtStatus* st, const char* where, char* err, size_t err_len) {
@@ -979,13 +1151,27 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
     return HostFail(EP_HOST_PROTOCOL, "a fused group in a graph of one node", err, err_len);
 
   // ---- session resources
-  OrtAllocator* allocator = nullptr;
-  if (OrtStatus* st = ep->CreateAllocator(ep, device_mem, &allocator)) return Fail(st, "CreateAllocator", err, err_len);
+  OrtAllocator* ep_allocator = nullptr;
+  if (OrtStatus* st = ep->CreateAllocator(ep, device_mem, &ep_allocator)) return Fail(st, "CreateAllocator", err, err_len);
   struct AllocGuard {
     OrtEpFactory* f;
     OrtAllocator* a;
     ~AllocGuard() { f->ReleaseAllocator(f, a); }
-  } alloc_guard{factory, allocator};
+  } alloc_guard{factory, ep_allocator};
+  // every device value below dies before the arena (declared later = destroyed earlier), the arena before the
+  // plugin's allocator
+  ArenaAllocator arena(ep_allocator);
+  OrtAllocator* allocator = &arena;
+  struct ValuesGuard {  // device tensors go back to the arena before it is destroyed
+    std::vector<std::unique_ptr<OrtValue>>& v;
+    ~ValuesGuard() {
+      for (auto& x : v) x.reset();
+    }
+  } values_guard{device_values};
+  const int timing_iters = tl_timing_iters, timing_warmup = tl_timing_warmup;
+  tl_timing_iters = 0;
+  tl_stats = EpHostRunStats{};
+  tl_stats.device_us_per_compute = -1.0;
   OrtDataTransferImpl* transfer = nullptr;
   if (OrtStatus* st = factory->CreateDataTransfer(factory, &transfer)) return Fail(st, "CreateDataTransfer", err, err_len);
   struct TransferGuard {
@@ -1189,6 +1375,62 @@ int RunNode(const char* plugin_path, const EpHostNodeSpec& spec, const EpHostTen
       outs[o].produced = 1;
     }
   }
+  // ---- timing mode: the cost of one Compute call as ONNX Runtime's executor sees it.  The activation stays on the
+  // device (what the previous node would have produced), every call gets a fresh context whose output comes from the
+  // arena, and nothing synchronises between the calls.
+  if (rc == 0 && timing_iters > 0) {
+    OrtKernelImpl* from_host = nullptr;
+    if (OrtStatus* st = memcpy_kernel("MemcpyFromHost", host_values[0]->type, &from_host))
+      return Fail(st, "MemcpyFromHost creation", err, err_len);
+    KernelGuard from_guard{from_host};
+    OrtKernelContext copy_in{{host_values[0].get()}, {}, {false}, allocator, &cpu_mem, &stream};
+    copy_in.outputs.resize(1);
+    if (OrtStatus* st = from_host->Compute(from_host, &copy_in)) return Fail(st, "MemcpyFromHost", err, err_len);
+    auto one_compute = [&]() -> OrtStatus* {
+      OrtKernelContext ctx{{}, {}, {}, allocator, &cpu_mem, &stream};
+      ctx.outputs.resize(spec.num_outputs);
+      ctx.output_on_host.assign(spec.num_outputs, false);
+      ctx.output_skipped.assign(spec.num_outputs, false);
+      for (size_t o = 0; o < spec.num_outputs; ++o) ctx.output_skipped[o] = (spec.skipped_output_mask >> o) & 1;
+      if (compiled) {
+        ctx.inputs.assign(1, copy_in.outputs[0].get());
+        return compute_info.info->Compute(compute_info.info, compute_info.state, &ctx);
+      }
+      ctx.inputs.assign(node.inputs.size(), nullptr);
+      ctx.inputs[0] = copy_in.outputs[0].get();
+      for (size_t i = 1; i < node.inputs.size(); ++i)
+        if (!dropped[i] && fed_value(i)) ctx.inputs[i] = fed_value(i);
+      return kernel->Compute(kernel, &ctx);
+    };
+    for (int i = 0; i < timing_warmup; ++i)
+      if (OrtStatus* st = one_compute()) return Fail(st, "Compute (warm-up)", err, err_len);
+    if (OrtStatus* st = stream_impl->Flush(stream_impl)) return Fail(st, "stream Flush", err, err_len);
+    static HipEvents hip;
+    void* e0 = nullptr;
+    void* e1 = nullptr;
+    void* handle = stream_impl->GetHandle(stream_impl);
+    const bool events = hip.ok && hip.create(&e0) == 0 && hip.create(&e1) == 0;
+    const uint64_t ep_allocs_before = tl_stats.ep_allocs;
+    const auto t0 = std::chrono::steady_clock::now();
+    if (events) hip.record(e0, handle);
+    for (int i = 0; i < timing_iters; ++i)
+      if (OrtStatus* st = one_compute()) return Fail(st, "Compute (timed)", err, err_len);
+    if (events) hip.record(e1, handle);
+    const auto t1 = std::chrono::steady_clock::now();
+    if (OrtStatus* st = stream_impl->Flush(stream_impl)) return Fail(st, "stream Flush", err, err_len);
+    const auto t2 = std::chrono::steady_clock::now();
+    tl_stats.timed_computes = static_cast<uint64_t>(timing_iters);
+    tl_stats.host_us_per_compute = std::chrono::duration<double, std::micro>(t1 - t0).count() / timing_iters;
+    tl_stats.wall_us_per_compute = std::chrono::duration<double, std::micro>(t2 - t0).count() / timing_iters;
+    if (events) {
+      float ms = 0.f;
+      if (hip.sync(e1) == 0 && hip.elapsed(&ms, e0, e1) == 0) tl_stats.device_us_per_compute = ms * 1e3 / timing_iters;
+      hip.destroy(e0);
+      hip.destroy(e1);
+    }
+    trace.add("timed=%d ep_allocs_while_timed=%llu ", timing_iters,
+              static_cast<unsigned long long>(tl_stats.ep_allocs - ep_allocs_before));
+  }
   if (profiler != nullptr) {
     OrtProfilingEventsContainer container;
     if (OrtStatus* st = profiler->EndProfiling(profiler, &container)) return Fail(st, "EndProfiling", err, err_len);
@@ -1220,6 +1462,20 @@ __attribute__((visibility("default"))) void EpHostProfileNextRun(char* buf, size
   tl_profile_buf = len > 0 ? buf : nullptr;
   tl_profile_len = len;
 }
+
+// The next EpHostRun* call on the calling thread ends with `warmup` untimed and `iters` timed Compute calls on
+// device-resident inputs; EpHostLastRunStats then holds what one call cost.
+__attribute__((visibility("default"))) void EpHostTimeNextRun(int warmup, int iters) {
+  tl_timing_warmup = warmup;
+  tl_timing_iters = iters;
+}
+
+// How the next sessions on this thread answer KernelContext_GetScratchBuffer: 0 serve (default), 1 fail with a
+// status, 2 succeed with a NULL buffer, 3 return a buffer that is only 64-byte aligned.
+__attribute__((visibility("default"))) void EpHostSetScratchMode(int mode) { tl_scratch_mode = mode; }
+
+// Allocator and scratch statistics (and the timing figures) of the last EpHostRun* call on the calling thread.
+__attribute__((visibility("default"))) void EpHostLastRunStats(EpHostRunStats* out) { *out = tl_stats; }
 
 // Any operator of the com.microsoft domain the plugin registers (MatMulNBitsMlp, MatMulNBitsQkv, ...).
 __attribute__((visibility("default"))) int EpHostRunNode(const char* plugin_path, const EpHostNodeSpec* spec,

@@ -151,3 +151,42 @@ def test_accuracy_level_4_takes_int8_activations_only_with_the_sessions_consent(
         check_against_oracle(oracle, c8, y88)
     y_after, _ = host.run_matmul_nbits(N, K, bits, bs, c.A, c.B, c.scales, c.zero_points, bias=c.bias, accuracy_level=4)
     assert np.array_equal(y_after, y)
+
+
+def test_per_call_scratch_comes_from_the_sessions_allocator(oracle):
+    """Compute takes its workspace through KernelContext_GetScratchBuffer and hands it back through the allocator of
+    KernelContext_GetAllocator (onnxruntime_c_api.h:5269, :4929); when the host declines -- an error status, a NULL
+    buffer, a buffer the kernels cannot use -- the stream-ordered pool serves the call: same bits either way."""
+    # M = 100, K = 320 (not a whole number of the streaming kernel's chunks): a staged copy of A, hence a workspace
+    c = make_case(100, 320, 320, 4, 32, np.float16, has_zp=True, has_bias=True, seed=21)
+    y0, _ = _run(c, repeat=3)
+    st = host.last_run_stats()
+    assert st["scratch_requests"] == 3 and st["scratch_served"] == 3 and st["scratch_bytes_max"] > 0, st
+    assert st["scratch_freed"] == 3 and st["allocator_requests"] == st["allocators_released"] == 3, st
+    check_against_oracle(oracle, c, y0)
+    for mode in (1, 2, 3):
+        with host.scratch_mode(mode):
+            y, _ = _run(c, repeat=2)
+        st = host.last_run_stats()
+        assert st["scratch_requests"] == 2 and st["allocator_requests"] == st["allocators_released"] == 2, (mode, st)
+        assert st["scratch_served"] == (2 if mode == 3 else 0), (mode, st)
+        assert np.array_equal(y.view(np.uint8), y0.view(np.uint8)), mode
+    # the unpacked route packs into scratch as well
+    y_unpacked, trace = _run(c, constant=("B",), repeat=2)
+    st = host.last_run_stats()
+    assert "prepacked= " in trace and st["scratch_served"] == 2 and st["scratch_freed"] == 2, (trace, st)
+    assert np.array_equal(y_unpacked.view(np.uint8), y0.view(np.uint8))
+    # a decode call needs no workspace: no request at all
+    d = make_case(1, 512, 1024, 4, 128, np.float16, seed=22)
+    _run(d)
+    assert host.last_run_stats()["scratch_requests"] == 0
+
+
+def test_timing_mode_reports_one_compute_call():
+    c = make_case(1, 1024, 1024, 4, 128, np.float16, seed=23)
+    host.time_next_run(5, 50)
+    _, trace = _run(c)
+    st = host.last_run_stats()
+    assert st["timed_computes"] == 50 and "ep_allocs_while_timed=0" in trace, (st, trace)  # the arena serves the outputs
+    assert 0 < st["host_us_per_compute"] <= st["wall_us_per_compute"] < 1e4, st
+    assert st["device_us_per_compute"] > 0, st

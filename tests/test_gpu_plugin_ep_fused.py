@@ -103,3 +103,21 @@ def test_fused_nodes_left_to_the_cpu_provider_or_rejected():
     bad = (g.B[:, :-1], g.scales, None)
     with pytest.raises(host.EpHostError, match="quantized_weight"):
         host.run_mlp(N, K, 4, 32, g.A, gm, bad)
+
+
+def test_fused_nodes_take_their_scratch_from_the_session():
+    """The Mlp / Qkv kernels' workspace (and per-call packing) comes from KernelContext_GetScratchBuffer; a host that
+    declines is served from the stream-ordered pool with the same bits."""
+    rng = np.random.default_rng(5)
+    M, N, K, bits, bs = 40, 96, 256, 4, 32
+    from onnxruntime_amd.synthetic import make_case
+    g = make_case(M, N, K, bits, bs, np.float16, has_bias=True, seed=31)
+    u = make_case(M, N, K, bits, bs, np.float16, has_bias=False, seed=32)
+    gamma = rng.uniform(0.5, 1.5, K).astype(np.float16)
+    y0, _, _ = host.run_mlp(N, K, bits, bs, g.A, (g.B, g.scales, g.bias), (u.B, u.scales, None), norm_scale=gamma)
+    st = host.last_run_stats()
+    assert st["scratch_requests"] == 1 and st["scratch_served"] == 1 and st["scratch_freed"] == 1, st
+    with host.scratch_mode(1):
+        y1, _, _ = host.run_mlp(N, K, bits, bs, g.A, (g.B, g.scales, g.bias), (u.B, u.scales, None), norm_scale=gamma)
+    assert host.last_run_stats()["scratch_served"] == 0
+    assert np.array_equal(y0.view(np.uint8), y1.view(np.uint8))
