@@ -116,13 +116,23 @@ MNB_API int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int 
                     const void* a_dev, size_t lda, const void* packed_dev, const void* bias_dev, void* c_dev,
                     size_t ldc, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Health of the last MnbGemm launch that used this workspace for the same problem.  No counterpart in the reference.
+ * Only the tile GEMM's cut along K (case (b) of MnbGemmWorkspaceSize) has anything to report: its workgroups hand
+ * partial sums to one another through the workspace and wait for one another with a bound; a wait that gave up has
+ * written NaN into its output tile and set a word in the workspace.  *gave_up = 1 then, else 0 (also for problems and
+ * workspaces that do not take the cut).  The call waits for `stream`.  The word is cleared by the next launch that
+ * uses the workspace. */
+MNB_API int MnbGemmWorkspaceStatus(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
+                                   int a_dtype, const void* workspace_dev, size_t workspace_bytes, void* stream,
+                                   int* gave_up);
+
 /* MnbGemm for callers that cannot allocate or carry device memory of their own: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results
  * as MnbGemm (bit for bit) minus the workspace: the scratch MnbGemm would ask for lives in a device array inside the
- * library (MnbGemmStaticScratchCapacity bytes, 32 MiB, held on every device the library runs on until the process
+ * library (MnbGemmStaticScratchCapacity bytes, 32 MiB + 64 KiB, held on every device the library runs on until the process
  * ends).  The call allocates and frees nothing.  A problem whose MnbGemmWorkspaceSize exceeds the capacity is rejected
- * with MNB_INVALID_ARGUMENT, unless the scratch would only serve the tile GEMM's optional cut of tiles along K: that
- * kernel then runs without the cut (the same sums in another fp32 order).  Every call on a device shares that device's array: calls that may overlap on one device
+ * with MNB_INVALID_ARGUMENT, unless the kernel that serves the call without a workspace needs none: the tile GEMM then
+ * runs without its optional cut of tiles along K (the same sums in another fp32 order).  Every call on a device shares that device's array: calls that may overlap on one device
  * (different streams, several threads) race on it and must be serialised by the caller. */
 MNB_API size_t MnbGemmStaticScratchCapacity(void);
 MNB_API int MnbGemmStaticScratch(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,

@@ -62,6 +62,8 @@ SIGNATURES = {
     "MnbGemmWorkspaceSize": (c_size_t, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int]),
     "MnbGemm": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
                         c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "MnbGemmWorkspaceStatus": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t,
+                                       c_void_p, ctypes.POINTER(c_int)]),
     "MnbGemmStaticScratchCapacity": (c_size_t, []),
     "MnbGemmStaticScratch": (c_int, [c_size_t, c_size_t, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p,
                                      c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -323,6 +323,26 @@ int MnbGemm(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero
                       c_dev, ldc, workspace_dev, workspace_bytes, stream);
 }
 
+int MnbGemmWorkspaceStatus(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
+                           const void* workspace_dev, size_t workspace_bytes, void* stream, int* gave_up) {
+  const char* fn = "MnbGemmWorkspaceStatus";
+  if (!gave_up) return fail(MNB_INVALID_ARGUMENT, "%s: gave_up must not be NULL", fn);
+  *gave_up = 0;
+  if (int rc = check_config(fn, bits, block_size, a_dtype)) return rc;
+  if (M == 0 || N == 0 || K == 0 || a_dtype != kMnbDtypeFloat16 || M <= 16) return MNB_OK;
+  const MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
+  if (!mnb_prefer_gemm256(L, (int64_t)M)) return MNB_OK;  // another kernel: its workspace holds no status
+  const uint32_t* word = mnb_gemm256_status_word(L, (int64_t)M, kMnbIoModel, workspace_dev, workspace_bytes);
+  if (word == nullptr) return MNB_OK;  // the launch ran uncut
+  uint32_t v = 0;
+  hipStream_t s = (hipStream_t)stream;
+  hipError_t e = hipMemcpyAsync(&v, word, sizeof(v), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) return hip_fail(e, fn);
+  *gave_up = v != 0;
+  return MNB_OK;
+}
+
 size_t MnbGemmInt8WorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                 int a_dtype) {
   if (check_config("MnbGemmInt8WorkspaceSize", bits, block_size, a_dtype) != MNB_OK || M == 0 || N == 0 || K == 0) return 0;
@@ -372,7 +392,8 @@ int MnbGemmInt8(size_t M, size_t N, size_t K, int bits, int block_size, int has_
 // The per-call scratch of MnbGemm (the streaming kernel's copy of A in matrix-core operand order) as a file-scope
 // device array: every device the library runs on holds its own copy, at its own address, until the process ends.
 // In host code the array's name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
-constexpr size_t kMnbStaticScratchBytes = (size_t)32 << 20;
+// 32 MiB of partial tiles (128 workgroups x 256 KiB, the usual cut of a tall problem along K) plus their flags
+constexpr size_t kMnbStaticScratchBytes = ((size_t)32 << 20) + ((size_t)64 << 10);
 static __device__ __align__(256) unsigned char scratch[kMnbStaticScratchBytes];
 
 namespace {
@@ -412,14 +433,15 @@ int MnbGemmStaticScratch(size_t M, size_t N, size_t K, int bits, int block_size,
   if (M == 0 || N == 0) return MNB_OK;
   size_t need = MnbGemmWorkspaceSize(M, N, K, bits, block_size, has_zero_points, a_dtype);
   if (need > kMnbStaticScratchBytes) {
-    // The tile GEMM uses scratch only to cut tiles along K across workgroups and runs without it otherwise; every
-    // other use of scratch (the streaming kernel's staged activations) is indispensable.
+    // The tile GEMM uses scratch only to cut tiles along K across workgroups and runs without it otherwise, and the
+    // kernels a call without a workspace falls back to need none; only the streaming kernel's staged copy of the
+    // activations is indispensable.
     MnbGemmArgs probe{};
     probe.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
     probe.M = (int64_t)M;
     probe.A = a_dev;
-    probe.lda = (int64_t)lda;
-    if (mnb_select_kernel(probe) != kMnbKernelGemm256)
+    probe.lda = (int64_t)lda;  // (no workspace: the kernel this call would run without one)
+    if (mnb_select_kernel(probe) == kMnbKernelMid && !mnb_mid_direct(probe))
       return fail(MNB_INVALID_ARGUMENT,
                   "MnbGemmStaticScratch: this problem needs %zu bytes of scratch, the static array holds %zu; use "
                   "MnbGemm with a workspace of MnbGemmWorkspaceSize bytes",

@@ -40,8 +40,25 @@
 // is needed: the finalising part starts from it instead of from zero (no burst of reads when all workgroups finish
 // together).  Partials of workgroups whose whole share lies inside the tile arrive as late as the finalising part
 // itself ends and are added then, nearest first.  The order of summation is fixed by the shares, so results are the
-// same from run to run.  Partials and flags travel with device-scope atomic stores and loads (write-through, no
-// cache maintenance); the flags are cleared by a small kernel in front of the launch.
+// same from run to run.
+// The hand-over of a partial.  Every access to partials and flags is a relaxed device-scope atomic, which on this
+// hardware is an access that bypasses the per-XCD caches (sc1: stores write through to, and loads are served from,
+// the level all XCDs share); no fence instruction is involved.  What orders data before flag:
+//   writer: s_waitcnt vmcnt(0) between the partial's stores and the flag's store -- a write-through store is counted
+//           as outstanding until that shared level has acknowledged it, so the flag cannot become visible first;
+//   reader: the partial's loads are issued behind the branch that leaves the polling loop, and the branch needs the
+//           flag's value: a wavefront issues in order and never speculates past a branch, so no load of the partial
+//           is in flight before a poll has returned 1.
+// The compiler is held to the same order by signal fences (no instructions) on both sides.  Device-scope release /
+// acquire fences in their place (MNB_SPLIT_FENCES=1: the writer's becomes a write-back of its XCD's L2, the reader's
+// an invalidation) were measured at +12 to +18 us per launch on every split shape (M = 1024, N = 4096, K = 14336:
+// 134.2 against 119.7 us; M = 512, N = K = 8192: 90.0 against 73.5 us) with bit-identical results, and are not used.
+// Progress.  A workgroup waits only for workgroups with smaller indices, and the plan never splits into more than
+// two rounds of workgroups: what is relied on is that workgroup w is not dispatched before workgroups 0 .. w-1
+// (one-dimensional grids are dispatched in index order).  Should that ever fail, a wait ends after spin_limit polls:
+// it poisons its tile with NaN and sets the status word behind the flags, which MnbGemmWorkspaceStatus reads back.
+// Flags and status word are cleared by a small kernel in front of the launch, so a workspace must not be shared by
+// launches that may overlap.
 // Without a workspace the grid is one workgroup per tile and nothing is split.
 #include <cstdlib>
 #include <type_traits>
@@ -50,6 +67,10 @@
 #include "mnb_buffer.hip.h"
 #include "mnb_device.hip.h"
 #include "mnb_internal.h"
+
+#if !defined(MNB_SPLIT_FENCES)
+#define MNB_SPLIT_FENCES 0  // 1 (calibration builds): device-scope release / acquire fences around the flag hand-over
+#endif
 
 namespace {
 
@@ -137,7 +158,10 @@ struct Gemm256Params {
   int64_t share_q, share_r;
   uint64_t* partials;       // one slot of tile_rows x tile_cols floats per workgroup (NULL: grid == tiles, nothing is split)
   uint32_t* flags;          // one word per workgroup and wavefront, zero when the kernel starts
+  uint32_t* status;         // one word behind the flags, zero when the kernel starts: set to 1 by a wait that gave up
   int spin_limit;           // polls of a flag before the wait gives up and the tile is poisoned with NaN
+  int test_drop_odd_lower;  // test builds only: the lower parts of odd-numbered tiles are not computed (their flags
+                            // stay zero, so the finalising parts of those tiles run into the bounded wait)
   int c_vec_ok;  // C allows 16-byte stores of 8 columns: aligned base and pitch, N a multiple of 8
   // several matrices packed as one (mnb_layout.h); these kinds always take the 16-byte store path
   int epi_kind;            // kMnbFusedNone / kMnbFusedMlp: C[M][n_out0] = silu(gate) * up / kMnbFusedQkv: three outputs
@@ -492,6 +516,11 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
       }
       __builtin_amdgcn_s_sleep(16);
     }
+    if (!ok && lane == 0) __hip_atomic_store(p.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);  // the compiler keeps the partial's loads behind the loop (file header)
+#if MNB_SPLIT_FENCES
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#endif
     uint32_t lane_here = lane;
     asm volatile("" : "+v"(lane_here));  // no address arithmetic in front of the loop over the parts (see the store)
     const uint64_t* src = p.partials + (size_t)w * SLOT_PAIRS + wave_pairs;
@@ -526,6 +555,9 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
     const int ks_begin = (int)(part_lo - tile_lo) * 2, ks_end = (int)(u_hi - tile_lo) * 2;
     const bool finalises = ks_end == p.ksteps;  // this part holds the tile's last unit
     u_hi = part_lo;
+#if defined(MNB_TEST_HOOKS)
+    if (!finalises && p.test_drop_odd_lower && (tile & 1)) continue;
+#endif
 
     // column-fastest tile order: the workgroups at work on neighbouring tiles share a slab of A
     m0 = (tile / p.tiles_n) * BM;
@@ -597,7 +629,14 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
             __hip_atomic_store(grp + q * 64 + lane_here, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
+      // release: every store of this wavefront is visible to the device before the flag is
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
+#if MNB_SPLIT_FENCES
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#else
       __builtin_amdgcn_s_waitcnt(0);  // every store of this wavefront has been acknowledged by the memory system
+#endif
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
       if (lane == 0) __hip_atomic_store(p.flags + wg * 8 + wave, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       continue;
     }
@@ -848,8 +887,10 @@ inline double cycles_narrow(int vi, int64_t grid, int64_t steps, int64_t cus) {
 }  // namespace plan_model
 
 namespace {
+// [flags: 8 per workgroup][status word] rounded up to 256 bytes, then one partial tile per workgroup
+size_t split_flag_bytes(int64_t grid) { return round256(((size_t)grid * 8 + 1) * sizeof(uint32_t)); }
 size_t split_workspace_bytes(int64_t grid, int rows, int cols) {
-  return round256((size_t)grid * 8 * sizeof(uint32_t)) + (size_t)grid * rows * cols * sizeof(float);
+  return split_flag_bytes(grid) + (size_t)grid * rows * cols * sizeof(float);
 }
 }  // namespace
 
@@ -924,6 +965,28 @@ bool mnb_gemm256_fused_ok(const MnbEpilogue& e) {
   return true;
 }
 
+#if defined(MNB_TEST_HOOKS)
+// Test builds (tests/hooks): the host chooses the bound of the cross-workgroup wait and may leave the lower parts of
+// odd-numbered tiles uncomputed, so that the give-up path runs with every kernel still ending normally.
+static int g_test_spin_limit = 0;
+static int g_test_drop_odd_lower = 0;
+extern "C" __attribute__((visibility("default"))) void MnbTestSetSplitHooks(int spin_limit, int drop_odd_lower) {
+  g_test_spin_limit = spin_limit;
+  g_test_drop_odd_lower = drop_odd_lower;
+}
+#endif
+
+// Device address of the status word of a split launch's workspace (NULL when this problem's plan does not split or
+// the workspace is too small for it): 1 after a launch in which a cross-workgroup wait gave up.
+const uint32_t* mnb_gemm256_status_word(const MnbLayout& L, int64_t M, int io, const void* workspace,
+                                        size_t workspace_bytes) {
+  const MnbGemm256Plan plan = mnb_gemm256_plan(L, M, true, io);
+  if (!plan.split || workspace == nullptr || workspace_bytes < plan.workspace_bytes ||
+      reinterpret_cast<uintptr_t>(workspace) % 8 != 0)
+    return nullptr;
+  return reinterpret_cast<const uint32_t*>(workspace) + plan.grid * 8;
+}
+
 hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   if (!mnb_gemm256_addressable(a.lda, a.L.Npad)) return hipErrorInvalidValue;  // the dispatcher never sends these
   // a matrix packed for an fp32 model is run in a 16-bit type named by a.io; fused outputs exist for fp16 models only
@@ -957,11 +1020,15 @@ hipError_t mnb_launch_gemm256(const MnbGemmArgs& a, hipStream_t s) {
   p.share_q = units / plan.grid;
   p.share_r = units % plan.grid;
   p.spin_limit = 1 << 20;  // polls half a microsecond apart: seconds, where a healthy wait takes microseconds
+#if defined(MNB_TEST_HOOKS)
+  if (g_test_spin_limit > 0) p.spin_limit = g_test_spin_limit;
+  p.test_drop_odd_lower = g_test_drop_odd_lower;
+#endif
   if (plan.split) {
     p.flags = reinterpret_cast<uint32_t*>(a.workspace);
-    p.partials = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(a.workspace) +
-                                             round256((size_t)plan.grid * 8 * sizeof(uint32_t)));
-    mnb_gemm256_clear_flags_kernel<<<dim3(1), dim3(256), 0, s>>>(p.flags, (int)plan.grid * 8);
+    p.status = p.flags + plan.grid * 8;
+    p.partials = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(a.workspace) + split_flag_bytes(plan.grid));
+    mnb_gemm256_clear_flags_kernel<<<dim3(1), dim3(256), 0, s>>>(p.flags, (int)plan.grid * 8 + 1);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
   }
   const unsigned grid = (unsigned)plan.grid;

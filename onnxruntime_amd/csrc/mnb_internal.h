@@ -102,6 +102,9 @@ struct MnbGemm256Plan {
 };
 // io: element type of the activations when it is not the packed matrix's own (MnbGemmArgs::io)
 MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspace, int io = kMnbIoModel);
+// device address of the status word in a split launch's workspace; NULL when the plan for this problem does not split
+const uint32_t* mnb_gemm256_status_word(const MnbLayout& L, int64_t M, int io, const void* workspace,
+                                        size_t workspace_bytes);
 bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM's 16-byte stores
 // the tile GEMM's 32-bit per-lane offsets reach every element of this problem
 uint64_t mnb_gemm256_max_lane_offset(int64_t lda);

@@ -136,3 +136,63 @@ def test_narrow_tiles_against_the_oracle_and_unit_vectors(oracle, M, N, K, bits,
     y1, _ = _gemm(c, op, dev(A), None, True)
     w = oracle.C.dequantize(c.B, c.scales, c.zero_points, N, K, bits, bs)
     assert np.array_equal(y1.cpu().numpy().view(np.uint16), np.ascontiguousarray(w[:, ks].T).view(np.uint16))
+
+
+def test_a_wait_that_gives_up_poisons_its_tile_and_is_reported(oracle):
+    """The bounded cross-workgroup wait, exercised from the host's choice of arguments: a test build of the library
+    (tests/hooks) leaves the lower parts of odd-numbered tiles uncomputed, so their flags stay zero, and bounds the
+    wait at a few polls.  The finalising parts of those tiles give up: every kernel ends normally, exactly the
+    odd-numbered tiles hold NaN, the even ones the product's own bits, and MnbGemmWorkspaceStatus reports it."""
+    from pathlib import Path
+    hooks_path = Path(__file__).resolve().parent / "hooks" / "libmnb_test_hooks.so"
+    assert hooks_path.exists(), "tests/hooks/libmnb_test_hooks.so is missing: python -m tests.hooks.build"
+    lib = _lib.load()
+    hooked = ctypes.CDLL(str(hooks_path))
+    for name in ("MnbGemm", "MnbGemmWorkspaceSize", "MnbGemmWorkspaceStatus", "MnbGemmTilePlan"):
+        getattr(hooked, name).restype, getattr(hooked, name).argtypes = _lib.SIGNATURES[name]
+    hooked.MnbTestSetSplitHooks.restype = None
+    hooked.MnbTestSetSplitHooks.argtypes = [ctypes.c_int, ctypes.c_int]
+    M, N, K, bits, bs = 1024, 4096, 8192, 4, 128
+    tr, tc, parts = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    hooked.MnbGemmTilePlan(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16, ctypes.byref(tr), ctypes.byref(tc), ctypes.byref(parts))
+    assert parts.value > 1, "the case is meant to be cut along K"
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, has_bias=True, seed=7)
+    op = MatMulNBits(K, N, bits, bs, dtype=torch.float16, has_zero_points=True, has_bias=True)
+    assert op.PrePack(dev(c.B), dev(c.scales), dev(c.zero_points))
+    a, bias = dev(c.A), dev(c.bias)
+    need = hooked.MnbGemmWorkspaceSize(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16)
+    assert need == lib.MnbGemmWorkspaceSize(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16) > 0
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    gave_up = ctypes.c_int(-1)
+
+    def run(l):
+        y = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+        _lib.check(l.MnbGemm(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16, _ptr(a), K, _ptr(op.packed), _ptr(bias), _ptr(y),
+                             N, _ptr(ws), need, stream))
+        torch.cuda.synchronize()
+        _lib.check(l.MnbGemmWorkspaceStatus(M, N, K, bits, bs, 1, _lib.DTYPE_FLOAT16, _ptr(ws), need, stream,
+                                            ctypes.byref(gave_up)))
+        return y
+
+    y_good = run(lib)
+    assert gave_up.value == 0 and not torch.isnan(y_good).any()
+    hooked.MnbTestSetSplitHooks(0, 0)                       # the hook build with its hooks off is the product
+    assert torch.equal(run(hooked).view(torch.int16), y_good.view(torch.int16)) and gave_up.value == 0
+    hooked.MnbTestSetSplitHooks(64, 1)                      # 64 polls, odd tiles lose their lower parts
+    try:
+        y_bad = run(hooked)
+    finally:
+        hooked.MnbTestSetSplitHooks(0, 0)
+    assert gave_up.value == 1
+    tiles_n = -(-N // tc.value)
+    nan = torch.isnan(y_bad)
+    for t in range((-(-M // tr.value)) * tiles_n):
+        r0, c0 = (t // tiles_n) * tr.value, (t % tiles_n) * tc.value
+        blk = (slice(r0, min(r0 + tr.value, M)), slice(c0, min(c0 + tc.value, N)))
+        if t & 1:
+            assert bool(nan[blk].all()), t
+        else:
+            assert not bool(nan[blk].any()) and torch.equal(y_bad[blk].view(torch.int16), y_good[blk].view(torch.int16)), t
+    # the next healthy launch clears the report
+    assert not torch.isnan(run(lib)).any() and gave_up.value == 0

@@ -53,21 +53,25 @@ PAIRS = [
     ((128, 4096, 4096, 4, 128), (17, 333, 200, 8, 64)),    # a large staged copy, then a ragged small one
     ((64, 512, 512, 4, 128), (1, 512, 1024, 4, 128)),      # scratch, then the decode kernel (no scratch)
     ((5, 100, 200, 4, 32), (3, 100, 200, 4, 32)),          # M <= 16 with K that is not whole chunks: staged route
+    ((1024, 4096, 8192, 4, 128), (300, 520, 1024, 4, 32)),  # tile GEMM cut along K (flags + partials fit), then staged
 ]
 
 
 @pytest.mark.parametrize("first,second", PAIRS)
 def test_same_bits_as_the_entry_point_with_a_workspace(oracle, first, second):
     used_scratch = False
+    lib = _lib.load()
     for (M, N, K, bits, bs) in (first, second):
         c = make_case(M, N, K, bits, bs, np.float16, has_zp=True, has_bias=True, seed=M + N)
         y_ref, y_new, need = _both(c)
+        assert need <= lib.MnbGemmStaticScratchCapacity()      # (the cut along K included: nothing is dropped)
         used_scratch |= need > 0
         assert not torch.isnan(y_new).any()
         assert torch.equal(_bits(y_ref), _bits(y_new)), (M, N, K, bits, bs)
         # and MnbGemm itself is right (the oracle's reference-semantics result, fp16 gate)
-        want = oracle.C.matmul(c.A, c.B, c.scales, c.zero_points, c.bias, c.N, c.K, c.bits, c.block_size).astype(np.float64)
-        got = y_new.cpu().numpy().astype(np.float64)
+        rows = np.arange(M) if M <= 300 else np.array([0, 127, 128, 255, 256, M - 1])
+        want = oracle.C.matmul(c.A[rows], c.B, c.scales, c.zero_points, c.bias, c.N, c.K, c.bits, c.block_size).astype(np.float64)
+        got = y_new.cpu().numpy()[rows].astype(np.float64)
         assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 5e-3
     assert used_scratch
 
@@ -88,7 +92,7 @@ def test_fp32_and_tile_gemm_need_no_scratch():
 def test_problems_beyond_the_capacity_are_rejected():
     lib = _lib.load()
     cap = lib.MnbGemmStaticScratchCapacity()
-    assert cap == 32 << 20
+    assert cap == (32 << 20) + (64 << 10)
     M, N, K = 1024, 4096, 32768 + 64                        # K not a multiple of 128: the streaming kernel at any M
     need = lib.MnbGemmWorkspaceSize(M, N, K, 4, 32, 0, _lib.DTYPE_FLOAT16)
     assert need > cap
@@ -97,3 +101,16 @@ def test_problems_beyond_the_capacity_are_rejected():
                                   None)
     assert rc == _lib.INVALID_ARGUMENT
     assert "the static array holds" in _lib.last_error()
+
+
+def test_the_common_cut_along_k_fits_the_array():
+    """128 workgroups x 256 KiB of partial tiles plus flags: the workspace of the usual split shapes."""
+    import ctypes as C
+    lib = _lib.load()
+    if lib.MnbGetDeviceCount() == 0:
+        pytest.skip("no device")
+    r, c, p = C.c_int(), C.c_int(), C.c_int()
+    for (M, N, K) in [(1024, 4096, 14336), (1024, 4096, 8192), (512, 8192, 8192)]:
+        lib.MnbGemmTilePlan(M, N, K, 4, 128, 1, _lib.DTYPE_FLOAT16, C.byref(r), C.byref(c), C.byref(p))
+        need = lib.MnbGemmWorkspaceSize(M, N, K, 4, 128, 1, _lib.DTYPE_FLOAT16)
+        assert p.value > 1 and 0 < need <= lib.MnbGemmStaticScratchCapacity(), (M, N, K, p.value, need)
