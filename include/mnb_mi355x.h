@@ -306,12 +306,14 @@ MNB_API int MnbVariantDequantize(float* dst_dev, const void* b_dev, const void* 
  * tested against, onnxruntime/test/mlas/unittest/test_sqnbitgemm.cpp:94-170).  A is quantised per row and block of
  * block_size elements (scale = max|a| / 127, round half away from zero), every block's dot product with the 4-bit
  * weights is exact integer arithmetic, and Y = bias + sum over blocks of float(dot) * a_scale * b_scale in fp32,
- * blocks in k order, narrowed once.  Same packed weights as MnbGemm.  Implemented for bits = 4, a_dtype float16 and
- * block sizes 32 ... 256 (MNB_NOT_IMPLEMENTED otherwise).  accuracy_level is a permission, not a demand: MnbGemm
- * computes the same nodes at full accuracy and is faster for every block size (measured on prefill shapes: 1.2 times
- * at blocks of 128, 1.5 at 256, 19 times at blocks of 32, where every 32-deep matrix instruction is followed by a
- * rescale of its 16 sums on the vector unit), so nothing chooses this entry point by itself.  The workspace (16-byte aligned, MnbGemmInt8WorkspaceSize bytes, 0 = not implemented for
- * these arguments) receives the quantised activations. */
+ * blocks in k order, narrowed once.  Same packed weights as MnbGemm.  Implemented for bits = 4, a_dtype float16,
+ * block sizes 64 ... 256 and M * K / block_size below 2^29 (MNB_NOT_IMPLEMENTED otherwise).  Blocks of 32 -- the block
+ * size the reference's own int8 kernels are built around -- are declined on purpose: the contract fixes one fp32
+ * multiply-add chain per output and 32-deep block, 80 vector instructions behind every matrix instruction, which ran
+ * 19 times slower than MnbGemm on a prefill shape.  accuracy_level is a permission, not a demand: MnbGemm computes the
+ * same nodes at full accuracy and is faster for every block size (measured on prefill shapes: 1.2 times at blocks of
+ * 128, 1.5 at 256), so nothing chooses this entry point by itself.  The workspace (16-byte aligned,
+ * MnbGemmInt8WorkspaceSize bytes, 0 = not implemented for these arguments) receives the quantised activations. */
 MNB_API size_t MnbGemmInt8WorkspaceSize(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points,
                                         int a_dtype);
 MNB_API int MnbGemmInt8(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,

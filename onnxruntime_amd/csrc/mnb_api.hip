@@ -347,7 +347,7 @@ size_t MnbGemmInt8WorkspaceSize(size_t M, size_t N, size_t K, int bits, int bloc
                                 int a_dtype) {
   if (check_config("MnbGemmInt8WorkspaceSize", bits, block_size, a_dtype) != MNB_OK || M == 0 || N == 0 || K == 0) return 0;
   const MnbLayout L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
-  return mnb_gemm_i8_supported(L) ? mnb_gemm_i8_workspace_bytes(L, (int64_t)M) : 0;
+  return mnb_gemm_i8_supported(L, (int64_t)M) ? mnb_gemm_i8_workspace_bytes(L, (int64_t)M) : 0;
 }
 
 int MnbGemmInt8(size_t M, size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype,
@@ -364,11 +364,12 @@ int MnbGemmInt8(size_t M, size_t N, size_t K, int bits, int block_size, int has_
     return fail(MNB_INVALID_ARGUMENT, "%s: M, N and K must fit in 31 bits", fn);
   MnbGemmArgs a{};
   a.L = mnb_make_layout((int64_t)N, (int64_t)K, bits, block_size, a_dtype, has_zero_points);
-  if (!mnb_gemm_i8_supported(a.L))
+  if (!mnb_gemm_i8_supported(a.L, (int64_t)M))
     return fail(MNB_NOT_IMPLEMENTED,
-                "%s: int8 activations are implemented for 4-bit weights, float16 models and block sizes 32 to 256 "
-                "(got bits=%d, block_size=%d, a_dtype=%d); MnbGemm computes these at full accuracy",
-                fn, bits, block_size, a_dtype);
+                "%s: int8 activations are implemented for 4-bit weights, float16 models, block sizes 64 to 256 and "
+                "M * K / block_size below 2^29 (got M=%zu, K=%zu, bits=%d, block_size=%d, a_dtype=%d); MnbGemm "
+                "computes these at full accuracy",
+                fn, M, K, bits, block_size, a_dtype);
   const size_t need = mnb_gemm_i8_workspace_bytes(a.L, (int64_t)M);
   if (!workspace_dev || workspace_bytes < need || reinterpret_cast<uintptr_t>(workspace_dev) % 16 != 0)
     return fail(MNB_INVALID_ARGUMENT, "%s: a 16-byte aligned workspace of %zu bytes is needed (MnbGemmInt8WorkspaceSize), %zu given",

@@ -23,11 +23,15 @@
 // is the packed layout's nibble order (e0 e4 e1 e5 e2 e6 e3 e7 per word); the quantiser writes the activations in the
 // same order, so no permutation happens in the loop.
 //
-// This route is slower than the fp16 one on this hardware for every block size below 256 and is therefore never
-// chosen by the dispatcher: it runs when the caller asks for it (MnbGemmInt8).  The per-block rescale costs five
-// vector instructions per output (integer correction, conversion, two multiplies, one add) against one matrix
-// instruction per 32 x 32 x 32 products: with 32-wide blocks 80 instructions per matrix instruction, with 128-wide
-// blocks 20; the fp16 route folds the scale into the weights and pays 3.5 per matrix instruction of half the depth.
+// This route is slower than the fp16 one on this hardware for every block size and is therefore never chosen by the
+// dispatcher: it runs when the caller asks for it (MnbGemmInt8).  The per-block rescale costs five vector
+// instructions per output (integer correction, conversion, two multiplies, one add) against one matrix instruction
+// per 32 x 32 x 32 products: with 128-wide blocks 20 instructions per matrix instruction, with 64-wide blocks 40; the
+// fp16 route folds the scale into the weights and pays 3.5 per matrix instruction of half the depth.
+// Blocks of 32 are declined (MNB_NOT_IMPLEMENTED): every matrix instruction would be followed by the rescale of its
+// 16 sums, 80 vector instructions -- 320 issue cycles against the 32 the matrix instruction takes.  The contract fixes
+// one fp32 multiply-add chain per output and block, so no arrangement of the loop removes them; the instantiation
+// that existed took 4.0 ms where the full-accuracy route takes 0.21 ms (M = 2048, N = 14336, K = 4096).
 #include <hip/hip_runtime.h>
 
 #include "mnb_buffer.hip.h"
@@ -312,7 +316,6 @@ __global__ void __launch_bounds__(256) mnb_gemm_i8_kernel(GemmI8Params p) {
 template <bool HAS_ZP>
 hipError_t launch_bs(const GemmI8Params& p, int bs, dim3 grid, hipStream_t s) {
   switch (bs) {
-    case 32: mnb_gemm_i8_kernel<HAS_ZP, 1><<<grid, dim3(256), 0, s>>>(p); break;
     case 64: mnb_gemm_i8_kernel<HAS_ZP, 2><<<grid, dim3(256), 0, s>>>(p); break;
     case 128: mnb_gemm_i8_kernel<HAS_ZP, 4><<<grid, dim3(256), 0, s>>>(p); break;
     case 256: mnb_gemm_i8_kernel<HAS_ZP, 8><<<grid, dim3(256), 0, s>>>(p); break;
@@ -323,14 +326,14 @@ hipError_t launch_bs(const GemmI8Params& p, int bs, dim3 grid, hipStream_t s) {
 
 }  // namespace
 
-bool mnb_gemm_i8_supported(const MnbLayout& L) {
-  // a block of 16 is half a matrix instruction; 8-bit weights do not fit the signed int8 operand as they are
-  return L.src_bits == 4 && L.bits == 4 && L.dtype == kMnbDtypeFloat16 && L.bs >= 32 && L.bs <= 256 &&
-         L.Kpad < ((int64_t)1 << 24);
-}
-
 // the kernel's 32-bit offsets into the activation scales and sums reach every row of this problem
 static bool offsets_fit(const MnbLayout& L, int64_t Mpad) { return 2 * L.KBp * Mpad * 4 < ((int64_t)1 << 32); }
+
+bool mnb_gemm_i8_supported(const MnbLayout& L, int64_t M) {
+  // 8-bit weights do not fit the signed int8 operand as they are; blocks below 64 are declined (file header)
+  return L.src_bits == 4 && L.bits == 4 && L.dtype == kMnbDtypeFloat16 && L.bs >= 64 && L.bs <= 256 &&
+         L.Kpad < ((int64_t)1 << 24) && offsets_fit(L, mnb_round_up(M, TILE));
+}
 
 size_t mnb_gemm_i8_workspace_bytes(const MnbLayout& L, int64_t M) {
   const int64_t Mpad = mnb_round_up(M, TILE);
@@ -340,7 +343,7 @@ size_t mnb_gemm_i8_workspace_bytes(const MnbLayout& L, int64_t M) {
 hipError_t mnb_launch_gemm_i8(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
   const int64_t Mpad = mnb_round_up(a.M, TILE);
-  if (!mnb_gemm_i8_supported(L) || !offsets_fit(L, Mpad) || a.workspace == nullptr ||
+  if (!mnb_gemm_i8_supported(L, a.M) || a.workspace == nullptr ||
       a.workspace_bytes < mnb_gemm_i8_workspace_bytes(L, a.M) || reinterpret_cast<uintptr_t>(a.workspace) % 16 != 0)
     return hipErrorInvalidValue;  // the caller checks before coming here
   QuantAParams q{};

@@ -110,8 +110,9 @@ bool mnb_gemm256_fused_ok(const MnbEpilogue& e);  // outputs allow the tile GEMM
 uint64_t mnb_gemm256_max_lane_offset(int64_t lda);
 bool mnb_gemm256_addressable(int64_t lda, int64_t Npad);
 hipError_t mnb_launch_gemm_generic(const MnbGemmArgs& a, hipStream_t s);
-// int8 activations (accuracy_level 4; mnb_gemm_i8.hip): 4-bit weights, fp16 model, block sizes 32 ... 256
-bool mnb_gemm_i8_supported(const MnbLayout& L);
+// int8 activations (accuracy_level 4; mnb_gemm_i8.hip): 4-bit weights, fp16 model, block sizes 64 ... 256, M rows
+// within the reach of the kernel's 32-bit offsets
+bool mnb_gemm_i8_supported(const MnbLayout& L, int64_t M);
 size_t mnb_gemm_i8_workspace_bytes(const MnbLayout& L, int64_t M);
 hipError_t mnb_launch_gemm_i8(const MnbGemmArgs& a, hipStream_t s);
 bool mnb_gemm32_applicable(const MnbGemmArgs& a);

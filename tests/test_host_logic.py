@@ -243,3 +243,19 @@ def test_fused_workspace_covers_the_streaming_kernel_on_split_shapes():
                 need = lib.MnbMlpWorkspaceSize(M, N, K, 4, 128, _lib.DTYPE_FLOAT16, 0)
                 assert split > 0 and need >= max(split, mid), (M, N, K, split, mid, need)
     assert seen >= 8
+
+
+def test_int8_route_sizes_agree_with_what_the_kernel_accepts():
+    """MnbGemmInt8WorkspaceSize is 0 exactly where MnbGemmInt8 declines, so callers that ask first fall back to the
+    full-accuracy route instead of running into an error: blocks of 32, and activations whose scales and sums lie
+    beyond the kernel's 32-bit offsets (2 * ceil(K / bs) * roundup(M, 128) * 4 bytes must stay below 4 GiB)."""
+    lib = _lib.load()
+    f16 = _lib.DTYPE_FLOAT16
+    assert lib.MnbGemmInt8WorkspaceSize(64, 256, 512, 4, 64, 0, f16) > 0
+    assert lib.MnbGemmInt8WorkspaceSize(64, 256, 512, 4, 32, 0, f16) == 0
+    K, bs = 1 << 20, 64                      # 16384 blocks per row
+    m_ok, m_big = 32640, 32768               # 2 * 16384 * M * 4 < 2^32  <=>  M < 32768
+    assert lib.MnbGemmInt8WorkspaceSize(m_ok, 256, K, 4, bs, 0, f16) > 0
+    assert lib.MnbGemmInt8WorkspaceSize(m_big, 256, K, 4, bs, 0, f16) == 0
+    assert lib.MnbGemmInt8(m_big, 256, K, 4, bs, 0, f16, 256, K, 256, None, 256, 256, 256, 1 << 40, None) == _lib.NOT_IMPLEMENTED
+    assert "M * K / block_size below 2^29" in _lib.last_error()
