@@ -140,6 +140,8 @@ def load_probe():
     lib.MnbProbeReadBandwidth.restype = ctypes.c_int
     lib.MnbProbeReadBandwidth.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                           ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeReadBandwidthResident.restype = ctypes.c_int
+    lib.MnbProbeReadBandwidthResident.argtypes = lib.MnbProbeReadBandwidth.argtypes
     lib.MnbProbeMfmaRate.restype = ctypes.c_int
     lib.MnbProbeMfmaRate.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     lib.MnbProbeRelease.restype = None
@@ -312,9 +314,22 @@ def main() -> int:
                     assert rc == 0, f"read probe failed ({rc})"
                     sweep_rows.append((v.value, threads, inflight, batches))
         best = max(sweep_rows)
+        # the same bytes waiting in the Infinity Cache (every launch re-reads one buffer): the eight best configurations
+        resident_rows = []
+        for _, threads, inflight, batches in sorted(sweep_rows, reverse=True)[:8]:
+            assert probe.MnbProbeReadBandwidthResident(bytes_per_launch, LAYERS, threads, inflight, batches,
+                                                       ctypes.byref(v)) == 0
+            resident_rows.append((v.value, threads, inflight, batches))
         probe.MnbProbeRelease()
-        assert probe.MnbProbeReadBandwidth(1 << 30, 2, 256, 8, 1, ctypes.byref(v)) == 0
-        read_big = v.value
+        # 1 GiB per launch, where launch ramp and tail no longer count: the same 36 configurations
+        big_rows = []
+        for threads in (256, 512, 1024):
+            for inflight in (4, 8, 16, 32):
+                for batches in (1, 2, 4):
+                    assert probe.MnbProbeReadBandwidth(1 << 30, 2, threads, inflight, batches, ctypes.byref(v)) == 0
+                    big_rows.append((v.value, threads, inflight, batches))
+        big_best = max(big_rows)
+        read_big = big_best[0]
         probe.MnbProbeRelease()
         out["roofline"]["measured_ceiling"] = {
             "read_only_kernel_same_bytes_per_launch_GBs": round(best[0], 1),
@@ -322,13 +337,25 @@ def main() -> int:
             "read_only_kernel_sweep_GBs_min_median_max": [round(x, 1) for x in (
                 min(sweep_rows)[0], sorted(sweep_rows)[len(sweep_rows) // 2][0], best[0])],
             "read_only_kernel_configs_swept": len(sweep_rows),
+            "read_only_kernel_same_bytes_in_infinity_cache_GBs": round(max(resident_rows)[0], 1),
             "read_only_kernel_1GiB_per_launch_GBs": round(read_big, 1),
+            "read_only_kernel_1GiB_best_config": {"threads": big_best[1], "loads_in_flight": big_best[2],
+                                                  "batches": big_best[3]},
+            "read_only_kernel_1GiB_sweep_GBs_min_median_max": [round(x, 1) for x in (
+                min(big_rows)[0], sorted(big_rows)[len(big_rows) // 2][0], big_best[0])],
+            "read_only_kernel_1GiB_frac_of_hbm_peak": round(read_big / HBM_PEAK_GBS, 4),
             "frac_of_read_only_kernel": round(gbs / best[0], 4) if best[0] > 0 else None,
         }
         if args.sweep:
             for r in sorted(sweep_rows, reverse=True):
                 print(f"read probe: {r[0]:8.1f} GB/s threads={r[1]} loads_in_flight={r[2]} batches={r[3]}",
                       file=sys.stderr)
+            for r in sorted(big_rows, reverse=True):
+                print(f"read probe 1 GiB: {r[0]:8.1f} GB/s threads={r[1]} loads_in_flight={r[2]} batches={r[3]}",
+                      file=sys.stderr)
+            for r in sorted(resident_rows, reverse=True):
+                print(f"read probe, data in the Infinity Cache: {r[0]:8.1f} GB/s threads={r[1]} loads_in_flight={r[2]} "
+                      f"batches={r[3]}", file=sys.stderr)
 
     # ---- prefill GEMM ----------------------------------------------------------------------------------------
     if not args.no_prefill:

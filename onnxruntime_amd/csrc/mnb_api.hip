@@ -778,7 +778,9 @@ const char* MnbGemmKernelNameStrided(size_t M, size_t N, size_t K, int bits, int
   a.lda = (int64_t)lda;
   a.A = nullptr;  // an aligned base
   a.workspace_bytes = ~(size_t)0;  // a caller that follows MnbGemmWorkspaceSize
-  return mnb_kernel_name(mnb_select_kernel(a), a.L);
+  const MnbKernelKind kind = mnb_select_kernel(a);
+  if (kind == kMnbKernelMid && mnb_mid_shared(a)) return "mnb_mid_shared_kernel";
+  return mnb_kernel_name(kind, a.L);
 }
 
 const char* MnbGemmKernelName(size_t M, size_t N, size_t K, int bits, int block_size, int a_dtype) {

@@ -789,6 +789,9 @@ constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
 template <int BITS, bool HAS_ZP, int MPS, int DT, bool HAS_256 = true>
 hipError_t launch_rows(const Gemm256Params& p, unsigned grid, hipStream_t s) {
   if (p.tile_cols == 128) {
+    if constexpr (DT == 0) {
+      if (p.tile_rows == 64) return launch_wm<BITS, HAS_ZP, MPS, 1, 1, DT, 4>(p, grid, s);
+    }
     if constexpr (DT == 0 || DT == 1)
       return p.tile_rows == 128 ? launch_wm<BITS, HAS_ZP, MPS, 2, 1, DT, 4>(p, grid, s) : hipErrorInvalidValue;
     else
@@ -932,9 +935,9 @@ MnbGemm256Plan mnb_gemm256_plan(const MnbLayout& L, int64_t M, bool with_workspa
   if (const char* e = mnb_tuning_env("MNB_GEMM256_PLAN")) {  // calibration: "<tile rows>,<parts>[,<tile columns>]"
     int rows = 0, parts = 0, cols = 256;
     const int got = sscanf(e, "%d,%d,%d", &rows, &parts, &cols);
-    if (got >= 2 && (rows == 128 || (rows == 256 && !only_128_rows)) && parts >= 1 && parts <= 8 &&
-        upt % parts == 0 && (parts == 1 || with_workspace) &&
-        (cols == 256 || (cols == 128 && rows == 128 && narrow_ok))) {
+    if (got >= 2 && (rows == 128 || (rows == 256 && !only_128_rows) || (rows == 64 && cols == 128 && io == kMnbIoModel)) &&
+        parts >= 1 && parts <= 8 && upt % parts == 0 && (parts == 1 || with_workspace) &&
+        (cols == 256 || (cols == 128 && rows <= 128 && narrow_ok))) {
       best = MnbGemm256Plan{};
       best.tile_rows = rows;
       best.tile_cols = cols;

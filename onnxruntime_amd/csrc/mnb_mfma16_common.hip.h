@@ -165,7 +165,13 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
     if constexpr (BITS == 4) load_meta_vec<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1);
   }
 #pragma unroll
-  for (int t = 0; t < T; ++t) R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + col0 + t * 16];
+  for (int t = 0; t < T; ++t) {
+#if defined(MNB_ABLATE_NO_LOADS)
+    R.w[t] = make_uint4((uint32_t)c, (uint32_t)kq, (uint32_t)t, 0x12345678u);  // calibration builds: no weight stream
+#else
+    R.w[t] = p.W[((int64_t)c * 4 + kq) * p.Npad + col0 + t * 16];
+#endif
+  }
 }
 
 // The same loads for slabs that do not start at a multiple of 64 columns (the meta entries of a lane's tiles are then
@@ -263,9 +269,11 @@ __device__ __forceinline__ h8_t raw4_bf16(uint32_t w, const UnpackConsts& u, uin
 // Sum the per-wavefront partial tiles (red[(w * T * 4 + t * 4 + r) * 64 + lane], written by NW wavefronts) in
 // wavefront order and write the result.  Lane l, register r of tile t is row m_base + 4 * (l / 16) + r, packed column
 // n0 + 16 t + l % 16.  bias is indexed by packed column.
+// `first` / `step`: the threads that share this slab of T tiles number themselves first, first + step, ... (by default
+// the whole workgroup: thread index, NW * 64).
 template <int T, int NW>
 __device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, const float* red, int m_base,
-                                                       int64_t n0) {
+                                                       int64_t n0, int first = threadIdx.x, int step = NW * 64) {
   auto total = [&](int tr, int l) {
     float sum = 0.f;
 #pragma unroll
@@ -276,7 +284,7 @@ __device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, co
   if (p.epi.kind == kMnbFusedMlp) {
     // adjacent tiles (2u, 2u + 1) are gate and up of output columns [n0 / 2 + 16 u, +16)
     if constexpr (T >= 2) {
-      for (int i = threadIdx.x; i < (T / 2) * 4 * 64; i += NW * 64) {
+      for (int i = first; i < (T / 2) * 4 * 64; i += step) {
         const int l = i & 63, ur = i >> 6;
         const int u = ur >> 2, r = ur & 3;
         const int m = m_base + 4 * (l >> 4) + r;
@@ -290,7 +298,7 @@ __device__ __forceinline__ void reduce_and_store_tiles(const SkinnyParams& p, co
     }
     return;
   }
-  for (int i = threadIdx.x; i < T * 4 * 64; i += NW * 64) {
+  for (int i = first; i < T * 4 * 64; i += step) {
     const int l = i & 63, tr = i >> 6;
     const int t = tr >> 2, r = tr & 3;
     const int m = m_base + 4 * (l >> 4) + r;

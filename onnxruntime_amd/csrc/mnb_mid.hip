@@ -279,6 +279,133 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, in
   }
 }
 
+// ---- activations shared through LDS ---------------------------------------------------------------------------------
+// The kernel above re-reads the activations once per 16 T columns: every workgroup walks all of K, and its wavefronts,
+// which split K between them, share nothing.  For wide matrices that stream is several times the weights' (64 rows,
+// K = 4096, N = 28672, 64 columns per workgroup: 448 x 512 KB = 229 MB against 59 MB of weights) and it is the level-2
+// caches, busy 70 % of the launch, that set the pace.  Here a workgroup's eight wavefronts form KGS = 4 teams of NG = 2:
+// the teams split K as before, the two wavefronts of a team own neighbouring slabs of 16 T columns and walk the same
+// chunks, and the chunk's activations (16 MT rows x 256 bytes) are fetched ONCE per team, from the caller's row-major A
+// straight into LDS (buffer_load ... lds, 16-byte pieces XOR-swizzled with the row so that neither the row-contiguous
+// fills nor the operand reads conflict on banks), one round ahead of the arithmetic, into one of two buffers.  Per
+// round: wait for the own fills of this round, barrier, start the fills of the next round, pick the operands up from
+// LDS, compute, reload the weight registers for the round after next.  No staged copy of A, no staging launch.
+// Needs K a whole number of chunks and 16-byte aligned rows of A; everything else takes the kernel above.
+template <int BITS, bool HAS_ZP, int T, int MT, int KGS, int NG>
+__global__ void __launch_bounds__(KGS * NG * 64) mnb_mid_shared_kernel(const uint4* hot_W, int64_t hot_Npad,
+                                                                        const _Float16* hot_A, const uint8_t* hot_meta,
+                                                                        int64_t hot_lda, int hot_chunks,
+                                                                        int hot_bs_shift, MidParams rest) {
+  MidParams mp = rest;
+  mp.s.W = hot_W;
+  mp.s.Npad = hot_Npad;
+  mp.s.A = hot_A;
+  mp.s.meta = hot_meta;
+  mp.s.lda = hot_lda;
+  mp.s.chunks = hot_chunks;
+  mp.s.bs_shift = hot_bs_shift;
+  const SkinnyParams& p = mp.s;
+  constexpr int NW = KGS * NG;
+  constexpr int GK = 128 / BITS, NI = GK / 8, CK = 4 * GK;
+  constexpr int PIECES = 4 * NI;                   // 16-byte pieces per row of a chunk
+  constexpr int ROWS = 16 * MT;                    // rows of A a workgroup works on
+  constexpr int CHUNK_BYTES = ROWS * PIECES * 16;  // one team's activations of one chunk
+  constexpr int RPI = 64 / PIECES;                 // rows one fill instruction covers
+  constexpr int A_PER_WAVE = ROWS / RPI / NG;      // fill instructions per wavefront and round
+  constexpr int W_LOADS = T + (BITS == 4 ? 2 : 1); // vector-memory instructions of load_chunk (MODE 1)
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kg = wave / NG, ng = wave % NG;
+  const int j = lane & 15, kq = lane >> 4;
+  const int64_t n0 = ((int64_t)blockIdx.x * NG + ng) * (16 * T);
+  const int64_t col0 = n0 + j;
+  const int m0 = blockIdx.y * ROWS;
+  auto swz = [](int row) { return PIECES == 16 ? (row & 15) : ((row >> 1) & 7); };
+
+  // this wavefront's share of a round's fills: instruction q covers rows q * RPI + lane / PIECES
+  uint32_t a_off[A_PER_WAVE];
+#pragma unroll
+  for (int u = 0; u < A_PER_WAVE; ++u) {
+    const int row = (ng * A_PER_WAVE + u) * RPI + lane / PIECES;
+    const int piece = (lane % PIECES) ^ swz(row);
+    const int grow = m0 + row < p.M ? m0 + row : p.M - 1;  // rows beyond M re-read the last row and are never stored
+    a_off[u] = (uint32_t)(((int64_t)grow * p.lda + piece * 8) * 2);
+  }
+  unsigned char* const team = smem + kg * CHUNK_BYTES;  // buffer b of the team: team + b * KGS * CHUNK_BYTES
+  auto fill = [&](int c, int b) {
+    const rsrc_t r = mnb_rsrc(p.A + (int64_t)c * CK);
+#pragma unroll
+    for (int u = 0; u < A_PER_WAVE; ++u)
+      mnb_buffer_load_lds_b128(r, a_off[u],
+                               (lds_ptr_t)(team + b * (KGS * CHUNK_BYTES) + (ng * A_PER_WAVE + u) * RPI * PIECES * 16));
+  };
+  f4_t y[MT][T];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < T; ++t) y[mt][t] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const UnpackConsts uc = make_unpack_consts();
+  h8_t af[MT][NI];
+  auto pick = [&](int b) {
+    const unsigned char* buf = team + b * (KGS * CHUNK_BYTES);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int row = mt * 16 + j;
+        af[mt][i] = *reinterpret_cast<const h8_t*>(buf + (row * PIECES + ((kq * NI + i) ^ swz(row))) * 16);
+      }
+  };
+
+  const int last = p.chunks - 1;
+  const int rounds = (p.chunks + KGS - 1) / KGS;
+  auto chunk_of = [&](int r) { return r * KGS + kg; };
+  ChunkRegs<BITS, T> R0, R1;
+  // One round.  On entry the fills of round r (issued a round earlier) are followed in issue order by exactly one
+  // set of weight loads, so "at most W_LOADS outstanding" means they have landed; the barrier makes that true of the
+  // team-mate's share, and tells everybody that the other buffer's readers are done with it.
+  auto round = [&](int r, ChunkRegs<BITS, T>& R, int b) {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(W_LOADS));
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    fill(min(chunk_of(r + 1), last), b ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+    pick(b);
+    if (chunk_of(r) < p.chunks) mid_compute_chunk<BITS, HAS_ZP, T, MT, false, kMnbIoModel>(R, af, nullptr, 0, uc, y);
+    __builtin_amdgcn_sched_barrier(0);
+    load_chunk<BITS, HAS_ZP, 1, T>(p, min(chunk_of(r + 2), last), kq, col0, R);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  load_chunk<BITS, HAS_ZP, 1, T>(p, min(chunk_of(0), last), kq, col0, R0);
+  __builtin_amdgcn_sched_barrier(0);
+  fill(min(chunk_of(0), last), 0);
+  __builtin_amdgcn_sched_barrier(0);
+  load_chunk<BITS, HAS_ZP, 1, T>(p, min(chunk_of(1), last), kq, col0, R1);
+  for (int r = 0; r < rounds; r += 2) {
+    round(r, R0, 0);
+    round(r + 1, R1, 1);  // (past the end: loads of valid memory, a barrier everybody reaches, no arithmetic)
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lds0(0));  // the last prefetches write LDS the reduction is about to reuse
+  __syncthreads();
+
+  // reduce over the teams, one row tile at a time; the KGS wavefronts that share a slab do its sums
+  float* red = reinterpret_cast<float*>(smem);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (mt > 0) __syncthreads();
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[((ng * KGS + kg) * T * 4 + t * 4 + r) * 64 + lane] = y[mt][t][r];
+    __syncthreads();
+    reduce_and_store_tiles<T, KGS>(p, red + ng * KGS * T * 4 * 64, m0 + mt * 16, n0, kg * 64 + lane, KGS * 64);
+  }
+}
+
 struct MidPlan {
   int t, mt, nw;
 };
@@ -314,8 +441,7 @@ MidPlan mid_plan(const MnbLayout& L, int64_t M, int min_t = 1) {
   // eight wavefronts split K further and hide more latency in a single round of workgroups; with several rounds of
   // the largest tile, two workgroups of four wavefronts share a CU instead
   pl.nw = chunks < 16 || (best_area == 16 && best_wgs >= 384) ? 4 : 8;
-  static const char* const plan_override = mnb_tuning_env("MNB_MID_PLAN");  // tuning override "<T>,<MT>,<NW>", read once
-  if (const char* e = plan_override) {
+  if (const char* e = mnb_tuning_env("MNB_MID_PLAN")) {  // calibration builds: "<T>,<MT>,<NW>"
     int t = 0, mt = 0, nw = 0;
     if (sscanf(e, "%d,%d,%d", &t, &mt, &nw) == 3 && (t == 1 || t == 2 || t == 4) && (mt == 2 || mt == 4) &&
         (nw == 4 || nw == 8)) {
@@ -385,6 +511,57 @@ hipError_t launch_io(const MidParams& p, const MidPlan& pl, int io, bool direct,
 
 int mid_row_tiles(int64_t M, int mt) { return (int)((M + 16 * mt - 1) / (16 * mt)) * mt; }
 
+// ---- the kernel with activations shared through LDS: when it applies, and its launch
+constexpr int kSharedT = 4, kSharedKgs = 4, kSharedNg = 2;  // 128 columns per workgroup, eight wavefronts
+
+bool mid_shared_applies(const MnbGemmArgs& a) {
+  const MnbLayout& L = a.L;
+  if (a.io != kMnbIoModel || L.dtype != kMnbDtypeFloat16 || a.M <= 16) return false;
+  const int CK = 4 * L.group_k;
+  const bool vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
+  // the fills address A with 32-bit byte offsets from the chunk's first column
+  const bool reach = (uint64_t)a.M * (uint64_t)a.lda * 2 + 512 < ((uint64_t)1 << 32);
+  if (!vec_ok || !reach || L.K % CK != 0) return false;
+  bool use;
+  if (const char* e = mnb_tuning_env("MNB_MID_SHARED")) {
+    use = e[0] != '0';
+  } else {
+    // A workgroup here needs the same time whatever the grid (eight rounds of 2 - 3 us at K = 4096), so the kernel pays
+    // where its 128-column slabs make one well-filled round of workgroups -- which is also where the activations'
+    // stream through the level-2 caches is largest.  Measured against the kernel above (K = 4096, 4-bit):
+    // N = 28672: M = 17 21.9 -> 17.7 us, M = 32 22.8 -> 17.6, M = 64 28.5 -> 25.5; N = 14336, M = 128 28.1 -> 24.8;
+    // N = 11008, M = 128 30.2 -> 25.2; N = 6144, M = 256 27.4 -> 24.0; with fewer workgroups than 5/8 of the compute
+    // units, or more than all of them, it loses (N = 14336, M = 64: 16.9 -> 24.0; N = 28672, M = 256: 82 -> 100).
+    const int64_t slabs = (L.N + 16 * kSharedT * kSharedNg - 1) / (16 * kSharedT * kSharedNg);
+    const int rows = a.M <= 32 ? 32 : 64;
+    const int64_t wgs = slabs * ((a.M + rows - 1) / rows), cus = mnb_device_info().cus;
+    use = wgs * 8 >= cus * 5 && wgs <= cus && L.K / CK >= 2 * kSharedKgs;
+  }
+  return use;
+}
+
+template <int BITS, bool HAS_ZP, int MT>
+hipError_t launch_shared_mt(const MidParams& mp, hipStream_t s) {
+  const SkinnyParams& p = mp.s;
+  constexpr int T = kSharedT, KGS = kSharedKgs, NG = kSharedNg, NW = KGS * NG;
+  constexpr size_t chunk_bytes = (size_t)16 * MT * (128 / BITS / 2) * 16;
+  constexpr size_t fills = 2 * KGS * chunk_bytes, red = (size_t)NW * T * 4 * 64 * sizeof(float);
+  constexpr size_t smem = fills > red ? fills : red;
+  auto kernel = mnb_mid_shared_kernel<BITS, HAS_ZP, T, MT, KGS, NG>;
+  if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      e != hipSuccess)
+    return e;
+  const dim3 grid((unsigned)((p.N + 16 * T * NG - 1) / (16 * T * NG)), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)));
+  kernel<<<grid, dim3(NW * 64), smem, s>>>(p.W, p.Npad, p.A, p.meta, p.lda, p.chunks, p.bs_shift, mp);
+  return hipGetLastError();
+}
+
+template <int BITS, bool HAS_ZP>
+hipError_t launch_shared(const MidParams& mp, hipStream_t s) {
+  return mp.s.M <= 32 ? launch_shared_mt<BITS, HAS_ZP, 2>(mp, s) : launch_shared_mt<BITS, HAS_ZP, 4>(mp, s);
+}
+
 }  // namespace
 
 bool mnb_mid_applicable(const MnbGemmArgs& a) {
@@ -402,7 +579,10 @@ size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M) {
 // Activations straight from A when its rows allow 16-byte loads and K is a whole number of chunks (the kernel then
 // reorders them itself, and no workspace is touched); otherwise, and for the widest tiles, a staging pass writes them
 // in operand order first.
+bool mnb_mid_shared(const MnbGemmArgs& a) { return mid_shared_applies(a); }
+
 bool mnb_mid_direct(const MnbGemmArgs& a) {
+  if (mid_shared_applies(a)) return true;  // (reads A in place as well)
   const MidPlan pl = mid_plan(a.L, a.M, a.epi.kind == kMnbFusedMlp ? 2 : 1);
   const bool vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0);
   bool direct = vec_ok && a.L.K % (4 * a.L.group_k) == 0 && !(pl.mt == 4 && pl.t == 4);
@@ -444,6 +624,10 @@ hipError_t mnb_launch_mid(const MnbGemmArgs& a, hipStream_t s) {
     p.epi.out2 = reinterpret_cast<_Float16*>(a.epi.out[2]);
     p.epi.ld1 = a.epi.ld[1];
     p.epi.ld2 = a.epi.ld[2];
+  }
+  if (mid_shared_applies(a)) {
+    if (L.bits == 4) return L.has_zp ? launch_shared<4, true>(mp, s) : launch_shared<4, false>(mp, s);
+    return L.has_zp ? launch_shared<8, true>(mp, s) : launch_shared<8, false>(mp, s);
   }
   mp.As = reinterpret_cast<const uint4*>(a.workspace);
   mp.row_tiles = mid_row_tiles(a.M, pl.mt);

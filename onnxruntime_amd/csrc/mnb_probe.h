@@ -22,6 +22,10 @@ extern "C" {
  * The buffers are kept between calls with the same sizes (a sweep allocates once); MnbProbeRelease frees them. */
 MNB_PROBE_API int MnbProbeReadBandwidth(size_t bytes_per_launch, int launches, int threads, int loads_in_flight,
                                         int batches, double* gb_per_s);
+/* The same with every launch reading the SAME buffer: what a kernel of that size reaches when its data waits in the
+ * Infinity Cache (bytes_per_launch well below 256 MB) instead of HBM. */
+MNB_PROBE_API int MnbProbeReadBandwidthResident(size_t bytes_per_launch, int launches, int threads,
+                                                int loads_in_flight, int batches, double* gb_per_s);
 MNB_PROBE_API void MnbProbeRelease(void);
 
 /* TFLOP/s of a loop of nothing but v_mfma_f32_32x32x16_f16 on every CU, with constant operands

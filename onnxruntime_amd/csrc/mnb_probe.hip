@@ -102,7 +102,9 @@ void launch_read(unsigned blocks, int threads, hipStream_t s, const uint4* p, si
 }
 
 // `launches` back-to-back kernels (one HIP graph), each reading its own `bytes` of device memory once.
-hipError_t probe_read(size_t bytes, int launches, int threads, int loads_in_flight, int batches, double* gb_per_s) {
+// same_buffer: every launch reads the first buffer again (30 MB stay in the 256 MB Infinity Cache between launches).
+hipError_t probe_read(size_t bytes, int launches, int threads, int loads_in_flight, int batches, bool same_buffer,
+                      double* gb_per_s) {
   *gb_per_s = 0.0;
   const size_t n_vec = bytes / 16;
   hipStream_t s = nullptr;
@@ -116,17 +118,17 @@ hipError_t probe_read(size_t bytes, int launches, int threads, int loads_in_flig
   };
   const size_t per_block = (size_t)threads * loads_in_flight * batches;
   const unsigned blocks = (unsigned)((n_vec + per_block - 1) / per_block);
-  ok(ensure_buffers(n_vec, launches));
+  ok(ensure_buffers(n_vec, same_buffer ? 1 : launches));
   if (ok(err) && ok(hipStreamCreateWithFlags(&s, hipStreamNonBlocking)) && ok(hipEventCreate(&e0)) &&
       ok(hipEventCreate(&e1)) && ok(hipDeviceSynchronize()) &&
       ok(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal))) {
     for (int i = 0; i < launches; ++i) {
       switch (loads_in_flight) {
-        case 2: launch_read<2>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
-        case 4: launch_read<4>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
-        case 8: launch_read<8>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
-        case 16: launch_read<16>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
-        default: launch_read<32>(blocks, threads, s, g_bufs[i], n_vec, batches); break;
+        case 2: launch_read<2>(blocks, threads, s, g_bufs[same_buffer ? 0 : i], n_vec, batches); break;
+        case 4: launch_read<4>(blocks, threads, s, g_bufs[same_buffer ? 0 : i], n_vec, batches); break;
+        case 8: launch_read<8>(blocks, threads, s, g_bufs[same_buffer ? 0 : i], n_vec, batches); break;
+        case 16: launch_read<16>(blocks, threads, s, g_bufs[same_buffer ? 0 : i], n_vec, batches); break;
+        default: launch_read<32>(blocks, threads, s, g_bufs[same_buffer ? 0 : i], n_vec, batches); break;
       }
     }
     ok(hipStreamEndCapture(s, &g));
@@ -199,7 +201,17 @@ int MnbProbeReadBandwidth(size_t bytes_per_launch, int launches, int threads, in
   if (!gb_per_s || bytes_per_launch < 16 || launches < 1 || (double)bytes_per_launch * launches > 8e9 || !u_ok ||
       threads < 64 || threads > 1024 || threads % 64 != 0 || batches < 1 || batches > 64)
     return 2;
-  return probe_read(bytes_per_launch, launches, threads, loads_in_flight, batches, gb_per_s) == hipSuccess ? 0 : 1;
+  return probe_read(bytes_per_launch, launches, threads, loads_in_flight, batches, false, gb_per_s) == hipSuccess ? 0 : 1;
+}
+
+int MnbProbeReadBandwidthResident(size_t bytes_per_launch, int launches, int threads, int loads_in_flight, int batches,
+                                  double* gb_per_s) {
+  const bool u_ok = loads_in_flight == 2 || loads_in_flight == 4 || loads_in_flight == 8 || loads_in_flight == 16 ||
+                    loads_in_flight == 32;
+  if (!gb_per_s || bytes_per_launch < 16 || launches < 1 || bytes_per_launch > ((size_t)1 << 31) || !u_ok ||
+      threads < 64 || threads > 1024 || threads % 64 != 0 || batches < 1 || batches > 64)
+    return 2;
+  return probe_read(bytes_per_launch, launches, threads, loads_in_flight, batches, true, gb_per_s) == hipSuccess ? 0 : 1;
 }
 
 void MnbProbeRelease(void) { release_buffers(); }

@@ -50,6 +50,16 @@ template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t* af, const BConst& bc,
                                               const UnpackConsts& uc, f4_t* y) {
   constexpr int NI = (128 / BITS) / 8;
+#if defined(MNB_ABLATE_NO_MATH)
+  // calibration builds: the loads are waited for and nothing is computed (what the arithmetic costs a launch)
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    asm volatile("; keep %0 %1 %2 %3 %4" ::"v"(R.w[t].x), "v"(R.w[t].y), "v"(R.w[t].z), "v"(R.w[t].w), "v"(R.m0[t]));
+  }
+#pragma unroll
+  for (int i = 0; i < NI; ++i) asm volatile("; keep %0" ::"v"(__builtin_bit_cast(u4_t, af[i])));
+  return;
+#endif
   if constexpr (MODE == 0 || MODE == 5) {
     // init[m] = -sum_k (off_k + zp) a[m][k] (no zero points) or -sum_k off_k a[m][k]; nc2[m] = -sum_k a[m][k].
     // The constant operands are the same in every lane, so every lane receives the value of its own rows.
@@ -191,6 +201,20 @@ template <int T, int NW>
 __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* red, const f4_t* y, int wave, int lane,
                                                 int64_t n0) {
   const int kq = lane >> 4;
+#if defined(MNB_ABLATE_NO_REDUCE)
+  // calibration builds: no exchange through LDS, no barrier; the first wavefront stores its own partial sums (what the
+  // reduction costs a launch; the result is wrong)
+  if (wave == 0) {
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int64_t n = n0 + t * 16 + (lane & 15);
+        if (4 * kq + r < p.M && n < p.N) p.C[(int64_t)(4 * kq + r) * p.ldc + n] = (_Float16)y[t][r];
+      }
+  }
+  return;
+#endif
 #pragma unroll
   for (int t = 0; t < T; ++t)
 #pragma unroll

@@ -210,6 +210,22 @@ def test_qkv_parity(oracle, dtype, norm, M, Nq, Nkv, K, bits, bs):
                          max(np.linalg.norm(want.astype(np.float64)), 1e-30)) <= 1e-3
 
 
+@pytest.mark.parametrize("M,N,K,bits,bs", [(64, 14336, 1024, 4, 128), (20, 10500, 1024, 8, 64)])
+def test_mlp_on_the_shared_activations_variant(oracle, M, N, K, bits, bs):
+    """Gate and up packed as one matrix of 2 N columns wide enough for the streaming kernel's variant that shares the
+    activations through LDS: the operator's output against the oracle, and against the two separate products."""
+    lib = _lib.load()
+    if lib.MnbGemmKernelName(M, 2 * ((N + 15) // 16 * 16), K, bits, bs, _lib.DTYPE_FLOAT16) != b"mnb_mid_shared_kernel":
+        pytest.skip("this device's compute-unit count does not select the shared-activations variant here")
+    g, _ = _mats(M, N, K, bits, bs, np.float16, True, 71)
+    u, _ = _mats(M, N, K, bits, bs, np.float16, True, 72)
+    op = MatMulNBitsMlp(K, N, bits, bs)
+    assert op.PrePack(dev(g.B), dev(g.scales), dev(g.bias), dev(u.B), dev(u.scales), dev(u.bias))
+    y = op.Compute(dev(g.A))
+    torch.cuda.synchronize()
+    _check_mlp(oracle, y.cpu().numpy(), g.A, g, u, N, K, bits, bs, np.float16)
+
+
 def test_tile_gemm_shape_with_unaligned_output_takes_the_streaming_kernel(oracle):
     """Where the shape selects the tile GEMM but Y does not allow 16-byte stores, the streaming kernel (whose scratch
     the workspace contract reserves) writes the outputs: same result, up to the narrowing of gate / up."""

@@ -212,6 +212,36 @@ def test_decode_with_more_slabs_than_compute_units(oracle, bits, bs, zp, N, K, M
         assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
 
 
+@pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (4, 16, True), (8, 64, True), (8, 16, False)])
+@pytest.mark.parametrize("N,K,M", [(28672, 1024, 64), (21000, 1024, 17), (28672, 2048, 32), (24000, 1024, 33),
+                                   (11008, 1024, 100), (14336, 1024, 128), (6144, 1024, 250)])
+def test_streaming_kernel_with_activations_shared_through_lds(oracle, bits, bs, zp, N, K, M):
+    """Wide matrices whose 128-column slabs make one well-filled round of workgroups: pairs of wavefronts share each
+    chunk of the activations through LDS (fetched straight from the caller's A, no staged copy).  Every row of Y against
+    the oracle on sampled rows; unit-vector rows return columns of W bit for bit; a misaligned A takes the staged route
+    and gives the same sums up to their order."""
+    from onnxruntime_amd import _lib
+    lib = _lib.load()
+    if lib.MnbGemmKernelName(M, N, K, bits, bs, _lib.DTYPE_FLOAT16) != b"mnb_mid_shared_kernel":
+        pytest.skip("this device's compute-unit count does not select the shared-activations variant here")
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + M)
+    y = run_case(c)
+    check_against_oracle(oracle, c, y)
+    ks = np.random.default_rng(N).choice(K, size=M, replace=False)
+    eye = np.zeros((M, K), np.float16)
+    eye[np.arange(M), ks] = 1
+    c0 = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + M)
+    w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
+    assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+    # rows that are not 16-byte aligned: the staged route
+    op = make_op(c)
+    wide = torch.zeros(M, K + 3, dtype=torch.float16, device="cuda")
+    wide[:, :K] = dev(c.A)
+    y2 = op.Compute(wide[:, :K], bias=dev(c.bias)).cpu().numpy()
+    d = np.abs(y2.astype(np.float64) - y.astype(np.float64))
+    assert d.max() <= 2e-3 * np.abs(y).max() + 1e-3
+
+
 @pytest.mark.parametrize("bits,bs,zp", [(4, 32, True), (4, 128, False), (4, 16, True), (8, 64, True)])
 @pytest.mark.parametrize("N,K", [(300, 4096), (4100, 8192), (1000, 14336), (8200, 4096)])
 @pytest.mark.parametrize("M", [1, 2, 4])

@@ -195,10 +195,12 @@ def test_dispatch_on_the_benchmark_layer_shapes():
         pytest.skip("device properties replace the defaults the expectations below were written for")
     from onnxruntime_amd.synthetic import C5_SHAPES
     want = {  # M -> kernel, whether the tile GEMM splits tiles along K
-        "qkv": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
+        # (qkv at M = 256: 48 slabs x 4 row blocks = 192 workgroups, one round: activations shared through LDS)
+        "qkv": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid_shared", 1), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
         # (o at M = 1024: 128 x 128 tiles, one per compute unit, instead of a cut along K)
         "o": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
-        "gate_up": {1: ("skinny", 0), 64: ("mid", 1), 256: ("gemm256", 0), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
+        # (gate+up at M = 64: 224 slabs of 128 columns, one round of workgroups: activations shared through LDS)
+        "gate_up": {1: ("skinny", 0), 64: ("mid_shared", 1), 256: ("gemm256", 0), 1024: ("gemm256", 0), 4096: ("gemm256", 0)},
         "down": {1: ("skinny", 0), 64: ("mid", 1), 256: ("mid", 1), 1024: ("gemm256", 1), 4096: ("gemm256", 0)},
     }
     for bits, bs in ((4, 128), (8, 64)):
