@@ -789,9 +789,13 @@ constexpr bool kBf16Has256Rows = !(HAS_ZP && MPS == 4);
 template <int BITS, bool HAS_ZP, int MPS, int DT, bool HAS_256 = true>
 hipError_t launch_rows(const Gemm256Params& p, unsigned grid, hipStream_t s) {
   if (p.tile_cols == 128) {
+#if defined(MNB_TUNING_HOOKS)
+    // calibration only: 64 x 128 tiles for 16 < M <= 256 measured no faster than the streaming kernel (one tile per
+    // workgroup leaves the k loop latency-bound: 29.5 us on M=64 N=28672 K=4096 against 25.5 us)
     if constexpr (DT == 0) {
       if (p.tile_rows == 64) return launch_wm<BITS, HAS_ZP, MPS, 1, 1, DT, 4>(p, grid, s);
     }
+#endif
     if constexpr (DT == 0 || DT == 1)
       return p.tile_rows == 128 ? launch_wm<BITS, HAS_ZP, MPS, 2, 1, DT, 4>(p, grid, s) : hipErrorInvalidValue;
     else
