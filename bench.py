@@ -144,6 +144,9 @@ def load_probe():
     lib.MnbProbeReadBandwidthResident.argtypes = lib.MnbProbeReadBandwidth.argtypes
     lib.MnbProbeMfmaRate.restype = ctypes.c_int
     lib.MnbProbeMfmaRate.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeIssueOverlap.restype = ctypes.c_int
+    lib.MnbProbeIssueOverlap.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                         ctypes.POINTER(ctypes.c_double)]
     lib.MnbProbeRelease.restype = None
     lib.MnbProbeRelease.argtypes = []
     return lib
@@ -389,7 +392,19 @@ def main() -> int:
             p4.a.copy_(a_saved)
             del a_saved
             tflops_zero = c4.flops() / (ms4_zero * 1e-3) / 1e12
+            # What the kernel's instruction mix costs with nothing else in the way: two wavefronts per SIMD, per matrix
+            # instruction two independent vector instructions (the dequantisation) and one 1 KB LDS read (its A
+            # operand: eight wavefronts x 1 KB per 32-cycle matrix instruction is the LDS's 128 bytes per clock).
+            slot = {}
+            for name, (valu, lds) in {"mfma_only": (0, 0), "mfma_2_vector": (2, 0), "mfma_lds_operand": (0, 2),
+                                      "mfma_2_vector_lds_operand": (2, 2)}.items():
+                assert probe.MnbProbeIssueOverlap(valu, 1, 2, lds, ctypes.byref(v)) == 0
+                slot[name] = v.value
             out["prefill"]["roofline"]["measured_ceiling"] = {
+                "issue_probe_ns_per_matrix_instruction_per_wavefront_two_per_simd": {k: round(x, 2)
+                                                                                    for k, x in slot.items()},
+                "issue_probe_instruction_mix_of_this_kernel_vs_mfma_only": round(
+                    slot["mfma_only"] / slot["mfma_2_vector_lds_operand"], 4),
                 "mfma_only_loop_constant_operands_TFLOPs": round(mfma_const, 1),
                 "mfma_only_loop_random_operands_TFLOPs": round(mfma_rand, 1),
                 "frac_of_mfma_only_random": round(tflops / mfma_rand, 4) if mfma_rand > 0 else None,

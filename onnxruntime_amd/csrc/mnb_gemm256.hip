@@ -241,6 +241,14 @@ __device__ __forceinline__ void slab_end() {
 // the matrix pipe idle while it issues its own vector instructions: 3217 cycles per k-step against 2460, 231.5 us
 // against 212.0 us on the same box although the power limit then allows 2.10 instead of 1.82 GHz; with the order inside a
 // slab section stated by hand (one matrix instruction, two vector instructions, one LDS read, one load) 244.7 us.
+// What bounds the 1 x 8 arrangement.  Every matrix instruction takes its A operand from LDS, 1 KB per wavefront: eight
+// wavefronts x 1 KB per 32-cycle instruction is 128 bytes per clock, all the LDS delivers, so LDS and matrix pipe are
+// saturated together and the dequantisation's vector instructions (two per matrix instruction), which the pipe alone
+// would hide, come on top.  A loop of nothing but that mix (mnb_probe.hip, two wavefronts per SIMD, constant
+// operands) needs 34.8 ns per matrix instruction and wavefront against 27.0 ns for matrix instructions alone, 28.0
+// with the vector instructions, 29.5 with the LDS reads: 1.24 x, and this kernel's k-step takes 2516 cycles against
+// the 2048 of its matrix instructions, 1.23 x.  Raising the priority of a wavefront around its matrix instructions
+// (s_setprio 1 or 3) costs 1.5 to 2 % on every shape.
 template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV, int CTW = WM>
 __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 : 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int THREADS = 64 * NWV;

@@ -18,6 +18,8 @@
 // into operand order in the caller's workspace, [chunk][word i][row tile][kq][j] in 16-byte units (zero-filled beyond
 // M and K, any alignment of the source), so that every operand load of a wavefront is 1 KiB contiguous.  The staged
 // copy is M x K halves (at most a few MB) and is re-read from L2 by every workgroup.
+#include <atomic>
+
 #include "mnb_mfma16_common.hip.h"
 
 namespace {
@@ -292,13 +294,20 @@ __global__ void __launch_bounds__(NW * 64) mnb_mid_kernel(const uint4* hot_W, in
 // LDS, compute, reload the weight registers for the round after next.  No staged copy of A, no staging launch.
 // Needs K a whole number of chunks and 16-byte aligned rows of A; everything else takes the kernel above.
 // Anatomy of a round (64 rows, N = 28672, K = 4096, 4-bit, time stamps of the shader clock in a calibration build):
-// the older wavefront of a SIMD needs 2800 cycles for its arithmetic (64 matrix instructions = 1024 cycles, 320
-// vector instructions = 1280 cycles: the two do not overlap), the younger one, which gets the issue slots the older
+// the older wavefront of a SIMD needs 2800 cycles for its arithmetic (64 matrix instructions, 1024 cycles of the matrix
+// pipe, and 320 vector instructions, 1280 issue cycles), the younger one, which gets the issue slots the older
 // leaves, 4250; then both wait about 1300 cycles for the fills they issued when the round began -- every workgroup
 // fills at the same moment, 22 MB per round chip-wide through level-2 caches that deliver about 11 TB/s, 2 us, against
 // 1.8 us of arithmetic.  A third buffer (fills two rounds ahead) does not fit the 160 KB of LDS, and would not lift
 // the bandwidth bound; the ablations agree: without the arithmetic the launch takes 16.0 us, without fills, operand
 // reads and arithmetic 10.9 us (the weights alone), all together 29.7 us.
+// Tried on top and not kept: dequantising the next operand between the matrix instructions of the current one (a
+// software pipeline inside mid_compute_chunk, also with the order forced by scheduling groups) -- bit-identical
+// results and the same times (+-1 %) on eight shapes of both kernels; cutting K into parts across workgroups for
+// matrices too narrow to fill the chip (fp32 partial tiles, an arrival counter per tile, the last workgroup to arrive
+// adds the parts in part order) -- correct, and slower than the kernel above on every narrow shape (N = 4096,
+// K = 14336, 64 rows: 27.5 against 19.7 us; K = 4096: 18.6 against 7.9 us), because a round costs 2.0 to 2.3 us
+// whatever the grid (the same with 32 workgroups as with 224) on top of about 8 us per launch.
 template <int BITS, bool HAS_ZP, int T, int MT, int KGS, int NG>
 __global__ void __launch_bounds__(KGS * NG * 64) mnb_mid_shared_kernel(const uint4* hot_W, int64_t hot_Npad,
                                                                         const _Float16* hot_A, const uint8_t* hot_meta,
@@ -556,10 +565,17 @@ hipError_t launch_shared_mt(const MidParams& mp, hipStream_t s) {
   constexpr size_t fills = 2 * KGS * chunk_bytes, red = (size_t)NW * T * 4 * 64 * sizeof(float);
   constexpr size_t smem = fills > red ? fills : red;
   auto kernel = mnb_mid_shared_kernel<BITS, HAS_ZP, T, MT, KGS, NG>;
-  if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-      e != hipSuccess)
-    return e;
+  // more than 64 KB of dynamic LDS has to be asked for, once per device (the attribute is kept per device)
+  static std::atomic<unsigned long long> asked{0};
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device >= 64 || !((asked.load(std::memory_order_relaxed) >> device) & 1ull)) {
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        e != hipSuccess)
+      return e;
+    if (device < 64) asked.fetch_or(1ull << device, std::memory_order_relaxed);
+  }
   const dim3 grid((unsigned)((p.N + 16 * T * NG - 1) / (16 * T * NG)), (unsigned)((p.M + 16 * MT - 1) / (16 * MT)));
   kernel<<<grid, dim3(NW * 64), smem, s>>>(p.W, p.Npad, p.A, p.meta, p.lda, p.chunks, p.bs_shift, mp);
   return hipGetLastError();

@@ -32,6 +32,14 @@ MNB_PROBE_API void MnbProbeRelease(void);
  * (random_operands = 0) or random fp16 operands (1): the sustained matrix-core clock depends on operand toggling. */
 MNB_PROBE_API int MnbProbeMfmaRate(int random_operands, double* tflops);
 
+/* Nanoseconds per "slot" of a loop that every wavefront of the chip runs (waves_per_simd = 1 or 2 wavefronts on each
+ * SIMD): a slot is one v_mfma_f32_32x32x16_f16 (when with_mfma) followed by valu_per_mfma (0, 1, 2, 4, 8) independent
+ * packed-fp16 multiply-adds; with lds_reads_per_two_mfma = 1 or 2 the matrix instruction's A operand comes from a
+ * 16-byte-per-lane LDS read issued two slots earlier (one read per matrix instruction, or one per two).  Comparing (mfma only), (vector only) and (both) tells whether the two kinds of
+ * instruction overlap on a SIMD or take turns. */
+MNB_PROBE_API int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int waves_per_simd,
+                                       int lds_reads_per_two_mfma, double* ns_per_slot);
+
 #ifdef __cplusplus
 }
 #endif

@@ -68,6 +68,55 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_mfma_kernel(float* out, int 
   out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
+// A loop of "slots": one v_mfma_f32_32x32x16_f16 (MFMA) followed by V packed-fp16 fused multiply-adds on registers
+// the matrix instruction does not touch, every instruction independent of its neighbours.  Timed with and without
+// either kind, it shows whether a SIMD overlaps the two or issues them one after the other.
+template <int V, bool MFMA, int LDS2>
+__global__ void __launch_bounds__(512, 2) mnb_probe_issue_kernel(float* out, int iters) {
+  __shared__ __align__(16) unsigned char tile[32768];
+  for (int i = threadIdx.x; i < 32768 / 16; i += blockDim.x)
+    reinterpret_cast<uint4*>(tile)[i] = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);  // ones
+  __syncthreads();
+  const int lane = threadIdx.x & 63;
+  h8_t fa[2];
+  f16_t acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+  h8_t a, b;
+  for (int i = 0; i < 8; ++i) a[i] = (_Float16)1.0f, b[i] = (_Float16)0.5f;
+  fa[0] = fa[1] = a;
+  typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+  h2v h[8];
+  for (int i = 0; i < 8; ++i) h[i] = h2v{(_Float16)(threadIdx.x & 7), (_Float16)i};
+  const h2v m = h2v{(_Float16)0.5f, (_Float16)0.25f}, c = h2v{(_Float16)1.0f, (_Float16)2.0f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // the operand of this slot was read from LDS two slots ago (16 bytes per lane, a different kilobyte each time)
+      if constexpr (MFMA) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(LDS2 ? fa[i & 1] : a, b, acc[i], 0, 0, 0);
+      if constexpr (LDS2 == 2 || (LDS2 == 1 && true))
+        if (LDS2 == 2 || (i & 1) == 0) {
+          fa[i & 1] = *reinterpret_cast<const h8_t*>(tile + ((it * 8 + i) & 31) * 1024 + lane * 16);
+        }
+#pragma unroll
+      for (int v = 0; v < V; ++v) h[(i * V + v) & 7] = h[(i * V + v) & 7] * m + c;
+      if constexpr (MFMA) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (LDS2 == 2 || (LDS2 == 1 && (i & 1) == 0)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      if constexpr (V > 0) __builtin_amdgcn_sched_group_barrier(0x002, V, 0);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    s += (float)h[i].x + (float)h[i].y;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[i][r];
+  }
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // Buffers of the read probe, kept between calls so that a sweep allocates once.
 std::vector<uint4*> g_bufs;
 size_t g_buf_vecs = 0;
@@ -190,6 +239,57 @@ hipError_t probe_mfma(int random_operands, double* tflops) {
   return err;
 }
 
+template <int V>
+void launch_issue(bool mfma, int lds2, int cus, int threads, float* out, int n) {
+  if (!mfma)
+    mnb_probe_issue_kernel<V, false, 0><<<cus, threads, 0, nullptr>>>(out, n);
+  else if (lds2 == 2)
+    mnb_probe_issue_kernel<V, true, 2><<<cus, threads, 0, nullptr>>>(out, n);
+  else if (lds2 == 1)
+    mnb_probe_issue_kernel<V, true, 1><<<cus, threads, 0, nullptr>>>(out, n);
+  else
+    mnb_probe_issue_kernel<V, true, 0><<<cus, threads, 0, nullptr>>>(out, n);
+}
+
+hipError_t probe_issue(int valu_per_mfma, int with_mfma, int waves_per_simd, int lds2, double* ns_per_slot) {
+  *ns_per_slot = 0.0;
+  int dev = 0, cus = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (err != hipSuccess) return err;
+  float* out = nullptr;
+  err = hipMalloc(&out, (size_t)cus * 512 * sizeof(float));
+  if (err != hipSuccess) return err;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  const int iters = 20000, threads = 256 * waves_per_simd;
+  auto launch = [&](int n) {
+    switch (valu_per_mfma) {
+      case 0: launch_issue<0>(with_mfma, lds2, cus, threads, out, n); break;
+      case 1: launch_issue<1>(with_mfma, lds2, cus, threads, out, n); break;
+      case 2: launch_issue<2>(with_mfma, lds2, cus, threads, out, n); break;
+      case 4: launch_issue<4>(with_mfma, lds2, cus, threads, out, n); break;
+      default: launch_issue<8>(with_mfma, lds2, cus, threads, out, n); break;
+    }
+  };
+  if ((err = hipEventCreate(&e0)) == hipSuccess && (err = hipEventCreate(&e1)) == hipSuccess) {
+    launch(iters);
+    if ((err = hipDeviceSynchronize()) == hipSuccess) {
+      (void)hipEventRecord(e0, nullptr);
+      launch(iters);
+      (void)hipEventRecord(e1, nullptr);
+      err = hipDeviceSynchronize();
+      float ms = 0.f;
+      if (err == hipSuccess && (err = hipEventElapsedTime(&ms, e0, e1)) == hipSuccess && ms > 0.f)
+        *ns_per_slot = (double)ms * 1e6 / ((double)iters * 8);
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(out);
+  return err;
+}
+
 }  // namespace
 
 extern "C" {
@@ -219,6 +319,17 @@ void MnbProbeRelease(void) { release_buffers(); }
 int MnbProbeMfmaRate(int random_operands, double* tflops) {
   if (!tflops) return 2;
   return probe_mfma(random_operands, tflops) == hipSuccess ? 0 : 1;
+}
+
+int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int waves_per_simd, int lds_reads_per_two_mfma,
+                         double* ns_per_slot) {
+  const bool v_ok = valu_per_mfma == 0 || valu_per_mfma == 1 || valu_per_mfma == 2 || valu_per_mfma == 4 ||
+                    valu_per_mfma == 8;
+  if (!ns_per_slot || !v_ok || (valu_per_mfma == 0 && !with_mfma) || (waves_per_simd != 1 && waves_per_simd != 2) ||
+      lds_reads_per_two_mfma < 0 || lds_reads_per_two_mfma > 2 || (lds_reads_per_two_mfma && !with_mfma))
+    return 2;
+  return probe_issue(valu_per_mfma, with_mfma, waves_per_simd, lds_reads_per_two_mfma, ns_per_slot) == hipSuccess ? 0
+                                                                                                                  : 1;
 }
 
 }  // extern "C"
