@@ -147,6 +147,8 @@ def load_probe():
     lib.MnbProbeIssueOverlap.restype = ctypes.c_int
     lib.MnbProbeIssueOverlap.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                          ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeDequantMfma16.restype = ctypes.c_int
+    lib.MnbProbeDequantMfma16.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     lib.MnbProbeRelease.restype = None
     lib.MnbProbeRelease.argtypes = []
     return lib
@@ -686,6 +688,14 @@ def sweep(torch, _lib, synthetic):
         del p
         torch.cuda.empty_cache()
 
+    # the streaming kernels' instruction mix on its own (two wavefronts per SIMD): per 32-bit word of 4-bit weights and
+    # column tile, 13 vector instructions make the operand and 4 matrix instructions (64 rows) use it
+    probe, v = load_probe(), ctypes.c_double(0.0)
+    for mode, what in enumerate(("4 matrix instructions alone", "13 vector instructions alone",
+                                 "operand made in front of its matrix instructions",
+                                 "next operand made between the matrix instructions")):
+        assert probe.MnbProbeDequantMfma16(mode, 2, ctypes.byref(v)) == 0
+        print(f"streaming mix probe: {v.value:6.2f} ns per step of two wavefronts on a SIMD, {what}", file=sys.stderr)
     one("C1 fp32 M=1 4096x4096 bs32 zp", synthetic.config_c1(), 16)
     for nm, (K, N) in synthetic.C3_SHAPES.items():
         for M in (1, 2, 4, 8, 16):

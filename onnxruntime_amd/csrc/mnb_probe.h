@@ -40,6 +40,13 @@ MNB_PROBE_API int MnbProbeMfmaRate(int random_operands, double* tflops);
 MNB_PROBE_API int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int waves_per_simd,
                                        int lds_reads_per_two_mfma, double* ns_per_slot);
 
+/* Nanoseconds per step of the streaming kernel's instruction mix, run by waves_per_simd (1 or 2) wavefronts on every
+ * SIMD: a step is 13 vector instructions that dequantise one 32-bit word of eight 4-bit weights into a matrix-core
+ * operand and four v_mfma_f32_16x16x32_f16 that use it.  mode 0: the matrix instructions alone; 1: the vector
+ * instructions alone; 2: the operand made right in front of its matrix instructions; 3: the next step's operand made
+ * between the matrix instructions of the current one. */
+MNB_PROBE_API int MnbProbeDequantMfma16(int mode, int waves_per_simd, double* ns_per_step);
+
 #ifdef __cplusplus
 }
 #endif

@@ -11,6 +11,7 @@
 
 #include <vector>
 
+#include "mnb_buffer.hip.h"
 #include "mnb_device.hip.h"
 
 namespace {
@@ -115,6 +116,80 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_issue_kernel(float* out, int
     for (int r = 0; r < 16; ++r) s += acc[i][r];
   }
   out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// The streaming kernel's instruction mix in isolation.  A step is what that kernel does per packed word and column
+// tile at 64 rows: 13 vector instructions turn a 32-bit word of eight 4-bit weights into the B operand (one shift,
+// four and-or, four packed adds, four packed multiplies), and four v_mfma_f32_16x16x32_f16 use it.
+// MODE 0: the matrix instructions alone; 1: the vector instructions alone; 2: operand made right in front of the
+// matrix instructions that read it; 3: the operand of the next step is made between the matrix instructions of this
+// one (order stated through scheduling groups).
+template <int MODE>
+__global__ void __launch_bounds__(512, 2) mnb_probe_dequant16_kernel(float* out, const uint32_t* words, int iters) {
+  typedef float f4v __attribute__((ext_vector_type(4)));
+  typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+  f4v acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = f4v{0.f, 0.f, 0.f, 0.f};
+  h8_t a[4];
+  for (int t = 0; t < 4; ++t)
+    for (int i = 0; i < 8; ++i) a[t][i] = (_Float16)1.0f;
+  uint32_t w = words[threadIdx.x & 63];  // (zero: keeps the arithmetic finite, and unknown to the compiler)
+  uint32_t mask_lo, mask_hi, magic_lo, magic_hi;
+  asm("s_mov_b32 %0, 0x000F000F" : "=s"(mask_lo));
+  asm("s_mov_b32 %0, 0x00F000F0" : "=s"(mask_hi));
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(magic_lo));
+  asm("v_mov_b32 %0, 0x54005400" : "=v"(magic_hi));
+  const h2v z_lo = h2v{(_Float16)-1032.0f, (_Float16)-1032.0f}, z_hi = h2v{(_Float16)-72.0f, (_Float16)-72.0f};
+  const h2v s2 = h2v{(_Float16)0.01f, (_Float16)0.01f};
+  auto as_h2 = [](uint32_t x) { return __builtin_bit_cast(h2v, x); };
+  auto as_u32 = [](h2v x) { return __builtin_bit_cast(uint32_t, x); };
+  auto make = [&](uint32_t word) {
+    const uint32_t w8 = word >> 8;
+    u4_t r;
+    r[0] = as_u32((as_h2((word & mask_lo) | magic_lo) + z_lo) * s2);
+    r[1] = as_u32((as_h2((word & mask_hi) | magic_hi) + z_hi) * s2);
+    r[2] = as_u32((as_h2((w8 & mask_lo) | magic_lo) + z_lo) * s2);
+    r[3] = as_u32((as_h2((w8 & mask_hi) | magic_hi) + z_hi) * s2);
+    return __builtin_bit_cast(h8_t, r);
+  };
+  h8_t b = make(w);
+  uint32_t sink = 0;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      w = w * 5u + 0x11111111u * (uint32_t)st;  // (one more vector instruction; the word changes from step to step)
+      if constexpr (MODE == 1) {
+        const h8_t nb = make(w);
+        sink ^= __builtin_bit_cast(u4_t, nb)[0] ^ __builtin_bit_cast(u4_t, nb)[3];
+      } else if constexpr (MODE == 0) {
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          acc[st * 4 + mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], b, acc[st * 4 + mt], 0, 0, 0);
+      } else if constexpr (MODE == 2) {
+        b = make(w);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          acc[st * 4 + mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], b, acc[st * 4 + mt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+        const h8_t nb = make(w);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          acc[st * 4 + mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[mt], b, acc[st * 4 + mt], 0, 0, 0);
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        }
+        b = nb;
+      }
+    }
+  }
+  float s = (float)sink;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s + (float)b[0];
 }
 
 // Buffers of the read probe, kept between calls so that a sweep allocates once.
@@ -290,6 +365,50 @@ hipError_t probe_issue(int valu_per_mfma, int with_mfma, int waves_per_simd, int
   return err;
 }
 
+hipError_t probe_dequant16(int mode, int waves_per_simd, double* ns_per_step) {
+  *ns_per_step = 0.0;
+  int dev = 0, cus = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (err != hipSuccess) return err;
+  float* out = nullptr;
+  uint32_t* words = nullptr;
+  if ((err = hipMalloc(&out, (size_t)cus * 512 * sizeof(float))) != hipSuccess) return err;
+  if ((err = hipMalloc(&words, 64 * sizeof(uint32_t))) != hipSuccess || (err = hipMemset(words, 0, 256)) != hipSuccess) {
+    (void)hipFree(out);
+    if (words) (void)hipFree(words);
+    return err;
+  }
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  const int iters = 40000, threads = 256 * waves_per_simd;
+  auto launch = [&](int n) {
+    switch (mode) {
+      case 0: mnb_probe_dequant16_kernel<0><<<cus, threads, 0, nullptr>>>(out, words, n); break;
+      case 1: mnb_probe_dequant16_kernel<1><<<cus, threads, 0, nullptr>>>(out, words, n); break;
+      case 2: mnb_probe_dequant16_kernel<2><<<cus, threads, 0, nullptr>>>(out, words, n); break;
+      default: mnb_probe_dequant16_kernel<3><<<cus, threads, 0, nullptr>>>(out, words, n); break;
+    }
+  };
+  if ((err = hipEventCreate(&e0)) == hipSuccess && (err = hipEventCreate(&e1)) == hipSuccess) {
+    launch(iters);
+    if ((err = hipDeviceSynchronize()) == hipSuccess) {
+      (void)hipEventRecord(e0, nullptr);
+      launch(iters);
+      (void)hipEventRecord(e1, nullptr);
+      err = hipDeviceSynchronize();
+      float ms = 0.f;
+      if (err == hipSuccess && (err = hipEventElapsedTime(&ms, e0, e1)) == hipSuccess && ms > 0.f)
+        *ns_per_step = (double)ms * 1e6 / ((double)iters * 4);
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  (void)hipFree(out);
+  (void)hipFree(words);
+  return err;
+}
+
 }  // namespace
 
 extern "C" {
@@ -330,6 +449,11 @@ int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int waves_per_simd, i
     return 2;
   return probe_issue(valu_per_mfma, with_mfma, waves_per_simd, lds_reads_per_two_mfma, ns_per_slot) == hipSuccess ? 0
                                                                                                                   : 1;
+}
+
+int MnbProbeDequantMfma16(int mode, int waves_per_simd, double* ns_per_step) {
+  if (!ns_per_step || mode < 0 || mode > 3 || (waves_per_simd != 1 && waves_per_simd != 2)) return 2;
+  return probe_dequant16(mode, waves_per_simd, ns_per_step) == hipSuccess ? 0 : 1;
 }
 
 }  // extern "C"
