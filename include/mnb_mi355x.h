@@ -252,6 +252,17 @@ MNB_API int MnbSimplifiedLayerNorm(size_t M, size_t K, int a_dtype, const void* 
  *                    provider has no bfloat16 kernel.  The tile GEMM reads activations in place when they are 16-byte
  *                    aligned with a pitch that is a multiple of 8 and there is no g_idx, else from a copy in the
  *                    workspace; the other two take any alignment.
+ *                    One exception, with different (tighter) arithmetic: 4-bit weights in blocks of 128 and more on
+ *                    the decode kernel (M <= 16).  There no weight is narrowed to the activation type.  The matrix
+ *                    instruction multiplies the activations by the raw operand r = c + q, which is exact in the
+ *                    activation type (bfloat16: c = 128; float16: c = 1024, or 64 for the nibbles taken from bits
+ *                    4..7), two more matrix instructions per block against constant operands give S_c = sum(c * a) and
+ *                    S_1 = sum(a), and the block contributes  scale * (sum(a * r) - S_c - zp * S_1)  with every sum, the
+ *                    scale and the zero point in fp32 (scale and zp are the unrounded fp32 meta entries).  The result
+ *                    differs from the formula above by the weight rounding that formula contains and this one does
+ *                    not (relative L2 against float64: 1.7e-3 against 2.2e-3 for bfloat16, both dominated by the
+ *                    narrowing of Y), so the same model rounds slightly differently at M <= 16 than at M > 16; both
+ *                    are inside the operator's tolerance, and the reference holds no bfloat16 vectors to pin either.
  * Zero points are honoured together with g_idx for both zero-point types, as the schema defines; the reference's CPU
  * dequantiser reads uint8 zero points in that combination but then uses 8 (matmul_nbits_impl.cc:56-66).
  * Supported: g_idx with bits = 4; typed zero points with bits = 2 or 4 (the reference rejects 8, :1251-1252). */
