@@ -214,7 +214,8 @@ def test_decode_with_more_slabs_than_compute_units(oracle, bits, bs, zp, N, K, M
 
 @pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (4, 16, True), (8, 64, True), (8, 16, False)])
 @pytest.mark.parametrize("N,K,M", [(28672, 1024, 64), (21000, 1024, 17), (28672, 2048, 32), (24000, 1024, 33),
-                                   (11008, 1024, 100), (14336, 1024, 128), (6144, 1024, 250)])
+                                   (11008, 1024, 100), (14336, 1024, 128), (6144, 1024, 250),
+                                   (28672, 1152, 64), (21000, 1408, 40)])   # K: 9 and 11 chunks of 128
 def test_streaming_kernel_with_activations_shared_through_lds(oracle, bits, bs, zp, N, K, M):
     """Wide matrices whose 128-column slabs make one well-filled round of workgroups: pairs of wavefronts share each
     chunk of the activations through LDS (fetched straight from the caller's A, no staged copy).  Every row of Y against
@@ -233,8 +234,13 @@ def test_streaming_kernel_with_activations_shared_through_lds(oracle, bits, bs, 
     c0 = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + M)
     w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
     assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
-    # rows that are not 16-byte aligned: the staged route
+    # a pitch beyond K that keeps the rows 16-byte aligned: still read in place, the same bits
     op = make_op(c)
+    pitched = torch.zeros(M, K + 8, dtype=torch.float16, device="cuda")
+    pitched[:, :K] = dev(c.A)
+    y1 = op.Compute(pitched[:, :K], bias=dev(c.bias)).cpu().numpy()
+    assert np.array_equal(_bits_view(y1), _bits_view(y))
+    # rows that are not 16-byte aligned: the staged route
     wide = torch.zeros(M, K + 3, dtype=torch.float16, device="cuda")
     wide[:, :K] = dev(c.A)
     y2 = op.Compute(wide[:, :K], bias=dev(c.bias)).cpu().numpy()
