@@ -36,7 +36,7 @@ PROFILED_TRAFFIC_BYTES = {"c2_decode": int((14858.5 * 2.0 + 28.0) * 1024), "c4_p
 # (standalone MLAS build, SQNBIT_CompFp32, N sliced over 8 threads): quoted beside the port so that the port's
 # figure is not read as the reference's.
 REFERENCE_MLAS_US_SURVEY = {"us_per_call": 1353.0, "threads": 8, "algorithmic_GBs": 23.1,
-                            "source": "BASELINE.md section 2 (survey container, not this host)"}
+                            "source": "the baseline survey of the reference (its container, not this host)"}
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published (no sparsity)
 LAYERS = 32
