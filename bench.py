@@ -394,9 +394,9 @@ def main() -> int:
             p4.a.copy_(a_saved)
             del a_saved
             tflops_zero = c4.flops() / (ms4_zero * 1e-3) / 1e12
-            # What the kernel's instruction mix costs with nothing else in the way: two wavefronts per SIMD, per matrix
-            # instruction two independent vector instructions (the dequantisation) and one 1 KB LDS read (its A
-            # operand: eight wavefronts x 1 KB per 32-cycle matrix instruction is the LDS's 128 bytes per clock).
+            # What the kernel's instruction mix costs in issue slots, with nothing else in the way: two wavefronts per
+            # SIMD, per matrix instruction two independent vector instructions (the dequantisation) and one 1 KB LDS
+            # read (its A operand), issued a whole loop iteration ahead of its use; constant operands.
             slot = {}
             for name, (valu, lds) in {"mfma_only": (0, 0), "mfma_2_vector": (2, 0), "mfma_lds_operand": (0, 2),
                                       "mfma_2_vector_lds_operand": (2, 2)}.items():

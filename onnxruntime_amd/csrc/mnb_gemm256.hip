@@ -217,8 +217,17 @@ __device__ __forceinline__ h8_t dequant_word(uint32_t w0, uint32_t w1, const Unp
 // a hand-written order of "one MFMA, one LDS read, two loads, n VALU" per matrix instruction (measured: 1-2 % on every
 // shape).  A fence between sections keeps it from pulling the next slab's work forward, which pays everywhere (1-4 %)
 // except in the 256-row 4-bit kernel, where letting it mix the sections of a k-step is worth another 2 %.
-template <bool FENCE>
+template <bool FENCE, int INTERLEAVE = 0>
 __device__ __forceinline__ void slab_end() {
+  // INTERLEAVE matrix instructions, each followed by up to three vector instructions (one wavefront per SIMD: the
+  // dequantisation of the next slab has to sit between this slab's matrix instructions, nobody else fills the gaps)
+  if constexpr (INTERLEAVE > 0) {
+#pragma unroll
+    for (int k = 0; k < INTERLEAVE; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+    }
+  }
   if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -241,14 +250,21 @@ __device__ __forceinline__ void slab_end() {
 // the matrix pipe idle while it issues its own vector instructions: 3217 cycles per k-step against 2460, 231.5 us
 // against 212.0 us on the same box although the power limit then allows 2.10 instead of 1.82 GHz; with the order inside a
 // slab section stated by hand (one matrix instruction, two vector instructions, one LDS read, one load) 244.7 us.
-// What bounds the 1 x 8 arrangement.  Every matrix instruction takes its A operand from LDS, 1 KB per wavefront: eight
-// wavefronts x 1 KB per 32-cycle instruction is 128 bytes per clock, all the LDS delivers, so LDS and matrix pipe are
-// saturated together and the dequantisation's vector instructions (two per matrix instruction), which the pipe alone
-// would hide, come on top.  A loop of nothing but that mix (mnb_probe.hip, two wavefronts per SIMD, constant
-// operands) needs 34.8 ns per matrix instruction and wavefront against 27.0 ns for matrix instructions alone, 28.0
-// with the vector instructions, 29.5 with the LDS reads: 1.24 x, and this kernel's k-step takes 2516 cycles against
-// the 2048 of its matrix instructions, 1.23 x.  Raising the priority of a wavefront around its matrix instructions
-// (s_setprio 1 or 3) costs 1.5 to 2 % on every shape.
+// With the LDS reads of the next slab pinned to the head of each slab section and the dequantisation placed between
+// the matrix instructions by scheduling groups (what a wavefront that is alone on its SIMD needs; both apply to this
+// arrangement only) 1 x 4 comes to 229.3 against 210.9 us: 481 K against 389 K cycles per launch, 45 % of a
+// wavefront's cycles still spent in waits.
+// What bounds the launch is energy, not issue slots.  A loop of nothing but the kernel's mix (mnb_probe.hip: per
+// matrix instruction two vector instructions and one 1 KB LDS operand read issued a whole iteration ahead, two
+// wavefronts per SIMD, constant operands) runs at 29.0 ns per matrix instruction and wavefront against 27.05 ns for
+// the matrix instructions alone: the mix costs 7 % of the issue slots.  Ablation builds of this kernel on C4 (results
+// wrong on purpose) keep its cycle count and change its clock: complete 385 K cycles per launch in 208.7 us
+// (1.85 GHz); without the LDS operand reads 378 K in 186.2 us (2.03 GHz); without the dequantisation arithmetic
+// 382 K in 180.0 us (2.12 GHz); without both 361 K in 154.0 us (2.35 GHz, the time the complete kernel needs on
+// all-zero activations); without the step's barrier 372 K in 206.9 us.  The matrix cores on random fp16 operands
+// take most of the power budget; every LDS read and vector instruction beside them is paid for in clock.
+// Raising the priority of a wavefront around its matrix instructions (s_setprio 1 or 3) costs 1.5 to 2 % on every
+// shape.
 template <int BITS, bool HAS_ZP, int MPS, int TM, int WM, int DT, int NWV, int CTW = WM>
 __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 : 2) mnb_gemm256_kernel(Gemm256Params p) {
   constexpr int THREADS = 64 * NWV;
@@ -410,10 +426,15 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
         }
         FB[j] = dequant_word_wide<BITS, DT == 1>(w0, w1, sc, -zp * sc);
       } else {
+#if defined(MNB_ABLATE_NO_DEQUANT)  // (calibration builds: the packed bits go to the matrix cores as they are)
+        const u4_t raw = {w0, w1, (uint32_t)R.m[e][j], w0};
+        FB[j] = __builtin_bit_cast(h8_t, raw);
+#else
         h2_t s2;
         ZpH z;
         decode(R.m[e][j], j, s2, z);
         FB[j] = dequant_word<BITS>(w0, w1, uc, z, s2);
+#endif
       }
     }
   };
@@ -427,6 +448,11 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
     a_rd[kk] = (uint32_t)((wm * 32 * RT + li) * ROW_BYTES + ((chunk ^ ((li >> 1) & 7)) * 16));
   }
   auto read_a = [&](int stage_off, int kk, h8_t* FA) {
+#if defined(MNB_ABLATE_NO_LDS_READS)  // (calibration builds: the A operands keep whatever the registers hold)
+#pragma unroll
+    for (int t = 0; t < RT; ++t) asm volatile("; keep %0" : "+v"(FA[t]));
+    return;
+#endif
     const unsigned char* As = lds_bytes + stage_off + a_rd[kk];
 #pragma unroll
     for (int t = 0; t < RT; ++t) FA[t] = *reinterpret_cast<const h8_t*>(As + t * 32 * ROW_BYTES);
@@ -450,29 +476,38 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
   // One k-step.  On entry: the staged tile at `cur` holds A of step ks, the one at `nxt` is receiving A of step ks+1,
   // the one at `nn` is free (its readers passed the barrier of step ks-1); FA0/FB0 hold the operands of slab 0, Rc
   // holds the weights of step ks, Rn holds (or is receiving) those of step ks+1.
+  // One wavefront per SIMD (four wavefronts) has nobody to hide an LDS wait behind: the reads of the next slab's A
+  // operands stay where they are written, at the head of the section, a slab ahead of their use (left alone the
+  // scheduler sinks them to just in front of it to save registers).
+  auto reads_stay_here = [] {
+    if constexpr (NWV == 4 && CTW == 2) __builtin_amdgcn_sched_barrier(0);
+  };
   auto k_step = [&](int ks, Stage& Rc, Stage& Rn, int cur, int nxt, int nn) {
     // slab 0: operands of slab 1; A of step ks+2 on its way into the free tile
     load_a(ks + 2, nn);
     read_a(cur, 1, FA1);
+    reads_stay_here();
     if constexpr (Plan::slab_waits(1)) await_b(Slab<1>{}, Rc);
     make_b(1, Rc, FB1);
     mfma_slab(FA0, FB0);
     load_b_slot(ks + 2, Rc, 1);
-    slab_end<SLAB_FENCE>();
+    slab_end<SLAB_FENCE || (NWV == 4 && CTW == 2), (NWV == 4 && CTW == 2) ? RT * CT : 0>();
     // slab 1: operands of slab 2
     read_a(cur, 2, FA0);
+    reads_stay_here();
     if constexpr (Plan::slab_waits(2)) await_b(Slab<2>{}, Rc);
     make_b(2, Rc, FB0);
     mfma_slab(FA1, FB1);
     load_b_slot(ks + 2, Rc, 2);
-    slab_end<SLAB_FENCE>();
+    slab_end<SLAB_FENCE || (NWV == 4 && CTW == 2), (NWV == 4 && CTW == 2) ? RT * CT : 0>();
     // slab 2: operands of slab 3
     read_a(cur, 3, FA1);
+    reads_stay_here();
     if constexpr (Plan::slab_waits(3)) await_b(Slab<3>{}, Rc);
     make_b(3, Rc, FB1);
     mfma_slab(FA0, FB0);
     load_b_slot(ks + 2, Rc, 3);
-    slab_end<SLAB_FENCE>();
+    slab_end<SLAB_FENCE || (NWV == 4 && CTW == 2), (NWV == 4 && CTW == 2) ? RT * CT : 0>();
     // The barrier of the step.  Before it a wavefront makes sure that its own part of A of step ks+1 has landed in
     // LDS (issued in slab 0 of step ks-1) and that the weights of slab 0 of step ks+1 are there; LoadPlan counts the
     // operations younger than both.  The wavefront's LDS reads have completed too, so the tile at `cur` may be
@@ -481,16 +516,19 @@ __global__ void __launch_bounds__(64 * NWV, (2 * TM / WM) * CTW * 16 > 128 ? 1 :
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt(waitcnt_vm_lds0(Plan::wait_of_barrier()));
+#if !defined(MNB_ABLATE_NO_BARRIER)  // (calibration builds: what the step's barrier costs; results are then wrong)
     __builtin_amdgcn_s_barrier();
+#endif
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     // slab 3, behind the barrier: operands of slab 0 of step ks+1
     read_a(nxt, 0, FA0);
+    reads_stay_here();
     await_b(Slab<0>{}, Rn);
     make_b(0, Rn, FB0);
     mfma_slab(FA1, FB1);
     load_b_slot(ks + 3, Rn, 4);
-    slab_end<SLAB_FENCE>();
+    slab_end<SLAB_FENCE || (NWV == 4 && CTW == 2), (NWV == 4 && CTW == 2) ? RT * CT : 0>();
   };
 
   // bias and output in the model's 16-bit type (the pointers are typed _Float16 for both: bfloat16 travels as bits)

@@ -79,7 +79,7 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_issue_kernel(float* out, int
     reinterpret_cast<uint4*>(tile)[i] = make_uint4(0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u);  // ones
   __syncthreads();
   const int lane = threadIdx.x & 63;
-  h8_t fa[2];
+  h8_t fa[8];
   f16_t acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -87,7 +87,8 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_issue_kernel(float* out, int
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
   h8_t a, b;
   for (int i = 0; i < 8; ++i) a[i] = (_Float16)1.0f, b[i] = (_Float16)0.5f;
-  fa[0] = fa[1] = a;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) fa[i] = a;
   typedef _Float16 h2v __attribute__((ext_vector_type(2)));
   h2v h[8];
   for (int i = 0; i < 8; ++i) h[i] = h2v{(_Float16)(threadIdx.x & 7), (_Float16)i};
@@ -95,12 +96,12 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_issue_kernel(float* out, int
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      // the operand of this slot was read from LDS two slots ago (16 bytes per lane, a different kilobyte each time)
-      if constexpr (MFMA) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(LDS2 ? fa[i & 1] : a, b, acc[i], 0, 0, 0);
-      if constexpr (LDS2 == 2 || (LDS2 == 1 && true))
-        if (LDS2 == 2 || (i & 1) == 0) {
-          fa[i & 1] = *reinterpret_cast<const h8_t*>(tile + ((it * 8 + i) & 31) * 1024 + lane * 16);
-        }
+      // the operand of this slot was read from LDS eight slots ago, into a register set of its own (16 bytes per
+      // lane, a different kilobyte each time): the reads have a whole iteration to land
+      if constexpr (MFMA) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(LDS2 ? fa[i] : a, b, acc[i], 0, 0, 0);
+      if constexpr (LDS2 != 0)
+        if (LDS2 == 2 || (i & 1) == 0)
+          fa[i] = *reinterpret_cast<const h8_t*>(tile + ((it * 8 + i) & 31) * 1024 + lane * 16);
 #pragma unroll
       for (int v = 0; v < V; ++v) h[(i * V + v) & 7] = h[(i * V + v) & 7] * m + c;
       if constexpr (MFMA) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
