@@ -110,3 +110,27 @@ def test_random_fused_projections(oracle, seed):
     if want_sum:
         sm = out[-1].cpu().numpy()
         assert np.array_equal(sm, (A.astype(np.float32) + np.resize(skip.astype(np.float32), A.shape)).astype(dtype))
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_wide_matrices(oracle, seed):
+    """Wide fp16 matrices with more than sixteen rows: the widths at which the streaming kernel shares the activations
+    through LDS, at which the tile GEMM runs 128- and 256-row tiles or cuts tiles along K, and the ragged widths
+    between them.  A random sample of rows against the oracle (rows are independent)."""
+    rng = np.random.default_rng(9000 + seed)
+    bits = int(rng.choice([4, 4, 8, 2]))
+    bs = int(rng.choice([32, 64, 128]))
+    M = int(rng.choice([17, 31, 33, 64, 65, 100, 129, 257, 600]))
+    N = int(rng.integers(4500, 30000))
+    if rng.random() < 0.4:
+        N = (N // 128) * 128
+    K = int(rng.choice([1024, 1152, 1408, 2048, 2080, 4096]))
+    zp, bias = bool(rng.random() < 0.5), bool(rng.random() < 0.5)
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=bias, seed=seed)
+    op = MatMulNBits(K, N, bits, bs, dtype=torch.float16, has_zero_points=zp, has_bias=bias)
+    assert op.PrePack(dev(c.B), dev(c.scales), dev(c.zero_points))
+    a = _strided_activation(rng, c.A) if rng.random() < 0.5 else dev(c.A)
+    y = op.Compute(a, bias=dev(c.bias))
+    torch.cuda.synchronize()
+    rows = np.sort(rng.choice(M, size=min(M, 24), replace=False))
+    check_against_oracle(oracle, c, y.cpu().numpy()[rows], A=c.A[rows])
