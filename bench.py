@@ -149,6 +149,10 @@ def load_probe():
                                          ctypes.POINTER(ctypes.c_double)]
     lib.MnbProbeDequantMfma16.restype = ctypes.c_int
     lib.MnbProbeDequantMfma16.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeShaderClockStart.restype = ctypes.c_int
+    lib.MnbProbeShaderClockStart.argtypes = [ctypes.c_double]
+    lib.MnbProbeShaderClockFinish.restype = ctypes.c_int
+    lib.MnbProbeShaderClockFinish.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     lib.MnbProbeRelease.restype = None
     lib.MnbProbeRelease.argtypes = []
     return lib
@@ -391,9 +395,24 @@ def main() -> int:
             a_saved = p4.a.clone()
             p4.a.zero_()
             ms4_zero = time_steps(torch, p4.step, k4, max(1, args.warmup // 2), warm_ms=30.0) / 2
-            p4.a.copy_(a_saved)
-            del a_saved
             tflops_zero = c4.flops() / (ms4_zero * 1e-3) / 1e12
+
+            def clock_during(run_step, steps):
+                """GHz of the shader clock while `steps` steps run: a single wavefront on a stream of its own compares
+                the shader clock's cycle counter with the constant 100 MHz counter for 12 ms (chip already warm)."""
+                ghz, sampled = ctypes.c_double(0.0), ctypes.c_double(0.0)
+                assert probe.MnbProbeShaderClockStart(12.0) == 0
+                for _ in range(steps):
+                    run_step()
+                torch.cuda.synchronize()
+                assert probe.MnbProbeShaderClockFinish(ctypes.byref(ghz), ctypes.byref(sampled)) == 0
+                return round(ghz.value, 3)
+
+            p4.a.zero_()
+            clock_zero = clock_during(p4.step, k4)
+            p4.a.copy_(a_saved)
+            clock_random = clock_during(p4.step, k4)
+            del a_saved
             # What the kernel's instruction mix costs in issue slots, with nothing else in the way: two wavefronts per
             # SIMD, per matrix instruction two independent vector instructions (the dequantisation) and one 1 KB LDS
             # read (its A operand), issued a whole loop iteration ahead of its use; constant operands.
@@ -412,6 +431,8 @@ def main() -> int:
                 "frac_of_mfma_only_random": round(tflops / mfma_rand, 4) if mfma_rand > 0 else None,
                 "same_kernel_zero_activations_TFLOPs": round(tflops_zero, 1),
                 "same_kernel_zero_activations_ms_per_launch": round(ms4_zero, 4),
+                "shader_clock_ghz_during_these_launches": clock_random,
+                "shader_clock_ghz_during_the_zero_activation_launches": clock_zero,
             }
         del p4
         torch.cuda.empty_cache()

@@ -47,6 +47,13 @@ MNB_PROBE_API int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int wav
  * between the matrix instructions of the current one. */
 MNB_PROBE_API int MnbProbeDequantMfma16(int mode, int waves_per_simd, double* ns_per_step);
 
+/* The clock the shader engines run at while other work is on the chip: Start launches a single wavefront on a stream
+ * of its own that watches the shader clock's cycle counter against the constant 100 MHz counter for sample_ms
+ * milliseconds and returns at once; Finish waits for it and gives the ratio in GHz and the time actually sampled.
+ * Launch the kernels to be observed between the two calls. */
+MNB_PROBE_API int MnbProbeShaderClockStart(double sample_ms);
+MNB_PROBE_API int MnbProbeShaderClockFinish(double* ghz, double* sampled_ms);
+
 #ifdef __cplusplus
 }
 #endif

@@ -193,6 +193,22 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_dequant16_kernel(float* out,
   out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = s + (float)b[0];
 }
 
+// One wavefront that watches two counters for a while: the shader clock's cycle counter and the constant 100 MHz
+// counter.  Their ratio is the clock the chip runs at while other kernels are busy on it.
+__global__ void __launch_bounds__(64) mnb_probe_clock_kernel(unsigned long long* out, unsigned long long ticks) {
+  if (threadIdx.x != 0) return;
+  const unsigned long long r0 = __builtin_amdgcn_s_memrealtime(), c0 = __builtin_amdgcn_s_memtime();
+  unsigned long long r1 = r0;
+  for (int spins = 0; spins < (1 << 22) && r1 - r0 < ticks; ++spins) {  // bounded whatever the counters do
+    __builtin_amdgcn_s_sleep(64);
+    r1 = __builtin_amdgcn_s_memrealtime();
+  }
+  const unsigned long long c1 = __builtin_amdgcn_s_memtime();
+  r1 = __builtin_amdgcn_s_memrealtime();
+  out[0] = c1 - c0;
+  out[1] = r1 - r0;
+}
+
 // Buffers of the read probe, kept between calls so that a sweep allocates once.
 std::vector<uint4*> g_bufs;
 size_t g_buf_vecs = 0;
@@ -410,6 +426,33 @@ hipError_t probe_dequant16(int mode, int waves_per_simd, double* ns_per_step) {
   return err;
 }
 
+// state of a running clock sample
+hipStream_t g_clock_stream = nullptr;
+unsigned long long* g_clock_out = nullptr;
+
+hipError_t clock_start(double sample_ms) {
+  hipError_t err = hipSuccess;
+  if (!g_clock_stream && (err = hipStreamCreateWithFlags(&g_clock_stream, hipStreamNonBlocking)) != hipSuccess) return err;
+  if (!g_clock_out && (err = hipMalloc(&g_clock_out, 2 * sizeof(unsigned long long))) != hipSuccess) return err;
+  mnb_probe_clock_kernel<<<1, 64, 0, g_clock_stream>>>(g_clock_out, (unsigned long long)(sample_ms * 1e5));
+  return hipGetLastError();
+}
+
+hipError_t clock_finish(double* ghz, double* sampled_ms) {
+  *ghz = 0.0;
+  *sampled_ms = 0.0;
+  if (!g_clock_stream || !g_clock_out) return hipErrorNotReady;
+  hipError_t err = hipStreamSynchronize(g_clock_stream);
+  if (err != hipSuccess) return err;
+  unsigned long long v[2] = {0, 0};
+  if ((err = hipMemcpy(v, g_clock_out, sizeof(v), hipMemcpyDeviceToHost)) != hipSuccess) return err;
+  if (v[1] > 0) {
+    *ghz = (double)v[0] / (double)v[1] * 0.1;  // cycles per 10 ns tick
+    *sampled_ms = (double)v[1] * 1e-5;
+  }
+  return hipSuccess;
+}
+
 }  // namespace
 
 extern "C" {
@@ -455,6 +498,16 @@ int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int waves_per_simd, i
 int MnbProbeDequantMfma16(int mode, int waves_per_simd, double* ns_per_step) {
   if (!ns_per_step || mode < 0 || mode > 3 || (waves_per_simd != 1 && waves_per_simd != 2)) return 2;
   return probe_dequant16(mode, waves_per_simd, ns_per_step) == hipSuccess ? 0 : 1;
+}
+
+int MnbProbeShaderClockStart(double sample_ms) {
+  if (!(sample_ms > 0.0) || sample_ms > 1000.0) return 2;
+  return clock_start(sample_ms) == hipSuccess ? 0 : 1;
+}
+
+int MnbProbeShaderClockFinish(double* ghz, double* sampled_ms) {
+  if (!ghz || !sampled_ms) return 2;
+  return clock_finish(ghz, sampled_ms) == hipSuccess ? 0 : 1;
 }
 
 }  // extern "C"
