@@ -527,15 +527,18 @@ def main() -> int:
     # ---- the same decode kernel on larger matrices: how the fixed part of a launch weighs against its size ----------
     if not args.no_sizes:
         rows = []
-        for label, bits, bs in (("gate+up int4 bs128 zp", 4, 128), ("gate+up int8 bs64 zp", 8, 64)):
-            K5, N5 = synthetic.C5_SHAPES["gate_up"]
+        # (the 2-bit rows stream the copy of the weights in their own width: half the bytes of the 4-bit rows)
+        for label, bits, bs, shape in (("gate+up int4 bs128 zp", 4, 128, "gate_up"), ("gate+up int8 bs64 zp", 8, 64, "gate_up"),
+                                       ("gate+up int2 bs128 zp", 2, 128, "gate_up"),
+                                       ("configs[1] shape as int2 bs128 zp", 2, 128, None)):
+            K5, N5 = synthetic.C5_SHAPES[shape] if shape else (c2.K, c2.N)
             case = synthetic.make_case(1, N5, K5, bits, bs, np.float16, has_zp=True, seed=0)
-            copies = 8  # 8 x 60 / 123 MB of distinct weights: beyond the Infinity Cache
+            copies = 8 if shape else 32  # distinct weights beyond the 256 MB Infinity Cache
             p5 = Problem(case, copies, torch, _lib)
             g5 = graph_of(torch, p5.step)
             us5 = time_steps(torch, g5.replay, max(4, args.steps // 2), 2) / copies * 1e3
             gb5 = case.algorithmic_bytes() / (us5 * 1e-6) / 1e9
-            rows.append({"workload": f"BASELINE configs[4] M=1 K={K5} N={N5} {label} fp16", "kernel": p5.kernel,
+            rows.append({"workload": f"{'BASELINE configs[4] ' if shape else ''}M=1 K={K5} N={N5} {label} fp16", "kernel": p5.kernel,
                          "algorithmic_bytes_per_launch": case.algorithmic_bytes(), "us_per_launch": round(us5, 3),
                          "value": round(gb5, 1), "unit": "GB/s", "frac_of_hbm_peak": round(gb5 / HBM_PEAK_GBS, 4)})
             del g5, p5

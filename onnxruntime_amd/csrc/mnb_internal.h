@@ -72,6 +72,7 @@ bool mnb_rows16_f32_applicable(const MnbGemmArgs& a);
 hipError_t mnb_launch_rows16_f32(const MnbGemmArgs& a, hipStream_t s);
 size_t mnb_mid_workspace_bytes(const MnbLayout& L, int64_t M);  // staged copy of A
 bool mnb_mid_direct(const MnbGemmArgs& a);  // this call reads A in place: no staged copy, no workspace
+bool mnb_skinny_native2(const MnbGemmArgs& a);  // a decode call that streams the native copy of 2-bit weights
 bool mnb_mid_shared(const MnbGemmArgs& a);  // ... through the variant whose wavefront pairs share the activations in LDS
 // 16 < M: whether the tile GEMM's plan beats the streaming kernel's estimate for this shape (needs K % 128 == 0)
 bool mnb_prefer_gemm256(const MnbLayout& L, int64_t M);

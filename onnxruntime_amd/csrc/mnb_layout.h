@@ -15,6 +15,17 @@
 //                             order (n%16)*4 + (n%64)/16, so that the four 16-column tiles a matrix-core lane
 //                             works on are adjacent and arrive with one vector load (mnb_meta_col).
 //
+//   W2  [Kpad/64][Npad][16 B] 2-bit sources of fp16 models with blocks of 64 and more only, behind everything else: the
+//                             weights once more in their own width for the decode kernel (M <= 16 streams half the
+//                             bytes).  One 16-byte vector = 64 k of one column, the operands of eight matrix
+//                             instructions: vector 4 c + kq holds, as operand i, k = 256 c + 128 (i / 4) + 32 kq +
+//                             8 (i % 4) .. + 7 (mnb_w2_k), so that every matrix instruction of a wavefront -- it sums
+//                             over the four kq -- stays inside one block of 128; inside every 32-bit word
+//                             the fields of elements e0..e15 are stored e0 e2 .. e14 in the low half and e1 e3 .. e15
+//                             in the high half (LSB first), so that (w & 0x00030003), (w & 0x000C000C), (w & 0x00300030),
+//                             (w & 0x00C000C0) yield the pairs (e0,e1) (e2,e3) (e4,e5) (e6,e7) and the same masks on
+//                             w >> 8 the pairs (e8,e9) .. (e14,e15).  The meta entries are shared with W.
+//
 //   Npad = N rounded up to 256, Kpad = k_blocks*block_size rounded up to 128, KG = Kpad*bits/128, KBp = Kpad/bs.
 //   Padding columns and padding k hold zero weights and zero scales, so loads never need a bounds check.
 #pragma once
@@ -43,6 +54,7 @@ struct MnbLayout {
   int group_k;        // k covered by one 16-byte group: 32 (4-bit) or 16 (8-bit)
   int meta_bytes;     // bytes of one meta entry
   int64_t w_bytes, meta_off, total_bytes;
+  int64_t w2_off, w2_bytes;  // the native 2-bit copy for the decode kernel (0, 0: none)
 };
 
 MNB_HD int64_t mnb_round_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -54,10 +66,14 @@ MNB_HD int mnb_log2i(int v) {
   return s;
 }
 
+// first k of operand i (0..7) of vector g of the native 2-bit copy
+MNB_HD int64_t mnb_w2_k(int64_t g, int i) { return (g >> 2) * 256 + (int64_t)(i >> 2) * 128 + (g & 3) * 32 + (i & 3) * 8; }
+
 // position of column n inside a meta row
 MNB_HD int64_t mnb_meta_col(int64_t n) { return (n & ~(int64_t)63) | ((n & 15) << 2) | ((n >> 4) & 3); }
 
-MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dtype, int has_zp) {
+// native2: 2-bit sources also get the W2 section (single matrices; the fused and variant layouts do without)
+MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dtype, int has_zp, bool native2 = true) {
   MnbLayout L;
   L.N = N;
   L.K = K;
@@ -83,6 +99,13 @@ MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dty
   L.w_bytes = L.KG * L.Npad * 16;
   L.meta_off = mnb_round_up(L.w_bytes, 256);
   L.total_bytes = mnb_round_up(L.meta_off + L.KBp * L.Npad * L.meta_bytes, 256);
+  L.w2_off = 0;
+  L.w2_bytes = 0;
+  if (native2 && L.src_bits == 2 && dtype == kMnbDtypeFloat16 && bs >= 64) {
+    L.w2_off = L.total_bytes;
+    L.w2_bytes = (L.Kpad / 64) * L.Npad * 16;
+    L.total_bytes += mnb_round_up(L.w2_bytes, 256);
+  }
   return L;
 }
 
@@ -152,7 +175,7 @@ MNB_HD MnbFusedLayout mnb_make_fused_layout(int kind, int64_t n0, int64_t n1, in
     m.start[2] = m.start[1] + mnb_round_up(n1, 16);
     m.Np = m.start[2] + mnb_round_up(n1, 16);
   }
-  F.L = mnb_make_layout(m.Np, K, bits, bs, dtype, 0);
+  F.L = mnb_make_layout(m.Np, K, bits, bs, dtype, 0, false);
   F.bias_off = F.L.total_bytes;
   F.total_bytes = F.bias_off + mnb_round_up(m.Np * (dtype == kMnbDtypeFloat16 ? 2 : 4), 256);
   return F;

@@ -64,6 +64,36 @@ __device__ __forceinline__ h8_t raw4(uint32_t w, const UnpackConsts& u) {
   r.w = (w8 & u.mask_hi) | u.magic_hi;
   return __builtin_bit_cast(h8_t, r);
 }
+// 2-bit weights in their own width (the W2 section of the packed matrix): a 32-bit word holds 16 weights, the
+// operands of two matrix instructions.  Bits 0..7 of each half carry four fields; or-ing a field at bit 2 f into the
+// half whose unit in the last place is 2^(-2 f) gives 1024 + q, 256 + q, 64 + q, 16 + q (magic halves 0x6400, 0x5C00,
+// 0x5400, 0x4C00) -- one v_and_or_b32 per pair of weights, as for nibbles.  The second operand of a word is the same
+// on w >> 8.  Masks in SGPRs, magics in VGPRs (one SGPR operand per VALU instruction), by opaque moves.
+struct UnpackConsts2 {
+  uint32_t mask[4], magic[4];
+};
+
+__device__ __forceinline__ UnpackConsts2 make_unpack_consts2() {
+  UnpackConsts2 u;
+  asm("s_mov_b32 %0, 0x00030003" : "=s"(u.mask[0]));
+  asm("s_mov_b32 %0, 0x000C000C" : "=s"(u.mask[1]));
+  asm("s_mov_b32 %0, 0x00300030" : "=s"(u.mask[2]));
+  asm("s_mov_b32 %0, 0x00C000C0" : "=s"(u.mask[3]));
+  asm("v_mov_b32 %0, 0x64006400" : "=v"(u.magic[0]));
+  asm("v_mov_b32 %0, 0x5C005C00" : "=v"(u.magic[1]));
+  asm("v_mov_b32 %0, 0x54005400" : "=v"(u.magic[2]));
+  asm("v_mov_b32 %0, 0x4C004C00" : "=v"(u.magic[3]));
+  return u;
+}
+
+// raw magic halves of the low bytes of one word: {1024+e0,1024+e1,256+e2,256+e3,64+e4,64+e5,16+e6,16+e7}
+__device__ __forceinline__ h8_t raw2(uint32_t w, const UnpackConsts2& u) {
+  u4_t r;
+#pragma unroll
+  for (int f = 0; f < 4; ++f) r[f] = (w & u.mask[f]) | u.magic[f];
+  return __builtin_bit_cast(h8_t, r);
+}
+
 // 8-bit: two words -> 8 halves 1024+b
 __device__ __forceinline__ h8_t raw8(uint32_t w0, uint32_t w1) {
   uint4 r;
@@ -149,9 +179,11 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
   constexpr int CK = 4 * GK;
   // small loads first: memory returns in issue order, and the weights are waited for tile by tile
   const int64_t mcol = mnb_meta_col(col0);  // entries of columns col0 + 16 t follow at mcol + t
-  if constexpr (MODE == 0) {
+  if constexpr (MODE == 0 || MODE == 6) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0);
+    // MODE 6 (2-bit, blocks of 128): the second half of the chunk lies in the next block
+    if constexpr (MODE == 6) load_meta_vec<HAS_ZP, T>(p.meta, (kb + 1) * p.Npad + mcol, R.m1);
   } else if constexpr (MODE == 4 || MODE == 5) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
     load_meta_vec_f32<HAS_ZP, T>(p.meta, kb * p.Npad + mcol, R.m0, R.z0);
@@ -160,9 +192,11 @@ __device__ __forceinline__ void load_chunk(const SkinnyParams& p, int c, int kq,
     load_meta_vec_f32<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0, R.z0);
     if constexpr (BITS == 4) load_meta_vec_f32<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1, R.z1);
   } else {
-    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
+    // first k of the lane's vector; 2-bit vectors hold 32 k of each half of the chunk (mnb_w2_k)
+    const int64_t k0 = BITS == 2 ? (int64_t)c * CK + kq * 32 : ((int64_t)c * 4 + kq) * GK;
     load_meta_vec<HAS_ZP, T>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol, R.m0);
     if constexpr (BITS == 4) load_meta_vec<HAS_ZP, T>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol, R.m1);
+    if constexpr (BITS == 2) load_meta_vec<HAS_ZP, T>(p.meta, ((k0 + 128) >> p.bs_shift) * p.Npad + mcol, R.m1);
   }
 #pragma unroll
   for (int t = 0; t < T; ++t) {
@@ -181,10 +215,14 @@ __device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, in
                                                 const int32_t* mcol, ChunkRegs<BITS, T>& R) {
   constexpr int GK = 128 / BITS;
   constexpr int CK = 4 * GK;
-  if constexpr (MODE == 0) {
+  if constexpr (MODE == 0 || MODE == 6) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
     for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, kb * p.Npad + mcol[t], &R.m0[t]);
+    if constexpr (MODE == 6) {
+#pragma unroll
+      for (int t = 0; t < T; ++t) load_meta_vec<HAS_ZP, 1>(p.meta, (kb + 1) * p.Npad + mcol[t], &R.m1[t]);
+    }
   } else if constexpr (MODE == 4 || MODE == 5) {
     const int64_t kb = ((int64_t)c * CK) >> p.bs_shift;
 #pragma unroll
@@ -198,12 +236,14 @@ __device__ __forceinline__ void load_chunk_cols(const SkinnyParams& p, int c, in
         load_meta_vec_f32<HAS_ZP, 1>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol[t], &R.m1[t], &R.z1[t]);
     }
   } else {
-    const int64_t k0 = ((int64_t)c * 4 + kq) * GK;
+    const int64_t k0 = BITS == 2 ? (int64_t)c * CK + kq * 32 : ((int64_t)c * 4 + kq) * GK;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       load_meta_vec<HAS_ZP, 1>(p.meta, (k0 >> p.bs_shift) * p.Npad + mcol[t], &R.m0[t]);
       if constexpr (BITS == 4)
         load_meta_vec<HAS_ZP, 1>(p.meta, ((k0 + 16) >> p.bs_shift) * p.Npad + mcol[t], &R.m1[t]);
+      if constexpr (BITS == 2)
+        load_meta_vec<HAS_ZP, 1>(p.meta, ((k0 + 128) >> p.bs_shift) * p.Npad + mcol[t], &R.m1[t]);
     }
   }
 #pragma unroll
@@ -237,6 +277,12 @@ __device__ __forceinline__ BConst make_bconst() {
   const _Float16 hi = (_Float16)(-((BITS == 4 ? 64.0f : 1024.0f) + zp));
   const _Float16 m1 = (_Float16)(-1.0f);
   BConst bc;
+  if constexpr (BITS == 2) {  // 1024, 256, 64, 16 by field (raw2)
+    const _Float16 o1 = (_Float16)(-(256.0f + zp)), o2 = (_Float16)(-(64.0f + zp)), o3 = (_Float16)(-(16.0f + zp));
+    bc.off = h8_t{lo, lo, o1, o1, o2, o2, o3, o3};
+    bc.one = h8_t{m1, m1, m1, m1, m1, m1, m1, m1};
+    return bc;
+  }
   bc.off = h8_t{lo, lo, hi, hi, lo, lo, hi, hi};
   bc.one = h8_t{m1, m1, m1, m1, m1, m1, m1, m1};
   return bc;

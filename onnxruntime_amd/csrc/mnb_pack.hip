@@ -72,6 +72,34 @@ __global__ void __launch_bounds__(256) mnb_pack_weights_kernel(MnbPackSrc S, uin
   W[g * L.Npad + n] = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// The native copy of a 2-bit source for the decode kernel (W2 of mnb_layout.h): one thread per (column, vector).
+// Vector g = 4 c + kq belongs to lane quarter kq of chunk c (256 k); its operand i (8 weights, i = 0..7) covers
+// k = 256 c + 128 (i / 4) + 32 kq + 8 (i % 4) .. + 7 (mnb_w2_k).
+__global__ void __launch_bounds__(256) mnb_pack_weights2_native_kernel(MnbPackSrc S, uint4* __restrict__ W2, MnbLayout L) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t groups = L.Kpad / 64;
+  const int64_t n = idx / groups, g = idx % groups;
+  if (n >= L.Npad) return;
+  uint32_t w[4] = {0, 0, 0, 0};
+  const int64_t col_bytes = L.k_blocks * L.bs / 4;  // bytes of one canonical column
+  int m;
+  int64_t col;
+  if (mnb_map_col(S.map, n, &m, &col)) {
+    const uint8_t* src = S.B[m] + col * col_bytes;
+    for (int j = 0; j < 4; ++j) {
+      uint32_t r = 0;
+      for (int e = 0; e < 16; ++e) {
+        const int64_t k = mnb_w2_k(g, 2 * j + (e >> 3)) + (e & 7);
+        const uint32_t byte = (k >> 2) < col_bytes ? src[k >> 2] : 0u;
+        const uint32_t q = (byte >> (2 * (k & 3))) & 0x3u;
+        r |= q << (((e & 1) ? 16 : 0) + 2 * (e >> 1));
+      }
+      w[j] = r;
+    }
+  }
+  W2[g * L.Npad + n] = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // The same transformation as a tiled transpose, for 4- and 8-bit sources whose columns are whole 16-byte groups at
 // 16-byte aligned addresses (every block size but 16 with an odd block count).  In the kernel above a wavefront reads
 // 64 x 16 single bytes and writes 64 vectors to 64 different cache lines; here a workgroup moves a tile of 32 columns
@@ -129,6 +157,11 @@ static void mnb_pack_weights_dispatch(const MnbPackSrc& S, uint4* W, const MnbLa
   const dim3 grid((unsigned)((wn + 255) / 256)), blk(256);
   if (L.src_bits == 2) {
     mnb_pack_weights_kernel<2><<<grid, blk, 0, s>>>(S, W, L);
+    if (L.w2_bytes > 0) {
+      const int64_t vecs = L.Npad * (L.Kpad / 64);
+      mnb_pack_weights2_native_kernel<<<dim3((unsigned)((vecs + 255) / 256)), blk, 0, s>>>(
+          S, reinterpret_cast<uint4*>(reinterpret_cast<unsigned char*>(W) + L.w2_off), L);
+    }
     return;
   }
   bool tiled = (L.k_blocks * L.bs * L.bits) % 128 == 0 && L.Npad % kPackTile == 0;

@@ -27,6 +27,10 @@
 //    the bfloat16 128 + q, exact in its 8 significant bits.
 //  * MODE 5 (fp16 models with zero points in the activation type, block_size >= chunk): MODE 0 with the block's
 //    fp32 scale and zero point - the zero point enters the fp32 correction unrounded.
+//  * 2-bit weights stream from a copy in their own width (mnb_layout.h, W2): a vector holds 64 weights, the operands
+//    of eight matrix instructions, a chunk is 256 k.  MODE 0 for blocks of 256, MODE 1 for blocks of 64, and MODE 6
+//    for blocks of 128: MODE 0 with the two halves of a chunk (operands 0..3 and 4..7) in different blocks, each with
+//    its own corrections, block sum and meta entry.
 //  * The A operands come straight from global memory (L2 hits after the first workgroup) when the rows of A are
 //    16-byte aligned -- every load of a wavefront's first two chunks is issued before anything is waited for;
 //    otherwise the rows are staged in LDS phase by phase (zero-filled beyond K, any alignment).
@@ -46,10 +50,19 @@ __device__ __forceinline__ BConst bconst_of_mode() {
 }
 
 // One chunk: T column tiles x (4 k-groups) against the 16-row A operands af[].
+// the B operand i of a lane's vector as raw magic halves (MODE 0)
+template <int BITS>
+__device__ __forceinline__ h8_t raw_operand(const uint32_t* wd, int i, const UnpackConsts& uc, const UnpackConsts2& uc2) {
+  if constexpr (BITS == 4) return raw4(wd[i], uc);
+  else if constexpr (BITS == 8) return raw8(wd[2 * i], wd[2 * i + 1]);
+  else return raw2((i & 1) ? wd[i >> 1] >> 8 : wd[i >> 1], uc2);
+}
+
 template <int BITS, bool HAS_ZP, int MODE, int T>
 __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const h8_t* af, const BConst& bc,
-                                              const UnpackConsts& uc, f4_t* y) {
+                                              const UnpackConsts& uc, const UnpackConsts2& uc2, f4_t* y) {
   constexpr int NI = (128 / BITS) / 8;
+  static_assert(BITS != 2 || MODE <= 1 || MODE == 6, "2-bit weights in their own width: fp16 models only");
 #if defined(MNB_ABLATE_NO_MATH)
   // calibration builds: the loads are waited for and nothing is computed (what the arithmetic costs a launch)
 #pragma unroll
@@ -60,46 +73,54 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
   for (int i = 0; i < NI; ++i) asm volatile("; keep %0" ::"v"(__builtin_bit_cast(u4_t, af[i])));
   return;
 #endif
-  if constexpr (MODE == 0 || MODE == 5) {
+  if constexpr (MODE == 0 || MODE == 5 || MODE == 6) {
     // init[m] = -sum_k (off_k + zp) a[m][k] (no zero points) or -sum_k off_k a[m][k]; nc2[m] = -sum_k a[m][k].
     // The constant operands are the same in every lane, so every lane receives the value of its own rows.
+    // MODE 6 (2-bit weights in blocks of 128): a chunk is 256 k and its halves of 128 (operands 0..3 and 4..7) lie in
+    // different blocks, so each half has its own corrections, block sum and meta entry (m0, m1).
+    static_assert(MODE != 6 || BITS == 2, "two blocks per chunk: 2-bit weights only");
+    constexpr int SUB = MODE == 6 ? 2 : 1, PER = NI / SUB;
     const f4_t zero = f4_t{0.f, 0.f, 0.f, 0.f};
-    f4_t init = zero, nc2 = zero;
+    f4_t init[SUB], nc2[SUB];
 #pragma unroll
-    for (int i = 0; i < NI; ++i) init = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bc.off, init, 0, 0, 0);
-    if constexpr (HAS_ZP) {
+    for (int h = 0; h < SUB; ++h) {
+      init[h] = zero;
+      nc2[h] = zero;
 #pragma unroll
-      for (int i = 0; i < NI; ++i) nc2 = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bc.one, nc2, 0, 0, 0);
+      for (int i = h * PER; i < (h + 1) * PER; ++i)
+        init[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bc.off, init[h], 0, 0, 0);
+      if constexpr (HAS_ZP) {
+#pragma unroll
+        for (int i = h * PER; i < (h + 1) * PER; ++i)
+          nc2[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bc.one, nc2[h], 0, 0, 0);
+      }
     }
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-      float sf, zp;  // scale and zero point of the chunk's block
-      if constexpr (MODE == 5) {
-        sf = __uint_as_float(R.m0[t]);
-        zp = __uint_as_float(R.z0[t]);
-      } else {
-        _Float16 s, nz;
-        decode_meta<BITS, HAS_ZP>(R.m0[t], s, nz);
-        sf = (float)s;
-        zp = -(float)nz - 1024.0f;
-      }
       const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
-      f4_t d = init;
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        h8_t b;
-        if constexpr (BITS == 4)
-          b = raw4(wd[i], uc);
-        else
-          b = raw8(wd[2 * i], wd[2 * i + 1]);
-        d = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], b, d, 0, 0, 0);
-      }
-      if constexpr (HAS_ZP) {
+      for (int h = 0; h < SUB; ++h) {
+        float sf, zp;  // scale and zero point of the block
+        if constexpr (MODE == 5) {
+          sf = __uint_as_float(R.m0[t]);
+          zp = __uint_as_float(R.z0[t]);
+        } else {
+          _Float16 sc, nz;
+          decode_meta<BITS, HAS_ZP>(h == 0 ? R.m0[t] : R.m1[t], sc, nz);
+          sf = (float)sc;
+          zp = -(float)nz - 1024.0f;
+        }
+        f4_t d = init[h];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, __builtin_fmaf(zp, nc2[r], d[r]), y[t][r]);
-      } else {
+        for (int i = h * PER; i < (h + 1) * PER; ++i)
+          d = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], raw_operand<BITS>(wd, i, uc, uc2), d, 0, 0, 0);
+        if constexpr (HAS_ZP) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, d[r], y[t][r]);
+          for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, __builtin_fmaf(zp, nc2[h][r], d[r]), y[t][r]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) y[t][r] = __builtin_fmaf(sf, d[r], y[t][r]);
+        }
       }
     }
   } else if constexpr (MODE == 4) {
@@ -156,7 +177,7 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
       const uint32_t wd[4] = {R.w[t].x, R.w[t].y, R.w[t].z, R.w[t].w};
       _Float16 s0, s1, nz0, nz1;
       decode_meta<BITS, HAS_ZP>(R.m0[t], s0, nz0);
-      if constexpr (BITS == 4) {
+      if constexpr (BITS == 4 || BITS == 2) {
         decode_meta<BITS, HAS_ZP>(R.m1[t], s1, nz1);
       } else {
         s1 = s0;
@@ -166,10 +187,20 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         h2_t d[4];
-        const bool second = (BITS == 4) && i >= 2;
+        // words 2, 3 of a 4-bit vector may belong to the next block; operands 4..7 of a 2-bit vector lie in the other
+        // half of the chunk
+        const bool second = (BITS == 4 && i >= 2) || (BITS == 2 && i >= 4);
         const ZpH& z = second ? z1 : z0;
         const h2_t s2 = mnb_h2(second ? s1 : s0);
-        if constexpr (BITS == 4) {
+        if constexpr (BITS == 2) {
+          // -(256 + zp) and -(16 + zp) beside z.lo = -(1024 + zp) and z.hi = -(64 + zp); exact (integers below 2048)
+          const _Float16 nz = second ? nz1 : nz0;
+          const u4_t p = __builtin_bit_cast(u4_t, raw2((i & 1) ? wd[i >> 1] >> 8 : wd[i >> 1], uc2));
+          d[0] = mnb_as_h2(p[0]) + z.lo;
+          d[1] = mnb_as_h2(p[1]) + mnb_h2(nz + (_Float16)768.0f);
+          d[2] = mnb_as_h2(p[2]) + z.hi;
+          d[3] = mnb_as_h2(p[3]) + mnb_h2(nz + (_Float16)1008.0f);
+        } else if constexpr (BITS == 4) {
           mnb_unpack4_h(wd[i], z, d);
         } else {
           mnb_unpack8_h(wd[2 * i], z, d);
@@ -259,7 +290,11 @@ struct AStage {
       mine[row * PIECES + (piece ^ swz(row))] = g[I];
     }
 #pragma unroll
-    for (int i = 0; i < NI; ++i) af[i] = mine[j * PIECES + ((kq * NI + i) ^ swz(j))];
+    for (int i = 0; i < NI; ++i) {
+      // the 16-byte piece of the row's chunk that holds operand i of lane quarter kq (2-bit: mnb_w2_k)
+      const int piece = BITS == 2 ? (i >> 2) * 16 + kq * 4 + (i & 3) : kq * NI + i;
+      af[i] = mine[j * PIECES + (piece ^ swz(j))];
+    }
   }
 };
 
@@ -275,10 +310,12 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
   constexpr int NI = GK / 8;
   const int j = lane & 15, kq = lane >> 4;
   const int arow = j < p.M ? j : p.M - 1;  // rows >= M of the MFMA A operand re-read row M-1: they are never stored
-  const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * GK;
+  // first k of the lane's operands inside a chunk: kq GK, or for 2-bit vectors 32 kq in each half of the chunk
+  const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * (BITS == 2 ? 32 : GK);
   h8_t* mine = reinterpret_cast<h8_t*>(smem) + wave * (16 * AStage<BITS>::PIECES);  // A_LDS only
   const BConst bconst = bconst_of_mode<BITS, HAS_ZP, MODE>();
   const UnpackConsts uc = make_unpack_consts();
+  const UnpackConsts2 uc2 = make_unpack_consts2();  // (2-bit weights; unused moves are dropped)
 
   // the activation loads of chunk c: the operands themselves, or the row-contiguous pieces that pass through LDS
   auto fetch_a = [&](int c, h8_t* a) {
@@ -286,16 +323,18 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
       AStage<BITS>::fetch(p, c, lane, a);
     } else {
 #pragma unroll
-      for (int i = 0; i < NI; ++i) a[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK + 8 * i);
+      for (int i = 0; i < NI; ++i)
+        a[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK +
+                                              (BITS == 2 ? (i >> 2) * 128 + (i & 3) * 8 : 8 * i));
     }
   };
   auto run = [&](const ChunkRegs<BITS, T>& R, const h8_t* a) {
     if constexpr (A_LDS) {
       h8_t af[NI];
       AStage<BITS>::pass(mine, a, lane, af);
-      compute_chunk<BITS, HAS_ZP, MODE, T>(R, af, bconst, uc, y);
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R, af, bconst, uc, uc2, y);
     } else {
-      compute_chunk<BITS, HAS_ZP, MODE, T>(R, a, bconst, uc, y);
+      compute_chunk<BITS, HAS_ZP, MODE, T>(R, a, bconst, uc, uc2, y);
     }
   };
 
@@ -311,10 +350,10 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
 #pragma unroll
       for (int q = 0; q < CPW; ++q) AStage<BITS>::pass(mine, a[q], lane, af[q]);
 #pragma unroll
-      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], af[q], bconst, uc, y);
+      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], af[q], bconst, uc, uc2, y);
     } else {
 #pragma unroll
-      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, y);
+      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, uc2, y);
     }
   } else if constexpr (T <= 2) {
     // Two chunks in flight.  Loads under a run-time condition would leave the compiler unable to count the
@@ -479,6 +518,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
   for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
   const BConst bconst = bconst_of_mode<BITS, HAS_ZP, MODE>();
   const UnpackConsts uc = make_unpack_consts();
+  const UnpackConsts2 uc2 = make_unpack_consts2();
 
   for (int ph0 = 0; ph0 < p.chunks; ph0 += p.phase_chunks) {
     const int ph1 = min(ph0 + p.phase_chunks, p.chunks);
@@ -506,7 +546,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
       const _Float16* abase = As + arow * row_stride + ((c - ph0) * 4 + kq) * GK;
 #pragma unroll
       for (int i = 0; i < NI; ++i) af[i] = *reinterpret_cast<const h8_t*>(abase + 8 * i);
-      compute_chunk<BITS, HAS_ZP, MODE, T>(Rc, af, bconst, uc, y);
+      compute_chunk<BITS, HAS_ZP, MODE, T>(Rc, af, bconst, uc, uc2, y);
     }
   }
   __syncthreads();
@@ -529,7 +569,8 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   SkinnyPlan pl;
   const int GK = L.group_k, CK = 4 * GK;
   const int chunks = (int)((L.K + CK - 1) / CK);
-  pl.mode = (L.bs >= CK) ? 0 : 1;
+  // raw operands need every matrix instruction inside one block: a whole chunk, or half of a 2-bit chunk (mode 6)
+  pl.mode = (L.bs >= CK) ? 0 : (L.bits == 2 && L.bs == 128) ? 6 : 1;
   if (const char* e = mnb_tuning_env("MNB_SKINNY_MODE")) pl.mode = e[0] == '1' ? 1 : pl.mode;  // calibration: exact halves
   if (io != kMnbIoModel) {  // fp32 meta entries: raw operands where a chunk lies inside a block, else exact weights
     const bool raw = L.bits == 4 && L.bs >= CK;
@@ -543,6 +584,9 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   pl.t = tiles >= 800 ? 4 : tiles >= 320 ? 2 : 1;  // measured: N = 6144 prefers 2 (192 workgroups), N = 4096 prefers 1
   // wavefronts per workgroup: aim for >= 2 chunks per wavefront
   pl.nw = chunks >= 32 ? 16 : chunks >= 16 ? 8 : 4;
+  // 2-bit chunks are 256 k, twice the arithmetic of the others: one per wavefront already pays (measured at K = 4096,
+  // M = 1, blocks of 128: N = 14336 8.2 -> 7.3 us, N = 6144 5.6 -> 5.0 us; blocks of 64: 9.2 -> 8.0 us)
+  if (L.bits == 2) pl.nw = chunks >= 16 ? 16 : chunks >= 8 ? 8 : 4;
   // More four-tile slabs than compute units: sixteen-wavefront workgroups run one per unit, in rounds that each pay
   // their own first-load latency and reduction, and the last round is partly empty.  Smaller workgroups share a unit
   // and overlap these (measured at K = 4096 and 8192, N = 20480 ... 57344, M = 1, 8, 16: 3-26 % faster; 4-bit
@@ -556,7 +600,7 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
       pl.nw = L.bits == 4 ? 4 : 8;
     }
   }
-  static const char* const plan_override = mnb_tuning_env("MNB_SKINNY_PLAN");  // tuning override "<T>,<NW>", read once
+  const char* const plan_override = mnb_tuning_env("MNB_SKINNY_PLAN");  // calibration builds: "<T>,<NW>"
   if (const char* e = plan_override) {
     int t = 0, nw = 0;
     if (sscanf(e, "%d,%d", &t, &nw) == 2 && (t == 1 || t == 2 || t == 4) && (nw == 4 || nw == 8 || nw == 16)) {
@@ -693,7 +737,8 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
 #undef MNB_SKINNY_LAUNCH
   } else {
     // rare: A not 16-byte aligned or K not a multiple of 8 -- one configuration is enough
-    mnb_skinny_staged_kernel<BITS, HAS_ZP, MODE, T, 4><<<grid, dim3(256), pl.smem, s>>>(p);
+    if constexpr (BITS != 2) mnb_skinny_staged_kernel<BITS, HAS_ZP, MODE, T, 4><<<grid, dim3(256), pl.smem, s>>>(p);
+    else return hipErrorInvalidValue;  // (the native 2-bit copy is only taken with aligned activations)
   }
   return hipGetLastError();
 }
@@ -718,10 +763,17 @@ hipError_t launch_zp(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s)
     if constexpr (BITS == 4 && HAS_ZP) return launch_mode<BITS, HAS_ZP, 5>(p, pl, s);
     else return hipErrorInvalidValue;
   }
-  if (pl.mode == 2) return launch_mode<BITS, HAS_ZP, 2>(p, pl, s);
+  if (pl.mode == 2) {
+    if constexpr (BITS != 2) return launch_mode<BITS, HAS_ZP, 2>(p, pl, s);
+    else return hipErrorInvalidValue;  // (2-bit weights in their own width: fp16 models only)
+  }
   if (pl.mode == 3) {
     if constexpr (BITS == 4 && HAS_ZP) return launch_mode<BITS, HAS_ZP, 3>(p, pl, s);
     else return hipErrorInvalidValue;  // zero points in the activation type: 4-bit with zero points
+  }
+  if (pl.mode == 6) {
+    if constexpr (BITS == 2) return launch_mode<BITS, HAS_ZP, 6>(p, pl, s);
+    else return hipErrorInvalidValue;
   }
   return pl.mode == 0 ? launch_mode<BITS, HAS_ZP, 0>(p, pl, s) : launch_mode<BITS, HAS_ZP, 1>(p, pl, s);
 }
@@ -733,12 +785,26 @@ bool mnb_skinny_applicable(const MnbGemmArgs& a) {
   return (a.io != kMnbIoModel ? a.L.dtype == kMnbDtypeFloat : a.L.dtype == kMnbDtypeFloat16) && a.M >= 1 && a.M <= 16;
 }
 
+bool mnb_skinny_native2(const MnbGemmArgs& a) {
+  const MnbLayout& L = a.L;
+  return L.src_bits == 2 && L.w2_bytes > 0 && a.io == kMnbIoModel && a.epi.kind == kMnbFusedNone && a.M <= 16 &&
+         (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % 256 == 0);
+}
+
 hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
   if (!mnb_skinny_applicable(a) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
   // direct variant: 16-byte loads of whole chunks of A
-  const bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
-  SkinnyPlan pl = skinny_plan(L, a.io, a.M, a_vec_ok, a.epi.kind == kMnbFusedMlp ? 2 : 1);
+  bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
+  // 2-bit sources: the copy in their own width (half the bytes to stream) when the matrix has one, the operator is
+  // the plain one and whole chunks of 256 k can be read straight from aligned activations; else the nibble copy
+  const bool native2 = mnb_skinny_native2(a);
+  MnbLayout L2 = L;
+  if (native2) {
+    L2.bits = 2;
+    L2.group_k = 64;
+  }
+  SkinnyPlan pl = skinny_plan(native2 ? L2 : L, a.io, a.M, a_vec_ok, a.epi.kind == kMnbFusedMlp ? 2 : 1);
   SkinnyParams p{};
   p.A = reinterpret_cast<const _Float16*>(a.A);
   p.W = reinterpret_cast<const uint4*>(a.packed);
@@ -752,8 +818,9 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   p.N = (int)L.N;
   p.K = (int)L.K;
   p.bs_shift = mnb_log2i(L.bs);
-  const int CK = 4 * L.group_k;
+  const int CK = 4 * (native2 ? L2.group_k : L.group_k);
   p.chunks = (int)((L.K + CK - 1) / CK);
+  if (native2) p.W = reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(a.packed) + L.w2_off);
   p.phase_chunks = pl.phase_chunks;
   p.mtr = pl.mtr;
   p.a_vec_ok = a_vec_ok;
@@ -772,6 +839,7 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
     p.epi.ld1 = a.epi.ld[1];
     p.epi.ld2 = a.epi.ld[2];
   }
+  if (native2) return launch_zp<2, true>(p, pl, s);
   if (L.bits == 4) return L.has_zp ? launch_zp<4, true>(p, pl, s) : launch_zp<4, false>(p, pl, s);
   return L.has_zp ? launch_zp<8, true>(p, pl, s) : launch_zp<8, false>(p, pl, s);
 }

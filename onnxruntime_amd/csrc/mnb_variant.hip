@@ -285,7 +285,7 @@ int order_by_group(const int32_t* g_idx, size_t len, int64_t K, int bs, bool tab
 int64_t staged_ld(const MnbVariantPlan& p) { return (p.packed_k + 7) / 8 * 8; }
 
 MnbLayout packed_layout(const MnbVariantPlan& p) {
-  return mnb_make_layout(p.N, p.packed_k, p.bits, p.packed_block_size, p.compute_dtype, p.zp_kind != MNB_ZP_NONE);
+  return mnb_make_layout(p.N, p.packed_k, p.bits, p.packed_block_size, p.compute_dtype, p.zp_kind != MNB_ZP_NONE, false);
 }
 
 int check_plan(const char* fn, const MnbVariantPlan* p) {

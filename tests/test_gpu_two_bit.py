@@ -98,3 +98,48 @@ def test_quantiser_matches_the_oracle(oracle, dtype, bs, symmetric):
     assert np.array_equal(_bits_view(s.cpu().numpy()), _bits_view(ws))
     if not symmetric:
         assert np.array_equal(z.cpu().numpy(), wz)
+
+
+NATIVE = [
+    # M, N, K, bs, zp, bias: decode shapes whose K is whole chunks of 256: the copy in the weights' own width
+    (1, 512, 1024, 128, False, False), (1, 1000, 4096, 128, True, True), (2, 4096, 4096, 64, True, False),
+    (4, 6144, 4096, 128, False, True), (1, 14336, 4096, 128, True, False), (3, 11008, 4096, 256, True, True),
+    (5, 333, 256, 64, True, False), (8, 2048, 8192, 256, False, False), (9, 4100, 2048, 128, True, True),
+    (16, 520, 4096, 64, False, True), (16, 4096, 14336, 128, True, False), (1, 28672, 4096, 256, True, False),
+    (12, 14336, 512, 64, True, True), (7, 20480, 1024, 128, False, False),
+]
+
+
+@pytest.mark.parametrize("M,N,K,bs,zp,bias", NATIVE)
+def test_decode_streams_the_native_copy(oracle, M, N, K, bs, zp, bias):
+    """fp16 models, blocks of 64 and more, up to 16 rows, K a multiple of 256, aligned activations: the decode kernel
+    reads the 2-bit copy of the weights (half the bytes).  Against the oracle; unit-vector rows return columns of W
+    bit for bit; the nibble copy is not touched (it is overwritten first) while more than 16 rows still need it."""
+    c = make_case(M, N, K, 2, bs, np.float16, has_zp=zp, has_bias=bias, seed=M + N + K)
+    op = make_op(c)
+    y = op.Compute(dev(c.A), bias=dev(c.bias))
+    check_against_oracle(oracle, c, y.cpu().numpy())
+    ks = np.random.default_rng(N).choice(K, size=M, replace=False)
+    eye = np.zeros((M, K), np.float16)
+    eye[np.arange(M), ks] = 1
+    w = oracle.C.dequantize(c.B, c.scales, c.zero_points, N, K, 2, bs)
+    got = op.Compute(dev(eye)).cpu().numpy()   # (without the bias)
+    assert np.array_equal(_bits_view(got), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+    # activations that are not 16-byte aligned take the nibble copy: the same result up to the order of the sums
+    wide = torch.zeros(1 + M * (K + 3), dtype=torch.float16, device="cuda")[1:].view(M, K + 3)  # (base off by 2 bytes)
+    wide[:, :K] = dev(c.A)
+    y_nib = op.Compute(wide[:, :K], bias=dev(c.bias)).cpu().numpy()
+    d = np.abs(y_nib.astype(np.float64) - y.cpu().numpy().astype(np.float64))
+    assert d.max() <= 2e-3 * np.abs(y_nib).max() + 1e-3
+    # which copy is read: garbage in the nibble section changes nothing for aligned decode calls ...
+    n_pad, k_pad = -(-N // 256) * 256, -(-(-(-K // bs) * bs) // 128) * 128
+    w_bytes = k_pad // 32 * n_pad * 16
+    saved = op.packed[:w_bytes].clone()
+    op.packed[:w_bytes] = 0x5A
+    y_again = op.Compute(dev(c.A), bias=dev(c.bias))
+    assert torch.equal(y_again, y)
+    # ... and does for the calls that read it
+    y_broken = op.Compute(wide[:, :K], bias=dev(c.bias)).cpu().numpy()
+    assert not np.array_equal(y_broken, y_nib)
+    op.packed[:w_bytes] = saved
+    assert np.array_equal(op.Compute(wide[:, :K], bias=dev(c.bias)).cpu().numpy(), y_nib)
