@@ -72,7 +72,7 @@ MNB_HD int64_t mnb_w2_k(int64_t g, int i) { return (g >> 2) * 256 + (int64_t)(i 
 // position of column n inside a meta row
 MNB_HD int64_t mnb_meta_col(int64_t n) { return (n & ~(int64_t)63) | ((n & 15) << 2) | ((n >> 4) & 3); }
 
-// native2: 2-bit sources also get the W2 section (single matrices; the fused and variant layouts do without)
+// native2: 2-bit sources also get the W2 section (the variant layouts do without)
 MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dtype, int has_zp, bool native2 = true) {
   MnbLayout L;
   L.N = N;
@@ -175,7 +175,7 @@ MNB_HD MnbFusedLayout mnb_make_fused_layout(int kind, int64_t n0, int64_t n1, in
     m.start[2] = m.start[1] + mnb_round_up(n1, 16);
     m.Np = m.start[2] + mnb_round_up(n1, 16);
   }
-  F.L = mnb_make_layout(m.Np, K, bits, bs, dtype, 0, false);
+  F.L = mnb_make_layout(m.Np, K, bits, bs, dtype, 0);
   F.bias_off = F.L.total_bytes;
   F.total_bytes = F.bias_off + mnb_round_up(m.Np * (dtype == kMnbDtypeFloat16 ? 2 : 4), 256);
   return F;

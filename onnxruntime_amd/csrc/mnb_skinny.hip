@@ -787,7 +787,7 @@ bool mnb_skinny_applicable(const MnbGemmArgs& a) {
 
 bool mnb_skinny_native2(const MnbGemmArgs& a) {
   const MnbLayout& L = a.L;
-  return L.src_bits == 2 && L.w2_bytes > 0 && a.io == kMnbIoModel && a.epi.kind == kMnbFusedNone && a.M <= 16 &&
+  return L.src_bits == 2 && L.w2_bytes > 0 && a.io == kMnbIoModel && a.M <= 16 &&
          (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % 256 == 0);
 }
 
@@ -796,8 +796,8 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   if (!mnb_skinny_applicable(a) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
   // direct variant: 16-byte loads of whole chunks of A
   bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
-  // 2-bit sources: the copy in their own width (half the bytes to stream) when the matrix has one, the operator is
-  // the plain one and whole chunks of 256 k can be read straight from aligned activations; else the nibble copy
+  // 2-bit sources: the copy in their own width (half the bytes to stream) when the matrix has one and whole chunks
+  // of 256 k can be read straight from aligned activations; else the nibble copy
   const bool native2 = mnb_skinny_native2(a);
   MnbLayout L2 = L;
   if (native2) {

@@ -143,3 +143,27 @@ def test_decode_streams_the_native_copy(oracle, M, N, K, bs, zp, bias):
     assert not np.array_equal(y_broken, y_nib)
     op.packed[:w_bytes] = saved
     assert np.array_equal(op.Compute(wide[:, :K], bias=dev(c.bias)).cpu().numpy(), y_nib)
+
+
+@pytest.mark.parametrize("M,N,K,bs", [(1, 1408, 1024, 128), (3, 200, 256, 64), (8, 4096, 4096, 256), (16, 520, 2048, 128)])
+def test_fused_decode_streams_the_native_copy(oracle, M, N, K, bs):
+    """MatMulNBitsMlp / MatMulNBitsQkv with 2-bit weights, up to 16 rows: the packed matrix of all projections has the
+    copy in the weights' own width too, and decode reads it (the nibble copy is overwritten first)."""
+    from onnxruntime_amd.matmul_nbits import MatMulNBitsQkv
+    g = make_case(M, N, K, 2, bs, np.float16, has_bias=True, seed=N)
+    u = make_case(M, N, K, 2, bs, np.float16, seed=N + 1)
+    op = MatMulNBitsMlp(K, N, 2, bs)
+    assert op.PrePack(dev(g.B), dev(g.scales), dev(g.bias), dev(u.B), dev(u.scales), None)
+    n_pad, k_pad = -(-(2 * (-(-N // 16) * 16)) // 256) * 256, -(-(-(-K // bs) * bs) // 128) * 128
+    op.packed[:k_pad // 32 * n_pad * 16] = 0x5A
+    y = op.Compute(dev(g.A)).cpu().numpy().astype(np.float64)
+    want = oracle.C.mlp(g.A, (g.B, g.scales, g.bias), (u.B, u.scales, None), N, K, 2, bs).astype(np.float64)
+    assert float(np.linalg.norm(y - want) / np.linalg.norm(want)) <= 5e-3
+    nkv = max(N // 4, 16)
+    q, k, v = g, make_case(M, nkv, K, 2, bs, np.float16, has_bias=True, seed=N + 2), make_case(M, nkv, K, 2, bs, np.float16, seed=N + 3)
+    opq = MatMulNBitsQkv(K, N, nkv, 2, bs)
+    assert opq.PrePack(dev(q.B), dev(q.scales), dev(q.bias), dev(k.B), dev(k.scales), dev(k.bias), dev(v.B), dev(v.scales), None)
+    outs = opq.Compute(dev(q.A))
+    for got, c in zip(outs[:3], (q, k, v)):
+        y64, _ = oracle.C.matmul_f64(q.A, c.B, c.scales, None, c.bias, c.N, K, 2, bs, nthreads=8)
+        assert float(np.linalg.norm(got.cpu().numpy().astype(np.float64) - y64) / np.linalg.norm(y64)) <= 5e-3
