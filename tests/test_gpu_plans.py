@@ -1,0 +1,76 @@
+"""The planners' choices against the alternatives they could have made, timed on the device.
+
+Needs the calibration library (python -m onnxruntime_amd.calibration.build: the product sources with the planners'
+environment overrides compiled in); skipped when it has not been built.  For each problem the plan the library picks
+by itself must be within 25 % of the fastest forced alternative (HIP graphs of 20 launches, best of three): a plan
+that is off by more than box-to-box noise fails here instead of going unnoticed."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from onnxruntime_amd import _lib
+from onnxruntime_amd.calibration import build as cal_build
+from onnxruntime_amd.calibration import run as cal_run
+
+pytestmark = pytest.mark.gpu
+
+CAL = cal_build.lib_path()
+
+
+def _time(call, launches=20, reps=3):
+    best = float("inf")
+    for _ in range(reps):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(launches):
+                assert call() == 0
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) / (2 * launches) * 1e3)
+    return best
+
+
+# (M, N, K, bits, block, copies of the packed matrix), alternatives as environment settings
+CASES = [
+    ((1, 14336, 4096, 4, 128, 16), ["MNB_SKINNY_PLAN=4,8", "MNB_SKINNY_PLAN=2,16", "MNB_SKINNY_PLAN=2,8"]),
+    ((1, 6144, 4096, 4, 64, 16), ["MNB_SKINNY_PLAN=4,16", "MNB_SKINNY_PLAN=1,16", "MNB_SKINNY_PLAN=2,8"]),
+    ((1, 14336, 4096, 2, 128, 16), ["MNB_SKINNY_PLAN=4,8", "MNB_SKINNY_PLAN=2,16", "MNB_SKINNY_MODE=1"]),
+    ((64, 28672, 4096, 4, 128, 1), ["MNB_MID_SHARED=0", "MNB_MID_SHARED=0+MNB_MID_PLAN=4,4,8"]),
+    ((64, 4096, 14336, 4, 128, 1), ["MNB_MID_PLAN=1,4,8", "MNB_MID_PLAN=2,2,4", "MNB_MID_SHARED=1"]),
+    ((256, 6144, 4096, 4, 128, 1), ["MNB_MID_SHARED=0", "MNB_MID_MAX_M=64"]),
+    ((1024, 4096, 14336, 4, 128, 1), ["MNB_GEMM256_PLAN=256,1", "MNB_GEMM256_PLAN=128,2", "MNB_MID_MAX_M=4096"]),
+    ((2048, 14336, 4096, 4, 32, 1), ["MNB_GEMM256_PLAN=128,1", "MNB_GEMM256_WAVES=4"]),
+]
+
+
+@pytest.mark.skipif(not CAL.exists(), reason="the calibration library has not been built")
+@pytest.mark.parametrize("shape,alternatives", CASES)
+def test_the_plan_chosen_is_close_to_the_best_alternative(shape, alternatives):
+    M, N, K, bits, bs, copies = shape
+    lib = cal_run.load(str(CAL))
+    prob = cal_run.Problem(M, N, K, bits, bs, zp=True, bias=False, copies=copies)
+    times = {}
+    try:
+        for env in [""] + alternatives:
+            cal_run.set_env(dict(kv.split("=", 1) for kv in env.split("+") if kv))
+            call, _ = prob.caller(lib)
+            print("plan", env or "(chosen)", shape, flush=True)   # (names the case should a launch fault)
+            assert call() == 0
+            torch.cuda.synchronize()
+            for _ in range(50):   # clock and caches settled
+                call()
+            torch.cuda.synchronize()
+            times[env] = _time(call, launches=max(20, copies))
+    finally:
+        cal_run.set_env({})
+    chosen, best = times[""], min(times.values())
+    assert chosen <= 1.25 * best, f"{shape}: chosen {chosen:.1f} us, alternatives {times}"
