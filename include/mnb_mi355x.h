@@ -85,7 +85,7 @@ MNB_API int MnbCheckInputs(const MnbTensorInfo* quantized_weight, const MnbTenso
  * weights, scales and zero points of one [N, K] matrix in the gfx950 tiled layout; 0 if unsupported.
  * has_zero_points: 1 if the operator has a zero_points input (the packed meta then carries them).
  * 2-bit weights are stored widened to nibbles (every 4-bit kernel runs them) with their zero points always explicit;
- * float16 models with blocks of 64 and more also keep a copy in the weights' own width, N * K / 4 bytes, which the
+ * float16 models with blocks of 32 and more also keep a copy in the weights' own width, N * K / 4 bytes, which the
  * decode kernel streams for up to 16 rows when K is a multiple of 256 and the activations are 16-byte aligned. */
 MNB_API size_t MnbPackQuantBDataSize(size_t N, size_t K, int bits, int block_size, int has_zero_points, int a_dtype);
 

@@ -15,7 +15,7 @@
 //                             order (n%16)*4 + (n%64)/16, so that the four 16-column tiles a matrix-core lane
 //                             works on are adjacent and arrive with one vector load (mnb_meta_col).
 //
-//   W2  [Kpad/64][Npad][16 B] 2-bit sources of fp16 models with blocks of 64 and more only, behind everything else: the
+//   W2  [Kpad/64][Npad][16 B] 2-bit sources of fp16 models with blocks of 32 and more only, behind everything else: the
 //                             weights once more in their own width for the decode kernel (M <= 16 streams half the
 //                             bytes).  One 16-byte vector = 64 k of one column, the operands of eight matrix
 //                             instructions: vector 4 c + kq holds, as operand i, k = 256 c + 128 (i / 4) + 32 kq +
@@ -101,7 +101,7 @@ MNB_HD MnbLayout mnb_make_layout(int64_t N, int64_t K, int bits, int bs, int dty
   L.total_bytes = mnb_round_up(L.meta_off + L.KBp * L.Npad * L.meta_bytes, 256);
   L.w2_off = 0;
   L.w2_bytes = 0;
-  if (native2 && L.src_bits == 2 && dtype == kMnbDtypeFloat16 && bs >= 64) {
+  if (native2 && L.src_bits == 2 && dtype == kMnbDtypeFloat16 && bs >= 32) {
     L.w2_off = L.total_bytes;
     L.w2_bytes = (L.Kpad / 64) * L.Npad * 16;
     L.total_bytes += mnb_round_up(L.w2_bytes, 256);

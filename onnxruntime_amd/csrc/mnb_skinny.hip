@@ -28,7 +28,7 @@
 //  * MODE 5 (fp16 models with zero points in the activation type, block_size >= chunk): MODE 0 with the block's
 //    fp32 scale and zero point - the zero point enters the fp32 correction unrounded.
 //  * 2-bit weights stream from a copy in their own width (mnb_layout.h, W2): a vector holds 64 weights, the operands
-//    of eight matrix instructions, a chunk is 256 k.  MODE 0 for blocks of 256, MODE 1 for blocks of 64, and MODE 6
+//    of eight matrix instructions, a chunk is 256 k.  MODE 0 for blocks of 256, MODE 1 for blocks of 32 and 64, MODE 6
 //    for blocks of 128: MODE 0 with the two halves of a chunk (operands 0..3 and 4..7) in different blocks, each with
 //    its own corrections, block sum and meta entry.
 //  * The A operands come straight from global memory (L2 hits after the first workgroup) when the rows of A are
@@ -795,7 +795,7 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   const MnbLayout& L = a.L;
   if (!mnb_skinny_applicable(a) || (a.io != kMnbIoModel && a.epi.kind != kMnbFusedNone)) return hipErrorInvalidValue;
   // direct variant: 16-byte loads of whole chunks of A
-  bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
+  const bool a_vec_ok = (reinterpret_cast<uintptr_t>(a.A) % 16 == 0) && (a.lda % 8 == 0) && (L.K % (4 * L.group_k) == 0);
   // 2-bit sources: the copy in their own width (half the bytes to stream) when the matrix has one and whole chunks
   // of 256 k can be read straight from aligned activations; else the nibble copy
   const bool native2 = mnb_skinny_native2(a);

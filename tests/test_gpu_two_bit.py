@@ -107,12 +107,13 @@ NATIVE = [
     (5, 333, 256, 64, True, False), (8, 2048, 8192, 256, False, False), (9, 4100, 2048, 128, True, True),
     (16, 520, 4096, 64, False, True), (16, 4096, 14336, 128, True, False), (1, 28672, 4096, 256, True, False),
     (12, 14336, 512, 64, True, True), (7, 20480, 1024, 128, False, False),
+    (1, 4096, 4096, 32, True, False), (6, 1000, 1024, 32, False, True),
 ]
 
 
 @pytest.mark.parametrize("M,N,K,bs,zp,bias", NATIVE)
 def test_decode_streams_the_native_copy(oracle, M, N, K, bs, zp, bias):
-    """fp16 models, blocks of 64 and more, up to 16 rows, K a multiple of 256, aligned activations: the decode kernel
+    """fp16 models, blocks of 32 and more, up to 16 rows, K a multiple of 256, aligned activations: the decode kernel
     reads the 2-bit copy of the weights (half the bytes).  Against the oracle; unit-vector rows return columns of W
     bit for bit; the nibble copy is not touched (it is overwritten first) while more than 16 rows still need it."""
     c = make_case(M, N, K, 2, bs, np.float16, has_zp=zp, has_bias=bias, seed=M + N + K)

@@ -35,10 +35,10 @@ def test_availability_and_sizes():
     assert lib.MnbPackQuantBDataSize(14336, 4096, 4, 128, 0, _lib.DTYPE_FLOAT16) == 14336 * 2048 + 14336 * 32 * 2
     # 2-bit weights are stored as nibbles with explicit zero points: the 4-bit size with 4-byte meta entries ...
     four = lib.MnbPackQuantBDataSize(14336, 4096, 4, 128, 1, _lib.DTYPE_FLOAT16)
-    # ... plus, for fp16 models with blocks of 64 and more, a copy in their own width for the decode kernel (N*K/4)
+    # ... plus, for fp16 models with blocks of 32 and more, a copy in their own width for the decode kernel (N*K/4)
     assert lib.MnbPackQuantBDataSize(14336, 4096, 2, 128, 0, _lib.DTYPE_FLOAT16) == four + 14336 * 4096 // 4
-    assert lib.MnbPackQuantBDataSize(14336, 4096, 2, 32, 0, _lib.DTYPE_FLOAT16) == \
-        lib.MnbPackQuantBDataSize(14336, 4096, 4, 32, 1, _lib.DTYPE_FLOAT16)
+    assert lib.MnbPackQuantBDataSize(14336, 4096, 2, 16, 0, _lib.DTYPE_FLOAT16) == \
+        lib.MnbPackQuantBDataSize(14336, 4096, 4, 16, 1, _lib.DTYPE_FLOAT16)
     assert lib.MnbPackQuantBDataSize(14336, 4096, 2, 128, 0, _lib.DTYPE_FLOAT) == \
         lib.MnbPackQuantBDataSize(14336, 4096, 4, 128, 1, _lib.DTYPE_FLOAT)
     assert lib.MnbPackQuantBDataSize(14336, 4096, 4, 32, 1, _lib.DTYPE_FLOAT16) == 14336 * 2048 + 14336 * 128 * 4
