@@ -214,7 +214,7 @@ def test_decode_with_more_slabs_than_compute_units(oracle, bits, bs, zp, N, K, M
 
 @pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (4, 16, True), (8, 64, True), (8, 16, False)])
 @pytest.mark.parametrize("N,K,M", [(28672, 1024, 64), (21000, 1024, 17), (28672, 2048, 32), (24000, 1024, 33),
-                                   (11008, 1024, 100), (14336, 1024, 128), (6144, 1024, 250),
+                                   (11008, 1024, 100), (14336, 4096, 128), (6144, 1024, 250),
                                    (28672, 1152, 64), (21000, 1408, 40)])   # K: 9 and 11 chunks of 128
 def test_streaming_kernel_with_activations_shared_through_lds(oracle, bits, bs, zp, N, K, M):
     """Wide matrices whose 128-column slabs make one well-filled round of workgroups: pairs of wavefronts share each
