@@ -39,6 +39,35 @@ def test_identical_to_oracle(oracle, dtype, bits, bs, symmetric):
         assert np.array_equal(b.cpu().numpy(), Bq), (K, N, "weights")
 
 
+# (rows = K, columns = N, block) of the reference's quantise -> dequantise test, column-wise blocks
+# (onnxruntime/test/mlas/unittest/test_blockq4.cpp:191-229)
+QDQ_SHAPES = [(20, 1, 32), (52, 1, 32), (20, 3, 32), (52, 3, 32), (52, 3, 64), (32 * 9 + 17, 41, 32),
+              (32 * 9 + 17, 41, 64), (32 * 15 + 17, 63, 128), (256, 256, 32)]
+QDQ_TOLERANCE = {8: (1e-2, 5e-2), 4: (6e-2, 2e-1), 2: (2e-1, 5e-1)}   # |a - b| < err + |a| rel (test_blockq4.cpp:55-63)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_reference_round_trip_list(oracle, dtype, bits, symmetric):
+    """MlasBlockwiseQdqTest: weights from U(-1, 1), quantise, dequantise, compare with the reference's tolerance --
+    and every byte of the quantiser's and every bit of the dequantiser's output against the oracle."""
+    err, rel = QDQ_TOLERANCE[bits]
+    for (K, N, bs) in QDQ_SHAPES:
+        rng = np.random.default_rng(192373 + K + N + bs)
+        W = rng.uniform(-1.0, 1.0, size=(K, N)).astype(dtype)
+        b, sc, zp = quantize_blockwise(dev(W), bits, bs, symmetric)
+        w = dequantize_blockwise(b, sc, zp, N, K, bits, bs)
+        torch.cuda.synchronize()
+        Bq, s, z = oracle.C.quantize(W, bits, bs, symmetric)
+        assert np.array_equal(b.cpu().numpy(), Bq) and np.array_equal(_bits(sc.cpu().numpy()), _bits(s)), (K, N, bs)
+        assert (zp is None and z is None) or np.array_equal(zp.cpu().numpy(), z), (K, N, bs)
+        w = w.cpu().numpy()
+        assert np.array_equal(_bits(w), _bits(oracle.C.dequantize(Bq, s, z, N, K, bits, bs))), (K, N, bs)
+        a32, b32 = W.astype(np.float32), w.T.astype(np.float32)
+        assert np.all(np.abs(a32 - b32) < err + np.abs(a32) * rel), (K, N, bs, float(np.abs(a32 - b32).max()))
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("bs", [16, 64, 128])
 @pytest.mark.parametrize("symmetric", [False, True])

@@ -237,3 +237,51 @@ def test_basic_shapes(oracle):
         for option in ("", "zp"):
             for kind in ("f32", "f16"):
                 run_one(oracle, M, 128, 512, 4, 32, kind, option)
+
+
+# ---- the kernel library's own unit-test list (onnxruntime/test/mlas/unittest/test_sqnbitgemm.cpp:467-503) ------------
+def mlas_short_list():
+    """(M, N, K, with_bias) as SQNBitGemmShortExecuteTest registers them for one block length and symmetry."""
+    out = []
+    for b in range(1, 16):
+        out += [(b, b, b, False), (b, b, b, True)]
+    for b in (16, 32, 64, 128, 256):
+        out += [(b, b, b, False), (b, b, b, True)]
+    for b in range(256, 320, 32):
+        out += [(b, b, b, True)]
+    for b in range(1, 96):
+        out += [(1, b, 32, False), (1, 32, b, True), (1, b, b, False)]
+    out += [(43, 500, 401, True), (1, 2, 16, True), (1, 2, 16, False), (1, 1027, 1031, False), (11, 1027, 1031, False),
+            (1, 1027, 1031, True), (11, 1027, 1031, True), (1, 527, 2131, False), (11, 527, 2131, False),
+            (1, 527, 2131, True), (11, 527, 2131, True)]
+    return out
+
+
+def guard_buffer_pattern(n):
+    """The deterministic fill of the unit tests' buffers: 32, 39, 46, ... stepping by 7 and wrapping inside [21, 64)
+    (onnxruntime/test/mlas/unittest/test_util.h:123-138)."""
+    return (((11 + 7 * np.arange(n, dtype=np.int64)) % 43) + 21).astype(np.float32)
+
+
+@pytest.mark.parametrize("symmetric", [False, True])
+@pytest.mark.parametrize("bs", [16, 32, 64, 128, 256])
+def test_kernel_library_unit_test_list(oracle, bs, symmetric):
+    """fp32 activations, 4-bit weights quantised from the unit test's buffers (test_sqnbitgemm.cpp:209-274, 582-586);
+    fp16 on the same list for two block sizes, with A and W scaled by 1/64 so that the sums stay finite."""
+    kinds = ("f32", "f16") if bs in (32, 128) else ("f32",)
+    for (M, N, K, with_bias) in mlas_short_list():
+        for kind in kinds:
+            unit = np.float32(1.0 if kind == "f32" else 1.0 / 64)
+            a32 = guard_buffer_pattern(M * K).reshape(M, K) * unit
+            w32 = guard_buffer_pattern(N * K).reshape(K, N) * unit
+            bias32 = guard_buffer_pattern(N) * unit if with_bias else None
+            b, scales, zp = quantize_blockwise(torch.from_numpy(w32).to(DEV), 4, bs, symmetric=symmetric)
+            torch.cuda.synchronize()
+            B, Z = b.cpu().numpy(), None if zp is None else zp.cpu().numpy()
+            A, sc, bias = to_type(a32, kind), to_type(scales.cpu().numpy(), kind), to_type(bias32, kind)
+            op = MatMulNBits(K, N, 4, bs, dtype=TORCH[kind], has_zero_points=not symmetric, has_bias=with_bias)
+            assert op.PrePack(to_dev(B), to_dev(sc), to_dev(Z))
+            y = op.Compute(to_dev(A), bias=to_dev(bias))
+            torch.cuda.synchronize()
+            case = MatMulNBitsCase(M, N, K, 4, bs, np.dtype(A.dtype), A, B, sc, Z, bias)
+            check_against_oracle(oracle, case, y.cpu().numpy(), nthreads=4)
