@@ -285,3 +285,70 @@ def test_kernel_library_unit_test_list(oracle, bs, symmetric):
             torch.cuda.synchronize()
             case = MatMulNBitsCase(M, N, K, 4, bs, np.dtype(A.dtype), A, B, sc, Z, bias)
             check_against_oracle(oracle, case, y.cpu().numpy(), nthreads=4)
+
+
+# ---- 2-bit weights with zero points that are not integers (matmul_2bits_test.cc:579-1255) --------------------------
+def run_float_zero_points(M, N, K, bs, kind, zp_of, prepacked=True, uint8_zp=None):
+    """W ~ N(0, 0.25) quantised symmetrically to 2 bits, then paired with the zero points the test supplies; the
+    expectation is A x ((q - zp) scale) as the reference computes it (abs 0.1, rel 0.02), and this build's gates:
+    fp32 max |err| <= 1e-4 sum |a w|, fp16 relative L2 <= 5e-3."""
+    rng = np.random.default_rng(1234)
+    a32 = (rng.standard_normal((M, K)) * 0.25).astype(np.float32)
+    w32 = (rng.standard_normal((K, N)) * 0.25).astype(np.float32)
+    b, scales, _ = quantize_blockwise(torch.from_numpy(w32).to(DEV), 2, bs, symmetric=True)
+    torch.cuda.synchronize()
+    kb = (K + bs - 1) // bs
+    B, sc, A = b.cpu().numpy(), to_type(scales.cpu().numpy(), kind), to_type(a32, kind)
+    if uint8_zp is not None:
+        zp_in, zp_dtype = uint8_zp, torch.uint8
+        zp_val = oracle_mod.np_unpack_zp(uint8_zp, N, K, 2, bs).astype(np.float64)
+    else:
+        zp_in = to_type(np.array([[zp_of(n, blk) for blk in range(kb)] for n in range(N)], np.float32), kind)
+        zp_dtype, zp_val = TORCH[kind], to_f32(zp_in).astype(np.float64)
+    op = MatMulNBits(K, N, 2, bs, dtype=TORCH[kind], has_zero_points=True, zero_points_dtype=zp_dtype)
+    assert op.supported
+    if prepacked:
+        assert op.PrePack(to_dev(B), to_dev(sc), to_dev(zp_in))
+        y = op.Compute(to_dev(A))
+    else:   # zero points fed per run (Float32_2b_FloatZP_DynamicZP)
+        y = op.Compute(to_dev(A), to_dev(B), to_dev(sc), to_dev(zp_in))
+    torch.cuda.synchronize()
+    y = y.cpu().numpy().astype(np.float64)
+    q = oracle_mod.np_unpack_q(B, N, K, 2, bs).reshape(N, kb, bs).astype(np.float64)
+    w = ((q - zp_val[:, :, None]) * to_f32(sc).astype(np.float64)[:, :, None]).reshape(N, kb * bs)[:, :K]
+    a64 = to_f32(A).astype(np.float64)
+    expected, bound = a64 @ w.T, np.abs(a64) @ np.abs(w).T
+    err = np.abs(y - expected)
+    assert np.all(err <= 0.1 + 0.02 * np.abs(expected)), (M, N, K, bs, float(err.max()))
+    if kind == "f32":
+        assert float(np.max(err / (bound + 1e-30))) <= 1e-4, (M, N, K, bs)
+    else:
+        assert float(np.linalg.norm(err) / np.linalg.norm(expected)) <= 5e-3, (M, N, K, bs)
+
+
+def test_two_bit_float_zero_points():
+    # Float32_2b_FloatZP_QAD: zp = 1.5 maps {0, 1, 2, 3} to {-1, -1/3, 1/3, 1} x scale
+    for (M, N, K, bs, zp) in [(1, 128, 128, 32, 1.5), (1, 256, 256, 64, 1.5), (1, 128, 128, 32, 0.0),
+                              (1, 128, 128, 32, 2.0), (1, 128, 128, 32, 3.0)]:
+        run_float_zero_points(M, N, K, bs, "f32", lambda n, blk, zp=zp: zp)
+    # Float32_2b_FloatZP_VaryingPerBlock and _DynamicZP: a different zero point for every (column, block)
+    varying = lambda n, blk: 0.25 + 0.5 * blk + 0.01 * (n % 17)
+    run_float_zero_points(1, 128, 128, 32, "f32", varying)
+    run_float_zero_points(1, 128, 128, 32, "f32", varying, prepacked=False)
+    # Float32_2b_FloatZP_Fallback, _Fallback_NonAlignedK, MLFloat16_2b_MLFloat16ZP_Fallback
+    run_float_zero_points(1, 32, 32, 16, "f32", lambda n, blk: 1.5)
+    run_float_zero_points(1, 32, 48, 32, "f32", lambda n, blk: 1.5)
+    run_float_zero_points(1, 32, 32, 16, "f16", lambda n, blk: 1.5)
+
+
+def test_two_bit_uint8_zero_points_that_vary():
+    """MLFloat16_2b_Uint8ZP_Fallback and _Accuracy4 (matmul_2bits_test.cc:1102-1255): packed 2-bit zero points, the
+    second test with bytes (hi << 4) | lo, lo = 3 i mod 4, hi = (5 i + 1) mod 4, so that they differ from the default."""
+    N, K, bs = 32, 32, 16
+    rng = np.random.default_rng(7)
+    run_float_zero_points(1, N, K, bs, "f16", None, uint8_zp=rng.integers(0, 256, (N, 1), dtype=np.uint8))
+    N, K, bs = 32, 128, 64
+    i = np.arange(N)
+    zp = ((((5 * i + 1) % 4) << 4) | ((3 * i) % 4)).astype(np.uint8).reshape(N, 1)
+    run_float_zero_points(1, N, K, bs, "f16", None, uint8_zp=zp)
+    run_float_zero_points(1, N, K, bs, "f32", None, uint8_zp=zp)
