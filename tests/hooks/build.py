@@ -17,24 +17,39 @@ LIB = HERE / "libmnb_test_hooks.so"
 HOOKED = "mnb_gemm256.hip"
 
 
-def build() -> Path:
+def _product():
     sys.path.insert(0, str(HERE.parent.parent))
     from onnxruntime_amd import build as B
+    return B
+
+
+def compile_hooked() -> Path:
+    """The one object that differs from the product's (needs no product object, so it can run beside that build)."""
+    B = _product()
+    B.OBJ_DIR.mkdir(exist_ok=True)
+    obj = B.OBJ_DIR / (HOOKED + ".hooks.o")
+    cmd = [B.hipcc(), *B.HIPCC_FLAGS, *B.EXTRA_FLAGS.get(HOOKED, []), "-DMNB_TEST_HOOKS", "-c", str(B.CSRC / HOOKED),
+           "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {HOOKED} (test hooks):\n{r.stderr}")
+    return obj
+
+
+def link(hooked: Path) -> Path:
+    B = _product()
     objs = []
     for src in B.SOURCES:
-        obj = B.OBJ_DIR / (src + ".o")
-        if src == HOOKED:
-            obj = B.OBJ_DIR / (src + ".hooks.o")
-            cmd = [B.hipcc(), *B.HIPCC_FLAGS, *B.EXTRA_FLAGS.get(src, []), "-DMNB_TEST_HOOKS", "-c", str(B.CSRC / src),
-                   "-o", str(obj)]
-            r = subprocess.run(cmd, capture_output=True, text=True)
-            if r.returncode != 0:
-                raise RuntimeError(f"hipcc failed on {src} (test hooks):\n{r.stderr}")
-        elif not obj.exists():
+        obj = hooked if src == HOOKED else B.OBJ_DIR / (src + ".o")
+        if not obj.exists():
             raise RuntimeError(f"{obj} is missing: build the product library first (python -m onnxruntime_amd.build)")
         objs.append(str(obj))
     subprocess.check_call([B.hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *objs])
     return LIB
+
+
+def build() -> Path:
+    return link(compile_hooked())
 
 
 if __name__ == "__main__":
