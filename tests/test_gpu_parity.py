@@ -265,11 +265,14 @@ def test_fp32_few_rows_with_k_split_over_sixteen_wavefronts(oracle, bits, bs, zp
     assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
 
 
-def test_unpacked_route_matches_packed():
+def test_unpacked_route_matches_packed_and_the_oracle(oracle):
     for dtype in (np.float16, np.float32):
-        for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128)]:
+        for (M, N, K, bits, bs) in [(1, 96, 160, 4, 32), (40, 200, 256, 8, 64), (16, 64, 4096, 4, 128),
+                                    (3, 33, 93, 2, 16), (70, 130, 1234, 4, 16)]:
             c = make_case(M, N, K, bits, bs, dtype, has_zp=True, has_bias=True, seed=4)
-            assert np.array_equal(run_case(c, prepack=True), run_case(c, prepack=False))
+            y = run_case(c, prepack=False)
+            assert np.array_equal(run_case(c, prepack=True), y)
+            check_against_oracle(oracle, c, y)
 
 
 def test_batched_leading_dims_and_strided_a(oracle):
