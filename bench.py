@@ -144,6 +144,8 @@ def load_probe():
     lib.MnbProbeReadBandwidthResident.argtypes = lib.MnbProbeReadBandwidth.argtypes
     lib.MnbProbeMfmaRate.restype = ctypes.c_int
     lib.MnbProbeMfmaRate.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    lib.MnbProbeMfmaRateOperands.restype = ctypes.c_int
+    lib.MnbProbeMfmaRateOperands.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
     lib.MnbProbeIssueOverlap.restype = ctypes.c_int
     lib.MnbProbeIssueOverlap.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                          ctypes.POINTER(ctypes.c_double)]
@@ -390,6 +392,15 @@ def main() -> int:
             mfma_const = v.value
             assert probe.MnbProbeMfmaRate(1, ctypes.byref(v)) == 0
             mfma_rand = v.value
+            # the same loop on the operand classes of this kernel: A bell-shaped activations (class 3), B what the
+            # kernel feeds (dequantised weights with a scale per column, class 4), what it would feed if the scale were
+            # applied to the sums instead (integers, 5; the decode kernel's raw halves, 6), and zeros
+            by_class = {}
+            for name, (ca, cb) in {"activations_x_dequantised_weights": (3, 4), "activations_x_integer_weights": (3, 5),
+                                   "activations_x_raw_magic_halves": (3, 6), "dequantised_weights_x_activations": (4, 3),
+                                   "zero_x_dequantised_weights": (2, 4)}.items():
+                assert probe.MnbProbeMfmaRateOperands(ca, cb, ctypes.byref(v)) == 0
+                by_class[name] = round(v.value, 1)
             # the same kernel, same launches, on activations that are all zero: the instruction stream is identical,
             # only the switching activity of the operands (and with it the clock the power limit allows) differs
             a_saved = p4.a.clone()
@@ -429,6 +440,9 @@ def main() -> int:
                 "mfma_only_loop_constant_operands_TFLOPs": round(mfma_const, 1),
                 "mfma_only_loop_random_operands_TFLOPs": round(mfma_rand, 1),
                 "frac_of_mfma_only_random": round(tflops / mfma_rand, 4) if mfma_rand > 0 else None,
+                "mfma_only_loop_TFLOPs_by_operand_class": by_class,
+                "frac_of_mfma_only_on_this_kernels_operands": round(
+                    tflops / by_class["activations_x_dequantised_weights"], 4),
                 "same_kernel_zero_activations_TFLOPs": round(tflops_zero, 1),
                 "same_kernel_zero_activations_ms_per_launch": round(ms4_zero, 4),
                 "shader_clock_ghz_during_these_launches": clock_random,

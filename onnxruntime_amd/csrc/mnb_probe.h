@@ -31,6 +31,12 @@ MNB_PROBE_API void MnbProbeRelease(void);
 /* TFLOP/s of a loop of nothing but v_mfma_f32_32x32x16_f16 on every CU, with constant operands
  * (random_operands = 0) or random fp16 operands (1): the sustained matrix-core clock depends on operand toggling. */
 MNB_PROBE_API int MnbProbeMfmaRate(int random_operands, double* tflops);
+/* The same loop with the value class of each operand chosen (A = the first, B = the second source of the matrix
+ * instruction): 0 the constant 1, 1 uniform in (-1, 1), 2 zero, 3 bell-shaped with variance 1 (activations),
+ * 4 dequantised 4-bit weights (q - 8) * scale with a scale per column (what the prefill kernel feeds as B),
+ * 5 the integers q - 8, 6 the raw halves 1024 + q (what the decode kernel feeds), 7 a 4-bit grid under one scale.
+ * The instruction stream is the same for every class; only the operands' significant bits differ. */
+MNB_PROBE_API int MnbProbeMfmaRateOperands(int a_class, int b_class, double* tflops);
 
 /* Nanoseconds per "slot" of a loop that every wavefront of the chip runs (waves_per_simd = 1 or 2 wavefronts on each
  * SIMD): a slot is one v_mfma_f32_32x32x16_f16 (when with_mfma) followed by valu_per_mfma (0, 1, 2, 4, 8) independent

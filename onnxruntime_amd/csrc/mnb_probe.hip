@@ -35,8 +35,32 @@ __global__ void mnb_probe_read_kernel(const uint4* __restrict__ p, float* out, s
   if (s == 0x12345678u) out[0] = 1.f;  // keeps the loads alive; practically never taken
 }
 
-template <int RANDOM>
-__global__ void __launch_bounds__(512, 2) mnb_probe_mfma_kernel(float* out, int iters) {
+// Values of one operand class (MnbProbeMfmaRateOperands): what the matrix cores see decides their switching activity,
+// and with it the clock the power limit allows.
+__device__ __forceinline__ _Float16 mnb_probe_operand(int kind, uint32_t x, int lane) {
+  const float u = (float)(x >> 8) * (1.0f / 8388608.0f) - 1.0f;  // U(-1, 1)
+  const int q = (x >> 8) & 15;
+  switch (kind) {
+    case 1: return (_Float16)u;
+    case 2: return (_Float16)0.0f;
+    case 3: {  // sum of three uniforms: bell-shaped, variance 1
+      uint32_t y = x * 747796405u + 2891336453u;
+      float v = u + ((float)(y >> 8) * (1.0f / 8388608.0f) - 1.0f);
+      y = y * 747796405u + 2891336453u;
+      return (_Float16)(v + ((float)(y >> 8) * (1.0f / 8388608.0f) - 1.0f));
+    }
+    case 4: {  // a dequantised 4-bit weight: (q - 8) times the scale of the lane's column
+      const float s = 0.005f + 0.01f * (float)(((uint32_t)lane * 2654435761u >> 20) & 1023) * (1.0f / 1024.0f);
+      return (_Float16)((float)(q - 8) * s);
+    }
+    case 5: return (_Float16)(float)(q - 8);     // the same weight before its scale: four significant bits
+    case 6: return (_Float16)(float)(1024 + q);  // the raw "magic" half the decode kernel feeds
+    case 7: return (_Float16)((float)q * 0.01f - 0.08f);  // 4-bit grid under one scale
+    default: return (_Float16)1.0f;
+  }
+}
+
+__global__ void __launch_bounds__(512, 2) mnb_probe_mfma_kernel(float* out, int iters, int kind_a, int kind_b) {
   f16_t acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
@@ -47,12 +71,12 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_mfma_kernel(float* out, int 
   for (int t = 0; t < 4; ++t)
     for (int i = 0; i < 8; ++i) {
       x = x * 1664525u + 1013904223u;
-      a[t][i] = RANDOM ? (_Float16)((float)(x >> 8) * (1.0f / 8388608.0f) - 1.0f) : (_Float16)1.0f;  // U(-1, 1)
+      a[t][i] = mnb_probe_operand(kind_a, x, threadIdx.x & 63);
     }
   for (int t = 0; t < 2; ++t)
     for (int i = 0; i < 8; ++i) {
       x = x * 1664525u + 1013904223u;
-      b[t][i] = RANDOM ? (_Float16)((float)((x >> 8) & 15) * 0.01f - 0.08f) : (_Float16)0.5f;  // 4-bit grid
+      b[t][i] = mnb_probe_operand(kind_b, x, threadIdx.x & 63);
     }
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
@@ -60,6 +84,12 @@ __global__ void __launch_bounds__(512, 2) mnb_probe_mfma_kernel(float* out, int 
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         acc[i * 2 + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i * 2 + j], 0, 0, 0);
+    if ((it & 63) == 63) {  // keeps the sums finite whatever the operands are
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] *= 0.0009765625f;
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -294,7 +324,7 @@ hipError_t probe_read(size_t bytes, int launches, int threads, int loads_in_flig
   return err;
 }
 
-hipError_t probe_mfma(int random_operands, double* tflops) {
+hipError_t probe_mfma(int kind_a, int kind_b, double* tflops) {
   *tflops = 0.0;
   int dev = 0, cus = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -307,12 +337,7 @@ hipError_t probe_mfma(int random_operands, double* tflops) {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   // From idle the matrix-core clock needs about 15 ms of load to settle: one untimed launch of 25 ms, then the timed one.
   const int iters = 100000;
-  auto launch = [&](int n) {
-    if (random_operands)
-      mnb_probe_mfma_kernel<1><<<cus, 512, 0, nullptr>>>(out, n);
-    else
-      mnb_probe_mfma_kernel<0><<<cus, 512, 0, nullptr>>>(out, n);
-  };
+  auto launch = [&](int n) { mnb_probe_mfma_kernel<<<cus, 512, 0, nullptr>>>(out, n, kind_a, kind_b); };
   if ((err = hipEventCreate(&e0)) == hipSuccess && (err = hipEventCreate(&e1)) == hipSuccess) {
     launch(iters);
     if ((err = hipDeviceSynchronize()) == hipSuccess) {
@@ -481,7 +506,13 @@ void MnbProbeRelease(void) { release_buffers(); }
 
 int MnbProbeMfmaRate(int random_operands, double* tflops) {
   if (!tflops) return 2;
-  return probe_mfma(random_operands, tflops) == hipSuccess ? 0 : 1;
+  // (random: uniform activations against a 4-bit grid under one scale, as this probe has always run)
+  return probe_mfma(random_operands ? 1 : 0, random_operands ? 7 : 0, tflops) == hipSuccess ? 0 : 1;
+}
+
+int MnbProbeMfmaRateOperands(int a_class, int b_class, double* tflops) {
+  if (!tflops || a_class < 0 || a_class > 7 || b_class < 0 || b_class > 7) return 2;
+  return probe_mfma(a_class, b_class, tflops) == hipSuccess ? 0 : 1;
 }
 
 int MnbProbeIssueOverlap(int valu_per_mfma, int with_mfma, int waves_per_simd, int lds_reads_per_two_mfma,
