@@ -136,5 +136,54 @@ def ab(argv):
             flush=True)
 
 
+def stamps(argv):
+    """Anatomy of a direct decode launch from a library built with -DMNB_STAMPS: M N K BITS BLOCK ZP [COPIES].
+    A HIP graph of COPIES launches over as many copies of the packed matrix is replayed; the readings are those of
+    its last launch (100 MHz counter: 10 ns steps), printed relative to the first wavefront's entry."""
+    lib = load(argv[0])
+    lib.MnbCalibrationReadStamps.restype = ctypes.c_int
+    lib.MnbCalibrationReadStamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    M, N, K, bits, bs, zp = map(int, argv[1:7])
+    copies = int(argv[7]) if len(argv) > 7 else 32
+    call, _ = Problem(M, N, K, bits, bs, bool(zp), bias=False, copies=copies).caller(lib)
+    print("kernel:", lib.MnbGemmKernelName(M, N, K, bits, bs, _lib.DTYPE_FLOAT16).decode(), flush=True)
+    assert call() == 0
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(copies):
+            assert call() == 0
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    print(f"{e0.elapsed_time(e1) / copies * 1e3:.2f} us per launch with the readings compiled in", flush=True)
+    points, waves, groups = 8, 16, 4096
+    buf = np.zeros(groups * waves * points, dtype=np.uint64)
+    assert lib.MnbCalibrationReadStamps(buf.ctypes.data_as(ctypes.c_void_p), buf.size) == 0
+    t = buf.reshape(groups, waves, points).astype(np.int64)
+    live = t[:, :, 0] != 0
+    t0 = t[:, :, 0][live].min()
+    us = (t - t0) / 100.0
+    names = ["entry", "loads issued", "first chunk computed", "last chunk computed", "partials in LDS",
+             "past the barrier", "sums stored"]
+    print(f"{int(live.sum())} wavefronts in {int(live.any(axis=1).sum())} workgroups; microseconds after the first entry")
+    print(f"{'point':24s} {'min':>7s} {'p10':>7s} {'median':>7s} {'p90':>7s} {'max':>7s}")
+    for i, name in enumerate(names):
+        v = us[:, :, i][live]
+        print(f"{name:24s} {v.min():7.2f} {np.percentile(v, 10):7.2f} {np.median(v):7.2f} {np.percentile(v, 90):7.2f} "
+              f"{v.max():7.2f}")
+    ends = np.where(live, us[:, :, 6], -1).max(axis=1)
+    ends = ends[live.any(axis=1)]
+    print(f"workgroup ends: min {ends.min():.2f}  median {np.median(ends):.2f}  max {ends.max():.2f}")
+    lag = (us[:, :, 5] - us[:, :, 4])[live]
+    print(f"wait at the barrier per wavefront: median {np.median(lag):.2f}  p90 {np.percentile(lag, 90):.2f}  "
+          f"max {lag.max():.2f}")
+
+
 if __name__ == "__main__":
-    {"one": one, "ab": ab}[sys.argv[1]](sys.argv[2:])
+    {"one": one, "ab": ab, "stamps": stamps}[sys.argv[1]](sys.argv[2:])

@@ -41,6 +41,29 @@
 
 #include "mnb_mfma16_common.hip.h"
 
+#if defined(MNB_STAMPS)
+// Calibration builds (-DMNB_STAMPS): every wavefront of the direct decode kernels reads the constant 100 MHz counter
+// at seven points of its life and leaves the readings in a device array, [workgroup][wavefront][point], which
+// MnbCalibrationReadStamps copies out: 0 entry, 1 all loads of the first chunks issued, 2 first chunk computed,
+// 3 last chunk computed, 4 partial sums written to LDS, 5 past the barrier, 6 sums read back and stores issued.
+// (The scheduling barriers around a reading keep it where it is written; they also keep the load block in front of
+// the arithmetic, which the product build leaves to the scheduler -- measured: no difference in time.)
+constexpr int kStampPoints = 8, kStampWaves = 16, kStampGroups = 4096;
+__device__ unsigned long long mnb_stamps[kStampGroups * kStampWaves * kStampPoints];
+#define MNB_STAMP_PARAM , unsigned long long* stamp
+#define MNB_STAMP_ARG , stamp
+#define MNB_STAMP(i)                                      \
+  do {                                                    \
+    __builtin_amdgcn_sched_barrier(0);                    \
+    stamp[i] = __builtin_amdgcn_s_memrealtime();          \
+    __builtin_amdgcn_sched_barrier(0);                    \
+  } while (0)
+#else
+#define MNB_STAMP_PARAM
+#define MNB_STAMP_ARG
+#define MNB_STAMP(i)
+#endif
+
 namespace {
 
 template <int BITS, bool HAS_ZP, int MODE>
@@ -230,7 +253,7 @@ __device__ __forceinline__ void compute_chunk(const ChunkRegs<BITS, T>& R, const
 // Lane (j, kq), register r of tile t holds row 4*kq + r, column n0 + 16 t + j; only rows < M travel.
 template <int T, int NW>
 __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* red, const f4_t* y, int wave, int lane,
-                                                int64_t n0) {
+                                                int64_t n0 MNB_STAMP_PARAM) {
   const int kq = lane >> 4;
 #if defined(MNB_ABLATE_NO_REDUCE)
   // calibration builds: no exchange through LDS, no barrier; the first wavefront stores its own partial sums (what the
@@ -251,8 +274,11 @@ __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* re
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       if (4 * kq + r < p.M) red[(wave * T * 4 + t * 4 + r) * 64 + lane] = y[t][r];
+  MNB_STAMP(4);
   __syncthreads();
+  MNB_STAMP(5);
   reduce_and_store_tiles<T, NW>(p, red, 0, n0);
+  MNB_STAMP(6);
 }
 
 // ---- activations through LDS for 4 < M <= 16 -----------------------------------------------------------------------
@@ -305,7 +331,7 @@ struct AStage {
 // its own vector has landed.  CPW = 0: general loop with two chunks in flight.
 template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS, class LoadW>
 __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned char* smem, int wave, int lane,
-                                              const LoadW& load_w, f4_t* y) {
+                                              const LoadW& load_w, f4_t* y MNB_STAMP_PARAM) {
   constexpr int GK = 128 / BITS;
   constexpr int NI = GK / 8;
   const int j = lane & 15, kq = lane >> 4;
@@ -345,6 +371,7 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
     for (int q = 0; q < CPW; ++q) fetch_a(wave + q * NW, a[q]);
 #pragma unroll
     for (int q = 0; q < CPW; ++q) load_w(wave + q * NW, R[q]);
+    MNB_STAMP(1);
     if constexpr (A_LDS) {
       h8_t af[CPW][NI];
 #pragma unroll
@@ -353,8 +380,12 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
       for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], af[q], bconst, uc, uc2, y);
     } else {
 #pragma unroll
-      for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, uc2, y);
+      for (int q = 0; q < CPW; ++q) {
+        compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], a[q], bconst, uc, uc2, y);
+        if (q == 0) MNB_STAMP(2);
+      }
     }
+    MNB_STAMP(3);
   } else if constexpr (T <= 2) {
     // Two chunks in flight.  Loads under a run-time condition would leave the compiler unable to count the
     // outstanding loads at the join, and every wait of the loop would then be for all of them, the prefetch issued
@@ -457,10 +488,20 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(MNB_SKINNY_H
   f4_t y[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+#if defined(MNB_STAMPS)
+  unsigned long long stamp[kStampPoints] = {};
+  MNB_STAMP(0);
+#endif
   skinny_chunks<BITS, HAS_ZP, MODE, T, NW, CPW, A_LDS>(
       p, smem, wave, lane,
-      [&](int c, ChunkRegs<BITS, T>& R) { load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R); }, y);
-  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
+      [&](int c, ChunkRegs<BITS, T>& R) { load_chunk<BITS, HAS_ZP, MODE, T>(p, c, kq, col0, R); }, y MNB_STAMP_ARG);
+  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0 MNB_STAMP_ARG);
+#if defined(MNB_STAMPS)
+  if (lane == 0 && blockIdx.x < kStampGroups && wave < kStampWaves)
+#pragma unroll
+    for (int i = 0; i < kStampPoints; ++i)
+      mnb_stamps[((size_t)blockIdx.x * kStampWaves + wave) * kStampPoints + i] = stamp[i];
+#endif
 }
 
 // ---- direct variant for slabs of three tiles ----------------------------------------------------------------------
@@ -490,10 +531,14 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(MNB_SKINNY_HOT
   f4_t y[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) y[t] = f4_t{0.f, 0.f, 0.f, 0.f};
+#if defined(MNB_STAMPS)
+  unsigned long long stamp[kStampPoints] = {};  // (only the kernel above keeps its readings)
+#endif
   skinny_chunks<BITS, HAS_ZP, MODE, T, NW, CPW, A_LDS>(
       p, smem, wave, lane,
-      [&](int c, ChunkRegs<BITS, T>& R) { load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c, kq, colw, mcol, R); }, y);
-  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
+      [&](int c, ChunkRegs<BITS, T>& R) { load_chunk_cols<BITS, HAS_ZP, MODE, T>(p, c, kq, colw, mcol, R); },
+      y MNB_STAMP_ARG);
+  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0 MNB_STAMP_ARG);
 }
 
 // ---- staged variant: any alignment of A; rows staged in LDS phase by phase -------------------------------------
@@ -550,7 +595,10 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
     }
   }
   __syncthreads();
-  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0);
+#if defined(MNB_STAMPS)
+  unsigned long long stamp[kStampPoints] = {};
+#endif
+  skinny_epilogue<T, NW>(p, reinterpret_cast<float*>(smem), y, wave, lane, n0 MNB_STAMP_ARG);
 }
 
 struct SkinnyPlan {
@@ -843,3 +891,13 @@ hipError_t mnb_launch_skinny(const MnbGemmArgs& a, hipStream_t s) {
   if (L.bits == 4) return L.has_zp ? launch_zp<4, true>(p, pl, s) : launch_zp<4, false>(p, pl, s);
   return L.has_zp ? launch_zp<8, true>(p, pl, s) : launch_zp<8, false>(p, pl, s);
 }
+
+#if defined(MNB_STAMPS)
+// Copies the readings of the last direct decode launch out (count = number of 64-bit values, at most the array's).
+extern "C" __attribute__((visibility("default"))) int MnbCalibrationReadStamps(unsigned long long* dst, size_t count) {
+  if (!dst || count > (size_t)kStampGroups * kStampWaves * kStampPoints) return 2;
+  if (hipDeviceSynchronize() != hipSuccess) return 1;
+  return hipMemcpyFromSymbol(dst, HIP_SYMBOL(mnb_stamps), count * sizeof(unsigned long long), 0,
+                             hipMemcpyDeviceToHost) == hipSuccess ? 0 : 1;
+}
+#endif
