@@ -174,6 +174,9 @@ def stamps(argv):
     print(f"{int(live.sum())} wavefronts in {int(live.any(axis=1).sum())} workgroups; microseconds after the first entry")
     print(f"{'point':24s} {'min':>7s} {'p10':>7s} {'median':>7s} {'p90':>7s} {'max':>7s}")
     for i, name in enumerate(names):
+        if not (t[:, :, i][live] != 0).all():   # (points 1-3 exist only where a wavefront's chunks are straight-line code)
+            print(f"{name:24s} not recorded by this instantiation")
+            continue
         v = us[:, :, i][live]
         print(f"{name:24s} {v.min():7.2f} {np.percentile(v, 10):7.2f} {np.median(v):7.2f} {np.percentile(v, 90):7.2f} "
               f"{v.max():7.2f}")
