@@ -289,29 +289,37 @@ __device__ __forceinline__ void skinny_epilogue(const SkinnyParams& p, float* re
 // through a private 4 KiB of LDS and picks its operands up from there.  No barrier is involved: the region belongs
 // to one wavefront and LDS executes a wavefront's accesses in order.  16-byte pieces are XOR-swizzled with the row
 // so that both the row-contiguous writes and the operand reads are free of bank conflicts.
-template <int BITS>
+// Up to four rows take the same road for another reason: read straight from A, a chunk costs a wavefront one load
+// instruction per operand (four for 4-bit weights) that all fetch the same few bytes sixteen times over, and on
+// single- and two-tile slabs those instructions outnumber the weight loads and fill the memory pipeline (measured
+// without them: N = 4096, K = 14336 10.4 -> 8.7 us at one row, 11.3 -> 8.8 us at four).  With ROWS = 4 one
+// instruction fetches the chunk of all four rows (two for 2-bit weights) and LDS hands the operands out.
+template <int BITS, int ROWS = 16>
 struct AStage {
   static constexpr int GK = 128 / BITS, NI = GK / 8;
   static constexpr int PIECES = 4 * NI;     // 16-byte pieces per row of a chunk
   static constexpr int RPI = 64 / PIECES;   // rows per load instruction; 16 / RPI == NI instructions
+  static constexpr int LOADS = (ROWS + RPI - 1) / RPI;  // load instructions per chunk
+  static constexpr int HELD = LOADS * RPI < 16 ? LOADS * RPI : 16;  // rows that pass through LDS
   static __device__ __forceinline__ int swz(int row) { return PIECES == 16 ? row : (row >> 1); }
 
   // global -> registers: g[I] = piece (lane % PIECES) of row I * RPI + lane / PIECES (rows >= M re-read row M - 1)
   static __device__ __forceinline__ void fetch(const SkinnyParams& p, int c, int lane, h8_t* g) {
     const int piece = lane % PIECES, r0 = lane / PIECES;
 #pragma unroll
-    for (int I = 0; I < NI; ++I) {
+    for (int I = 0; I < LOADS; ++I) {
       int row = I * RPI + r0;
       row = row < p.M ? row : p.M - 1;
       g[I] = *reinterpret_cast<const h8_t*>(p.A + (int64_t)row * p.lda + (int64_t)c * 4 * GK + piece * 8);
     }
   }
-  // registers -> LDS -> operands of lane (j, kq)
+  // registers -> LDS -> operands of lane (j, kq); rows the matrix instruction has beyond those held repeat them
+  // (they are never stored)
   static __device__ __forceinline__ void pass(h8_t* mine, const h8_t* g, int lane, h8_t* af) {
     const int piece = lane % PIECES, r0 = lane / PIECES;
-    const int j = lane & 15, kq = lane >> 4;
+    const int j = (lane & 15) % HELD, kq = lane >> 4;
 #pragma unroll
-    for (int I = 0; I < NI; ++I) {
+    for (int I = 0; I < LOADS; ++I) {
       const int row = I * RPI + r0;
       mine[row * PIECES + (piece ^ swz(row))] = g[I];
     }
@@ -329,35 +337,45 @@ struct AStage {
 // CPW = chunks per wavefront when that is 1 or 2 for every wavefront (chunks == CPW * NW): everything is loaded up
 // front in straight-line code, so the compiler's s_waitcnt counts are exact and each tile is processed as soon as
 // its own vector has landed.  CPW = 0: general loop with two chunks in flight.
-template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS, class LoadW>
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, int A_LDS, class LoadW>
 __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned char* smem, int wave, int lane,
                                               const LoadW& load_w, f4_t* y MNB_STAMP_PARAM) {
   constexpr int GK = 128 / BITS;
   constexpr int NI = GK / 8;
+  using Stage = AStage<BITS, A_LDS == 0 ? 16 : A_LDS>;  // A_LDS: rows of a chunk that pass through LDS (4, 8, 16), 0 = operands straight from A
   const int j = lane & 15, kq = lane >> 4;
   const int arow = j < p.M ? j : p.M - 1;  // rows >= M of the MFMA A operand re-read row M-1: they are never stored
   // first k of the lane's operands inside a chunk: kq GK, or for 2-bit vectors 32 kq in each half of the chunk
   const _Float16* arow_ptr = p.A + (int64_t)arow * p.lda + kq * (BITS == 2 ? 32 : GK);
-  h8_t* mine = reinterpret_cast<h8_t*>(smem) + wave * (16 * AStage<BITS>::PIECES);  // A_LDS only
+  h8_t* mine = reinterpret_cast<h8_t*>(smem) + wave * (16 * Stage::PIECES);  // A_LDS only
   const BConst bconst = bconst_of_mode<BITS, HAS_ZP, MODE>();
   const UnpackConsts uc = make_unpack_consts();
   const UnpackConsts2 uc2 = make_unpack_consts2();  // (2-bit weights; unused moves are dropped)
 
   // the activation loads of chunk c: the operands themselves, or the row-contiguous pieces that pass through LDS
   auto fetch_a = [&](int c, h8_t* a) {
-    if constexpr (A_LDS) {
-      AStage<BITS>::fetch(p, c, lane, a);
+    if constexpr (A_LDS != 0) {
+      Stage::fetch(p, c, lane, a);
     } else {
+#if defined(MNB_ABLATE_NO_A_LOADS)
+      // calibration builds: no activation loads (what they cost a launch; the result is wrong)
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const uint32_t v = 0x3c003c00u + (uint32_t)c;
+        a[i] = __builtin_bit_cast(h8_t, u4_t{v, v, v, v});
+      }
+#else
 #pragma unroll
       for (int i = 0; i < NI; ++i)
         a[i] = *reinterpret_cast<const h8_t*>(arow_ptr + (int64_t)c * 4 * GK +
                                               (BITS == 2 ? (i >> 2) * 128 + (i & 3) * 8 : 8 * i));
+#endif
     }
   };
   auto run = [&](const ChunkRegs<BITS, T>& R, const h8_t* a) {
-    if constexpr (A_LDS) {
+    if constexpr (A_LDS != 0) {
       h8_t af[NI];
-      AStage<BITS>::pass(mine, a, lane, af);
+      Stage::pass(mine, a, lane, af);
       compute_chunk<BITS, HAS_ZP, MODE, T>(R, af, bconst, uc, uc2, y);
     } else {
       compute_chunk<BITS, HAS_ZP, MODE, T>(R, a, bconst, uc, uc2, y);
@@ -372,10 +390,10 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
 #pragma unroll
     for (int q = 0; q < CPW; ++q) load_w(wave + q * NW, R[q]);
     MNB_STAMP(1);
-    if constexpr (A_LDS) {
+    if constexpr (A_LDS != 0) {
       h8_t af[CPW][NI];
 #pragma unroll
-      for (int q = 0; q < CPW; ++q) AStage<BITS>::pass(mine, a[q], lane, af[q]);
+      for (int q = 0; q < CPW; ++q) Stage::pass(mine, a[q], lane, af[q]);
 #pragma unroll
       for (int q = 0; q < CPW; ++q) compute_chunk<BITS, HAS_ZP, MODE, T>(R[q], af[q], bconst, uc, uc2, y);
     } else {
@@ -452,7 +470,7 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
       }
     }
   }
-  if constexpr (A_LDS) __syncthreads();  // the reduction buffer overlays the staging regions of all wavefronts
+  if constexpr (A_LDS != 0) __syncthreads();  // the reduction buffer overlays the staging regions of all wavefronts
 }
 
 // What a wavefront needs to issue its first loads comes as leading scalar kernel arguments, which the build asks the
@@ -476,7 +494,7 @@ __device__ __forceinline__ SkinnyParams with_hot_params(SkinnyParams p, MNB_SKIN
 }
 #define MNB_SKINNY_HOT_NAMES hot_W, hot_Npad, hot_A, hot_lda, hot_meta, hot_M, hot_chunks, hot_bs_shift
 
-template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS>
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, int A_LDS>
 __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(MNB_SKINNY_HOT_PARAMS, SkinnyParams rest) {
   const SkinnyParams p = with_hot_params(rest, MNB_SKINNY_HOT_NAMES);
   extern __shared__ __align__(16) unsigned char smem[];
@@ -512,7 +530,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_direct_kernel(MNB_SKINNY_H
 // (Slabs with half a tile at the end - 56 columns for N = 14336, which would put exactly one workgroup on every
 // compute unit - were measured too: the half tile costs the instructions of a whole one, and the run time did not
 // improve.)
-template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, bool A_LDS>
+template <int BITS, bool HAS_ZP, int MODE, int T, int NW, int CPW, int A_LDS>
 __global__ void __launch_bounds__(NW * 64) mnb_skinny_slab_kernel(MNB_SKINNY_HOT_PARAMS, SkinnyParams rest) {
   const SkinnyParams p = with_hot_params(rest, MNB_SKINNY_HOT_NAMES);
   extern __shared__ __align__(16) unsigned char smem[];
@@ -603,7 +621,7 @@ __global__ void __launch_bounds__(NW * 64) mnb_skinny_staged_kernel(SkinnyParams
 
 struct SkinnyPlan {
   int mode, t, nw, phase_chunks, mtr;
-  bool a_lds;  // activations row-contiguously through LDS (more than four rows, one or two chunks per wavefront)
+  int a_lds;   // rows of a chunk of the activations that pass through LDS: 0 (operands read straight from A), 4, 8 or 16
   size_t smem;
 };
 
@@ -690,10 +708,36 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   // of 4-bit weights cannot hold in their 128 registers: those run with eight (K = 14336, M = 16: 20 -> 13 us).
   static const int a_lds_from = mnb_tuning_env("MNB_SKINNY_ALDS_FROM") ? atoi(mnb_tuning_env("MNB_SKINNY_ALDS_FROM")) : 5;
   const bool up_front = chunks == pl.nw || chunks == 2 * pl.nw;  // everything loaded before the first wait
-  pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4);
+  pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4) ? 16 : 0;
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
   // the fp32 scales and zero points of modes 2 to 4 do not fit the 128 registers of sixteen wavefronts in the general loop
   if (pl.mode >= 2 && !up_front && pl.nw == 16) pl.nw = 8;
+  // Up to eight rows on single- and two-tile slabs: read straight from A, a chunk costs a wavefront one load
+  // instruction per operand, and on these slabs those loads outnumber the weight loads and fill the memory pipeline.
+  // AStage with four or eight rows fetches the chunk of all rows with one or two instructions and hands the operands
+  // out through LDS; bit-identical results.  Measured, weights from HBM, zero points, 4-bit blocks of 128 unless noted:
+  //   N = 4096, K = 14336   1 / 2 / 4 rows 10.4 / 10.6 / 11.3 -> 9.0 us; 5 / 8 rows (were sixteen rows through LDS)
+  //                         10.7 -> 9.6, 10.8 -> 10.2; blocks of 64 11.9 -> 9.9 (8 rows 12.1 -> 11.0); 2-bit 9.3 -> 7.3
+  //                         (8 rows 11.0 -> 9.0); 8-bit 13.8 -> 13.5 (4 rows 14.3 -> 13.6, 8 rows 14.3 -> 14.1)
+  //   N = 4096, K = 11008   8.6 -> 7.5 (8 rows 9.0 -> 8.6)
+  //   N = K = 4096          4.6 -> 4.3 (4 rows 5.2 -> 4.5, 8 rows 5.0 -> 4.7); blocks of 32 5.3 -> 5.1
+  //   N = 6144, K = 4096    5.6 -> 5.2 (4 rows 5.8 -> 5.2, 8 rows 6.3 -> 5.7); 8-bit 6.8 -> 6.7 (8 rows 7.7 -> 7.2)
+  //   raw 4-bit operands over more than 32 chunks on two-tile slabs, which ran sixteen wavefronts (no LDS form in
+  //   their 128 registers), with eight: N = K = 8192 8.8 -> 8.5 (4 rows 9.1 -> 8.7), N = 6144 8.0 -> 7.3,
+  //   N = 5120, K = 14336 12.0 -> 10.2, N = 8192, K = 28672 24.0 -> 23.4.
+  // Four-tile slabs do not gain (C2 without any activation load: 7.8 -> 7.7 us): there the weight loads dominate.
+  const bool few_rows = !(mnb_tuning_env("MNB_SKINNY_A4") && mnb_tuning_env("MNB_SKINNY_A4")[0] == '0');
+  if (few_rows && direct && pl.t <= 2 && M <= 8) {
+    const bool no_lds_form = L.bits == 4 && pl.nw == 16 && !up_front;  // (the general loop of sixteen 4-bit wavefronts)
+    if (pl.a_lds == 16) {
+      pl.a_lds = 8;  // (single-tile slabs, five to eight rows)
+    } else if (M <= 4) {
+      if (no_lds_form && pl.mode == 0) pl.nw = 8;
+      if (!(L.bits == 4 && pl.nw == 16 && !up_front)) pl.a_lds = 4;
+    } else if (!no_lds_form) {
+      pl.a_lds = 8;  // (two-tile slabs, five to eight rows)
+    }
+  }
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
   pl.phase_chunks = chunks < max_phase ? chunks : max_phase;
@@ -723,18 +767,18 @@ hipError_t launch_slab(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t 
   do {                                                              \
     if (pl.a_lds) {                                                 \
       if (cpw == 1)                                                 \
-        MNB_SLAB_LAUNCH(NW_, 1, true);                              \
+        MNB_SLAB_LAUNCH(NW_, 1, 16);                              \
       else if (cpw == 2)                                            \
-        MNB_SLAB_LAUNCH(NW_, 2, true);                              \
+        MNB_SLAB_LAUNCH(NW_, 2, 16);                              \
       else if constexpr (!(BITS == 4 && NW_ == 16))                 \
-        MNB_SLAB_LAUNCH(NW_, 0, true);                              \
+        MNB_SLAB_LAUNCH(NW_, 0, 16);                              \
     } else {                                                        \
       if (cpw == 1)                                                 \
-        MNB_SLAB_LAUNCH(NW_, 1, false);                             \
+        MNB_SLAB_LAUNCH(NW_, 1, 0);                             \
       else if (cpw == 2)                                            \
-        MNB_SLAB_LAUNCH(NW_, 2, false);                             \
+        MNB_SLAB_LAUNCH(NW_, 2, 0);                             \
       else if constexpr (!(MODE >= 2 && NW_ == 16))                 \
-        MNB_SLAB_LAUNCH(NW_, 0, false);                             \
+        MNB_SLAB_LAUNCH(NW_, 0, 0);                             \
     }                                                               \
   } while (0)
   switch (pl.nw) {
@@ -754,26 +798,45 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
     const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
     // not instantiated, never planned: LDS route in the general loop of four-tile slabs or of sixteen 4-bit wavefronts
     if (pl.a_lds && cpw == 0 && (T == 4 || (BITS == 4 && pl.nw == 16))) return hipErrorInvalidConfiguration;
+    if (pl.a_lds != 0 && pl.a_lds != 16 && T > 2) return hipErrorInvalidConfiguration;  // (four or eight rows: narrow slabs only)
     if (MODE >= 2 && cpw == 0 && pl.nw == 16) return hipErrorInvalidConfiguration;  // (nor the fp32-entry modes at all)
 #define MNB_SKINNY_LAUNCH(NW_, CPW_, LDS_) \
   mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_>                \
       <<<grid, dim3(NW_ * 64), pl.smem, s>>>(MNB_SKINNY_HOT_ARGS(p), p)
 #define MNB_SKINNY_CPW(NW_)                                         \
   do {                                                              \
-    if (pl.a_lds) {                                                 \
+    if (pl.a_lds == 4) {                                            \
+      if constexpr (T <= 2) {                                       \
+        if (cpw == 1)                                               \
+          MNB_SKINNY_LAUNCH(NW_, 1, 4);                             \
+        else if (cpw == 2)                                          \
+          MNB_SKINNY_LAUNCH(NW_, 2, 4);                             \
+        else if constexpr (!(BITS == 4 && NW_ == 16))               \
+          MNB_SKINNY_LAUNCH(NW_, 0, 4);                             \
+      }                                                             \
+    } else if (pl.a_lds == 8) {                                     \
+      if constexpr (T <= 2) {                                       \
+        if (cpw == 1)                                               \
+          MNB_SKINNY_LAUNCH(NW_, 1, 8);                             \
+        else if (cpw == 2)                                          \
+          MNB_SKINNY_LAUNCH(NW_, 2, 8);                             \
+        else if constexpr (!(BITS == 4 && NW_ == 16))               \
+          MNB_SKINNY_LAUNCH(NW_, 0, 8);                             \
+      }                                                             \
+    } else if (pl.a_lds) {                                          \
       if (cpw == 1)                                                 \
-        MNB_SKINNY_LAUNCH(NW_, 1, true);                            \
+        MNB_SKINNY_LAUNCH(NW_, 1, 16);                              \
       else if (cpw == 2)                                            \
-        MNB_SKINNY_LAUNCH(NW_, 2, true);                            \
+        MNB_SKINNY_LAUNCH(NW_, 2, 16);                              \
       else if constexpr (!(BITS == 4 && NW_ == 16) && T < 4)        \
-        MNB_SKINNY_LAUNCH(NW_, 0, true);                            \
+        MNB_SKINNY_LAUNCH(NW_, 0, 16);                              \
     } else {                                                        \
       if (cpw == 1)                                                 \
-        MNB_SKINNY_LAUNCH(NW_, 1, false);                           \
+        MNB_SKINNY_LAUNCH(NW_, 1, 0);                               \
       else if (cpw == 2)                                            \
-        MNB_SKINNY_LAUNCH(NW_, 2, false);                           \
+        MNB_SKINNY_LAUNCH(NW_, 2, 0);                               \
       else if constexpr (!(MODE >= 2 && NW_ == 16))                 \
-        MNB_SKINNY_LAUNCH(NW_, 0, false);                           \
+        MNB_SKINNY_LAUNCH(NW_, 0, 0);                               \
     }                                                               \
   } while (0)
     switch (pl.nw) {

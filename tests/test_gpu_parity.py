@@ -175,10 +175,10 @@ def test_decode_with_three_tile_slabs(oracle, bits, bs, zp, N, K, M):
 @pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (8, 64, True), (8, 128, False)])
 @pytest.mark.parametrize("N,K", [(100, 4096), (6144, 2048), (9000, 1024), (14400, 512), (200, 14336), (5200, 8320),
                                  (300, 4160)])
-@pytest.mark.parametrize("M", [5, 9, 16])
+@pytest.mark.parametrize("M", [5, 8, 9, 16])
 def test_decode_with_activations_through_lds(oracle, bits, bs, zp, N, K, M):
-    """More than four rows (single-tile slabs) or eight: the decode kernel reads its chunk of A row-contiguously and
-    passes it through LDS in a swizzled layout.  Shapes cover one, two and many chunks per wavefront (also unevenly
+    """More than four rows: the decode kernel reads its chunk of A row-contiguously and passes it through LDS in a
+    swizzled layout (eight rows of it up to M = 8 on single- and two-tile slabs, sixteen otherwise).  Shapes cover one, two and many chunks per wavefront (also unevenly
     many), slabs of one to four tiles, and long K on 4-bit weights (eight wavefronts); with unit-vector rows the
     product must return columns of W bit for bit, so a wrong piece, row or swizzle cannot hide in a tolerance."""
     c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + M)
@@ -186,6 +186,28 @@ def test_decode_with_activations_through_lds(oracle, bits, bs, zp, N, K, M):
     if N <= 300:
         rng = np.random.default_rng(M + K)
         ks = rng.choice(K, size=M, replace=False)
+        eye = np.zeros((M, K), np.float16)
+        eye[np.arange(M), ks] = 1
+        c0 = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + M)
+        w = oracle.C.dequantize(c0.B, c0.scales, c0.zero_points, N, K, bits, bs)
+        assert np.array_equal(_bits_view(run_case(c0, A=eye)), _bits_view(np.ascontiguousarray(w[:, ks].T)))
+
+
+@pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (4, 64, True), (8, 64, True), (8, 128, False),
+                                        (2, 128, True), (2, 64, False)])
+@pytest.mark.parametrize("N,K", [(100, 1024), (4096, 2048), (4090, 4096), (300, 14336), (200, 11008), (6144, 4096),
+                                 (6150, 8192), (5200, 2304), (260, 4352)])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+def test_decode_of_up_to_four_rows_on_narrow_slabs(oracle, bits, bs, zp, N, K, M):
+    """Up to four rows on single- and two-tile slabs (N < 12800): one load fetches a chunk of all four rows and LDS hands
+    the operands out (rows beyond M repeat row M - 1 and are never stored).  Shapes cover one, two and many chunks per
+    wavefront, uneven chunk counts, ragged N, both slab widths, the three weight widths and both dequantisation
+    modes; with unit-vector rows the product must return columns of W bit for bit, so a wrong row, piece or swizzle
+    cannot hide in a tolerance, and distinct unit vectors per row catch rows that were swapped or repeated."""
+    c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + M)
+    check_against_oracle(oracle, c, run_case(c))
+    if N <= 300 or K <= 2304:
+        ks = np.random.default_rng(M + K + N).choice(K, size=M, replace=False)
         eye = np.zeros((M, K), np.float16)
         eye[np.arange(M), ks] = 1
         c0 = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, seed=N + K + M)
