@@ -21,7 +21,9 @@ CSRC = PKG / "csrc"
 LIB = PKG / "libmnb_mi355x.so"
 OBJ_DIR = PKG / "build"
 
-SOURCES = ["mnb_api.hip", "mnb_pack.hip", "mnb_quant.hip", "mnb_gemv.hip", "mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_gemm_i8.hip", "mnb_gemm32.hip", "mnb_rows16_f32.hip", "mnb_fused.hip", "mnb_variant.hip"]
+# (the decode kernel's four translation units come first: they compile longest)
+SKINNY_UNITS = ["mnb_skinny_w4.hip", "mnb_skinny_w4zp.hip", "mnb_skinny_w8.hip", "mnb_skinny_w2.hip"]
+SOURCES = [*SKINNY_UNITS, "mnb_api.hip", "mnb_pack.hip", "mnb_quant.hip", "mnb_gemv.hip", "mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_gemm_i8.hip", "mnb_gemm32.hip", "mnb_rows16_f32.hip", "mnb_fused.hip", "mnb_variant.hip"]
 PROBE_LIB = PKG / "libmnb_probe.so"
 PROBE_SOURCES = ["mnb_probe.hip"]
 
@@ -43,7 +45,7 @@ def hipcc() -> str:
 # asked to have those preloaded into SGPRs at wavefront start (firmware without the feature runs the compatibility
 # prologue the compiler emits in front of the kernel, which loads them the usual way).
 _PRELOAD = ["-mllvm", "-amdgpu-kernarg-preload-count=14"]
-EXTRA_FLAGS = {"mnb_skinny.hip": _PRELOAD, "mnb_gemv.hip": _PRELOAD, "mnb_mid.hip": _PRELOAD}
+EXTRA_FLAGS = {**{u: _PRELOAD for u in SKINNY_UNITS}, "mnb_gemv.hip": _PRELOAD, "mnb_mid.hip": _PRELOAD}
 
 
 def _compile(src: str, extra=()) -> Path:
@@ -59,7 +61,7 @@ def _compile(src: str, extra=()) -> Path:
     return obj
 
 
-def build(force: bool = True, jobs: int = 4) -> Path:
+def build(force: bool = True, jobs: int = 6) -> Path:
     """Compiles every HIP source and links the shared library. Always recompiles when force is set."""
     srcs = [CSRC / s for s in SOURCES]
     hdrs = list(CSRC.glob("*.h")) + [PKG.parent / "include" / "mnb_mi355x.h"]

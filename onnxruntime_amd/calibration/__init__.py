@@ -13,6 +13,6 @@ from.  Nothing here is loaded by the operator: the product library has none of t
       ENV is KEY=VALUE[+KEY=VALUE...], empty for none; reports whether outputs are bit-identical to the first variant
   python -m onnxruntime_amd.calibration.run stamps LIB M N K BITS BLOCK ZP [COPIES]
       anatomy of a direct decode launch (M <= 16) from a library built with --tag stamps -D MNB_STAMPS --only
-      mnb_skinny.hip: every wavefront's readings of the 100 MHz counter at seven points of its life
+      mnb_skinny.hip (names the decode kernel's four translation units): every wavefront's readings of the 100 MHz counter at seven points of its life
 LIB is a path or the word `product`.
 """

@@ -16,11 +16,13 @@ def lib_path(tag: str = "") -> Path:
     return HERE / (f"libmnb_calibration_{tag}.so" if tag else "libmnb_calibration.so")
 
 
-def build(tag: str = "", defines=(), only=(), jobs: int = 4, force: bool = False) -> Path:
+def build(tag: str = "", defines=(), only=(), jobs: int = 6, force: bool = False) -> Path:
     OBJ_DIR.mkdir(exist_ok=True)
 
     def compile_one(src: str) -> str:
-        extra = [f"-D{d}" for d in defines] if (not only or src in only) else []
+        # (mnb_skinny.hip names the decode kernel as a whole: its kernels live in the units of build.SKINNY_UNITS)
+        named = not only or src in only or (src in B.SKINNY_UNITS and "mnb_skinny.hip" in only)
+        extra = [f"-D{d}" for d in defines] if named else []
         obj = OBJ_DIR / f"{src}.{tag if extra else 'hooks'}.o"
         if not force and not extra and obj.exists() and obj.stat().st_mtime >= max(
                 p.stat().st_mtime for p in [B.CSRC / src, *B.CSRC.glob("*.h"), B.PKG.parent / "include" / "mnb_mi355x.h"]):

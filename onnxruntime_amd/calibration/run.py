@@ -141,9 +141,12 @@ def stamps(argv):
     A HIP graph of COPIES launches over as many copies of the packed matrix is replayed; the readings are those of
     its last launch (100 MHz counter: 10 ns steps), printed relative to the first wavefront's entry."""
     lib = load(argv[0])
-    lib.MnbCalibrationReadStamps.restype = ctypes.c_int
-    lib.MnbCalibrationReadStamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
     M, N, K, bits, bs, zp = map(int, argv[1:7])
+    # the readings live in the translation unit that holds the kernels of the weight format
+    unit = {4: "w4zp" if zp else "w4", 8: "w8", 2: "w2"}[bits]
+    read_stamps = getattr(lib, "MnbCalibrationReadStamps_" + unit)
+    read_stamps.restype = ctypes.c_int
+    read_stamps.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
     copies = int(argv[7]) if len(argv) > 7 else 32
     call, _ = Problem(M, N, K, bits, bs, bool(zp), bias=False, copies=copies).caller(lib)
     print("kernel:", lib.MnbGemmKernelName(M, N, K, bits, bs, _lib.DTYPE_FLOAT16).decode(), flush=True)
@@ -164,7 +167,7 @@ def stamps(argv):
     print(f"{e0.elapsed_time(e1) / copies * 1e3:.2f} us per launch with the readings compiled in", flush=True)
     points, waves, groups = 8, 16, 4096
     buf = np.zeros(groups * waves * points, dtype=np.uint64)
-    assert lib.MnbCalibrationReadStamps(buf.ctypes.data_as(ctypes.c_void_p), buf.size) == 0
+    assert read_stamps(buf.ctypes.data_as(ctypes.c_void_p), buf.size) == 0
     t = buf.reshape(groups, waves, points).astype(np.int64)
     live = t[:, :, 0] != 0
     t0 = t[:, :, 0][live].min()

@@ -1,0 +1,8 @@
+// Decode kernel (mnb_skinny_kernels.hip.h): the kernels for 4-bit weights with zero points.
+#include "mnb_skinny_kernels.hip.h"
+
+hipError_t mnb_skinny_launch_w4zp(const void* params, const void* plan, hipStream_t s) {
+  return launch_zp<4, true>(*static_cast<const SkinnyParams*>(params), *static_cast<const SkinnyPlan*>(plan), s);
+}
+
+MNB_STAMPS_READER(MnbCalibrationReadStamps_w4zp)

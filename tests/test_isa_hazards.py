@@ -13,15 +13,30 @@ CSRC = Path(__file__).resolve().parents[1] / "onnxruntime_amd" / "csrc"
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 
-@pytest.mark.skipif(not Path(HIPCC).exists(), reason="hipcc not available")
-@pytest.mark.parametrize("source", ["mnb_skinny.hip", "mnb_mid.hip", "mnb_gemm256.hip", "mnb_rows16_f32.hip"])
-def test_no_early_read_of_mfma_results(source):
+SOURCES = ["mnb_skinny_w4.hip", "mnb_skinny_w4zp.hip", "mnb_skinny_w8.hip", "mnb_skinny_w2.hip", "mnb_mid.hip",
+           "mnb_gemm256.hip", "mnb_rows16_f32.hip"]
+
+
+@pytest.fixture(scope="module")
+def assembly():
+    """Every source compiled to assembly once, side by side (the decode kernel's four units take a minute or two
+    each)."""
+    from concurrent.futures import ThreadPoolExecutor
     from onnxruntime_amd.build import HIPCC_FLAGS
     with tempfile.TemporaryDirectory() as tmp:
-        out = Path(tmp) / (source + ".s")
-        subprocess.run([HIPCC, *HIPCC_FLAGS, "-S", "--cuda-device-only", str(CSRC / source), "-o", str(out)],
-                       check=True, capture_output=True, timeout=600)
-        findings = scan(out.read_text())
+        def compile_one(source):
+            out = Path(tmp) / (source + ".s")
+            subprocess.run([HIPCC, *HIPCC_FLAGS, "-S", "--cuda-device-only", str(CSRC / source), "-o", str(out)],
+                           check=True, capture_output=True, timeout=900)
+            return source, scan(out.read_text())
+        with ThreadPoolExecutor(max_workers=7) as ex:
+            yield dict(ex.map(compile_one, SOURCES))
+
+
+@pytest.mark.skipif(not Path(HIPCC).exists(), reason="hipcc not available")
+@pytest.mark.parametrize("source", SOURCES)
+def test_no_early_read_of_mfma_results(assembly, source):
+    findings = assembly[source]
     assert not findings, "\n".join(f"{f}: {w} wait states: {a} -> {b}" for f, w, a, b in findings[:10])
 
 
