@@ -542,17 +542,23 @@ def main() -> int:
     if not args.no_sizes:
         rows = []
         # (the 2-bit rows stream the copy of the weights in their own width: half the bytes of the 4-bit rows)
-        for label, bits, bs, shape in (("gate+up int4 bs128 zp", 4, 128, "gate_up"), ("gate+up int8 bs64 zp", 8, 64, "gate_up"),
-                                       ("gate+up int2 bs128 zp", 2, 128, "gate_up"),
-                                       ("configs[1] shape as int2 bs128 zp", 2, 128, None)):
+        # (the down rows run single-tile slabs, where the activations reach the operand registers through LDS: one load per
+        # chunk of up to four rows)
+        for label, bits, bs, shape, M5 in (("gate+up int4 bs128 zp", 4, 128, "gate_up", 1),
+                                           ("gate+up int8 bs64 zp", 8, 64, "gate_up", 1),
+                                           ("gate+up int2 bs128 zp", 2, 128, "gate_up", 1),
+                                           ("configs[1] shape as int2 bs128 zp", 2, 128, None, 1),
+                                           ("down int4 bs128 zp", 4, 128, "down", 1),
+                                           ("down int4 bs128 zp", 4, 128, "down", 4),
+                                           ("down int2 bs128 zp", 2, 128, "down", 1)):
             K5, N5 = synthetic.C5_SHAPES[shape] if shape else (c2.K, c2.N)
-            case = synthetic.make_case(1, N5, K5, bits, bs, np.float16, has_zp=True, seed=0)
-            copies = 8 if shape else 32  # distinct weights beyond the 256 MB Infinity Cache
+            case = synthetic.make_case(M5, N5, K5, bits, bs, np.float16, has_zp=True, seed=0)
+            copies = 8 if shape == "gate_up" else 32  # distinct weights beyond the 256 MB Infinity Cache
             p5 = Problem(case, copies, torch, _lib)
             g5 = graph_of(torch, p5.step)
             us5 = time_steps(torch, g5.replay, max(4, args.steps // 2), 2) / copies * 1e3
             gb5 = case.algorithmic_bytes() / (us5 * 1e-6) / 1e9
-            rows.append({"workload": f"{'BASELINE configs[4] ' if shape else ''}M=1 K={K5} N={N5} {label} fp16", "kernel": p5.kernel,
+            rows.append({"workload": f"{'BASELINE configs[4] ' if shape else ''}M={M5} K={K5} N={N5} {label} fp16", "kernel": p5.kernel,
                          "algorithmic_bytes_per_launch": case.algorithmic_bytes(), "us_per_launch": round(us5, 3),
                          "value": round(gb5, 1), "unit": "GB/s", "frac_of_hbm_peak": round(gb5 / HBM_PEAK_GBS, 4)})
             del g5, p5
