@@ -408,7 +408,7 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
       }
     }
     MNB_STAMP(3);
-  } else if constexpr (T <= 2) {
+  } else if constexpr (T <= 2 || (BITS == 4 && NW <= 8)) {
     // Two chunks in flight.  Loads under a run-time condition would leave the compiler unable to count the
     // outstanding loads at the join, and every wait of the loop would then be for all of them, the prefetch issued
     // a moment earlier included.  So the steady state and each possible tail are straight-line code, and the two
@@ -446,8 +446,11 @@ __device__ __forceinline__ void skinny_chunks(const SkinnyParams& p, unsigned ch
       run(R0, a0);
     }
   } else {
-    // Wide slabs keep the loop with conditional prefetches: the straight-line form needs 30-50 registers more
-    // there, which 16 wavefronts do not have (measured 11 % slower for T = 4; 2-9 % faster for T = 1, 2).
+    // Wide slabs keep the loop with conditional prefetches where registers are short: the straight-line form needs
+    // 30-50 registers more, which 16 wavefronts do not have (measured 11 % slower for T = 4; 2-9 % faster for
+    // T = 1, 2).  Workgroups of four or eight wavefronts have them: 4-bit weights gain 6-7 % there (N = 28672,
+    // K = 4096 14.6 -> 13.6 us at one row, 15.4 -> 14.5 at eight, blocks of 32 17.7 -> 16.7; N = 14336, K = 8192
+    // 13.5 -> 12.6 us), 8-bit weights lose 2-5 % (23.0 -> 23.5 us) and stay here.
     ChunkRegs<BITS, T> R0, R1;
     h8_t a0[NI], a1[NI];
     int c = wave;
