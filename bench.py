@@ -267,6 +267,12 @@ def main() -> int:
     g2hot = graph_of(torch, lambda: [p2.launch(0) for _ in range(LAYERS)])
     ms_hot = time_steps(torch, g2hot.replay, args.steps, args.warmup)
 
+    # the same chain four times over in one graph (128 launches): what a step loses to the hand-over from one graph
+    # replay to the next, which is not part of any launch (reported beside the headline)
+    g2long = graph_of(torch, lambda: [p2.launch(i % LAYERS) for i in range(4 * LAYERS)])
+    ms_long = time_steps(torch, g2long.replay, max(2, args.steps // 4), 1)
+    del g2long
+
     # and as two independent chains of 16: the head and tail of one launch overlap with its neighbour's streaming.
     # Reported beside the headline, never as the headline: `value` is the serialised chain.
     g2two = graph_of_chains(torch, p2.launch, LAYERS, 2)
@@ -295,6 +301,7 @@ def main() -> int:
             "prepack_ms_per_matrix": round(p2.prepack_ms, 3),
             "prepack_device_us_per_matrix": round(p2.prepack_device_us, 1),
             "us_per_launch_weights_in_infinity_cache": round(ms_hot * 1e3 / LAYERS, 3),
+            "us_per_launch_in_graphs_of_128_launches": round(ms_long * 1e3 / (4 * LAYERS), 3),
             "us_per_launch_as_two_independent_chains": round(ms_two * 1e3 / LAYERS, 3),
             "GBs_as_two_independent_chains": round(bytes_per_launch / (ms_two * 1e-3 / LAYERS) / 1e9, 1),
         },
@@ -555,8 +562,9 @@ def main() -> int:
             case = synthetic.make_case(M5, N5, K5, bits, bs, np.float16, has_zp=True, seed=0)
             copies = 8 if shape == "gate_up" else 32  # distinct weights beyond the 256 MB Infinity Cache
             p5 = Problem(case, copies, torch, _lib)
-            g5 = graph_of(torch, p5.step)
-            us5 = time_steps(torch, g5.replay, max(4, args.steps // 2), 2) / copies * 1e3
+            per_graph = max(copies, 32)  # (a graph replay hands over to the next in several microseconds: 32 launches share it)
+            g5 = graph_of(torch, lambda: [p5.launch(i % copies) for i in range(per_graph)])
+            us5 = time_steps(torch, g5.replay, max(4, args.steps // 2), 2) / per_graph * 1e3
             gb5 = case.algorithmic_bytes() / (us5 * 1e-6) / 1e9
             rows.append({"workload": f"{'BASELINE configs[4] ' if shape else ''}M={M5} K={K5} N={N5} {label} fp16", "kernel": p5.kernel,
                          "algorithmic_bytes_per_launch": case.algorithmic_bytes(), "us_per_launch": round(us5, 3),
@@ -718,11 +726,17 @@ def sweep(torch, _lib, synthetic):
     from onnxruntime_amd.synthetic import make_case
     rows = []
 
+    def copies_from_hbm(case):
+        """Distinct packed matrices whose total lies beyond twice the 256 MB Infinity Cache: every launch streams from HBM."""
+        return max(8, min(64, -(-600_000_000 // case.algorithmic_bytes())))
+
     def one(name, case, copies):
+        copies = copies or copies_from_hbm(case)
         p = Problem(case, copies, torch, _lib)
         if p.M <= 64:
-            g = graph_of(torch, p.step)
-            ms = time_steps(torch, g.replay, 20, 3) / copies
+            per_graph = max(copies, 32)  # (as in the decode legs: the hand-over between graph replays is shared by 32 launches)
+            g = graph_of(torch, lambda: [p.launch(i % copies) for i in range(per_graph)])
+            ms = time_steps(torch, g.replay, 20, 3) / per_graph
         else:
             ms = time_steps(torch, p.step, 20, 1, warm_ms=30.0) / copies
         gb = case.algorithmic_bytes() / (ms * 1e-3) / 1e9
@@ -740,14 +754,16 @@ def sweep(torch, _lib, synthetic):
                                  "next operand made between the matrix instructions")):
         assert probe.MnbProbeDequantMfma16(mode, 2, ctypes.byref(v)) == 0
         print(f"streaming mix probe: {v.value:6.2f} ns per step of two wavefronts on a SIMD, {what}", file=sys.stderr)
-    one("C1 fp32 M=1 4096x4096 bs32 zp", synthetic.config_c1(), 16)
+    c1 = synthetic.config_c1()
+    one("C1 fp32 M=1 4096x4096 bs32 zp", c1, copies_from_hbm(c1))
     for nm, (K, N) in synthetic.C3_SHAPES.items():
         for M in (1, 2, 4, 8, 16):
-            one(f"C3 {nm} M={M} K={K} N={N} bs64 zp", make_case(M, N, K, 4, 64, np.float16, has_zp=True), 16)
+            case = make_case(M, N, K, 4, 64, np.float16, has_zp=True)
+            one(f"C3 {nm} M={M} K={K} N={N} bs64 zp", case, copies_from_hbm(case))
     for bits, bs in ((4, 128), (8, 64)):
         for nm, (K, N) in synthetic.C5_SHAPES.items():
             for M in (1, 64, 256, 1024, 4096):
-                copies = 8 if M <= 64 else 1
+                copies = 0 if M <= 64 else 1  # (0: as many as stream from HBM, from the case itself)
                 one(f"C5 {nm} M={M} K={K} N={N} b{bits} bs{bs} zp",
                     make_case(M, N, K, bits, bs, np.float16, has_zp=True), copies)
     return rows
