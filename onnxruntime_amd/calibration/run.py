@@ -16,7 +16,7 @@ from onnxruntime_amd.synthetic import make_case
 ENV_KEYS = ("MNB_GEMM256_PLAN", "MNB_GEMM256_WAVES", "MNB_GEMM256_WAVE_ROWS", "MNB_GEMM32", "MNB_GEMV16_NW",
             "MNB_MID_DIRECT", "MNB_MID_MAX_M", "MNB_MID_PLAN", "MNB_MID_SHARED", "MNB_NATIVE_ROUTE", "MNB_ROWS16_M",
             "MNB_ROWS16_NW", "MNB_ROWS16_T", "MNB_SKINNY_A4", "MNB_SKINNY_ALDS_FROM", "MNB_SKINNY_MODE", "MNB_SKINNY_NW",
-            "MNB_SKINNY_PLAN", "MNB_SKINNY_WIDE_EXACT")
+            "MNB_SKINNY_PLAN", "MNB_SKINNY_T4LDS", "MNB_SKINNY_WIDE_EXACT")
 
 
 def load(path: str):

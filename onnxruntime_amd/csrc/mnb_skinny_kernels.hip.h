@@ -715,7 +715,18 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   // of 4-bit weights cannot hold in their 128 registers: those run with eight (K = 14336, M = 16: 20 -> 13 us).
   static const int a_lds_from = mnb_tuning_env("MNB_SKINNY_ALDS_FROM") ? atoi(mnb_tuning_env("MNB_SKINNY_ALDS_FROM")) : 5;
   const bool up_front = chunks == pl.nw || chunks == 2 * pl.nw;  // everything loaded before the first wait
-  pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4) ? 16 : 0;
+  // (four-tile slabs have an LDS form where all chunks are loaded up front, and in the straight-line chunk loop of
+  // 4-bit weights in workgroups of four or eight wavefronts)
+  const bool t4_hook = !(mnb_tuning_env("MNB_SKINNY_T4LDS") && mnb_tuning_env("MNB_SKINNY_T4LDS")[0] == '0');
+  // Long K on four-tile slabs from nine rows on (fp16 models): sixteen wavefronts run the loop with conditional
+  // prefetches, eight the straight-line one, with room for the LDS form.  N = 14336, K = 8192 at 12 / 16 rows
+  // 15.7 -> 14.2, 16.7 -> 14.6 us; K = 14336 at 16 rows 27.6 -> 23.2 us; exact operands (blocks of 64, N = 16384,
+  // K = 8192, 9 rows) 18.0 -> 16.7 us with eight wavefronts and 18.2 us with the LDS form on top, so they go without.
+  if (t4_hook && direct && L.bits == 4 && pl.t == 4 && pl.nw == 16 && !up_front && M >= 9 && pl.mode <= 1) pl.nw = 8;
+  // (at K = 4096 the form gains from thirteen rows on: N = 28672 at 9 / 12 / 16 rows 14.8 -> 15.2, 15.7 -> 15.5,
+  // 16.5 -> 15.9 us)
+  const bool t4_loop_lds = t4_hook && L.bits == 4 && pl.nw <= 8 && pl.mode == 0 && (M >= 13 || chunks > 32);
+  pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4 || t4_loop_lds) ? 16 : 0;
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
   // the fp32 scales and zero points of modes 2 to 4 do not fit the 128 registers of sixteen wavefronts in the general loop
   if (pl.mode >= 2 && !up_front && pl.nw == 16) pl.nw = 8;
@@ -751,6 +762,8 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   if (few_rows && direct && M <= 8 && !pl.a_lds) {
     const bool all_rows_of_c2 = mnb_tuning_env("MNB_SKINNY_A4") && mnb_tuning_env("MNB_SKINNY_A4")[0] == '3';
     if (pl.t == 3 && !(L.bits == 4 && pl.nw == 16 && !up_front)) pl.a_lds = M <= 4 ? 4 : 8;
+    // (in the chunk loop of four-tile slabs the forms for up to eight rows do not pay: N = 28672, K = 4096 at 2 / 4 / 6
+    // rows 13.8 -> 14.1, 14.1 -> 14.2, 14.1 -> 14.3 us, at 8 rows 14.7 -> 14.3 on one box and 14.6 -> 15.5 on another)
     if (pl.t == 4 && up_front && (M >= 2 || all_rows_of_c2)) pl.a_lds = M <= 4 ? 4 : 8;
   }
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
@@ -823,7 +836,8 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
   if (p.a_vec_ok) {
     const int cpw = (p.chunks == pl.nw) ? 1 : (p.chunks == 2 * pl.nw) ? 2 : 0;
     // not instantiated, never planned: LDS route in the general loop of four-tile slabs or of sixteen 4-bit wavefronts
-    if (pl.a_lds && cpw == 0 && (T == 4 || (BITS == 4 && pl.nw == 16))) return hipErrorInvalidConfiguration;
+    if (pl.a_lds && cpw == 0 && ((T == 4 && !(BITS == 4 && pl.nw <= 8)) || (BITS == 4 && pl.nw == 16)))
+      return hipErrorInvalidConfiguration;
     if (MODE >= 2 && cpw == 0 && pl.nw == 16) return hipErrorInvalidConfiguration;  // (nor the fp32-entry modes at all)
 #define MNB_SKINNY_LAUNCH(NW_, CPW_, LDS_) \
   mnb_skinny_direct_kernel<BITS, HAS_ZP, MODE, T, NW_, CPW_, LDS_>                \
@@ -835,7 +849,7 @@ hipError_t launch_t(const SkinnyParams& p, const SkinnyPlan& pl, hipStream_t s) 
         MNB_LDS_ROWS(MNB_SKINNY_LAUNCH, NW_, 1);                    \
       else if (cpw == 2)                                            \
         MNB_LDS_ROWS(MNB_SKINNY_LAUNCH, NW_, 2);                    \
-      else if constexpr (!(BITS == 4 && NW_ == 16) && T < 4)        \
+      else if constexpr (!(BITS == 4 && NW_ == 16) && (T < 4 || (BITS == 4 && NW_ <= 8))) \
         MNB_LDS_ROWS(MNB_SKINNY_LAUNCH, NW_, 0);                    \
     } else {                                                        \
       if (cpw == 1)                                                 \
