@@ -718,13 +718,16 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   // (four-tile slabs have an LDS form where all chunks are loaded up front, and in the straight-line chunk loop of
   // 4-bit weights in workgroups of four or eight wavefronts)
   const bool t4_hook = !(mnb_tuning_env("MNB_SKINNY_T4LDS") && mnb_tuning_env("MNB_SKINNY_T4LDS")[0] == '0');
-  // Long K on four-tile slabs from nine rows on (fp16 models): sixteen wavefronts run the loop with conditional
-  // prefetches, eight the straight-line one, with room for the LDS form.  N = 14336, K = 8192 at 12 / 16 rows
-  // 15.7 -> 14.2, 16.7 -> 14.6 us; K = 14336 at 16 rows 27.6 -> 23.2 us; exact operands (blocks of 64, N = 16384,
-  // K = 8192, 9 rows) 18.0 -> 16.7 us with eight wavefronts and 18.2 us with the LDS form on top, so they go without.
-  if (t4_hook && direct && L.bits == 4 && pl.t == 4 && pl.nw == 16 && !up_front && M >= 9 && pl.mode <= 1) pl.nw = 8;
-  // (at K = 4096 the form gains from thirteen rows on: N = 28672 at 9 / 12 / 16 rows 14.8 -> 15.2, 15.7 -> 15.5,
-  // 16.5 -> 15.9 us)
+  // K beyond 4096 on four-tile slabs of 4-bit weights (fp16 models): sixteen wavefronts run the loop with conditional
+  // prefetches, eight the straight-line one, with room for the LDS form.  Measured, N = 14336 unless noted:
+  //   nine rows and more: K = 8192 at 12 / 16 rows 15.7 -> 14.2, 16.7 -> 14.6 us; K = 14336 at 16 rows 27.6 -> 23.2 us;
+  //     exact operands (blocks of 64, N = 16384, K = 8192, 9 rows) 18.0 -> 16.7 us with eight wavefronts and 18.2 us
+  //     with the LDS form on top, so they go without it;
+  //   up to eight rows, exact operands (blocks of 32 and 64; N = 14336 and 16384, K = 8192, 11008, 14336, 1 / 4 / 8
+  //     rows: 36 cases): 2-9 % faster in every one (K = 8192, blocks of 64: 16.1 -> 14.8, 16.6 -> 15.2, 17.1 -> 16.0 us);
+  //   up to eight rows, raw operands below 64 chunks (K = 5120 ... 7168): 0-5 % (K = 6144: 10.7 -> 10.3 us, four rows
+  //     11.1 -> 10.5 us).
+  if (t4_hook && direct && L.bits == 4 && pl.t == 4 && pl.nw == 16 && !up_front && pl.mode <= 1) pl.nw = 8;
   const bool t4_loop_lds = t4_hook && L.bits == 4 && pl.nw <= 8 && pl.mode == 0 && (M >= 13 || chunks > 32);
   pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4 || t4_loop_lds) ? 16 : 0;
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
