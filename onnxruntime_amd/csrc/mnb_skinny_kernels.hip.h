@@ -728,6 +728,10 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   //   up to eight rows, raw operands below 64 chunks (K = 5120 ... 7168): 0-5 % (K = 6144: 10.7 -> 10.3 us, four rows
   //     11.1 -> 10.5 us).
   if (t4_hook && direct && L.bits == 4 && pl.t == 4 && pl.nw == 16 && !up_front && pl.mode <= 1) pl.nw = 8;
+  // Three-tile slabs likewise up to 64 chunks (N = 11008, K = 8192: 12.0 -> 11.0 us, four rows 12.8 -> 11.4, blocks of
+  // 64 15.8 -> 13.2; N = 12288, blocks of 32, four rows 17.0 -> 15.6; N = 9216, K = 6144 9.4 -> 8.5 us); beyond that
+  // sixteen wavefronts keep more chunks in flight (N = 12288, K = 14336: 19.6 us against 22.6 with eight).
+  if (t4_hook && direct && L.bits == 4 && pl.t == 3 && pl.nw == 16 && !up_front && pl.mode <= 1 && chunks <= 64) pl.nw = 8;
   const bool t4_loop_lds = t4_hook && L.bits == 4 && pl.nw <= 8 && pl.mode == 0 && (M >= 13 || chunks > 32);
   pl.a_lds = direct && M >= a_lds_from && (M >= 9 || pl.t == 1) && (up_front || pl.t < 4 || t4_loop_lds) ? 16 : 0;
   if (pl.a_lds && !up_front && pl.nw == 16 && L.bits == 4) pl.nw = 8;
