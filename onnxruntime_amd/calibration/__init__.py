@@ -5,7 +5,7 @@ from.  Nothing here is loaded by the operator: the product library has none of t
       builds onnxruntime_amd/calibration/libmnb_calibration[_T].so: every source with -DMNB_TUNING_HOOKS (the planners
       then read their decisions from the environment: the names in run.ENV_KEYS), the sources named by --only also with the -D switches
       (ablations: MNB_ABLATE_NO_LOADS, MNB_ABLATE_NO_MATH, MNB_ABLATE_NO_REDUCE; MNB_SPLIT_FENCES=1)
-  python -m onnxruntime_amd.calibration.run one  LIB M N K BITS BLOCK ZP [--launches N]
+  python -m onnxruntime_amd.calibration.run one  LIB M N K BITS BLOCK ZP [--launches N] [--copies C]
       launches one problem N times (for rocprofv3 --kernel-trace / --pmc); the variant comes from the environment
   python -m onnxruntime_amd.calibration.run ab   "LIB[;LIB...]" "ENV[;ENV...]" "M,N,K,BITS,BLOCK[,ZP[,COPIES]][;...]"
       alternating timing of libraries x environment variants on the same problems (HIP graphs of 20 launches, or of

@@ -79,7 +79,8 @@ def one(argv):
     lib = load(argv[0])
     M, N, K, bits, bs, zp = map(int, argv[1:7])
     launches = int(argv[argv.index("--launches") + 1]) if "--launches" in argv else 30
-    call, _ = Problem(M, N, K, bits, bs, bool(zp), bias=False).caller(lib)
+    copies = int(argv[argv.index("--copies") + 1]) if "--copies" in argv else 1   # > 1: weights stream from HBM
+    call, _ = Problem(M, N, K, bits, bs, bool(zp), bias=False, copies=copies).caller(lib)
     print("kernel:", lib.MnbGemmKernelName(M, N, K, bits, bs, _lib.DTYPE_FLOAT16).decode(), flush=True)
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < 0.05:   # the matrix-core clock settles
