@@ -44,6 +44,11 @@ CASES = [
     ((1, 14336, 4096, 4, 128, 16), ["MNB_SKINNY_PLAN=4,8", "MNB_SKINNY_PLAN=2,16", "MNB_SKINNY_PLAN=2,8"]),
     ((1, 6144, 4096, 4, 64, 16), ["MNB_SKINNY_PLAN=4,16", "MNB_SKINNY_PLAN=1,16", "MNB_SKINNY_PLAN=2,8"]),
     ((1, 14336, 4096, 2, 128, 16), ["MNB_SKINNY_PLAN=4,8", "MNB_SKINNY_PLAN=2,16", "MNB_SKINNY_MODE=1"]),
+    # few rows on single-tile slabs (activations through LDS or read straight from A), long K on four-tile slabs
+    # (eight wavefronts with the straight-line loop or sixteen with conditional prefetches), the gate+up decode plan
+    ((4, 4096, 14336, 4, 128, 32), ["MNB_SKINNY_A4=0", "MNB_SKINNY_PLAN=2,8", "MNB_SKINNY_PLAN=1,16"]),
+    ((16, 14336, 8192, 4, 128, 16), ["MNB_SKINNY_T4LDS=0", "MNB_SKINNY_PLAN=2,8"]),
+    ((1, 28672, 4096, 4, 128, 16), ["MNB_SKINNY_PLAN=4,8", "MNB_SKINNY_PLAN=2,8", "MNB_SKINNY_PLAN=2,4"]),
     ((64, 28672, 4096, 4, 128, 1), ["MNB_MID_SHARED=0", "MNB_MID_SHARED=0+MNB_MID_PLAN=4,4,8"]),
     ((64, 4096, 14336, 4, 128, 1), ["MNB_MID_PLAN=1,4,8", "MNB_MID_PLAN=2,2,4", "MNB_MID_SHARED=1"]),
     ((256, 6144, 4096, 4, 128, 1), ["MNB_MID_SHARED=0", "MNB_MID_MAX_M=64"]),
