@@ -691,13 +691,18 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
   //    4-bit operands at K = 4096 from four rows on: 0-10 % (at K = 8192 they lose 1-4 %);
   //  * raw 4-bit operands on slabs of two or four tiles with five to eight rows of A read straight from memory (two
   //    cache lines per row and load), and four-tile slabs with K >= 8192: 0-11 %, most with zero points.
+  //  * raw 4-bit operands with zero points on four-tile slabs, up to four rows: the corrections of the zero points
+  //    leave sixteen wavefronts short of registers, and eight run the straight-line chunk loop (K = 4096, blocks of
+  //    128: N = 14336 at 1 / 2 / 4 rows 8.5 -> 7.9, 8.3 -> 7.9, 8.4 -> 8.1 us; N = 16384 9.0 -> 8.3; blocks of 256,
+  //    N = 13312 8.0 -> 7.5; without zero points 7.8 / 7.9 us either way: the C2 plan stays).
   // Exact 4-bit operands (blocks of 32 and 64) on two-tile slabs do not gain.
   if (plan_override == nullptr && direct && pl.nw == 16 && pl.mode <= 1) {
     const bool raw4 = L.bits == 4 && pl.mode == 0;
     if (pl.t == 1 ? (M <= 8 || chunks <= 64)
                   : (pl.t == 2 && ((L.bits == 8 && chunks <= 64) || (raw4 && chunks <= 32))) ||
                         (pl.t == 3 && raw4 && chunks <= 32 && M >= 4) ||
-                        (raw4 && (pl.t == 2 || pl.t == 4) && M <= 8 && (M >= 5 || (pl.t == 4 && chunks >= 64))))
+                        (raw4 && (pl.t == 2 || pl.t == 4) && M <= 8 && (M >= 5 || (pl.t == 4 && chunks >= 64))) ||
+                        (raw4 && pl.t == 4 && L.has_zp && M <= 4))
       pl.nw = 8;
   }
   // 16-bit models on fp32 entries: only raw operands on single-tile slabs with up to four rows gain (N = K = 4096

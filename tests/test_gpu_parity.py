@@ -218,14 +218,16 @@ def test_decode_of_up_to_four_rows_on_narrow_slabs(oracle, bits, bs, zp, N, K, M
 @pytest.mark.parametrize("bits,bs,zp", [(4, 128, True), (4, 32, False), (8, 64, True), (8, 16, False)])
 @pytest.mark.parametrize("N,K,M", [(20480, 4096, 1), (20490, 4096, 8), (24576, 4096, 16), (28672, 4096, 1),
                                    (28672, 4096, 9), (33000, 8192, 3), (4096, 8192, 2), (4096, 11008, 8),
-                                   (14400, 8192, 9), (16000, 14336, 16), (14336, 8320, 12), (28672, 4096, 13)])
+                                   (14400, 8192, 9), (16000, 14336, 16), (14336, 8320, 12), (28672, 4096, 13),
+                                   (14336, 4096, 1), (13000, 4096, 4), (16384, 4096, 3)])
 def test_decode_with_more_slabs_than_compute_units(oracle, bits, bs, zp, N, K, M):
     """More four-tile slabs than compute units (N > 16384 on 256 units) with a K deep enough for sixteen wavefronts:
     the decode kernel runs smaller workgroups instead - two-tile slabs up to 1.6 slabs per unit, four or eight
     wavefronts with the general chunk loop beyond - and 8-bit weights over K >= 8192 run eight wavefronts on
     single-tile slabs.  The last four shapes are four-tile slabs whose 4-bit weights run the straight-line chunk loop in
     eight wavefronts from nine rows on (long K) with the activations through LDS (raw operands), also over an uneven
-    number of chunks.  Every row of Y against the oracle; unit-vector rows return columns of W bit for bit."""
+    number of chunks; the last three are raw 4-bit operands with zero points at K = 4096 and up to four rows, which run
+    eight wavefronts as well.  Every row of Y against the oracle; unit-vector rows return columns of W bit for bit."""
     c = make_case(M, N, K, bits, bs, np.float16, has_zp=zp, has_bias=True, seed=N + K + M)
     check_against_oracle(oracle, c, run_case(c))
     if K == 4096 and M >= 8:
