@@ -776,7 +776,9 @@ SkinnyPlan skinny_plan(const MnbLayout& L, int io, int64_t M, bool direct, int m
     if (pl.t == 3 && !(L.bits == 4 && pl.nw == 16 && !up_front)) pl.a_lds = M <= 4 ? 4 : 8;
     // (in the chunk loop of four-tile slabs the forms for up to eight rows do not pay: N = 28672, K = 4096 at 2 / 4 / 6
     // rows 13.8 -> 14.1, 14.1 -> 14.2, 14.1 -> 14.3 us, at 8 rows 14.7 -> 14.3 on one box and 14.6 -> 15.5 on another)
-    if (pl.t == 4 && up_front && (M >= 2 || all_rows_of_c2)) pl.a_lds = M <= 4 ? 4 : 8;
+    // (2-bit weights take eight activation loads per chunk when read straight from A: one row gains too - N = 14336,
+    // K = 4096, blocks of 128 7.4 -> 6.2 us, blocks of 256 6.8 -> 6.1, N = 16384 7.6 -> 6.5, K = 2048 5.6 -> 5.1)
+    if (pl.t == 4 && up_front && (M >= 2 || L.bits == 2 || all_rows_of_c2)) pl.a_lds = M <= 4 ? 4 : 8;
   }
   // LDS: staged A rows (<= 48 KiB per phase) and, afterwards, the reduction buffer (<= 64 KiB)
   const int max_phase = (48 * 1024 / 2 / pl.mtr - kLdsPad) / CK;  // >= 11 chunks for 16 rows
